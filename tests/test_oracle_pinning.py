@@ -1,0 +1,388 @@
+"""Pins the CPU oracle against things that are not the oracle: brute force,
+closed forms, library routines and special cases.  Each check is chosen so a
+plausible slip (dropped term, wrong sign/index, transposed operand, wrong tie
+order) fails it."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fm_oracle as O
+
+
+def g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ------------------------------------------------------------------ a14
+def test_init_centroids_reproducible():
+    a = O.init_centroids(8, 4)
+    ref = np.random.RandomState(42).randn(8, 4)
+    assert a.dtype == torch.float32
+    assert np.array_equal(a.numpy(), ref.astype(np.float32))
+    # first draw of MT19937(42) standard normal, a published constant
+    assert abs(ref[0, 0] - 0.4967141530112327) < 1e-15
+
+
+# ------------------------------------------------------------------ a1
+def test_project_tiny_hand_case():
+    A = torch.tensor([[[1., 2.], [0., -1.]]])          # H=1,C=2,d=2
+    K = torch.tensor([[[3., 4.], [5., 6.], [-1., 0.5]]])  # N=3
+    Y = O.project(A, K)
+    assert Y.shape == (1, 2, 3)
+    assert Y.tolist() == [[[11., 17., 0.], [-4., -6., -0.5]]]
+
+
+def test_project_matches_matmul():
+    A = torch.randn(3, 5, 16, generator=g(1))
+    K = torch.randn(3, 40, 16, generator=g(2))
+    Y = O.project(A, K)
+    ref = torch.matmul(A.double(), K.double().transpose(1, 2)).float()
+    assert torch.equal(Y, ref)
+    # a transposed operand would give another shape / values
+    assert Y.shape == (3, 5, 40)
+
+
+# ------------------------------------------------------------------ a2
+def brute_topz(row, Z):
+    """rank(i) = #{j : y_j > y_i or (y_j == y_i and j < i)}; take rank < Z."""
+    n = len(row)
+    rank = [sum(1 for j in range(n) if (row[j] > row[i]) or (row[j] == row[i] and j < i)) for i in range(n)]
+    out = [0] * min(Z, n)
+    for i, r in enumerate(rank):
+        if r < len(out):
+            out[r] = i
+    return out
+
+
+def test_argtopz_documented_tie_example():
+    y = torch.tensor([[1., 3., 3., 2., 3., 0., 3., 3.]])
+    assert O.argtopz(y, 3).tolist() == [[1, 2, 4]]
+
+
+def test_argtopz_brute_force_with_ties_zero_inf():
+    rng = np.random.default_rng(3)
+    for trial in range(20):
+        n = int(rng.integers(1, 40))
+        vals = rng.integers(-3, 4, size=n).astype(np.float32)      # heavy ties
+        if n > 4:
+            vals[rng.integers(n)] = np.inf
+            vals[rng.integers(n)] = -np.inf
+            vals[rng.integers(n)] = -0.0
+            vals[rng.integers(n)] = 0.0
+        Z = int(rng.integers(1, n + 3))                             # includes Z > N clamp
+        got = O.argtopz(torch.from_numpy(vals)[None], Z)[0].tolist()
+        assert got == brute_topz(vals.tolist(), Z), (vals, Z)
+
+
+def test_argtopz_neg_zero_equals_pos_zero():
+    y = torch.tensor([[-0.0, 0.0, -0.0, 0.0, -1.0]])
+    assert O.argtopz(y, 4).tolist() == [[0, 1, 2, 3]]
+
+
+def test_argtopz_invariants_random():
+    Y = torch.randn(4, 6, 257, generator=g(4))
+    Z = 31
+    idx = O.argtopz(Y, Z)
+    assert idx.shape == (4, 6, Z)
+    sel = torch.gather(Y, -1, idx)
+    assert (sel[..., :-1] >= sel[..., 1:]).all()                     # sorted descending
+    m = torch.ones_like(Y, dtype=torch.bool).scatter_(-1, idx, False)
+    assert (sel.min(-1)[0] >= Y.masked_fill(~m, -math.inf).max(-1)[0]).all()
+    assert all(len(set(r.tolist())) == Z for r in idx.reshape(-1, Z))
+    # agrees with torch.topk as a multiset of values
+    assert torch.equal(sel, torch.topk(Y, Z, dim=-1)[0])
+
+
+# ------------------------------------------------------------------ a3
+def test_qhash_first_max_and_brute_force():
+    A = torch.randn(2, 7, 8, generator=g(5))
+    q = torch.randn(2, 11, 8, generator=g(6))
+    A[0, 5] = A[0, 2]                                               # exact tie between buckets 2 and 5
+    h = O.qhash(A, q)
+    sc = O.qhash_scores(A, q)
+    for b in range(2):
+        for i in range(11):
+            row = sc[b, i].tolist()
+            first = min(j for j, x in enumerate(row) if x == max(row))
+            assert h[b, i].item() == first
+    assert not (h[0] == 5).any()
+    assert O.argmax_first(torch.tensor([[1., 5., 5., 2.]])).tolist() == [1]
+
+
+# ------------------------------------------------------------------ a5 / a16
+def test_group_queries_roundtrip_and_partition():
+    C = 9
+    qh = torch.randint(0, C, (3, 50), generator=g(7))
+    perm, gb, gc, go = O.group_queries(qh, C)
+    sorted_h = torch.gather(qh, 1, perm)
+    assert (sorted_h[:, 1:] >= sorted_h[:, :-1]).all()
+    # stable: equal hashes keep ascending original index
+    for b in range(3):
+        for c in range(C):
+            p = perm[b][sorted_h[b] == c]
+            assert (p[1:] > p[:-1]).all()
+    assert gc.sum().item() == qh.numel()
+    assert go.tolist() == [0] + np.cumsum(gc.numpy())[:-1].tolist()
+    flat = sorted_h.reshape(-1)
+    for z, n, o in zip(gb.tolist(), gc.tolist(), go.tolist()):
+        assert (flat[o:o + n] == z).all()
+    inv = torch.empty_like(perm)
+    inv.scatter_(1, perm, torch.arange(50).expand(3, -1))
+    assert torch.equal(torch.gather(sorted_h, 1, inv), qh)
+    bc = O.bin_counts(qh, C)
+    assert torch.equal(bc, torch.stack([torch.bincount(r, minlength=C) for r in qh]))
+
+
+def test_bucket_offsets_exclusive_scan():
+    c = torch.tensor([[2, 0, 3], [1, 4, 0]])
+    assert O.bucket_offsets(c).tolist() == [[0, 2, 2], [5, 6, 10]]
+
+
+def test_window_filter_counts_and_rebase():
+    kh = torch.tensor([[[0, 5, 9], [4, 3, 8]]])
+    flat, cnt = O.window_filter(kh, 4, 9)
+    assert cnt.tolist() == [[1, 2]]
+    assert flat.tolist() == [1, 0, 4]
+
+
+# ------------------------------------------------------------------ a6-a8
+def make_case(seed, B, S, N, C, Z, d, dtype=torch.float32, ragged=True):
+    gen = g(seed)
+    q = (torch.randn(B, S, d, generator=gen) * 0.5).to(dtype)
+    k = (torch.randn(B, N, d, generator=gen) * 0.5).to(dtype)
+    v = (torch.randn(B, N, d, generator=gen) * 0.5).to(dtype)
+    qh = torch.randint(0, C, (B, S), generator=gen)
+    kh = torch.topk(torch.rand(B, C, N, generator=gen), Z, dim=-1)[1]
+    if ragged:
+        mask = kh < int(N * 0.9)                                     # the reference test's window (tk:319-320)
+    else:
+        mask = torch.ones_like(kh, dtype=torch.bool)
+    return q, k, v, kh[mask], mask.sum(-1), qh
+
+
+def test_attention_two_formulations_agree():
+    q, k, v, kh, cnt, qh = make_case(20, 2, 24, 96, 8, 16, 16)
+    o1, l1 = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 16 ** -0.5)
+    o2, l2 = O.hashed_attention_dense_masked(q, k, v, kh, cnt, qh, 16 ** -0.5)
+    assert torch.allclose(o1, o2, atol=1e-6, rtol=0)
+    assert torch.allclose(l1, l2, atol=1e-6, rtol=0)
+    o3, l3 = O.hashed_attention_blocked(q, k, v, kh, cnt, qh, 16 ** -0.5, block_k=8)
+    assert torch.allclose(o1, o3, atol=1e-5, rtol=0)
+    assert torch.allclose(l1, l3, atol=1e-5, rtol=0)
+
+
+def test_attention_full_bucket_is_plain_softmax():
+    # C=1, Z=N: reduces to softmax(q K^T s) V and torch.logsumexp
+    B, S, N, d = 2, 5, 33, 8
+    gen = g(21)
+    q, k, v = (torch.randn(B, n, d, generator=gen) for n in (S, N, N))
+    kh = torch.stack([torch.randperm(N, generator=gen) for _ in range(B)]).reshape(-1)
+    cnt = torch.full((B, 1), N)
+    qh = torch.zeros(B, S, dtype=torch.long)
+    out, lse = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 0.3)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double(), scale=0.3)
+    assert torch.allclose(out.double(), ref, atol=1e-6)
+    assert torch.allclose(lse.double(), torch.logsumexp(q.double() @ k.double().transpose(1, 2) * 0.3, -1), atol=1e-6)
+
+
+def test_attention_single_key_bucket():
+    # Z=1: out = V[idx], lse = s * q.k
+    B, S, N, d, C = 1, 6, 10, 4, 3
+    gen = g(22)
+    q, k, v = (torch.randn(B, n, d, generator=gen) for n in (S, N, N))
+    kh = torch.tensor([7, 2, 5])
+    cnt = torch.ones(B, C, dtype=torch.long)
+    qh = torch.tensor([[0, 1, 2, 2, 1, 0]])
+    out, lse = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 0.7)
+    assert torch.allclose(out[0], v[0, kh[qh[0]]], atol=1e-6)
+    assert torch.allclose(lse[0], 0.7 * (q[0] * k[0, kh[qh[0]]]).sum(-1), atol=1e-6)
+
+
+def test_attention_empty_bucket_defined_behaviour():
+    B, S, N, d, C = 1, 4, 10, 4, 2
+    gen = g(23)
+    q, k, v = (torch.randn(B, n, d, generator=gen) for n in (S, N, N))
+    kh = torch.tensor([1, 2, 3])
+    cnt = torch.tensor([[3, 0]])
+    qh = torch.tensor([[0, 1, 1, 0]])
+    for fn in (O.hashed_attention_gather, O.hashed_attention_dense_masked, O.hashed_attention_blocked):
+        out, lse = fn(q, k, v, kh, cnt, qh, 0.5)
+        assert (out[0, 1] == 0).all() and (out[0, 2] == 0).all()
+        assert lse[0, 1].item() == torch.finfo(torch.float32).min
+        assert lse[0, 0].item() > -50
+
+
+def test_attention_invariants():
+    q, k, v, kh, cnt, qh = make_case(24, 2, 40, 128, 6, 20, 8, ragged=False)
+    s = 8 ** -0.5
+    out, lse = O.hashed_attention_gather(q, k, v, kh, cnt, qh, s)
+    Z = 20
+    table = kh.reshape(2, 6, Z)
+    for b in range(2):
+        for i in range(40):
+            idx = table[b, qh[b, i]]
+            sc = (k[b, idx] @ q[b, i]) * s
+            assert sc.max() - 1e-5 <= lse[b, i] <= sc.max() + math.log(Z) + 1e-5
+            vb = v[b, idx]
+            assert (out[b, i] <= vb.max(0)[0] + 1e-5).all() and (out[b, i] >= vb.min(0)[0] - 1e-5).all()
+    # permuting a bucket's list does not change the result
+    perm = torch.randperm(Z, generator=g(25))
+    out2, lse2 = O.hashed_attention_gather(q, k, v, table[:, :, perm].reshape(-1), cnt, qh, s)
+    assert torch.allclose(out, out2, atol=1e-6) and torch.allclose(lse, lse2, atol=1e-6)
+    # query-permutation equivariance
+    qp = torch.randperm(40, generator=g(26))
+    out3, lse3 = O.hashed_attention_gather(q[:, qp], k, v, kh, cnt, qh[:, qp], s)
+    assert torch.allclose(out[:, qp], out3, atol=1e-6) and torch.allclose(lse[:, qp], lse3, atol=1e-6)
+
+
+def test_ring_masked_forward_matches_ref_formulation():
+    C, H, G, S, N, Z, d = 5, 2, 2, 7, 30, 6, 8
+    gen = g(27)
+    q = torch.randn(1, H * G, S, d, generator=gen)
+    k = torch.randn(1, H, N, d, generator=gen)
+    v = torch.randn(1, H, N, d, generator=gen)
+    world = 2
+    kh = torch.topk(torch.rand(C, H, world * N, generator=gen), Z, dim=-1)[1]      # global indices
+    qh = torch.randint(0, C, (H, G, S), generator=gen)
+    for rank in range(world):
+        o1, l1 = O.ring_attention_masked_forward(kh, qh, q, k, v, 0.4, rank)
+        o2, l2 = O.ring_attention_masked_forward_ref(kh, qh, q, k, v, 0.4, rank)
+        ok = l1 > -1e30
+        assert torch.allclose(o1[ok], o2[ok], atol=1e-6)
+        assert torch.allclose(l1[ok], l2[ok], atol=1e-5)
+
+
+# ------------------------------------------------------------------ a10
+def test_merge_closed_form_and_first_call():
+    gen = g(30)
+    oa, ob = torch.randn(3, 5, 8, generator=gen), torch.randn(3, 5, 8, generator=gen)
+    la, lb = torch.randn(3, 5, generator=gen) * 4, torch.randn(3, 5, generator=gen) * 4
+    o0, l0 = O.update_out_and_lse(None, None, oa, la)
+    assert l0.shape == (3, 5, 1) and o0.dtype == torch.float32
+    o1, l1 = O.update_out_and_lse(o0.clone(), l0.clone(), ob, lb)
+    oc, lc = O.lse_merge_closed_form(oa, la, ob, lb)
+    assert torch.allclose(l1.squeeze(-1).double(), torch.logaddexp(la.double(), lb.double()), atol=1e-6)
+    assert torch.allclose(l1.squeeze(-1).double(), lc, atol=1e-6)
+    assert torch.allclose(o1.double(), oc, atol=1e-6)
+    # commutative
+    o2, l2 = O.update_out_and_lse(*O.update_out_and_lse(None, None, ob, lb), oa, la)
+    assert torch.allclose(o1, o2, atol=1e-6) and torch.allclose(l1, l2, atol=1e-6)
+
+
+def test_merge_split_test_equals_joint_softmax():
+    # attention over (bucket U local) == merge(attention over bucket, attention over local)
+    gen = g(31)
+    d, n1, n2 = 8, 13, 9
+    q = torch.randn(4, d, generator=gen)
+    k = torch.randn(n1 + n2, d, generator=gen)
+    v = torch.randn(n1 + n2, d, generator=gen)
+
+    def attn(ks, vs):
+        s = q.double() @ ks.double().T * 0.35
+        l = torch.logsumexp(s, -1)
+        return torch.exp(s - l[:, None]) @ vs.double(), l
+
+    oj, lj = attn(k, v)
+    o1, l1 = attn(k[:n1], v[:n1])
+    o2, l2 = attn(k[n1:], v[n1:])
+    om, lm = O.update_out_and_lse(*O.update_out_and_lse(None, None, o1.float(), l1.float()), o2.float(), l2.float())
+    assert torch.allclose(om.double(), oj, atol=1e-5)
+    assert torch.allclose(lm.squeeze(-1).double(), lj, atol=1e-5)
+
+
+def test_merge_with_empty_block_is_identity():
+    o = torch.randn(2, 3, 4, generator=g(32))
+    l = torch.randn(2, 3, generator=g(33))
+    o0, l0 = O.update_out_and_lse(None, None, o, l)
+    empty_lse = torch.full((2, 3), torch.finfo(torch.float32).min)
+    o1, l1 = O.update_out_and_lse(o0.clone(), l0.clone(), torch.zeros(2, 3, 4), empty_lse)
+    assert torch.equal(o1, o0) and torch.equal(l1, l0)
+
+
+# ------------------------------------------------------------------ a11
+def test_local_attention_vs_sdpa():
+    gen = g(40)
+    H, G, S, d = 2, 3, 17, 8
+    q = torch.randn(1, H * G, S, d, generator=gen)
+    k = torch.randn(1, H, S, d, generator=gen)
+    v = torch.randn(1, H, S, d, generator=gen)
+    out, lse = O.local_attention(q, k, v, 0.3, True)
+    kk = k.repeat_interleave(G, dim=1)
+    vv = v.repeat_interleave(G, dim=1)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double(), kk.double(), vv.double(), is_causal=True, scale=0.3)
+    assert torch.allclose(out.double(), ref, atol=1e-6)
+    s = (q.double() @ kk.double().transpose(-1, -2)) * 0.3
+    s = s.masked_fill(~torch.tril(torch.ones(S, S, dtype=torch.bool)), -math.inf)
+    assert torch.allclose(lse.double(), torch.logsumexp(s, -1), atol=1e-5)
+    # rectangular (decode): 1 query sees all L keys
+    q1 = q[:, :, -1:, :]
+    o1, l1 = O.local_attention(q1, k, v, 0.3, True)
+    ref1 = torch.nn.functional.scaled_dot_product_attention(q1.double(), kk.double(), vv.double(), scale=0.3)
+    assert torch.allclose(o1.double(), ref1, atol=1e-6)
+
+
+# ------------------------------------------------------------------ a12
+def test_compute_centroids_topk1_is_nearest_unit_key():
+    gen = g(50)
+    H, G, N, d, C = 2, 1, 30, 6, 4
+    kq = torch.randn(H * G, N, d, generator=gen)
+    cent = torch.randn(C, d, generator=gen)
+    A = O.compute_centroids(kq, cent, C, G, centroid_topk=1)
+    assert A.shape == (C, H, d)
+    xn = kq / kq.norm(dim=-1, keepdim=True)
+    for c in range(C):
+        for h in range(H):
+            best = torch.argmax(xn[h] @ cent[c])
+            assert torch.allclose(A[c, h], xn[h, best], atol=1e-6)
+
+
+def test_compute_centroids_loop_version():
+    gen = g(51)
+    H, G, N, d, C, topk = 2, 2, 25, 5, 3, 4
+    kq = torch.randn(H * G, N, d, generator=gen)
+    cent = torch.randn(C, d, generator=gen)
+    A = O.compute_centroids(kq, cent, C, G, centroid_topk=topk)
+    xn = (kq.double() / kq.double().norm(dim=-1, keepdim=True))
+    for c in range(C):
+        for h in range(H):
+            rows = []
+            for gq in range(G):
+                hg = h * G + gq                                       # head index = h*G + g (mem:228)
+                sc = xn[hg] @ cent[c].double()
+                order = sorted(range(N), key=lambda i: (-sc[i].item(), i))[:topk]
+                rows += [xn[hg, i] for i in order]
+            m = torch.stack(rows).mean(0)
+            m = m / m.norm()
+            assert torch.allclose(A[c, h].double(), m, atol=1e-6)
+    assert torch.allclose(A.norm(dim=-1), torch.ones(C, H), atol=1e-5)
+
+
+# ------------------------------------------------------------------ a13
+def test_kmeans_objective_monotone_and_unit_rows():
+    gen = g(60)
+    X = O.l2_normalize(torch.randn(400, 8, generator=gen))
+    init = O.l2_normalize(O.init_centroids(10, 8))
+    prev_obj = -1e9
+    cent = init.double()
+    for it in range(4):
+        labels = O.kmeans_assign(X, cent)
+        obj = (X.double() @ cent.T).max(-1)[0].sum().item()
+        assert obj >= prev_obj - 1e-9
+        prev_obj = obj
+        cent = O.kmeans_update(X, labels, cent)
+        assert torch.allclose(cent.norm(dim=-1), torch.ones(10, dtype=torch.float64), atol=1e-9)
+    c2, _ = O.kmeans_spherical(X, init, 4)
+    assert torch.allclose(c2, cent)
+
+
+def test_kmeans_update_brute_force_and_empty_cluster():
+    X = O.l2_normalize(torch.tensor([[1., 0.], [1., 1.], [0., 1.], [-1., 0.1]]))
+    prev = O.l2_normalize(torch.tensor([[1., 0.2], [0., 1.], [0., -1.]]))
+    labels = O.kmeans_assign(X, prev)
+    assert labels.tolist() == [0, 0, 1, 1]
+    new = O.kmeans_update(X, labels, prev)
+    m0 = (X[0] + X[1]).double() / 2
+    assert torch.allclose(new[0], m0 / m0.norm(), atol=1e-7)
+    assert torch.allclose(new[2], prev[2].double())                 # empty cluster keeps its centroid

@@ -1,0 +1,14 @@
+"""fast_memory_amd: MI355X (gfx950) implementation of the indexed-memory
+attention path of notbadai/fast_memory behind the reference's Python API.
+
+All compute runs in hand-written HIP kernels reached through the C ABI of
+``libfastmem.so`` (``include/fastmem.h``); PyTorch supplies device memory and
+streams.  There is no CPU path.
+"""
+from .hash_attention import attention_hash, attention_hash_varlen  # noqa: F401
+from .memory import (Memory, compute_centroids, fit_projection, init_centroids, kmeans_spherical,  # noqa: F401
+                     merge, ring_attention_masked_forward, update_out_and_lse)
+
+__all__ = ["attention_hash", "attention_hash_varlen", "Memory", "compute_centroids", "fit_projection",
+           "init_centroids", "kmeans_spherical", "merge", "ring_attention_masked_forward",
+           "update_out_and_lse"]

@@ -1,0 +1,125 @@
+// C entry points of the attention operators; picks the MFMA kernels for the
+// shapes they are built for and the generic kernels otherwise.
+#include "common.hpp"
+
+namespace fm {
+int hash_attn_generic(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                      const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                      const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
+                      float* lse, int Sq, int N, int d, int C, float sm_scale, int dtype,
+                      hipStream_t st);
+int local_attn_generic(const void* q, const void* k, const void* v, void* out, float* lse, int H,
+                       int G, int S, int L, int d, float sm_scale, int causal, int dtype,
+                       hipStream_t st);
+bool hash_attn_mfma_supported(int d, int dtype);
+int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                   const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                   const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
+                   float* lse, int Sq, int N, int d, int C, float sm_scale, hipStream_t st);
+bool local_attn_mfma_supported(int d, int dtype);
+int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
+                    int S, int L, int d, float sm_scale, int causal, hipStream_t st);
+
+// 0 = automatic, 1 = force the generic kernels (used by tests to compare paths)
+static int g_force_generic = 0;
+}  // namespace fm
+
+extern "C" void fm_debug_force_generic(int on) { fm::g_force_generic = on; }
+
+extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                                const int64_t* bucket_off, const int32_t* bucket_cnt,
+                                const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                                int64_t max_items, void* out, float* lse, int H, int Sq, int N,
+                                int d, int C, float sm_scale, int dtype, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
+             "fm_hash_attn_fwd: H=%d Sq=%d N=%d C=%d d=%d", H, Sq, N, C, d);
+  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_hash_attn_fwd: dtype=%d", dtype);
+  FM_REQUIRE(q && k && v && k_idx && bucket_off && bucket_cnt && q_perm && items && n_items && out &&
+                 lse,
+             FM_ERR_ARG, "fm_hash_attn_fwd: null pointer");
+  FM_REQUIRE(max_items >= 1 && max_items <= 0x7fffffffLL, FM_ERR_ARG,
+             "fm_hash_attn_fwd: max_items=%lld", (long long)max_items);
+  hipStream_t st = as_stream(stream);
+  if (!g_force_generic && hash_attn_mfma_supported(d, dtype))
+    return hash_attn_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items,
+                          out, lse, Sq, N, d, C, sm_scale, st);
+  return hash_attn_generic(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
+                           max_items, out, lse, Sq, N, d, C, sm_scale, dtype, st);
+}
+
+// workspace layout of the one-call operator
+namespace fm {
+struct VarlenWs {
+  size_t off_bucket_off, off_q_perm, off_bin_count, off_bin_off, off_items, off_n_items, off_group,
+      total;
+  int64_t max_items;
+};
+static VarlenWs varlen_layout(int H, int C, int Sq) {
+  VarlenWs w;
+  size_t o = 0;
+  auto take = [&](size_t bytes) {
+    size_t r = o;
+    o = align_up(o + bytes, 256);
+    return r;
+  };
+  w.max_items = fm_group_max_items(H, C, Sq);
+  w.off_bucket_off = take(size_t(H) * C * sizeof(int64_t));
+  w.off_q_perm = take(size_t(H) * Sq * sizeof(int32_t));
+  w.off_bin_count = take(size_t(H) * C * sizeof(int32_t));
+  w.off_bin_off = take(size_t(H) * C * sizeof(int32_t));
+  w.off_items = take(size_t(w.max_items) * sizeof(fm_item));
+  w.off_n_items = take(sizeof(int32_t));
+  w.off_group = take(fm_group_queries_workspace(H, C, Sq));
+  w.total = o;
+  return w;
+}
+}  // namespace fm
+
+extern "C" size_t fm_attention_hash_varlen_workspace(int H, int C, int Sq) {
+  if (H < 1 || C < 1 || Sq < 1) return 0;
+  return fm::varlen_layout(H, C, Sq).total;
+}
+
+extern "C" int fm_attention_hash_varlen(const void* q, const void* k, const void* v,
+                                        const int32_t* k_idx, const int32_t* bucket_cnt,
+                                        const int32_t* q_hash, void* out, float* lse, int H, int Sq,
+                                        int N, int d, int C, float sm_scale, int dtype, void* ws,
+                                        size_t ws_bytes, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1, FM_ERR_ARG,
+             "fm_attention_hash_varlen: H=%d Sq=%d N=%d C=%d", H, Sq, N, C);
+  FM_REQUIRE(ws && bucket_cnt && q_hash, FM_ERR_ARG, "fm_attention_hash_varlen: null pointer");
+  VarlenWs w = varlen_layout(H, C, Sq);
+  FM_REQUIRE(ws_bytes >= w.total, FM_ERR_WORKSPACE, "fm_attention_hash_varlen: workspace %zu < %zu",
+             ws_bytes, w.total);
+  char* base = static_cast<char*>(ws);
+  int64_t* bucket_off = reinterpret_cast<int64_t*>(base + w.off_bucket_off);
+  int32_t* q_perm = reinterpret_cast<int32_t*>(base + w.off_q_perm);
+  int32_t* bin_count = reinterpret_cast<int32_t*>(base + w.off_bin_count);
+  int32_t* bin_off = reinterpret_cast<int32_t*>(base + w.off_bin_off);
+  fm_item* items = reinterpret_cast<fm_item*>(base + w.off_items);
+  int32_t* n_items = reinterpret_cast<int32_t*>(base + w.off_n_items);
+  int rc = fm_bucket_offsets(bucket_cnt, int64_t(H) * C, bucket_off, stream);
+  if (rc) return rc;
+  rc = fm_group_queries(q_hash, H, C, Sq, q_perm, bin_count, bin_off, items, n_items, w.max_items,
+                        base + w.off_group, fm_group_queries_workspace(H, C, Sq), stream);
+  if (rc) return rc;
+  return fm_hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
+                          w.max_items, out, lse, H, Sq, N, d, C, sm_scale, dtype, stream);
+}
+
+extern "C" int fm_local_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                                 int H, int G, int S, int L, int d, float sm_scale, int causal,
+                                 int dtype, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && G >= 1 && S >= 1 && L >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
+             "fm_local_attn_fwd: H=%d G=%d S=%d L=%d d=%d", H, G, S, L, d);
+  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_local_attn_fwd: dtype=%d", dtype);
+  FM_REQUIRE(q && k && v && out && lse, FM_ERR_ARG, "fm_local_attn_fwd: null pointer");
+  FM_REQUIRE(int64_t(H) * G <= 65535, FM_ERR_UNSUPPORTED, "fm_local_attn_fwd: H*G > 65535");
+  hipStream_t st = as_stream(stream);
+  if (!g_force_generic && local_attn_mfma_supported(d, dtype))
+    return local_attn_mfma(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, st);
+  return local_attn_generic(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, dtype, st);
+}

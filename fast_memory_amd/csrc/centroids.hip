@@ -1,0 +1,152 @@
+// Construction of the projection matrix A: row normalisation and the
+// top-k-mean step of compute_centroids (memory.py:209-231, 256-258), and the
+// centroid update of spherical K-means (README.md:37-45).  Sums run in a fixed
+// order (member order of the index lists), so results do not depend on
+// scheduling.
+#include "common.hpp"
+
+namespace fm {
+
+__device__ __forceinline__ float block_sum_256(float v, float* sh) {
+  v = wave_sum(v);
+  if (lane_id() == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = sh[0] + sh[1] + sh[2] + sh[3];
+  __syncthreads();
+  return r;
+}
+
+// rows / max(||row||, eps); one wave per row
+template <typename T>
+__global__ __launch_bounds__(256) void l2_normalize_kernel(const T* __restrict__ X,
+                                                           T* __restrict__ Xn, int64_t rows, int d,
+                                                           float eps) {
+  const int64_t r = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const T* x = X + r * d;
+  float ss = 0.f;
+  for (int k = lane_id(); k < d; k += kWave) {
+    float v = Elem<T>::load(x + k);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.f / fmaxf(sqrtf(ss), eps);
+  for (int k = lane_id(); k < d; k += kWave) Elem<T>::store(Xn + r * d + k, Elem<T>::load(x + k) * inv);
+}
+
+// A[c,h,:] = normalise( mean over g<G, j<k of Xn[h*G+g, top_idx[c,h*G+g,j], :] )
+// one workgroup per (c,h); thread = dimension (d <= 256)
+template <typename T>
+__global__ __launch_bounds__(256) void topk_mean_kernel(const T* __restrict__ Xn,
+                                                        const int32_t* __restrict__ top_idx,
+                                                        T* __restrict__ A_out, int H, int G, int N,
+                                                        int k, int d, int normalize) {
+  __shared__ float sh[4];
+  const int c = blockIdx.x, h = blockIdx.y, t = threadIdx.x;
+  float acc = 0.f;
+  for (int g = 0; g < G; ++g) {
+    const int hg = h * G + g;
+    const int32_t* ti = top_idx + (int64_t(c) * H * G + hg) * k;
+    const T* xb = Xn + int64_t(hg) * N * d;
+    for (int j = 0; j < k; ++j) {
+      int row = min(max(ti[j], 0), N - 1);
+      if (t < d) acc += Elem<T>::load(xb + int64_t(row) * d + t);
+    }
+  }
+  acc /= float(G * k);
+  if (normalize) {
+    float ss = block_sum_256(t < d ? acc * acc : 0.f, sh);
+    acc /= sqrtf(ss);
+  }
+  if (t < d) Elem<T>::store(A_out + (int64_t(c) * H + h) * d + t, acc);
+}
+
+// cent[h,c,:] = normalise( mean of X[h, perm[...], :] over the cluster's members )
+// members = perm[seg_off[h,c] .. +seg_cnt[h,c]) (positions over the flattened
+// [H*N] sorted axis, values are row indices inside head h); empty -> prev.
+template <typename T>
+__global__ __launch_bounds__(256) void segment_mean_kernel(
+    const T* __restrict__ X, const int32_t* __restrict__ perm, const int32_t* __restrict__ seg_off,
+    const int32_t* __restrict__ seg_cnt, const T* __restrict__ prev, T* __restrict__ out, int C,
+    int N, int d) {
+  __shared__ float sh[4];
+  const int c = blockIdx.x, h = blockIdx.y, t = threadIdx.x;
+  const int64_t hc = int64_t(h) * C + c;
+  const int cnt = seg_cnt[hc];
+  const int32_t* mem = perm + seg_off[hc];
+  const T* xb = X + int64_t(h) * N * d;
+  float acc = 0.f;
+  for (int j = 0; j < cnt; ++j) {
+    int row = min(max(mem[j], 0), N - 1);
+    if (t < d) acc += Elem<T>::load(xb + int64_t(row) * d + t);
+  }
+  if (cnt > 0) acc /= float(cnt);
+  float ss = block_sum_256(t < d ? acc * acc : 0.f, sh);
+  float nrm = sqrtf(ss);
+  if (t < d) {
+    if (cnt == 0 || nrm < 1e-12f)
+      out[hc * d + t] = prev[hc * d + t];
+    else
+      Elem<T>::store(out + hc * d + t, acc / nrm);
+  }
+}
+
+}  // namespace fm
+
+extern "C" int fm_l2_normalize(const void* X, void* Xn, int64_t rows, int d, float eps, int dtype,
+                               void* stream) {
+  using namespace fm;
+  FM_REQUIRE(rows >= 0 && d >= 1, FM_ERR_ARG, "fm_l2_normalize: rows=%lld d=%d", (long long)rows, d);
+  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_l2_normalize: dtype=%d", dtype);
+  if (rows == 0) return FM_OK;
+  FM_REQUIRE(X && Xn, FM_ERR_ARG, "fm_l2_normalize: null pointer");
+  FM_REQUIRE(ceil_div(rows, 4) <= 0x7fffffffLL, FM_ERR_UNSUPPORTED, "fm_l2_normalize: too many rows");
+  dim3 grid = dim3(unsigned(ceil_div(rows, 4)));
+  if (dtype == FM_F32)
+    hipLaunchKernelGGL(l2_normalize_kernel<float>, grid, dim3(256), 0, as_stream(stream),
+                       (const float*)X, (float*)Xn, rows, d, eps);
+  else
+    hipLaunchKernelGGL(l2_normalize_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)X, (bf16_t*)Xn, rows, d, eps);
+  return launch_status("fm_l2_normalize");
+}
+
+extern "C" int fm_topk_mean(const void* Xn, const int32_t* top_idx, void* A_out, int C, int H, int G,
+                            int N, int k, int d, int normalize, int dtype, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(C >= 1 && H >= 1 && G >= 1 && N >= 1 && k >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
+             "fm_topk_mean: C=%d H=%d G=%d N=%d k=%d d=%d", C, H, G, N, k, d);
+  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_topk_mean: dtype=%d", dtype);
+  FM_REQUIRE(Xn && top_idx && A_out, FM_ERR_ARG, "fm_topk_mean: null pointer");
+  FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_topk_mean: H > 65535");
+  dim3 grid = dim3(unsigned(C), unsigned(H));
+  if (dtype == FM_F32)
+    hipLaunchKernelGGL(topk_mean_kernel<float>, grid, dim3(256), 0, as_stream(stream),
+                       (const float*)Xn, top_idx, (float*)A_out, H, G, N, k, d, normalize);
+  else
+    hipLaunchKernelGGL(topk_mean_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)Xn, top_idx, (bf16_t*)A_out, H, G, N, k, d, normalize);
+  return launch_status("fm_topk_mean");
+}
+
+extern "C" int fm_segment_mean(const void* X, const int32_t* perm, const int32_t* seg_off,
+                               const int32_t* seg_cnt, const void* prev, void* cent_out, int H,
+                               int C, int N, int d, int dtype, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
+             "fm_segment_mean: H=%d C=%d N=%d d=%d", H, C, N, d);
+  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_segment_mean: dtype=%d", dtype);
+  FM_REQUIRE(X && perm && seg_off && seg_cnt && prev && cent_out, FM_ERR_ARG,
+             "fm_segment_mean: null pointer");
+  FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_segment_mean: H > 65535");
+  dim3 grid = dim3(unsigned(C), unsigned(H));
+  if (dtype == FM_F32)
+    hipLaunchKernelGGL(segment_mean_kernel<float>, grid, dim3(256), 0, as_stream(stream),
+                       (const float*)X, perm, seg_off, seg_cnt, (const float*)prev,
+                       (float*)cent_out, C, N, d);
+  else
+    hipLaunchKernelGGL(segment_mean_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)X, perm, seg_off, seg_cnt, (const bf16_t*)prev,
+                       (bf16_t*)cent_out, C, N, d);
+  return launch_status("fm_segment_mean");
+}

@@ -1,0 +1,267 @@
+// Device-side bookkeeping around the attention kernel: prefix sums of bucket
+// sizes (triton_kernel.py:86-88), grouping of queries by (row, bucket)
+// (triton_kernel.py:75-88) with the occupancy histogram (memory.py:285-286),
+// and the window filter of bucket lists (memory.py:128-142).  All of it is
+// integer work with data-independent launch shapes: nothing here reads a count
+// back to the host.
+#include "common.hpp"
+
+namespace fm {
+
+constexpr int kGrpBlock = 256;  // queries per ranking block
+
+__global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+  int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  for (; i < n; i += stride) p[i] = v;
+}
+
+// Single-workgroup exclusive scan int32 -> int64 over n elements.
+__global__ __launch_bounds__(1024) void excl_scan_i32_i64_kernel(const int32_t* __restrict__ in,
+                                                                 int64_t n,
+                                                                 int64_t* __restrict__ out) {
+  __shared__ long long tmp[17];
+  long long carry = 0;
+  for (int64_t base = 0; base < n; base += 1024) {
+    int64_t i = base + threadIdx.x;
+    long long v = i < n ? in[i] : 0;
+    long long total;
+    long long ex = block_excl_scan_ll(v, tmp, &total);
+    if (i < n) out[i] = carry + ex;
+    carry += total;
+  }
+}
+
+// ---- grouping --------------------------------------------------------------
+// Pass 1: per block of 256 consecutive queries of a row, rank every query among
+// the earlier queries of the block with the same bucket; the first query of
+// each bucket in the block records the block's count for that bucket.
+// block_hist is [H][NB][C], zeroed beforehand.
+__global__ __launch_bounds__(kGrpBlock) void group_rank_kernel(const int32_t* __restrict__ q_hash,
+                                                               int C, int Sq, int NB,
+                                                               int32_t* __restrict__ block_hist,
+                                                               int32_t* __restrict__ bad) {
+  __shared__ int sh[kGrpBlock];
+  const int h = blockIdx.y, blk = blockIdx.x, t = threadIdx.x;
+  const int i = blk * kGrpBlock + t;
+  int b = -1;
+  if (i < Sq) {
+    b = q_hash[int64_t(h) * Sq + i];
+    if (b < 0 || b >= C) {
+      atomicOr(bad, 1);
+      b = -1;
+    }
+  }
+  sh[t] = b;
+  __syncthreads();
+  if (b < 0) return;
+  int before = 0, total = 0;
+  for (int j = 0; j < kGrpBlock; ++j) {
+    int e = (sh[j] == b);
+    total += e;
+    before += (j < t) ? e : 0;
+  }
+  if (before == 0) block_hist[(int64_t(h) * NB + blk) * C + b] = total;
+}
+
+// Pass 2: per (row, bucket) turn the per-block counts into exclusive offsets
+// over blocks; the total is the bucket's occupancy.
+__global__ void group_colscan_kernel(int32_t* __restrict__ block_hist, int H, int C, int NB,
+                                     int32_t* __restrict__ bin_count) {
+  int64_t g = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (g >= int64_t(H) * C) return;
+  int h = int(g / C), c = int(g - int64_t(h) * C);
+  int run = 0;
+  for (int blk = 0; blk < NB; ++blk) {
+    int64_t a = (int64_t(h) * NB + blk) * C + c;
+    int v = block_hist[a];
+    block_hist[a] = run;
+    run += v;
+  }
+  bin_count[g] = run;
+}
+
+// Pass 3: one workgroup scans the flattened [H*C] occupancies: bin_off = first
+// sorted position of the bucket; item offsets = prefix sum of ceil(cnt/QTILE);
+// items are written in (row, bucket, tile) order.
+__global__ __launch_bounds__(1024) void group_items_kernel(const int32_t* __restrict__ bin_count,
+                                                           int64_t n, int C,
+                                                           int32_t* __restrict__ bin_off,
+                                                           fm_item* __restrict__ items,
+                                                           int32_t* __restrict__ n_items,
+                                                           int64_t max_items) {
+  __shared__ int tmp[17];
+  int carry_q = 0, carry_i = 0;
+  for (int64_t base = 0; base < n; base += 1024) {
+    int64_t g = base + threadIdx.x;
+    int cnt = g < n ? bin_count[g] : 0;
+    int tiles = (cnt + FM_QTILE - 1) / FM_QTILE;
+    int tq, ti;
+    int exq = block_excl_scan(cnt, tmp, &tq);
+    int exi = block_excl_scan(tiles, tmp, &ti);
+    if (g < n) {
+      int off = carry_q + exq;
+      bin_off[g] = off;
+      int row = int(g / C), bucket = int(g - int64_t(row) * C);
+      for (int t = 0; t < tiles; ++t) {
+        int64_t slot = int64_t(carry_i) + exi + t;
+        if (slot < max_items) {
+          fm_item it;
+          it.row = row;
+          it.bucket = bucket;
+          it.q_start = off + t * FM_QTILE;
+          it.n_q = min(FM_QTILE, cnt - t * FM_QTILE);
+          items[slot] = it;
+        }
+      }
+    }
+    carry_q += tq;
+    carry_i += ti;
+  }
+  if (threadIdx.x == 0) *n_items = int32_t(min(int64_t(carry_i), max_items));
+}
+
+// Pass 4: scatter.  position = bucket start + queries of the bucket in earlier
+// blocks + rank inside the block  => stable ascending order.
+__global__ __launch_bounds__(kGrpBlock) void group_scatter_kernel(
+    const int32_t* __restrict__ q_hash, int C, int Sq, int NB,
+    const int32_t* __restrict__ block_hist, const int32_t* __restrict__ bin_off,
+    int32_t* __restrict__ q_perm) {
+  __shared__ int sh[kGrpBlock];
+  const int h = blockIdx.y, blk = blockIdx.x, t = threadIdx.x;
+  const int i = blk * kGrpBlock + t;
+  int b = -1;
+  if (i < Sq) {
+    b = q_hash[int64_t(h) * Sq + i];
+    if (b < 0 || b >= C) b = -1;
+  }
+  sh[t] = b;
+  __syncthreads();
+  if (b < 0) return;
+  int before = 0;
+  for (int j = 0; j < t; ++j) before += (sh[j] == b);
+  int pos = bin_off[int64_t(h) * C + b] + block_hist[(int64_t(h) * NB + blk) * C + b] + before;
+  q_perm[pos] = i;  // pos runs over the flattened [H*Sq] sorted axis
+}
+
+// ---- window filter ----------------------------------------------------------
+__global__ __launch_bounds__(256) void window_count_kernel(const int32_t* __restrict__ idx_in,
+                                                           int64_t nb, int Z, int64_t lo,
+                                                           int64_t hi, int32_t* __restrict__ cnt) {
+  int64_t b = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (b >= nb) return;
+  const int32_t* p = idx_in + b * Z;
+  int c = 0;
+  for (int j = lane_id(); j < Z; j += kWave) {
+    int64_t v = p[j];
+    c += (v >= lo && v < hi);
+  }
+  c = wave_sum_i(c);
+  if (lane_id() == 0) cnt[b] = c;
+}
+
+__global__ __launch_bounds__(256) void window_compact_kernel(const int32_t* __restrict__ idx_in,
+                                                             int64_t nb, int Z, int64_t lo,
+                                                             int64_t hi,
+                                                             const int64_t* __restrict__ off,
+                                                             int32_t* __restrict__ idx_out) {
+  int64_t b = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (b >= nb) return;
+  const int32_t* p = idx_in + b * Z;
+  int32_t* o = idx_out + off[b];
+  int base = 0;
+  const int l = lane_id();
+  for (int j0 = 0; j0 < Z; j0 += kWave) {  // order inside the bucket is preserved
+    int j = j0 + l;
+    int64_t v = j < Z ? int64_t(p[j]) : -1;
+    bool keep = (j < Z) && v >= lo && v < hi;
+    unsigned long long m = __ballot(keep);
+    int rank = __popcll(m & ((1ull << l) - 1ull));
+    if (keep) o[base + rank] = int32_t(v - lo);
+    base += __popcll(m);
+  }
+}
+
+static int launch_fill(int32_t* p, int64_t n, int32_t v, hipStream_t st) {
+  if (n <= 0) return FM_OK;
+  unsigned blocks = unsigned(std::min<int64_t>(ceil_div(n, 256), 4096));
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(blocks), dim3(256), 0, st, p, n, v);
+  return launch_status("fill");
+}
+
+}  // namespace fm
+
+extern "C" int fm_bucket_offsets(const int32_t* cnt, int64_t n, int64_t* off_out, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(n >= 0, FM_ERR_ARG, "fm_bucket_offsets: n=%lld", (long long)n);
+  if (n == 0) return FM_OK;
+  FM_REQUIRE(cnt && off_out, FM_ERR_ARG, "fm_bucket_offsets: null pointer");
+  hipLaunchKernelGGL(excl_scan_i32_i64_kernel, dim3(1), dim3(1024), 0, as_stream(stream), cnt, n,
+                     off_out);
+  return launch_status("fm_bucket_offsets");
+}
+
+extern "C" int64_t fm_group_max_items(int H, int C, int Sq) {
+  // sum over buckets of ceil(cnt/QTILE) <= #non-empty buckets + Sq/QTILE per row
+  int64_t nonempty = C < Sq ? C : Sq;
+  return int64_t(H) * (nonempty + Sq / FM_QTILE) + 1;
+}
+
+extern "C" size_t fm_group_queries_workspace(int H, int C, int Sq) {
+  int64_t NB = fm::ceil_div(Sq, fm::kGrpBlock);
+  return fm::align_up(size_t(H) * size_t(NB) * size_t(C) * sizeof(int32_t), 256) + 256;
+}
+
+extern "C" int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int32_t* q_perm,
+                                int32_t* bin_count, int32_t* bin_off, fm_item* items,
+                                int32_t* n_items, int64_t max_items, void* ws, size_t ws_bytes,
+                                void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && C >= 1 && Sq >= 1, FM_ERR_ARG, "fm_group_queries: H=%d C=%d Sq=%d", H, C, Sq);
+  FM_REQUIRE(q_hash && q_perm && bin_count && bin_off && items && n_items && ws, FM_ERR_ARG,
+             "fm_group_queries: null pointer");
+  FM_REQUIRE(int64_t(H) * Sq <= 0x7fffffffLL && int64_t(H) * C <= 0x7fffffffLL, FM_ERR_UNSUPPORTED,
+             "fm_group_queries: H*Sq or H*C exceeds int32");
+  FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_group_queries: H=%d > 65535", H);
+  FM_REQUIRE(max_items >= fm_group_max_items(H, C, Sq), FM_ERR_ARG,
+             "fm_group_queries: max_items=%lld < %lld", (long long)max_items,
+             (long long)fm_group_max_items(H, C, Sq));
+  FM_REQUIRE(ws_bytes >= fm_group_queries_workspace(H, C, Sq), FM_ERR_WORKSPACE,
+             "fm_group_queries: workspace %zu < %zu", ws_bytes, fm_group_queries_workspace(H, C, Sq));
+  hipStream_t st = as_stream(stream);
+  const int NB = int(ceil_div(Sq, kGrpBlock));
+  int32_t* block_hist = static_cast<int32_t*>(ws);
+  int32_t* bad = block_hist + int64_t(H) * NB * C;  // one flag word after the table (inside the +256)
+  int rc = launch_fill(block_hist, int64_t(H) * NB * C + 1, 0, st);
+  if (rc) return rc;
+  hipLaunchKernelGGL(group_rank_kernel, dim3(NB, H), dim3(kGrpBlock), 0, st, q_hash, C, Sq, NB,
+                     block_hist, bad);
+  hipLaunchKernelGGL(group_colscan_kernel, dim3(unsigned(ceil_div(int64_t(H) * C, 256))), dim3(256),
+                     0, st, block_hist, H, C, NB, bin_count);
+  hipLaunchKernelGGL(group_items_kernel, dim3(1), dim3(1024), 0, st, bin_count, int64_t(H) * C, C,
+                     bin_off, items, n_items, max_items);
+  hipLaunchKernelGGL(group_scatter_kernel, dim3(NB, H), dim3(kGrpBlock), 0, st, q_hash, C, Sq, NB,
+                     block_hist, bin_off, q_perm);
+  return launch_status("fm_group_queries");
+}
+
+extern "C" size_t fm_window_filter_workspace(int64_t) { return 0; }
+
+extern "C" int fm_window_filter(const int32_t* idx_in, int64_t nb, int Z, int64_t lo, int64_t hi,
+                                int32_t* idx_out, int32_t* cnt_out, int64_t* off_out, void* ws,
+                                size_t ws_bytes, void* stream) {
+  using namespace fm;
+  (void)ws;
+  (void)ws_bytes;
+  FM_REQUIRE(nb >= 0 && Z >= 1, FM_ERR_ARG, "fm_window_filter: nb=%lld Z=%d", (long long)nb, Z);
+  if (nb == 0) return FM_OK;
+  FM_REQUIRE(idx_in && idx_out && cnt_out && off_out, FM_ERR_ARG, "fm_window_filter: null pointer");
+  hipStream_t st = as_stream(stream);
+  unsigned blocks = unsigned(ceil_div(nb, 4));
+  hipLaunchKernelGGL(window_count_kernel, dim3(blocks), dim3(256), 0, st, idx_in, nb, Z, lo, hi,
+                     cnt_out);
+  hipLaunchKernelGGL(excl_scan_i32_i64_kernel, dim3(1), dim3(1024), 0, st, cnt_out, nb, off_out);
+  hipLaunchKernelGGL(window_compact_kernel, dim3(blocks), dim3(256), 0, st, idx_in, nb, Z, lo, hi,
+                     off_out, idx_out);
+  return launch_status("fm_window_filter");
+}

@@ -1,0 +1,282 @@
+// Projection Y = A.K^T (memory.py:261, triton_kernel.py:277) and query hashing
+// argmax_c A.q (memory.py:281-283, triton_kernel.py:280-281).
+#include "common.hpp"
+#include "mfma_tile.hpp"
+
+namespace fm {
+
+// ---------------------------------------------------------------------------
+// bf16 projection on MFMA: one workgroup = 128 buckets x 128 keys, the whole
+// contraction (d <= 256) staged once in LDS, four waves in a 2x2 grid of 64x64
+// sub-tiles, each 2x2 MFMA 32x32x16 tiles.  Lanes run along the key axis in
+// the accumulator layout, so stores are 128-byte segments of a Y row.
+// Bound: HBM write of Y (4 B per multiply-add column of 2*d flops).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void project_bf16_kernel(const bf16_t* __restrict__ A,
+                                                           const bf16_t* __restrict__ K,
+                                                           float* __restrict__ Y, int C, int N,
+                                                           int d, int64_t ldy) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int lds_ld = d + 8;  // bf16 elements per staged row (16 B pad: conflict-free b128 reads)
+  bf16_t* sA = reinterpret_cast<bf16_t*>(smem);
+  bf16_t* sB = sA + 128 * lds_ld;
+  const int h = blockIdx.z;
+  const int c0 = blockIdx.y * 128;
+  const int n0 = blockIdx.x * 128;
+  const bf16_t* Ah = A + int64_t(h) * C * d;
+  const bf16_t* Kh = K + int64_t(h) * N * d;
+  stage_rows_bf16(sA, lds_ld, Ah, c0, C, d, 128);
+  stage_rows_bf16(sB, lds_ld, Kh, n0, N, d, 128);
+  __syncthreads();
+  const int w = threadIdx.x >> 6, l = lane_id();
+  const int wm = w >> 1, wn = w & 1;
+  f32x16 acc[2][2];
+  mfma_tile_64x64(sA + (wm * 64) * lds_ld, sB + (wn * 64) * lds_ld, lds_ld, d, acc);
+  float* Yh = Y + int64_t(h) * C * ldy;
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni) {
+      int n = n0 + wn * 64 + ni * 32 + (l & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int c = c0 + wm * 64 + mi * 32 + acc_row_32(r, l);
+        if (c < C && n < N) Yh[int64_t(c) * ldy + n] = acc[mi][ni][r];
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Generic projection (any d <= 256, fp32 or bf16 storage, fp32 FMA chain over
+// k = 0..d-1).  64 keys staged in LDS per workgroup; lane = key, waves stride
+// over buckets.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void project_generic_kernel(const T* __restrict__ A,
+                                                              const T* __restrict__ K,
+                                                              float* __restrict__ Y, int C, int N,
+                                                              int d, int64_t ldy) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* sK = reinterpret_cast<float*>(smem);  // [64][d+1]
+  const int ld = d + 1;
+  const int h = blockIdx.y;
+  const int n0 = blockIdx.x * 64;
+  const T* Kh = K + int64_t(h) * N * d;
+  const T* Ah = A + int64_t(h) * C * d;
+  for (int e = threadIdx.x; e < 64 * d; e += 256) {
+    int r = e / d, k = e - r * d;
+    int n = n0 + r;
+    sK[r * ld + k] = n < N ? Elem<T>::load(Kh + int64_t(n) * d + k) : 0.f;
+  }
+  __syncthreads();
+  const int w = threadIdx.x >> 6, l = lane_id();
+  const int n = n0 + l;
+  float* Yh = Y + int64_t(h) * C * ldy;
+  for (int c = w; c < C; c += 4) {
+    const T* a = Ah + int64_t(c) * d;
+    float s = 0.f;
+    for (int k = 0; k < d; ++k) s = fmaf(Elem<T>::load(a + k), sK[l * ld + k], s);
+    if (n < N) Yh[int64_t(c) * ldy + n] = s;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Generic query hash: 64 queries staged in LDS, lane = query, each wave scans a
+// quarter of the buckets keeping (best score, first index), waves combined with
+// the same rule: larger score wins, equal scores keep the lower bucket.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void qhash_generic_kernel(const T* __restrict__ A,
+                                                            const T* __restrict__ q,
+                                                            int32_t* __restrict__ hash_out,
+                                                            float* __restrict__ scores_out, int C,
+                                                            int Sq, int d) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* sQ = reinterpret_cast<float*>(smem);  // [64][d+1]
+  __shared__ float s_best[4][64];
+  __shared__ int s_idx[4][64];
+  const int ld = d + 1;
+  const int h = blockIdx.y;
+  const int i0 = blockIdx.x * 64;
+  const T* qh = q + int64_t(h) * Sq * d;
+  const T* Ah = A + int64_t(h) * C * d;
+  for (int e = threadIdx.x; e < 64 * d; e += 256) {
+    int r = e / d, k = e - r * d;
+    int i = i0 + r;
+    sQ[r * ld + k] = i < Sq ? Elem<T>::load(qh + int64_t(i) * d + k) : 0.f;
+  }
+  __syncthreads();
+  const int w = threadIdx.x >> 6, l = lane_id();
+  const int i = i0 + l;
+  const int per = (C + 3) / 4;
+  const int cb = w * per, ce = min(C, cb + per);
+  float best = -INFINITY;
+  int besti = 0x7fffffff;
+  for (int c = cb; c < ce; ++c) {
+    const T* a = Ah + int64_t(c) * d;
+    float s = 0.f;
+    for (int k = 0; k < d; ++k) s = fmaf(Elem<T>::load(a + k), sQ[l * ld + k], s);
+    if (scores_out && i < Sq) scores_out[(int64_t(h) * Sq + i) * C + c] = s;
+    if (besti == 0x7fffffff || s > best) {
+      best = s;
+      besti = c;
+    }
+  }
+  s_best[w][l] = best;
+  s_idx[w][l] = besti;
+  __syncthreads();
+  if (w == 0 && i < Sq) {
+    for (int ww = 1; ww < 4; ++ww) {
+      float b = s_best[ww][l];
+      int bi = s_idx[ww][l];
+      if (bi != 0x7fffffff && (besti == 0x7fffffff || b > best)) {  // later waves hold higher buckets
+        best = b;
+        besti = bi;
+      }
+    }
+    hash_out[int64_t(h) * Sq + i] = besti;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// bf16 query hash on MFMA: workgroup = 128 queries of one KV head; loops over
+// bucket tiles of 128 staged in LDS; accumulator layout puts one query per lane
+// column, so the running (max, first index) is kept per lane without shuffles
+// and combined across the two lane halves and the two bucket-side waves at the
+// end.  Scores are the same MFMA sums fm_project would produce for these rows.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void qhash_bf16_kernel(const bf16_t* __restrict__ A,
+                                                         const bf16_t* __restrict__ q,
+                                                         int32_t* __restrict__ hash_out,
+                                                         float* __restrict__ scores_out, int C,
+                                                         int Sq, int d) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int lds_ld = d + 8;
+  bf16_t* sA = reinterpret_cast<bf16_t*>(smem);  // bucket tile (M side)
+  bf16_t* sB = sA + 128 * lds_ld;                // query tile  (N side)
+  __shared__ float s_best[2][128];
+  __shared__ int s_idx[2][128];
+  const int h = blockIdx.y;
+  const int i0 = blockIdx.x * 128;
+  const bf16_t* Ah = A + int64_t(h) * C * d;
+  const bf16_t* qh = q + int64_t(h) * Sq * d;
+  const int w = threadIdx.x >> 6, l = lane_id();
+  const int wm = w >> 1, wn = w & 1;
+  stage_rows_bf16(sB, lds_ld, qh, i0, Sq, d, 128);
+  float best[2] = {-INFINITY, -INFINITY};
+  int besti[2] = {0x7fffffff, 0x7fffffff};
+  for (int c0 = 0; c0 < C; c0 += 128) {
+    __syncthreads();  // previous tile consumed (and sB staged on the first trip)
+    stage_rows_bf16(sA, lds_ld, Ah, c0, C, d, 128);
+    __syncthreads();
+    f32x16 acc[2][2];
+    mfma_tile_64x64(sA + (wm * 64) * lds_ld, sB + (wn * 64) * lds_ld, lds_ld, d, acc);
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni) {
+      int i = i0 + wn * 64 + ni * 32 + (l & 31);
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {  // rows ascend with r inside a tile
+          int c = c0 + wm * 64 + mi * 32 + acc_row_32(r, l);
+          float s = acc[mi][ni][r];
+          if (c < C) {
+            if (scores_out && i < Sq) scores_out[(int64_t(h) * Sq + i) * C + c] = s;
+            if (besti[ni] == 0x7fffffff || s > best[ni] || (s == best[ni] && c < besti[ni])) {
+              best[ni] = s;
+              besti[ni] = c;
+            }
+          }
+        }
+    }
+  }
+  // combine lane halves (rows interleave between the halves, so compare indices on ties)
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    float ob = __shfl_xor(best[ni], 32);
+    int oi = __shfl_xor(besti[ni], 32);
+    if (oi != 0x7fffffff && (besti[ni] == 0x7fffffff || ob > best[ni] || (ob == best[ni] && oi < besti[ni]))) {
+      best[ni] = ob;
+      besti[ni] = oi;
+    }
+    if (l < 32) {
+      s_best[wm][wn * 64 + ni * 32 + l] = best[ni];
+      s_idx[wm][wn * 64 + ni * 32 + l] = besti[ni];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 128) {
+    int i = i0 + threadIdx.x;
+    float b0 = s_best[0][threadIdx.x], b1 = s_best[1][threadIdx.x];
+    int i0x = s_idx[0][threadIdx.x], i1x = s_idx[1][threadIdx.x];
+    int res = i0x;
+    if (i1x != 0x7fffffff && (i0x == 0x7fffffff || b1 > b0 || (b1 == b0 && i1x < i0x))) res = i1x;
+    if (i < Sq) hash_out[int64_t(h) * Sq + i] = res;
+  }
+}
+
+}  // namespace fm
+
+extern "C" int fm_project(const void* A, const void* K, float* Y, int H, int C, int N, int d,
+                          int64_t ldy, int dtype, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 0 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
+             "fm_project: H=%d C=%d N=%d d=%d", H, C, N, d);
+  FM_REQUIRE(ldy >= N, FM_ERR_ARG, "fm_project: ldy=%lld < N=%d", (long long)ldy, N);
+  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_project: dtype=%d", dtype);
+  if (H == 0) return FM_OK;
+  FM_REQUIRE(A && K && Y, FM_ERR_ARG, "fm_project: null pointer");
+  FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_project: H=%d > 65535", H);
+  hipStream_t st = as_stream(stream);
+  if (dtype == FM_BF16 && d % 16 == 0) {
+    FM_REQUIRE(ceil_div(C, 128) <= 65535, FM_ERR_UNSUPPORTED, "fm_project: C too large");
+    size_t lds = size_t(2) * 128 * (d + 8) * sizeof(bf16_t);
+    FM_ALLOW_LDS(project_bf16_kernel, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_project: lds");
+    dim3 grid = dim3(unsigned(ceil_div(N, 128)), unsigned(ceil_div(C, 128)), unsigned(H));
+    hipLaunchKernelGGL(project_bf16_kernel, grid, dim3(256), lds, st, (const bf16_t*)A,
+                       (const bf16_t*)K, Y, C, N, d, ldy);
+  } else {
+    size_t lds = size_t(64) * (d + 1) * sizeof(float);
+    dim3 grid = dim3(unsigned(ceil_div(N, 64)), unsigned(H));
+    FM_ALLOW_LDS(project_generic_kernel<float>, 64 * (FM_MAX_D + 1) * 4, "fm_project: lds");
+    FM_ALLOW_LDS(project_generic_kernel<bf16_t>, 64 * (FM_MAX_D + 1) * 4, "fm_project: lds");
+    if (dtype == FM_F32)
+      hipLaunchKernelGGL(project_generic_kernel<float>, grid, dim3(256), lds, st, (const float*)A,
+                         (const float*)K, Y, C, N, d, ldy);
+    else
+      hipLaunchKernelGGL(project_generic_kernel<bf16_t>, grid, dim3(256), lds, st,
+                         (const bf16_t*)A, (const bf16_t*)K, Y, C, N, d, ldy);
+  }
+  return launch_status("fm_project");
+}
+
+extern "C" int fm_qhash(const void* A, const void* q, int32_t* hash_out, float* scores_out, int H,
+                        int C, int Sq, int d, int dtype, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 0 && C >= 1 && Sq >= 0 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
+             "fm_qhash: H=%d C=%d Sq=%d d=%d", H, C, Sq, d);
+  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_qhash: dtype=%d", dtype);
+  if (H == 0 || Sq == 0) return FM_OK;
+  FM_REQUIRE(A && q && hash_out, FM_ERR_ARG, "fm_qhash: null pointer");
+  FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_qhash: H=%d > 65535", H);
+  hipStream_t st = as_stream(stream);
+  if (dtype == FM_BF16 && d % 16 == 0) {
+    size_t lds = size_t(2) * 128 * (d + 8) * sizeof(bf16_t);
+    FM_ALLOW_LDS(qhash_bf16_kernel, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_qhash: lds");
+    dim3 grid = dim3(unsigned(ceil_div(Sq, 128)), unsigned(H));
+    hipLaunchKernelGGL(qhash_bf16_kernel, grid, dim3(256), lds, st, (const bf16_t*)A,
+                       (const bf16_t*)q, hash_out, scores_out, C, Sq, d);
+  } else {
+    size_t lds = size_t(64) * (d + 1) * sizeof(float);
+    FM_ALLOW_LDS(qhash_generic_kernel<float>, 64 * (FM_MAX_D + 1) * 4, "fm_qhash: lds");
+    FM_ALLOW_LDS(qhash_generic_kernel<bf16_t>, 64 * (FM_MAX_D + 1) * 4, "fm_qhash: lds");
+    dim3 grid = dim3(unsigned(ceil_div(Sq, 64)), unsigned(H));
+    if (dtype == FM_F32)
+      hipLaunchKernelGGL(qhash_generic_kernel<float>, grid, dim3(256), lds, st, (const float*)A,
+                         (const float*)q, hash_out, scores_out, C, Sq, d);
+    else
+      hipLaunchKernelGGL(qhash_generic_kernel<bf16_t>, grid, dim3(256), lds, st, (const bf16_t*)A,
+                         (const bf16_t*)q, hash_out, scores_out, C, Sq, d);
+  }
+  return launch_status("fm_qhash");
+}

@@ -1,0 +1,85 @@
+"""Operator-level API with the reference's names and argument order
+(triton_kernel.py): ``attention_hash_varlen`` and ``attention_hash``.
+
+The grouping of queries (sort / unique / cumsum in the reference, with host
+synchronisations), the kernel and the un-permute run inside libfastmem; nothing
+here reads a value back from the device.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import ops
+
+
+def _as_i32(t: torch.Tensor) -> torch.Tensor:
+    return t if t.dtype == torch.int32 else t.to(torch.int32)
+
+
+def attention_hash_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                          k_hashes: torch.Tensor, k_hash_counts: torch.Tensor,
+                          q_hashes: torch.Tensor, sm_scale: float,
+                          lse_dtype: Optional[torch.dtype] = torch.float32) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Drop-in for ``attention_hash_varlen`` (triton_kernel.py:51-119).
+
+    :param q: ``[batch_size, q_seq_len, d_head]``
+    :param k: ``[batch_size, kv_seq_len, d_head]``
+    :param v: ``[batch_size, kv_seq_len, d_head]``
+    :param k_hashes: flat key indices of all buckets, row-major ``(batch, bucket)``
+    :param k_hash_counts: ``[batch_size, C]`` keys per bucket
+    :param q_hashes: ``[batch_size, q_seq_len]`` bucket of every query
+    :param sm_scale: softmax scale
+    :param lse_dtype: ``torch.float32`` (default) returns the fp32 natural-log
+        LSE; ``None`` reproduces the reference's rounding of the LSE to q's
+        dtype (triton_kernel.py:111-117).
+    :return: ``(out [batch, q_seq_len, d_head], lse [batch, q_seq_len])``;
+        a query whose bucket holds no key gets ``out = 0`` and
+        ``lse = finfo(lse.dtype).min``.
+    """
+    batch_size, q_seq_len, d_head = q.shape
+    _, kv_seq_len, _ = k.shape
+    _, n_buckets = k_hash_counts.shape
+
+    assert k.shape[0] == batch_size
+    assert k_hash_counts.shape[0] == batch_size
+    assert q_hashes.shape[0] == batch_size
+    assert q_hashes.shape[1] == q_seq_len, f'{q_hashes.shape} != {q_seq_len}'
+    assert d_head == k.shape[-1] == v.shape[-1]
+    assert q.is_contiguous()
+    assert k.is_contiguous()
+    assert v.is_contiguous()
+    assert k.stride() == v.stride()
+
+    out, lse = ops.attention_hash_varlen_i32(q, k, v, _as_i32(k_hashes).contiguous(),
+                                             _as_i32(k_hash_counts).contiguous(),
+                                             _as_i32(q_hashes).contiguous(), sm_scale)
+    if lse_dtype is None:
+        # the reference scales after rounding: lse2.to(q.dtype) * ln2, then nan_to_num
+        lse = lse.to(q.dtype)
+        lse = torch.nan_to_num(lse, nan=0.0, posinf=torch.finfo(lse.dtype).max,
+                               neginf=torch.finfo(lse.dtype).min)
+    elif lse_dtype != torch.float32:
+        lse = torch.nan_to_num(lse.to(lse_dtype), neginf=torch.finfo(lse_dtype).min)
+    return out, lse
+
+
+def attention_hash(q, k, v, centroids, bucket_size, sm_scale, window=None):
+    """Drop-in for the single-device composite ``attention_hash``
+    (triton_kernel.py:275-286): project, arg-top-Z, hash, attend.
+
+    ``centroids [batch, C, d]``.  The reference hard-codes a benchmark window
+    of key indices at triton_kernel.py:283; ``window=(lo, hi)`` gives the same
+    filter, default all keys."""
+    k_hashes = ops.build_index(centroids, k, bucket_size)
+    q_hashes = ops.qhash(centroids, q)
+    if window is None:
+        B, C, Z = k_hashes.shape
+        counts = torch.full((B, C), Z, dtype=torch.int32, device=q.device)
+        flat = k_hashes.reshape(-1)
+    else:
+        lo, hi = window
+        flat, counts, _ = ops.window_filter(k_hashes, lo, hi)
+        flat = flat + lo if lo else flat
+    return ops.attention_hash_varlen_i32(q, k, v, flat, counts, q_hashes, sm_scale)

@@ -1,0 +1,184 @@
+"""Module-level API of the indexed memory (the reference's memory.py), on one
+MI355X: LSE merge, construction of the projection matrix, the per-window
+attention step, and the ``Memory`` object the README describes (build a memory
+from past keys, query it, get attention output plus log-sum-exp).
+
+Ring send/receive, collectives, the autograd wrapper and the model hook of the
+reference are not part of this package.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import ops
+from .hash_attention import attention_hash_varlen
+
+
+# --------------------------------------------------------------------------
+def update_out_and_lse(out: Optional[torch.Tensor], lse: Optional[torch.Tensor],
+                       block_out: torch.Tensor, block_lse: torch.Tensor
+                       ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Drop-in for ``update_out_and_lse`` (memory.py:54-71): merges a partial
+    attention into the running fp32 ``(out, lse[..., None])`` pair, in place."""
+    if out is None:
+        return block_out.to(torch.float32), block_lse.to(torch.float32).unsqueeze(dim=-1)
+    assert out.dtype == torch.float32 and lse.dtype == torch.float32
+    assert out.is_contiguous() and lse.is_contiguous()
+    ops.lse_merge_(out, lse, block_out.contiguous(), block_lse.to(torch.float32).contiguous())
+    return out, lse
+
+
+# --------------------------------------------------------------------------
+def init_centroids(n_buckets: int, d: int, device, dtype) -> torch.Tensor:
+    """The reference's initial centroids (memory.py:489-493)."""
+    rng = np.random.RandomState(42)
+    return torch.tensor(rng.randn(n_buckets, d), device=device, dtype=dtype, requires_grad=False)
+
+
+@torch.no_grad()
+def compute_centroids(kq: torch.Tensor, centroids: torch.Tensor, n_hashes: int, n_groups: int,
+                      centroid_topk: int, normalize: bool = False) -> torch.Tensor:
+    """Drop-in for ``compute_centroids`` (memory.py:209-231); ``centroid_topk``
+    replaces the reference's module-global ``consts.centroid_topk``.
+
+    ``kq [H*G, N, d]``, ``centroids [C, d]`` -> ``[C, H, d]``.  With
+    ``normalize`` the rows are L2-normalised as the caller does at
+    memory.py:258 (the all-reduce before it is the identity on one device)."""
+    n_heads, context_len, d_qkv = kq.shape
+    k_heads = n_heads // n_groups
+    assert centroids.shape == (n_hashes, d_qkv)
+    kq_hash = ops.l2_normalize(kq.contiguous(), 1e-6)
+    # scores[hg, c, i] = centroids[c] . kq_hash[hg, i]; rows ordered (hg, c)
+    A = centroids.to(kq.dtype).unsqueeze(0).expand(n_heads, -1, -1).contiguous()
+    top = ops.build_index(A, kq_hash, centroid_topk)                 # [HG, C, k]
+    top = top.permute(1, 0, 2).contiguous()                          # [C, HG, k]
+    return ops.topk_mean(kq_hash, top, k_heads, n_groups, normalize=normalize)
+
+
+@torch.no_grad()
+def kmeans_spherical(X: torch.Tensor, init: torch.Tensor, iters: int):
+    """Spherical K-means (README.md:37-45): ``X [H,N,d]`` unit rows, ``init
+    [H,C,d]`` -> centroids ``[H,C,d]`` (unit rows) and the labels of the last
+    assignment ``[H,N]`` int32."""
+    cent = init.contiguous()
+    C = cent.shape[1]
+    labels = None
+    for _ in range(iters):
+        labels = ops.qhash(cent, X)
+        groups = ops.group_queries(labels, C)
+        cent = ops.segment_mean(X, groups, cent)
+    return cent, labels
+
+
+def fit_projection(keys: torch.Tensor, n_buckets: int, iters: int = 2,
+                   init: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A ``[H,C,d]`` from ``iters`` spherical K-means iterations on the
+    L2-normalised keys ``[H,N,d]`` (README.md:33-45), starting from the
+    reference's seeded random centroids, normalised."""
+    H, N, d = keys.shape
+    X = ops.l2_normalize(keys.contiguous(), 1e-6)
+    if init is None:
+        c0 = init_centroids(n_buckets, d, keys.device, torch.float32)
+        c0 = (c0 / c0.norm(dim=-1, keepdim=True)).to(keys.dtype)
+        init = c0.unsqueeze(0).expand(H, -1, -1).contiguous()
+    cent, _ = kmeans_spherical(X, init, iters)
+    return cent
+
+
+# --------------------------------------------------------------------------
+def ring_attention_masked_forward(k_hashes, q_hashes, q, k, v, sm_scale, rank,
+                                  lse_dtype: Optional[torch.dtype] = torch.float32):
+    """Drop-in for ``ring_attention_masked_forward`` (memory.py:106-163).
+
+    :param k_hashes: ``[n_buckets, k_heads, bucket_size]`` global key indices
+    :param q_hashes: ``[k_heads, n_groups, seq_len]``
+    :param q: ``[1, n_heads, seq_len, d]``
+    :param k, v: ``[1, k_heads, context_len, d]`` -- the window of keys with
+        global indices ``[rank*context_len, (rank+1)*context_len)``
+    :return: ``(out [1,n_heads,seq_len,d], lse [1,n_heads,seq_len])``; the
+        LSE is fp32 unless ``lse_dtype=None`` asks for the reference's rounding
+        to q's dtype.
+    """
+    batch_size, n_heads, seq_len, d_head = q.shape
+    _, k_heads, context_len, _ = k.shape
+    n_groups = n_heads // k_heads
+    assert batch_size == 1
+    assert k_hashes.shape[1] == k_heads
+    assert q_hashes.shape[0] == k_heads
+    assert q_hashes.shape[1] == n_groups
+    assert q_hashes.shape[2] == seq_len
+    assert k_hashes.numel() > 0, k_hashes.shape
+
+    kh = k_hashes.permute(1, 0, 2).to(torch.int32).contiguous()     # H C Z
+    flat, counts, _ = ops.window_filter(kh, rank * context_len, (rank + 1) * context_len)
+    out, lse = attention_hash_varlen(q.reshape(k_heads, -1, d_head), k.reshape(k_heads, -1, d_head),
+                                     v.reshape(k_heads, -1, d_head), flat, counts,
+                                     q_hashes.reshape(k_heads, -1), sm_scale, lse_dtype=lse_dtype)
+    return out.reshape(batch_size, n_heads, seq_len, d_head), lse.reshape(batch_size, n_heads, seq_len)
+
+
+# --------------------------------------------------------------------------
+class Memory:
+    """Indexed memory over one sequence's past keys (README.md:5-7).
+
+    ``keys, values [H,N,d]``; ``A [H,C,d]`` projection rows; ``Z`` bucket
+    capacity.  ``attend`` returns the attention over the hashed bucket and its
+    log-sum-exp so the caller can merge it with attention over other keys
+    (``merge`` / ``update_out_and_lse``).
+    """
+
+    def __init__(self, keys: torch.Tensor, values: torch.Tensor, A: torch.Tensor, bucket_idx: torch.Tensor):
+        self.keys, self.values, self.A, self.bucket_idx = keys, values, A, bucket_idx
+        H, C, Z = bucket_idx.shape
+        self.bucket_cnt = torch.full((H, C), Z, dtype=torch.int32, device=keys.device)
+        self.bucket_off = (torch.arange(H * C, dtype=torch.int64, device=keys.device) * Z).reshape(H, C)
+
+    @classmethod
+    def build(cls, keys: torch.Tensor, values: torch.Tensor, A: torch.Tensor, Z: int,
+              workspace_bytes: int = 8 << 30) -> "Memory":
+        keys, values, A = keys.contiguous(), values.contiguous(), A.contiguous()
+        assert keys.shape == values.shape and A.shape[0] == keys.shape[0] and A.shape[2] == keys.shape[2]
+        return cls(keys, values, A, ops.build_index(A, keys, Z, workspace_bytes))
+
+    @property
+    def n_buckets(self) -> int:
+        return self.A.shape[1]
+
+    def hash(self, q: torch.Tensor) -> torch.Tensor:
+        """q ``[H,Sq,d]`` -> bucket ids ``[H,Sq]`` int32."""
+        return ops.qhash(self.A, q.contiguous())
+
+    def attend(self, q: torch.Tensor, sm_scale: float, q_hash: Optional[torch.Tensor] = None):
+        """q ``[H,Sq,d]`` (Sq = G*S, query head h*G+g) -> ``(out [H,Sq,d], lse [H,Sq] fp32)``."""
+        q = q.contiguous()
+        if q_hash is None:
+            q_hash = self.hash(q)
+        groups = ops.group_queries(q_hash, self.n_buckets)
+        return ops.hash_attn_fwd(q, self.keys, self.values, self.bucket_idx.reshape(-1), self.bucket_off,
+                                 self.bucket_cnt, groups, sm_scale)
+
+    def attend_with_local(self, q: torch.Tensor, k_local: torch.Tensor, v_local: torch.Tensor,
+                          sm_scale: float, n_groups: int, causal: bool = True):
+        """Memory attention LSE-merged with dense attention over local keys
+        (memory.py:302-305, 319-332).  q ``[H,G*S,d]`` with ``G = n_groups``;
+        k_local, v_local ``[H,L,d]``.  Returns fp32 ``(out [H,G*S,d], lse
+        [H,G*S])``."""
+        H, Sq, d = q.shape
+        S = Sq // n_groups
+        q = q.contiguous()
+        lo, ll = ops.local_attn_fwd(q.reshape(H * n_groups, S, d), k_local.contiguous(),
+                                    v_local.contiguous(), sm_scale, causal)
+        out, lse = update_out_and_lse(None, None, lo.reshape(H, Sq, d), ll.reshape(H, Sq))
+        mo, ml = self.attend(q, sm_scale)
+        out, lse = update_out_and_lse(out.contiguous(), lse.contiguous(), mo, ml)
+        return out, lse.squeeze(-1)
+
+
+def merge(out_a, lse_a, out_b, lse_b):
+    """Functional LSE merge of two partial attentions (memory.py:54-71)."""
+    out, lse = update_out_and_lse(None, None, out_a, lse_a)
+    out, lse = update_out_and_lse(out.clone().contiguous(), lse.clone().contiguous(), out_b, lse_b)
+    return out, lse.squeeze(-1)

@@ -1,0 +1,248 @@
+"""Tensor-level wrappers over the C ABI: shape/dtype checks, output and
+workspace allocation (torch owns device memory and streams), one C call each."""
+from __future__ import annotations
+
+from typing import NamedTuple, Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import check
+
+_DT = {torch.float32: _lib.FM_F32, torch.bfloat16: _lib.FM_BF16}
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype not in _DT:
+        raise TypeError(f"unsupported dtype {t.dtype}; libfastmem takes float32 and bfloat16")
+    return _DT[t.dtype]
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _dev(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if not t.is_cuda:
+            raise RuntimeError("libfastmem operators take GPU tensors only (there is no CPU path)")
+        if not t.is_contiguous():
+            raise AssertionError("tensor must be contiguous")
+
+
+def _ws(nbytes: int, like: torch.Tensor) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=like.device)
+
+
+# --------------------------------------------------------------------- a1
+def project(A: torch.Tensor, K: torch.Tensor) -> torch.Tensor:
+    """Y[h,c,n] = sum_d A[h,c,d] K[h,n,d], fp32 (memory.py:261)."""
+    _dev(A, K)
+    H, C, d = A.shape
+    H2, N, d2 = K.shape
+    assert H == H2 and d == d2 and A.dtype == K.dtype
+    Y = torch.empty((H, C, N), dtype=torch.float32, device=A.device)
+    check(_lib.load().fm_project(_p(A), _p(K), _p(Y), H, C, N, d, N, _dt(A), _stream(A)))
+    return Y
+
+
+# --------------------------------------------------------------------- a2
+def argtopz(Y: torch.Tensor, Z: int) -> torch.Tensor:
+    """Indices of the min(Z,N) largest entries per row: value desc, index asc (memory.py:273)."""
+    _dev(Y)
+    assert Y.dtype == torch.float32
+    N = Y.shape[-1]
+    rows = Y.numel() // N if N else 0
+    Zc = min(int(Z), N)
+    out = torch.empty((*Y.shape[:-1], Zc), dtype=torch.int32, device=Y.device)
+    check(_lib.load().fm_argtopz_f32(_p(Y), rows, N, N, int(Z), _p(out), None, 0, _stream(Y)))
+    return out
+
+
+def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int = 8 << 30) -> torch.Tensor:
+    """Bucket lists [H,C,min(Z,N)] int32 (memory.py:260-278 on one device)."""
+    _dev(A, K)
+    H, C, d = A.shape
+    _, N, _ = K.shape
+    assert K.shape[0] == H and K.shape[2] == d and A.dtype == K.dtype
+    lib = _lib.load()
+    full = lib.fm_build_index_workspace(H, C, N, d, int(Z), C)
+    one = lib.fm_build_index_workspace(H, C, N, d, int(Z), 1)
+    ws = _ws(max(one, min(full, int(workspace_bytes))), A)
+    out = torch.empty((H, C, min(int(Z), N)), dtype=torch.int32, device=A.device)
+    check(lib.fm_build_index(_p(A), _p(K), _p(out), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(), _stream(A)))
+    return out
+
+
+# --------------------------------------------------------------------- a3
+def qhash(A: torch.Tensor, q: torch.Tensor, return_scores: bool = False):
+    """h_q = argmax_c A[h,c,:].q, first maximum wins (memory.py:281-283).  q [H,Sq,d]."""
+    _dev(A, q)
+    H, C, d = A.shape
+    H2, Sq, d2 = q.shape
+    assert H == H2 and d == d2 and A.dtype == q.dtype
+    out = torch.empty((H, Sq), dtype=torch.int32, device=q.device)
+    scores = torch.empty((H, Sq, C), dtype=torch.float32, device=q.device) if return_scores else None
+    check(_lib.load().fm_qhash(_p(A), _p(q), _p(out), _p(scores), H, C, Sq, d, _dt(A), _stream(q)))
+    return (out, scores) if return_scores else out
+
+
+# --------------------------------------------------------------------- a4
+def window_filter(k_idx: torch.Tensor, lo: int, hi: int):
+    """Keep bucket entries in [lo,hi), re-base by -lo (memory.py:128-142).
+
+    k_idx [H,C,Z] int32 -> (flat int32 buffer of H*C*Z slots of which the first
+    sum(cnt) are valid, cnt [H,C] int32, off [H,C] int64)."""
+    _dev(k_idx)
+    assert k_idx.dtype == torch.int32 and k_idx.dim() == 3
+    H, C, Z = k_idx.shape
+    flat = torch.empty(H * C * Z, dtype=torch.int32, device=k_idx.device)
+    cnt = torch.empty((H, C), dtype=torch.int32, device=k_idx.device)
+    off = torch.empty((H, C), dtype=torch.int64, device=k_idx.device)
+    check(_lib.load().fm_window_filter(_p(k_idx), H * C, Z, int(lo), int(hi), _p(flat), _p(cnt), _p(off),
+                                       None, 0, _stream(k_idx)))
+    return flat, cnt, off
+
+
+def bucket_offsets(cnt: torch.Tensor) -> torch.Tensor:
+    """Exclusive prefix sum over the flattened counts (triton_kernel.py:86-88)."""
+    _dev(cnt)
+    assert cnt.dtype == torch.int32
+    off = torch.empty(cnt.shape, dtype=torch.int64, device=cnt.device)
+    check(_lib.load().fm_bucket_offsets(_p(cnt), cnt.numel(), _p(off), _stream(cnt)))
+    return off
+
+
+# --------------------------------------------------------------------- a5
+class QueryGroups(NamedTuple):
+    q_perm: torch.Tensor      # [H,Sq] int32
+    bin_count: torch.Tensor   # [H,C]  int32
+    bin_off: torch.Tensor     # [H,C]  int32
+    items: torch.Tensor       # [max_items,4] int32
+    n_items: torch.Tensor     # [1] int32
+    max_items: int
+
+
+def group_queries(q_hash: torch.Tensor, C: int) -> QueryGroups:
+    """Stable grouping of queries by (row, bucket) on the device (triton_kernel.py:75-88)."""
+    _dev(q_hash)
+    assert q_hash.dtype == torch.int32 and q_hash.dim() == 2
+    H, Sq = q_hash.shape
+    lib = _lib.load()
+    dev = q_hash.device
+    max_items = lib.fm_group_max_items(H, C, Sq)
+    q_perm = torch.empty((H, Sq), dtype=torch.int32, device=dev)
+    bin_count = torch.empty((H, C), dtype=torch.int32, device=dev)
+    bin_off = torch.empty((H, C), dtype=torch.int32, device=dev)
+    items = torch.empty((max_items, 4), dtype=torch.int32, device=dev)
+    n_items = torch.empty(1, dtype=torch.int32, device=dev)
+    ws = _ws(lib.fm_group_queries_workspace(H, C, Sq), q_hash)
+    check(lib.fm_group_queries(_p(q_hash), H, C, Sq, _p(q_perm), _p(bin_count), _p(bin_off), _p(items),
+                               _p(n_items), max_items, _p(ws), ws.numel(), _stream(q_hash)))
+    return QueryGroups(q_perm, bin_count, bin_off, items, n_items, max_items)
+
+
+# --------------------------------------------------------------------- a6-a8
+def hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, sm_scale: float):
+    """Bucket-gathered attention (triton_kernel.py:137-272).  q [H,Sq,d], k,v [H,N,d].
+    Returns out [H,Sq,d] (q dtype) and lse [H,Sq] fp32 natural log, original query order."""
+    _dev(q, k, v, k_idx, bucket_off, bucket_cnt)
+    H, Sq, d = q.shape
+    _, N, _ = k.shape
+    C = bucket_cnt.shape[-1]
+    assert k.shape == v.shape and k.shape[0] == H and k.shape[2] == d
+    assert q.dtype == k.dtype == v.dtype
+    assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and bucket_off.dtype == torch.int64
+    out = torch.empty_like(q)
+    lse = torch.empty((H, Sq), dtype=torch.float32, device=q.device)
+    check(_lib.load().fm_hash_attn_fwd(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
+                                       _p(groups.q_perm), _p(groups.items), _p(groups.n_items),
+                                       groups.max_items, _p(out), _p(lse), H, Sq, N, d, C,
+                                       float(sm_scale), _dt(q), _stream(q)))
+    return out, lse
+
+
+def attention_hash_varlen_i32(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: float):
+    """The reference operator in one C call (triton_kernel.py:51-119) on int32 index tensors."""
+    _dev(q, k, v, k_idx, bucket_cnt, q_hash)
+    H, Sq, d = q.shape
+    _, N, _ = k.shape
+    C = bucket_cnt.shape[-1]
+    assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and q_hash.dtype == torch.int32
+    lib = _lib.load()
+    ws = _ws(lib.fm_attention_hash_varlen_workspace(H, C, Sq), q)
+    out = torch.empty_like(q)
+    lse = torch.empty((H, Sq), dtype=torch.float32, device=q.device)
+    check(lib.fm_attention_hash_varlen(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_cnt), _p(q_hash), _p(out),
+                                       _p(lse), H, Sq, N, d, C, float(sm_scale), _dt(q), _p(ws),
+                                       ws.numel(), _stream(q)))
+    return out, lse
+
+
+# --------------------------------------------------------------------- a11
+def local_attn_fwd(q, k, v, sm_scale: float, causal: bool = True):
+    """Dense GQA attention with LSE (call site memory.py:302).  q [H*G,S,d], k,v [H,L,d]."""
+    _dev(q, k, v)
+    HG, S, d = q.shape
+    H, L, _ = k.shape
+    assert HG % H == 0 and k.shape == v.shape and k.shape[2] == d and q.dtype == k.dtype == v.dtype
+    out = torch.empty_like(q)
+    lse = torch.empty((HG, S), dtype=torch.float32, device=q.device)
+    check(_lib.load().fm_local_attn_fwd(_p(q), _p(k), _p(v), _p(out), _p(lse), H, HG // H, S, L, d,
+                                        float(sm_scale), int(bool(causal)), _dt(q), _stream(q)))
+    return out, lse
+
+
+# --------------------------------------------------------------------- a10
+def lse_merge_(out: torch.Tensor, lse: torch.Tensor, block_out: torch.Tensor, block_lse: torch.Tensor):
+    """In-place merge of (block_out, block_lse) into the fp32 running pair (memory.py:54-71)."""
+    _dev(out, lse, block_out, block_lse)
+    assert out.dtype == torch.float32 and lse.dtype == torch.float32 and block_lse.dtype == torch.float32
+    d = out.shape[-1]
+    Q = out.numel() // d
+    assert lse.numel() == Q and block_lse.numel() == Q and block_out.numel() == out.numel()
+    check(_lib.load().fm_lse_merge(_p(out), _p(lse), _p(block_out), _p(block_lse), Q, d, _dt(block_out),
+                                   _stream(out)))
+    return out, lse
+
+
+# --------------------------------------------------------------------- a12/a13
+def l2_normalize(X: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    _dev(X)
+    d = X.shape[-1]
+    Xn = torch.empty_like(X)
+    check(_lib.load().fm_l2_normalize(_p(X), _p(Xn), X.numel() // d, d, float(eps), _dt(X), _stream(X)))
+    return Xn
+
+
+def topk_mean(Xn: torch.Tensor, top_idx: torch.Tensor, H: int, G: int, normalize: bool = True) -> torch.Tensor:
+    """Xn [H*G,N,d] unit rows, top_idx [C,H*G,k] int32 -> A [C,H,d] (memory.py:224-229, 258)."""
+    _dev(Xn, top_idx)
+    HG, N, d = Xn.shape
+    C, HG2, k = top_idx.shape
+    assert HG == HG2 == H * G and top_idx.dtype == torch.int32
+    A = torch.empty((C, H, d), dtype=Xn.dtype, device=Xn.device)
+    check(_lib.load().fm_topk_mean(_p(Xn), _p(top_idx), _p(A), C, H, G, N, k, d, int(normalize), _dt(Xn),
+                                   _stream(Xn)))
+    return A
+
+
+def segment_mean(X: torch.Tensor, groups: QueryGroups, prev: torch.Tensor) -> torch.Tensor:
+    """Spherical K-means update: X [H,N,d] unit rows grouped by label -> centroids [H,C,d]."""
+    _dev(X, prev)
+    H, N, d = X.shape
+    _, C, _ = prev.shape
+    assert prev.dtype == X.dtype
+    out = torch.empty_like(prev)
+    check(_lib.load().fm_segment_mean(_p(X), _p(groups.q_perm), _p(groups.bin_off), _p(groups.bin_count),
+                                      _p(prev), _p(out), H, C, N, d, _dt(X), _stream(X)))
+    return out
+
+
+def force_generic_kernels(on: bool) -> None:
+    """Diagnostic switch: route attention through the generic kernels."""
+    _lib.load().fm_debug_force_generic(int(on))

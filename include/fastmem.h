@@ -1,0 +1,178 @@
+/*
+ * fastmem.h -- C ABI of libfastmem.so, the MI355X (gfx950) implementation of
+ * the indexed-memory attention hot path of notbadai/fast_memory.
+ *
+ * The reference has no native boundary: its only operator is the torch custom
+ * op `notbad::attention_hash_varlen` (triton_kernel.py:16-41) plus plain torch
+ * calls around it.  Each entry point below names the reference lines whose work
+ * it takes over.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the name ends in `_host`;
+ *   - tensors are dense, row-major, batch-first: A [H,C,d], K/V [H,N,d],
+ *     q/out [H,Sq,d] with Sq = G*S (query head hq = h*G + g, memory.py:281);
+ *   - `dtype` selects the element type of q/k/v/A: FM_F32 or FM_BF16; all
+ *     accumulation is fp32; log-sum-exp values are fp32 natural logarithms;
+ *   - all index tensors are int32;
+ *   - `stream` is a hipStream_t (NULL = the default stream); no entry point
+ *     synchronises the device or allocates memory; scratch space comes in
+ *     through `ws` / `ws_bytes`, sized by the matching *_workspace() query;
+ *   - return value: FM_OK (0) or an fm_status error code; fm_last_error()
+ *     returns the message of the calling thread's last failure;
+ *   - calls are re-entrant per stream as long as they do not share outputs or
+ *     workspace.
+ */
+#ifndef FASTMEM_H
+#define FASTMEM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  FM_OK = 0,
+  FM_ERR_ARG = 1,         /* null pointer, bad extent, bad enum              */
+  FM_ERR_UNSUPPORTED = 2, /* shape outside what the kernels are built for    */
+  FM_ERR_WORKSPACE = 3,   /* ws_bytes smaller than the *_workspace() answer  */
+  FM_ERR_LAUNCH = 4       /* HIP reported an error at launch                 */
+} fm_status;
+
+typedef enum { FM_F32 = 0, FM_BF16 = 1 } fm_dtype;
+
+/* Largest bucket capacity Z the selection kernels accept. */
+#define FM_MAX_Z 16384
+/* Largest head dimension. */
+#define FM_MAX_D 256
+/* Queries one attention work item carries (tile of one (row,bucket) group). */
+#define FM_QTILE 64
+
+int fm_version(void);
+const char* fm_last_error(void);
+
+/* ---- a1: projection  Y[h,c,n] = sum_d A[h,c,d] K[h,n,d]  (fp32 out) --------
+ * replaces einsum at memory.py:261 / triton_kernel.py:277.  bf16 inputs use
+ * MFMA with fp32 accumulation.  Y is [H,C,N] with row stride `ldy` elements
+ * (ldy >= N). */
+int fm_project(const void* A, const void* K, float* Y, int H, int C, int N, int d,
+               int64_t ldy, int dtype, void* stream);
+
+/* ---- a2: arg-top-Z over every row of an fp32 matrix -------------------------
+ * replaces torch.topk at memory.py:273 / triton_kernel.py:278.  Output row r =
+ * the min(Z,N) indices of the largest entries of Y[r,:], ordered by value
+ * descending then index ascending (the first Z entries of a stable descending
+ * sort; -0 == +0; NaN is the largest).  idx_out is [rows, min(Z,N)] int32. */
+size_t fm_argtopz_workspace(int64_t rows, int N, int Z);
+int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, int Z, int32_t* idx_out,
+                   void* ws, size_t ws_bytes, void* stream);
+
+/* ---- a1+a2: index build without handing Y to the caller ---------------------
+ * memory.py:260-278 on one device.  idx_out [H,C,min(Z,N)] int32.  The
+ * workspace holds fp32 projection rows for as many (head,bucket) rows as fit;
+ * any size from fm_build_index_workspace(...,1) up is accepted and larger ones
+ * mean fewer passes. */
+size_t fm_build_index_workspace(int H, int C, int N, int d, int Z, int64_t rows_per_pass);
+int fm_build_index(const void* A, const void* K, int32_t* idx_out, int H, int C, int N, int d,
+                   int Z, int dtype, void* ws, size_t ws_bytes, void* stream);
+
+/* ---- a3: query hash  h_q = argmax_c A[h,c,:].q  (first maximum wins) ---------
+ * replaces einsum+argmax at memory.py:281-283 / triton_kernel.py:280-281.
+ * hash_out [H,Sq] int32.  scores_out is optional ([H,Sq,C] fp32, may be NULL):
+ * the scores the argmax was taken over. */
+int fm_qhash(const void* A, const void* q, int32_t* hash_out, float* scores_out, int H, int C,
+             int Sq, int d, int dtype, void* stream);
+
+/* ---- a4: window filter of bucket lists -------------------------------------
+ * memory.py:128-142: keep entries in [lo,hi), re-base by -lo, flatten row-major.
+ * idx_in [H*C, Z]; idx_out holds up to H*C*Z entries; cnt_out/off_out [H*C]. */
+size_t fm_window_filter_workspace(int64_t n_buckets_total);
+int fm_window_filter(const int32_t* idx_in, int64_t n_buckets_total, int Z, int64_t lo, int64_t hi,
+                     int32_t* idx_out, int32_t* cnt_out, int64_t* off_out, void* ws,
+                     size_t ws_bytes, void* stream);
+
+/* ---- exclusive prefix sum of per-bucket counts (triton_kernel.py:86-88) ----- */
+int fm_bucket_offsets(const int32_t* cnt, int64_t n, int64_t* off_out, void* stream);
+
+/* ---- a5 + a16: group queries by (row, bucket) on the device -----------------
+ * replaces sort / unique_consecutive / cumsum at triton_kernel.py:75-88, with
+ * no host synchronisation.
+ *   q_hash    [H,Sq]   in   bucket of every query
+ *   q_perm    [H,Sq]   out  stable ascending sort permutation per row:
+ *                           q_perm[h,p] = original index of the p-th sorted query
+ *   bin_count [H,C]    out  queries per bucket (memory.py:285-286)
+ *   bin_off   [H,C]    out  first sorted position of the bucket, over the
+ *                           flattened H*Sq axis (triton_kernel.py:84)
+ *   items     [max_items] out  work items {row, bucket, first sorted position,
+ *                           number of queries <= FM_QTILE}
+ *   n_items   [1]      out  number of items written
+ * max_items must be >= fm_group_max_items(H, C, Sq). */
+typedef struct { int32_t row, bucket, q_start, n_q; } fm_item;
+int64_t fm_group_max_items(int H, int C, int Sq);
+size_t fm_group_queries_workspace(int H, int C, int Sq);
+int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int32_t* q_perm,
+                     int32_t* bin_count, int32_t* bin_off, fm_item* items, int32_t* n_items,
+                     int64_t max_items, void* ws, size_t ws_bytes, void* stream);
+
+/* ---- a6-a8: bucket-gathered attention forward ------------------------------
+ * replaces the Triton kernel _attn_fwd/_attn_fwd_inner (triton_kernel.py:
+ * 137-272) and the un-permute / unit conversion at triton_kernel.py:108-117.
+ *   q [H,Sq,d], k,v [H,N,d]           in original order
+ *   k_idx flat int32, bucket_off [H*C] int64, bucket_cnt [H*C] int32
+ *   q_perm, items, n_items            from fm_group_queries
+ *   out [H,Sq,d] (dtype of q), lse [H,Sq] fp32 natural log, original order.
+ * A query whose bucket is empty gets out = 0, lse = -FLT_MAX. */
+int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                     const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                     const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
+                     float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype,
+                     void* stream);
+
+/* ---- the reference operator in one call -------------------------------------
+ * attention_hash_varlen(q,k,v,k_hashes,k_hash_counts,q_hashes,sm_scale)
+ * (triton_kernel.py:51-119): bucket offsets + grouping + attention. */
+size_t fm_attention_hash_varlen_workspace(int H, int C, int Sq);
+int fm_attention_hash_varlen(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                             const int32_t* bucket_cnt, const int32_t* q_hash, void* out,
+                             float* lse, int H, int Sq, int N, int d, int C, float sm_scale,
+                             int dtype, void* ws, size_t ws_bytes, void* stream);
+
+/* ---- a11: dense local attention with LSE ------------------------------------
+ * the attention_forward(q,k_self,v_self,sm_scale,True) call at memory.py:302
+ * (the reference ships no definition).  q [H*G,S,d], k,v [H,L,d]; causal is
+ * bottom-right aligned: query i sees keys j <= i + (L - S). */
+int fm_local_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int H,
+                      int G, int S, int L, int d, float sm_scale, int causal, int dtype,
+                      void* stream);
+
+/* ---- a10: LSE merge, in place on the running pair ---------------------------
+ * update_out_and_lse (memory.py:54-71).  out [Q,d] fp32 and lse [Q] fp32 are
+ * updated with block_out [Q,d] (dtype) and block_lse [Q] fp32. */
+int fm_lse_merge(float* out, float* lse, const void* block_out, const float* block_lse, int64_t Q,
+                 int d, int dtype, void* stream);
+
+/* ---- a12/a13: construction of A ----------------------------------------------
+ * fm_l2_normalize: rows / max(norm, eps)        (memory.py:214-217)
+ * fm_topk_mean:    gather + mean + normalise    (memory.py:224-229, 258)
+ *                  Xn [HG,N,d]; top_idx [C,HG,k] int32; A_out [C,H,d]
+ * fm_segment_mean: spherical K-means centroid update (README.md:41-43):
+ *                  X [H,N,d] unit rows, perm/seg_off/seg_cnt from
+ *                  fm_group_queries on the labels; an empty cluster keeps
+ *                  prev; cent_out [H,C,d] in dtype, unit rows. */
+int fm_l2_normalize(const void* X, void* Xn, int64_t rows, int d, float eps, int dtype,
+                    void* stream);
+int fm_topk_mean(const void* Xn, const int32_t* top_idx, void* A_out, int C, int H, int G, int N,
+                 int k, int d, int normalize, int dtype, void* stream);
+int fm_segment_mean(const void* X, const int32_t* perm, const int32_t* seg_off,
+                    const int32_t* seg_cnt, const void* prev, void* cent_out, int H, int C, int N,
+                    int d, int dtype, void* stream);
+
+/* Diagnostic: 1 routes the attention entry points through the generic kernels
+ * (used by tests to compare the two implementations), 0 restores dispatch. */
+void fm_debug_force_generic(int on);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTMEM_H */

@@ -1,0 +1,61 @@
+"""CPU-side checks of the boundary: the library loads, exports every symbol the
+header declares, and rejects bad arguments with status codes before touching
+the GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from fast_memory_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "fastmem.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    syms = header_symbols()
+    assert len(syms) >= 20
+    for s in syms:
+        assert hasattr(lib, s), f"{s} declared in include/fastmem.h but not exported"
+        assert s in _lib.SIGNATURES, f"{s} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == set(syms)
+
+
+def test_version_and_error_string():
+    lib = _lib.load()
+    assert lib.fm_version() >= 100
+    assert isinstance(lib.fm_last_error(), bytes)
+
+
+def test_argument_errors_are_status_codes():
+    lib = _lib.load()
+    assert lib.fm_argtopz_f32(None, 4, 0, 0, 1, None, None, 0, None) == 1        # N = 0
+    assert b"fm_argtopz_f32" in lib.fm_last_error()
+    assert lib.fm_project(None, None, None, 1, 1, 1, 1000, 1, 0, None) == 1      # d > FM_MAX_D
+    assert lib.fm_qhash(None, None, None, None, 1, 1, 1, 8, 7, None) == 1        # bad dtype
+    assert lib.fm_lse_merge(None, None, None, None, 5, 8, 0, None) == 1          # null pointers
+    assert lib.fm_group_queries(None, 1, 1, 1, None, None, None, None, None, 0, None, 0, None) == 1
+    with pytest.raises(ValueError):
+        _lib.check(1)
+
+
+def test_workspace_queries():
+    lib = _lib.load()
+    assert lib.fm_group_max_items(8, 2048, 32768) == 8 * (2048 + 512) + 1
+    assert lib.fm_build_index_workspace(8, 2048, 1048576, 128, 16384, 1) == 1048576 * 4
+    assert lib.fm_attention_hash_varlen_workspace(2, 16, 100) > 0
+    assert lib.fm_group_queries_workspace(1, 8, 24) >= 8 * 4
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+    from fast_memory_amd import ops
+    with pytest.raises(RuntimeError):
+        ops.project(torch.zeros(1, 2, 8), torch.zeros(1, 4, 8))

@@ -1,0 +1,403 @@
+"""GPU parity tests: every call goes through the C ABI (libfastmem.so) and is
+checked against the CPU oracle on the same seeded inputs.  Integer results
+(bucket lists, hashes, grouping) must match bit for bit; attention outputs are
+held to atol 2e-2 / rtol 1e-2 for bf16 and 1e-4 for fp32, the fp32 LSE to 1e-3
+absolute."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fm_oracle as O
+from tests.util import (assert_attn_close, dev, gen, make_attn_case)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from fast_memory_amd import ops as _ops
+    from fast_memory_amd import _lib
+    _lib.load()
+    assert torch.cuda.is_available()
+    return _ops
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------ a1
+@pytest.mark.parametrize("dtype,H,C,N,d", [
+    (torch.float32, 1, 64, 4096, 64),
+    (torch.float32, 2, 5, 130, 16),
+    (torch.bfloat16, 2, 256, 1000, 128),
+    (torch.bfloat16, 1, 130, 257, 64),
+    (torch.bfloat16, 3, 7, 33, 24),         # d not a multiple of 16: generic kernel
+])
+def test_project(ops, dtype, H, C, N, d):
+    g = gen(100)
+    A = torch.randn(H, C, d, generator=g).to(dtype)
+    K = torch.randn(H, N, d, generator=g).to(dtype)
+    Y = ops.project(*dev(A, K)).cpu()
+    ref = O.project(A, K)
+    assert Y.shape == ref.shape
+    # fp32 accumulation of d products of magnitude ~1: a few ulp of sqrt(d)
+    assert torch.allclose(Y, ref, atol=2e-4 * math.sqrt(d), rtol=1e-5), (Y - ref).abs().max()
+
+
+# ------------------------------------------------------------------ a2
+def check_topz(ops, Y, Z):
+    got = ops.argtopz(dev(Y), Z).cpu()
+    ref = O.argtopz(Y, Z)
+    assert got.dtype == torch.int32 and got.shape == ref.shape
+    assert torch.equal(got.long(), ref), "bucket lists differ from the stable-sort definition"
+
+
+def test_argtopz_random_rows(ops):
+    g = gen(200)
+    check_topz(ops, torch.randn(3, 7, 5000, generator=g), 256)
+    check_topz(ops, torch.randn(64, 4096, generator=g), 256)
+    check_topz(ops, torch.randn(5, 1023, generator=g) * 1e-3, 1)
+
+
+def test_argtopz_heavy_ties(ops):
+    g = gen(201)
+    # bf16-valued scores: thousands of exactly equal values straddle the cut
+    Y = torch.randn(6, 20000, generator=g).to(torch.bfloat16).float()
+    check_topz(ops, Y, 1024)
+    # integer-valued rows and an all-equal row (pure index order)
+    Yi = torch.randint(-3, 4, (4, 3000), generator=g).float()
+    Yi[1] = 2.0
+    check_topz(ops, Yi, 500)
+
+
+def test_argtopz_special_values(ops):
+    g = gen(202)
+    Y = torch.randn(4, 2048, generator=g)
+    Y[0, 5] = math.inf
+    Y[0, 77] = -math.inf
+    Y[1, ::3] = 0.0
+    Y[1, 1::3] = -0.0
+    Y[2] = -Y[2].abs() * 1e-40          # negative denormals
+    Y[3, 100:200] = math.inf
+    for Z in (1, 64, 700, 2048):
+        check_topz(ops, Y, Z)
+
+
+def test_argtopz_clamps_to_n_and_unaligned_rows(ops):
+    g = gen(203)
+    Y = torch.randn(3, 333, generator=g)
+    check_topz(ops, Y, 1000)                                        # Z > N -> full sort of the row
+    check_topz(ops, torch.randn(9, 1021, generator=g), 100)          # rows not 16-byte aligned
+
+
+def test_argtopz_max_z_long_row(ops):
+    g = gen(204)
+    Y = torch.randn(2, 300000, generator=g)
+    check_topz(ops, Y, 16384)
+
+
+def test_argtopz_rejects_oversize_z(ops):
+    Y = torch.zeros(1, 40000, device="cuda")
+    with pytest.raises(RuntimeError):
+        ops.argtopz(Y, 20000)
+
+
+def test_build_index_matches_project_then_select(ops):
+    g = gen(205)
+    A = torch.randn(2, 40, 128, generator=g).to(torch.bfloat16)
+    K = torch.randn(2, 3000, 128, generator=g).to(torch.bfloat16)
+    Ad, Kd = dev(A, K)
+    Y = ops.project(Ad, Kd)
+    lists = ops.build_index(Ad, Kd, 128, workspace_bytes=3000 * 4 * 7)   # forces several passes
+    assert torch.equal(lists, ops.argtopz(Y, 128))
+    assert torch.equal(lists.cpu().long(), O.argtopz(Y.cpu(), 128))
+
+
+# ------------------------------------------------------------------ a3
+@pytest.mark.parametrize("dtype,H,C,S,d", [
+    (torch.float32, 1, 64, 512, 64),
+    (torch.bfloat16, 2, 256, 1000, 128),
+    (torch.bfloat16, 2, 300, 77, 64),
+    (torch.float32, 3, 9, 40, 16),
+])
+def test_qhash(ops, dtype, H, C, S, d):
+    g = gen(300)
+    A = torch.randn(H, C, d, generator=g).to(dtype)
+    q = torch.randn(H, S, d, generator=g).to(dtype)
+    A[0, C - 1] = A[0, 2]                                            # exact tie: bucket 2 must win
+    h, sc = ops.qhash(*dev(A, q), return_scores=True)
+    h, sc = h.cpu(), sc.cpu()
+    assert torch.equal(h.long(), O.argmax_first(sc)), "hash is not the first argmax of the kernel's scores"
+    assert not (h[0] == C - 1).any()
+    ref_sc = O.qhash_scores(A, q)
+    assert torch.allclose(sc, ref_sc, atol=2e-4 * math.sqrt(d), rtol=1e-5)
+    ref_h = O.argmax_first(ref_sc)
+    diff = h.long() != ref_h
+    if diff.any():                                                   # only near-ties may differ
+        top2 = torch.topk(ref_sc, 2, dim=-1)[0]
+        assert ((top2[..., 0] - top2[..., 1])[diff] < 1e-3).all()
+    assert torch.equal(ops.qhash(*dev(A, q)).cpu(), h)
+
+
+# ------------------------------------------------------------------ a4/a5/a16
+@pytest.mark.parametrize("H,S,C", [(1, 24, 8), (3, 1000, 17), (8, 8160, 512), (2, 300, 2048)])
+def test_group_queries(ops, H, S, C):
+    qh = torch.randint(0, C, (H, S), generator=gen(400))
+    if S > 100:
+        qh[0, : S // 2] = 3                                          # a heavy bucket spanning several tiles
+    G = ops.group_queries(dev(qh.int()), C)
+    sync()
+    perm, gb, gc, go = O.group_queries(qh, C)
+    assert torch.equal(G.q_perm.cpu().long(), perm)
+    assert torch.equal(G.bin_count.cpu().long(), O.bin_counts(qh, C))
+    flat_cnt = G.bin_count.cpu().long().reshape(-1)
+    assert torch.equal(G.bin_off.cpu().long().reshape(-1), torch.cumsum(flat_cnt, 0) - flat_cnt)
+    n = int(G.n_items.item())
+    items = G.items[:n].cpu().long()
+    # items tile the groups in (row, bucket) order, at most 64 queries each
+    exp = []
+    for z, cnt, off in zip(gb.tolist(), gc.tolist(), go.tolist()):
+        row = off // S
+        for t in range(0, cnt, 64):
+            exp.append([row, z, off + t, min(64, cnt - t)])
+    assert items.tolist() == exp
+
+
+def test_bucket_offsets_and_window_filter(ops):
+    g = gen(401)
+    cnt = torch.randint(0, 50, (7, 300), generator=g).int()
+    off = ops.bucket_offsets(dev(cnt)).cpu()
+    assert torch.equal(off, O.bucket_offsets(cnt.long()))
+    kh = torch.randint(0, 1000, (3, 40, 33), generator=g).int()
+    flat, c, o = ops.window_filter(dev(kh), 250, 700)
+    rflat, rc = O.window_filter(kh.long(), 250, 700)
+    assert torch.equal(c.cpu().long(), rc)
+    assert torch.equal(o.cpu(), O.bucket_offsets(rc))
+    assert torch.equal(flat[: rflat.numel()].cpu().long(), rflat)
+
+
+# ------------------------------------------------------------------ a6-a8
+def run_varlen(q, k, v, kh, cnt, qh, scale):
+    from fast_memory_amd import attention_hash_varlen
+    qd, kd, vd, khd, cntd, qhd = dev(q, k, v, kh, cnt, qh)
+    out, lse = attention_hash_varlen(qd, kd, vd, khd, cntd, qhd, scale)
+    sync()
+    return out, lse
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_reference_small_shape(dtype):
+    # the reference's first test shape (triton_kernel.py:500): B=1,G=1,S=24,N=1024,C=8,Z=16,d=16
+    q, k, v, kh, cnt, qh = make_attn_case(20, 1, 24, 1024, 8, 16, 16, dtype)
+    out, lse = run_varlen(q, k, v, kh, cnt, qh, 16 ** -0.5)
+    ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 16 ** -0.5)
+    assert_attn_close(out, lse, ro, rl, dtype, "ref small")
+    ro2, rl2 = O.hashed_attention_dense_masked(q, k, v, kh, cnt, qh, 16 ** -0.5)
+    assert_attn_close(out, lse, ro2, rl2, dtype, "ref small (dense-masked)")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_reference_large_shape(dtype):
+    # the reference's second test shape (triton_kernel.py:502) with fewer rows so the CPU oracle
+    # finishes in seconds: G*S=8160 queries, N=61380, C=512, Z=1024, d=128; the N > 32K window
+    # leaves ~20% of the buckets empty
+    q, k, v, kh, cnt, qh = make_attn_case(20, 2, 4 * 2040, 1023 * 60, 512, 1024, 128, dtype)
+    assert (cnt == 0).any()
+    out, lse = run_varlen(q, k, v, kh, cnt, qh, 128 ** -0.5)
+    ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 128 ** -0.5)
+    assert_attn_close(out, lse, ro, rl, dtype, "ref large")
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.bfloat16, 64),
+                                     (torch.float32, 40), (torch.bfloat16, 256)])
+def test_attention_dense_buckets(dtype, d):
+    # full-length lists, skewed query groups (one bucket takes half the queries)
+    q, k, v, kh, cnt, qh = make_attn_case(21, 2, 700, 4096, 32, 300, d, dtype, window="all", std=1.0)
+    qh[0, :350] = 5
+    out, lse = run_varlen(q, k, v, kh, cnt, qh, d ** -0.5)
+    ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, d ** -0.5)
+    assert_attn_close(out, lse, ro, rl, dtype, f"dense d={d}")
+
+
+def test_attention_special_cases():
+    # C=1, Z=N: plain softmax attention; Z=1: out = V[idx]
+    g = gen(22)
+    B, S, N, d = 2, 9, 200, 64
+    q, k, v = (torch.randn(B, n, d, generator=g) for n in (S, N, N))
+    kh = torch.stack([torch.randperm(N, generator=g) for _ in range(B)]).reshape(-1)
+    out, lse = run_varlen(q, k, v, kh, torch.full((B, 1), N), torch.zeros(B, S, dtype=torch.long), 0.2)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, scale=0.2)
+    assert torch.allclose(out.cpu(), ref, atol=1e-4)
+    assert torch.allclose(lse.cpu(), torch.logsumexp(q @ k.transpose(1, 2) * 0.2, -1), atol=1e-4)
+    kh1 = torch.tensor([7, 2, 5, 1, 0, 3])
+    qh1 = torch.randint(0, 3, (B, S), generator=g)
+    out, lse = run_varlen(q, k, v, kh1, torch.ones(B, 3, dtype=torch.long), qh1, 0.7)
+    for b in range(B):
+        sel = kh1[b * 3 + qh1[b]]
+        assert torch.allclose(out[b].cpu(), v[b, sel], atol=1e-6)
+        assert torch.allclose(lse[b].cpu(), 0.7 * (q[b] * k[b, sel]).sum(-1), atol=1e-4)
+
+
+def test_attention_reference_lse_rounding_switch():
+    from fast_memory_amd import attention_hash_varlen
+    q, k, v, kh, cnt, qh = make_attn_case(23, 1, 50, 512, 4, 64, 64, torch.bfloat16, window="all")
+    table = kh.reshape(4, 64)
+    cnt = torch.tensor([[64, 0, 64, 64]])                            # bucket 1 emptied
+    kh = torch.cat([table[0], table[2], table[3]])
+    out, lse = attention_hash_varlen(*dev(q, k, v, kh, cnt, qh), 0.125, lse_dtype=None)
+    assert lse.dtype == torch.bfloat16
+    ro, rl = O.hashed_attention_blocked(q, k, v, kh, cnt, qh, 0.125, ref_lse_rounding=True)
+    empty = qh[0] == 1
+    assert (lse.cpu()[0][empty] == torch.finfo(torch.bfloat16).min).all()
+    assert torch.allclose(lse.cpu().float()[0][~empty], rl.float()[0][~empty], atol=0.07)
+
+
+# ------------------------------------------------------------------ a10
+def test_lse_merge(ops):
+    from fast_memory_amd import update_out_and_lse
+    g = gen(500)
+    oa = torch.randn(3, 40, 128, generator=g)
+    ob = torch.randn(3, 40, 128, generator=g).to(torch.bfloat16)
+    la = torch.randn(3, 40, generator=g) * 5
+    lb = torch.randn(3, 40, generator=g) * 5
+    lb[0, :5] = torch.finfo(torch.float32).min                      # empty block: identity
+    la[1, :5] = torch.finfo(torch.float32).min                      # empty running side: takes the block
+    o0, l0 = update_out_and_lse(None, None, dev(oa), dev(la))
+    assert l0.shape == (3, 40, 1) and o0.dtype == torch.float32
+    o1, l1 = update_out_and_lse(o0.clone(), l0.clone(), dev(ob), dev(lb))
+    rc_o, rc_l = O.lse_merge_closed_form(oa, la, ob.float(), lb)
+    assert torch.allclose(o1.cpu().double(), rc_o, atol=1e-5)
+    ok = rc_l > -1e30
+    assert torch.allclose(l1.squeeze(-1).cpu().double()[ok], rc_l[ok], atol=1e-5)
+    assert torch.equal(o1[0, :5], o0[0, :5]) and torch.equal(l1[0, :5], l0[0, :5])
+    assert torch.allclose(o1[1, :5].cpu(), ob[1, :5].float(), atol=1e-6)
+    # statement-for-statement restatement of the reference agrees where it is well conditioned
+    ro, rl = O.update_out_and_lse(oa.clone(), la.clone().unsqueeze(-1), ob, lb)
+    good = (la > -1e30) & (lb > -1e30)
+    assert torch.allclose(o1.cpu()[good], ro[good], atol=1e-5)
+    assert torch.allclose(l1.cpu().squeeze(-1)[good], rl.squeeze(-1)[good], atol=1e-5)
+
+
+# ------------------------------------------------------------------ a11
+@pytest.mark.parametrize("dtype,H,G,S,L,d,causal", [
+    (torch.float32, 2, 2, 33, 33, 64, True),
+    (torch.bfloat16, 2, 4, 200, 200, 128, True),
+    (torch.bfloat16, 2, 4, 1, 512, 128, True),          # decode: one query sees all local keys
+    (torch.float32, 1, 1, 16, 80, 32, True),            # rectangular, bottom-right aligned
+    (torch.bfloat16, 1, 2, 70, 130, 128, False),
+])
+def test_local_attention(ops, dtype, H, G, S, L, d, causal):
+    g = gen(600)
+    q = torch.randn(1, H * G, S, d, generator=g).to(dtype)
+    k = torch.randn(1, H, L, d, generator=g).to(dtype)
+    v = torch.randn(1, H, L, d, generator=g).to(dtype)
+    out, lse = ops.local_attn_fwd(dev(q[0]), dev(k[0]), dev(v[0]), d ** -0.5, causal)
+    ro, rl = O.local_attention(q, k, v, d ** -0.5, causal)
+    assert_attn_close(out, lse, ro[0], rl[0], dtype, "local")
+
+
+def test_memory_plus_local_equals_joint_softmax(ops):
+    # split test on the GPU path: merge(memory bucket, local keys) == one softmax over the union
+    from fast_memory_amd import Memory
+    g = gen(601)
+    H, G, S, N, L, d, C, Z = 2, 2, 16, 512, 16, 64, 8, 64
+    keys = torch.randn(H, N, d, generator=g)
+    vals = torch.randn(H, N, d, generator=g)
+    A = torch.randn(H, C, d, generator=g)
+    q = torch.randn(H, G * S, d, generator=g)
+    kl = torch.randn(H, L, d, generator=g)
+    vl = torch.randn(H, L, d, generator=g)
+    mem = Memory.build(*dev(keys, vals, A), Z)
+    out, lse = mem.attend_with_local(dev(q), dev(kl), dev(vl), 0.125, n_groups=G, causal=False)
+    lists = mem.bucket_idx.cpu().long()
+    qh = mem.hash(dev(q)).cpu().long()
+    for h in range(H):
+        for i in range(0, G * S, 5):
+            idx = lists[h, qh[h, i]]
+            kk = torch.cat([keys[h, idx], kl[h]]).double()
+            vv = torch.cat([vals[h, idx], vl[h]]).double()
+            s = kk @ q[h, i].double() * 0.125
+            assert abs(torch.logsumexp(s, 0).item() - lse[h, i].item()) < 1e-4
+            assert torch.allclose(torch.softmax(s, 0) @ vv, out[h, i].cpu().double(), atol=1e-4)
+
+
+# ------------------------------------------------------------------ a12/a13
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_compute_centroids(ops, dtype):
+    from fast_memory_amd import compute_centroids, init_centroids
+    g = gen(700)
+    H, G, N, d, C, topk = 2, 2, 600, 64, 16, 8
+    kq = torch.randn(H * G, N, d, generator=g).to(dtype)
+    cent = O.init_centroids(C, d, dtype)
+    assert torch.equal(init_centroids(C, d, "cuda", dtype).cpu(), cent)
+    A = compute_centroids(dev(kq), dev(cent), C, G, topk, normalize=True).cpu()
+    ref = O.compute_centroids(kq, cent, C, G, topk, normalize=True)
+    assert A.shape == (C, H, d)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(A.float(), ref.float(), atol=tol), (A.float() - ref.float()).abs().max()
+
+
+def test_kmeans_matches_oracle_fp32(ops):
+    from fast_memory_amd import kmeans_spherical
+    g = gen(701)
+    H, N, d, C = 2, 3000, 64, 24
+    X = O.l2_normalize(torch.randn(H, N, d, generator=g))
+    init = O.l2_normalize(O.init_centroids(C, d)).unsqueeze(0).expand(H, -1, -1).contiguous()
+    cent, labels = kmeans_spherical(dev(X), dev(init), 2)
+    for h in range(H):
+        rc, rl = O.kmeans_spherical(X[h], init[h], 2)
+        agree = (labels[h].cpu().long() == rl).float().mean().item()
+        assert agree > 0.999, agree                                 # fp32 vs fp64 near-ties only
+        assert torch.allclose(cent[h].cpu().double(), rc, atol=1e-4)
+    assert torch.allclose(cent.norm(dim=-1).cpu(), torch.ones(H, C), atol=1e-5)
+
+
+def test_l2_normalize(ops):
+    X = torch.randn(37, 128, generator=gen(702))
+    X[3] = 0
+    got = ops.l2_normalize(dev(X)).cpu()
+    assert torch.allclose(got, O.l2_normalize(X), atol=1e-6)
+    assert (got[3] == 0).all()
+
+
+# ------------------------------------------------------------------ a15 composite, config c1
+def test_config1_toy_end_to_end(ops):
+    from fast_memory_amd import Memory, fit_projection
+    g = gen(1001)
+    d, N, C, Z, S = 64, 4096, 64, 256, 512
+    K = torch.randn(1, N, d, generator=g)
+    V = torch.randn(1, N, d, generator=g)
+    Q = torch.randn(1, S, d, generator=g)
+    A = fit_projection(dev(K), C, iters=1)
+    Xn = O.l2_normalize(K[0])
+    ref_A, _ = O.kmeans_spherical(Xn, O.l2_normalize(O.init_centroids(C, d)), 1)
+    assert torch.allclose(A[0].cpu().double(), ref_A, atol=1e-4)
+    mem = Memory.build(dev(K), dev(V), A, Z)
+    Y = ops.project(A, dev(K)).cpu()
+    assert torch.equal(mem.bucket_idx.cpu().long(), O.argtopz(Y, Z))            # bit-exact given the same Y
+    qh, sc = ops.qhash(A, dev(Q), return_scores=True)
+    assert torch.equal(qh.cpu().long(), O.argmax_first(sc.cpu()))
+    out, lse = mem.attend(dev(Q), d ** -0.5)
+    cnt = torch.full((1, C), Z)
+    ro, rl = O.hashed_attention_gather(Q, K, V, mem.bucket_idx.cpu().long().reshape(-1), cnt, qh.cpu().long(),
+                                       d ** -0.5)
+    assert_attn_close(out, lse, ro, rl, torch.float32, "c1")
+
+
+def test_ring_attention_masked_forward_windows(ops):
+    from fast_memory_amd import ring_attention_masked_forward
+    g = gen(800)
+    C, H, G, S, N, Z, d, world = 6, 2, 2, 20, 256, 40, 64, 2
+    q = torch.randn(1, H * G, S, d, generator=g).to(torch.bfloat16)
+    kh = torch.stack([torch.stack([torch.randperm(world * N, generator=g)[:Z] for _ in range(H)]) for _ in range(C)])
+    qh = torch.randint(0, C, (H, G, S), generator=g)
+    for rank in range(world):
+        k = torch.randn(1, H, N, d, generator=g).to(torch.bfloat16)
+        v = torch.randn(1, H, N, d, generator=g).to(torch.bfloat16)
+        out, lse = ring_attention_masked_forward(*dev(kh, qh, q, k, v), 0.125, rank)
+        ro, rl = O.ring_attention_masked_forward(kh, qh, q, k, v, 0.125, rank)
+        assert out.shape == (1, H * G, S, d) and lse.shape == (1, H * G, S)
+        assert_attn_close(out[0], lse[0], ro[0], rl[0], torch.bfloat16, f"ring rank {rank}")

@@ -425,6 +425,7 @@ def compute_centroids(kq, centroids, n_hashes, n_groups, centroid_topk, normaliz
     H = n_heads // n_groups
     x = kq.double()
     x = x / x.norm(dim=-1, keepdim=True).clamp(min=1e-6)
+    x = x.to(kq.dtype).double()          # the reference keeps kq_hash in the input dtype (mem:217)
     scores = torch.einsum('zd,hid->zhi', centroids.double(), x)        # C HG N
     top = argtopz(scores.float(), centroid_topk)                        # C HG k
     h_idx = torch.arange(n_heads)

@@ -1,17 +1,353 @@
-// placeholder until the MFMA attention kernels land
+// bf16 attention on MFMA for head dimension 128 (gfx950): the bucket-gathered
+// forward (triton_kernel.py:137-272) and the dense local attention it is merged
+// with (call site memory.py:302).
+//
+// Work decomposition.  One workgroup (4 waves) per work item = up to 64 queries
+// that hashed to the same (row, bucket).  The bucket's key list is cut into
+// blocks of 32 keys dealt round-robin to the four waves; every wave runs its own
+// online softmax over its blocks for all the item's queries and the four partial
+// (m, l, O) triples are merged through LDS at the end.  K and V rows of a bucket
+// are therefore read from HBM once per item, whatever the number of queries.
+//
+// Data path.  No LDS in the main loop: gathered rows go from global memory
+// straight into MFMA operand registers.
+//   S^T = K.Q^T   v_mfma_f32_16x16x32_bf16, A = 16 gathered K rows (lane c of
+//                 lane group g reads 16 bytes at column 32s+8g of row c), B =
+//                 Q^T fragments kept in registers for the whole item.  Lane
+//                 (g,c) ends up with scores of keys 4g..4g+3 for query c.
+//   O^T += V^T.P^T  same instruction over a 32-key block: the accumulator
+//                 layout of S^T is already the B-operand layout (keys along
+//                 the contraction), so P needs no shuffle.  V rows are read
+//                 fully coalesced (16 lanes x 16 B = one 256-byte row): lane
+//                 (g,c) reads column chunk c of keys 4g..4g+3; transposing to
+//                 the A-operand layout is a per-lane repack because output
+//                 tile t takes column 8c+t of every chunk.  Lane (g,c) then
+//                 holds O[query c][32g .. 32g+31].
+// Softmax follows the reference kernel: base-2 with sm_scale*log2(e), fp32
+// running max / denominator, denominator from unrounded p, p rounded to bf16
+// before P.V (triton_kernel.py:248-263).
+//
+// Roofline: HBM.  Algorithmic bytes per item = cnt*(2*128*2 + 4) + n_q*(2*128*2
+// + 4).  Per 32-key block a wave issues 16 KiB of loads and keeps one block in
+// flight behind the one it is computing on.
 #include "common.hpp"
+
 namespace fm {
-bool hash_attn_mfma_supported(int, int) { return false; }
-int hash_attn_mfma(const void*, const void*, const void*, const int32_t*, const int64_t*,
-                   const int32_t*, const int32_t*, const fm_item*, const int32_t*, int64_t, void*,
-                   float*, int, int, int, int, float, hipStream_t) {
-  set_error("hash_attn_mfma: not built");
-  return FM_ERR_UNSUPPORTED;
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+constexpr int kD = 128;
+constexpr int kNQT = FM_QTILE / 16;  // query tiles of 16 per item
+constexpr int kBlk = 32;             // keys per block (two MFMA key tiles)
+
+struct KVRegs {
+  uint4 k[2][4];  // [key tile][contraction step]
+  uint4 v[2][4];  // [key tile][key 4g+j]
+};
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 u) {
+  union {
+    uint4 u;
+    bf16x8 b;
+  } x;
+  x.u = u;
+  return x.b;
 }
-bool local_attn_mfma_supported(int, int) { return false; }
-int local_attn_mfma(const void*, const void*, const void*, void*, float*, int, int, int, int, int,
-                    float, int, hipStream_t) {
-  set_error("local_attn_mfma: not built");
-  return FM_ERR_UNSUPPORTED;
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
 }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Issues the loads of one 32-key block.  `rows` holds, in lanes 0..31 (and again
+// in 32..63), the key row of block position lane%32 (already clamped to [0,N)).
+__device__ __forceinline__ void load_block(KVRegs& r, const bf16_t* __restrict__ Kb,
+                                           const bf16_t* __restrict__ Vb, int rows, int g, int c) {
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt) {
+    const int rk = __shfl(rows, kt * 16 + c);
+    const uint4* pk = reinterpret_cast<const uint4*>(Kb + int64_t(rk) * kD + 8 * g);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) r.k[kt][s] = pk[4 * s];  // column 32s + 8g
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int rv = __shfl(rows, kt * 16 + 4 * g + j);
+      r.v[kt][j] = *reinterpret_cast<const uint4*>(Vb + int64_t(rv) * kD + 8 * c);
+    }
+  }
+}
+
+// CAUSAL = false: gathered bucket (rows come from an index list).
+// CAUSAL = true : contiguous keys [0, cnt) with per-query visibility limit.
+template <bool CAUSAL>
+__device__ __forceinline__ void attend_item(
+    const bf16_t* __restrict__ Qb,   // query rows of this item's row/head: [*, 128]
+    const int* __restrict__ q_rows,  // LDS: row index (into Qb / out) of the item's queries
+    int n_q, const bf16_t* __restrict__ Kb, const bf16_t* __restrict__ Vb,
+    const int32_t* __restrict__ idx,  // bucket list (nullptr when CAUSAL)
+    int cnt, int N, int vis0,         // CAUSAL: query j of the item sees keys < vis0 + j + 1
+    float scale2, bf16_t* __restrict__ Ob, float* __restrict__ Lb, float* __restrict__ red) {
+  const int l = lane_id(), w = threadIdx.x >> 6;
+  const int g = l >> 4, c = l & 15;
+  const int nqt = (n_q + 15) >> 4;
+
+  // ---- Q^T fragments -------------------------------------------------------
+  uint4 qf[kNQT][4];
+#pragma unroll
+  for (int qt = 0; qt < kNQT; ++qt) {
+    const int j = qt * 16 + c;
+    const bool ok = (qt < nqt) && (j < n_q);
+    const uint4* pq = reinterpret_cast<const uint4*>(Qb + int64_t(ok ? q_rows[j] : 0) * kD + 8 * g);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) qf[qt][s] = ok ? pq[4 * s] : make_uint4(0, 0, 0, 0);
+  }
+
+  f32x4 O[kNQT][8];
+  float m[kNQT], lsum[kNQT];
+#pragma unroll
+  for (int qt = 0; qt < kNQT; ++qt) {
+    m[qt] = -INFINITY;
+    lsum[qt] = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) O[qt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int nblk = (cnt + kBlk - 1) / kBlk;
+  auto rows_of = [&](int b) -> int {
+    const int kp = b * kBlk + (l & 31);
+    int r = 0;
+    if (kp < cnt) r = CAUSAL ? kp : idx[kp];
+    return min(max(r, 0), N - 1);
+  };
+
+  auto compute = [&](const KVRegs& kv, int b) {
+    const int kp0 = b * kBlk;
+    // V^T fragments for the 8 output tiles: element t of the 8 loads of this lane
+    uint4 vf[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const int dw = t >> 1;
+      uint32_t a[8];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint4 x = kv.v[kt][j];
+          a[kt * 4 + j] = dw == 0 ? x.x : dw == 1 ? x.y : dw == 2 ? x.z : x.w;
+        }
+      uint32_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        o[e] = (t & 1) ? ((a[2 * e] >> 16) | (a[2 * e + 1] & 0xffff0000u))
+                       : ((a[2 * e] & 0xffffu) | (a[2 * e + 1] << 16));
+      vf[t] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    const bool tail = CAUSAL || (kp0 + kBlk > cnt);
+#pragma unroll
+    for (int qt = 0; qt < kNQT; ++qt) {
+      if (qt < nqt) {
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kv.k[0][s]), as_bf16x8(qf[qt][s]), s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kv.k[1][s]), as_bf16x8(qf[qt][s]), s1, 0, 0, 0);
+        }
+        float x[8];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          x[r] = s0[r] * scale2;
+          x[4 + r] = s1[r] * scale2;
+        }
+        if (tail) {
+          int lim = cnt;
+          if (CAUSAL) lim = min(cnt, vis0 + qt * 16 + c + 1);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            if (kp0 + 4 * g + r >= lim) x[r] = -INFINITY;
+            if (kp0 + 16 + 4 * g + r >= lim) x[4 + r] = -INFINITY;
+          }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])),
+                         fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m[qt], mx);
+        // a query that sees no key yet keeps m = -inf; subtract 0 instead of -inf
+        const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2(m[qt] - m_sub);
+        m[qt] = m_new;
+        float p[8], ps = 0.f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          p[r] = fast_exp2(x[r] - m_sub);
+          ps += p[r];
+        }
+        lsum[qt] = lsum[qt] * alpha + ps;
+        const uint4 pf = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]),
+                                    pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          f32x4 o = O[qt][t];
+          o[0] *= alpha;
+          o[1] *= alpha;
+          o[2] *= alpha;
+          o[3] *= alpha;
+          O[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[t]), as_bf16x8(pf), o, 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  // ---- main loop: this wave's blocks w, w+4, ..., one block in flight -------
+  KVRegs ra, rb;
+  int b = w;
+  // key rows are fetched two blocks ahead of the block being computed, K/V one ahead
+  if (b < nblk) load_block(ra, Kb, Vb, rows_of(b), g, c);
+  int r1 = rows_of(b + 4);
+  while (b < nblk) {
+    const int b1 = b + 4, b2 = b + 8;
+    const int r2 = rows_of(b2);
+    if (b1 < nblk) load_block(rb, Kb, Vb, r1, g, c);
+    compute(ra, b);
+    if (b1 >= nblk) break;
+    const int r3 = rows_of(b2 + 4);
+    if (b2 < nblk) load_block(ra, Kb, Vb, r2, g, c);
+    compute(rb, b1);
+    r1 = r3;
+    b = b2;
+  }
+
+  // ---- merge the four waves ---------------------------------------------------
+  // red layout (floats): O part [wave][qt][t][r][lane], then l [wave][qt][lane],
+  // then m [wave][qt][16]
+  float* redO = red;
+  float* redL = red + 4 * kNQT * 8 * 4 * 64;
+  float* redM = redL + 4 * kNQT * 64;
+#pragma unroll
+  for (int qt = 0; qt < kNQT; ++qt) {
+    if (qt < nqt) {
+#pragma unroll
+      for (int t = 0; t < 8; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) redO[(((w * kNQT + qt) * 8 + t) * 4 + r) * 64 + l] = O[qt][t][r];
+      redL[(w * kNQT + qt) * 64 + l] = lsum[qt];
+      if (g == 0) redM[(w * kNQT + qt) * 16 + c] = m[qt];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int qt = 0; qt < kNQT; ++qt) {
+    if (qt < nqt) {
+      float mw[4], mstar = -INFINITY;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) {
+        mw[ww] = redM[(ww * kNQT + qt) * 16 + c];
+        mstar = fmaxf(mstar, mw[ww]);
+      }
+      const int j = qt * 16 + c;
+      float f[4], lstar = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) {
+        f[ww] = (mw[ww] == -INFINITY) ? 0.f : fast_exp2(mw[ww] - mstar);
+        float lw = 0.f;
+#pragma unroll
+        for (int gg = 0; gg < 4; ++gg) lw += redL[(ww * kNQT + qt) * 64 + gg * 16 + c];
+        lstar += f[ww] * lw;
+      }
+      const bool empty = (mstar == -INFINITY);  // the query saw no key at all
+      const float inv = empty ? 0.f : 1.f / lstar;
+      // wave w finalises accumulator row r = w: columns 32g + 8w + (0..7) of query c
+      float o[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        float a = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < 4; ++ww) a += f[ww] * redO[(((ww * kNQT + qt) * 8 + t) * 4 + w) * 64 + l];
+        o[t] = a * inv;
+      }
+      if (j < n_q) {
+        const int64_t qr = q_rows[j];
+        uint4 st = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]),
+                              pack_bf16(o[6], o[7]));
+        *reinterpret_cast<uint4*>(Ob + qr * kD + 32 * g + 8 * w) = st;
+        if (w == 0 && g == 0) Lb[qr] = empty ? -FLT_MAX : (mstar + __builtin_amdgcn_logf(lstar)) * kLn2;
+      }
+    }
+  }
+}
+
+constexpr int kRedFloats = 4 * kNQT * 8 * 4 * 64 + 4 * kNQT * 64 + 4 * kNQT * 16;
+
+__global__ __launch_bounds__(256) void hash_attn_mfma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off,
+    const int32_t* __restrict__ bucket_cnt, const int32_t* __restrict__ q_perm,
+    const fm_item* __restrict__ items, const int32_t* __restrict__ n_items,
+    bf16_t* __restrict__ out, float* __restrict__ lse, int Sq, int N, int C, float scale2) {
+  extern __shared__ __attribute__((aligned(16))) float red[];
+  __shared__ int q_rows[FM_QTILE];
+  if (int(blockIdx.x) >= *n_items) return;
+  const fm_item it = items[blockIdx.x];
+  const int64_t bkt = int64_t(it.row) * C + it.bucket;
+  const int cnt = bucket_cnt[bkt];
+  if (threadIdx.x < it.n_q) q_rows[threadIdx.x] = q_perm[it.q_start + threadIdx.x];
+  __syncthreads();
+  const int64_t qbase = int64_t(it.row) * Sq;
+  attend_item<false>(q + qbase * kD, q_rows, it.n_q, k + int64_t(it.row) * N * kD,
+                     v + int64_t(it.row) * N * kD, k_idx + bucket_off[bkt], cnt, N, 0, scale2,
+                     out + qbase * kD, lse + qbase, red);
+}
+
+// Dense local attention: one workgroup per (query head, tile of 64 consecutive queries).
+__global__ __launch_bounds__(256) void local_attn_mfma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    bf16_t* __restrict__ out, float* __restrict__ lse, int G, int S, int L, float scale2,
+    int causal) {
+  extern __shared__ __attribute__((aligned(16))) float red[];
+  __shared__ int q_rows[FM_QTILE];
+  const int hq = blockIdx.y, hk = hq / G;
+  const int i0 = blockIdx.x * FM_QTILE;
+  const int n_q = min(FM_QTILE, S - i0);
+  if (threadIdx.x < FM_QTILE) q_rows[threadIdx.x] = i0 + threadIdx.x;
+  __syncthreads();
+  const int64_t qbase = int64_t(hq) * S;
+  // keys any query of the tile can see; per-query limit applied inside
+  int cnt = L, vis0 = L;  // non-causal: every query sees all L keys
+  if (causal) {
+    vis0 = i0 + (L - S);                       // query j of the tile sees keys < vis0 + j + 1
+    cnt = min(L, max(0, vis0 + n_q));
+  }
+  attend_item<true>(q + qbase * kD, q_rows, n_q, k + int64_t(hk) * L * kD, v + int64_t(hk) * L * kD,
+                    nullptr, cnt, L, vis0, scale2, out + qbase * kD, lse + qbase, red);
+}
+
+bool hash_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_BF16; }
+bool local_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_BF16; }
+
+int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                   const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                   const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
+                   float* lse, int Sq, int N, int d, int C, float sm_scale, hipStream_t st) {
+  (void)d;
+  FM_ALLOW_LDS(hash_attn_mfma_kernel, kRedFloats * sizeof(float), "fm_hash_attn_fwd: lds");
+  hipLaunchKernelGGL(hash_attn_mfma_kernel, dim3(unsigned(max_items)), dim3(256),
+                     kRedFloats * sizeof(float), st, (const bf16_t*)q, (const bf16_t*)k,
+                     (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
+                     (bf16_t*)out, lse, Sq, N, C, sm_scale * kLog2e);
+  return launch_status("fm_hash_attn_fwd(mfma)");
+}
+
+int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
+                    int S, int L, int d, float sm_scale, int causal, hipStream_t st) {
+  (void)d;
+  FM_ALLOW_LDS(local_attn_mfma_kernel, kRedFloats * sizeof(float), "fm_local_attn_fwd: lds");
+  dim3 grid = dim3(unsigned(ceil_div(S, FM_QTILE)), unsigned(H * G));
+  hipLaunchKernelGGL(local_attn_mfma_kernel, grid, dim3(256), kRedFloats * sizeof(float), st,
+                     (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)out, lse, G, S,
+                     L, sm_scale * kLog2e, causal);
+  return launch_status("fm_local_attn_fwd(mfma)");
+}
+
 }  // namespace fm

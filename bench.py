@@ -1,0 +1,254 @@
+#!/usr/bin/env python3
+"""Benchmark of the indexed-memory hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c5|c2|c1|c4]
+
+One "step" is one pass of the query path over the whole synthetic batch, inputs
+already resident in HBM: query hash -> grouping -> bucket-gathered attention ->
+(dense local attention -> LSE merge, where the configuration has local keys).
+``value`` is query-heads per second over K timed steps.  The index build
+(projection + arg-top-Z) and the K-means that produces A are timed beside it
+and reported in the same JSON line, as are the roofline figures of the
+dominant kernel and a CPU baseline on a bounded sample of the same workload.
+Prints exactly one JSON line on stdout; progress goes to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def ev_pair():
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def timed(fn, reps=1, warm=1):
+    """Average milliseconds of fn() over `reps` runs, HIP events on the current stream."""
+    for _ in range(warm):
+        fn()
+    a, b = ev_pair()
+    a.record()
+    for _ in range(reps):
+        r = fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps, r
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c5", choices=["c1", "c2", "c4", "c5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--workspace-gib", type=float, default=8.0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build measures one GPU (one MI355X holds a whole memory at its real "
+                 "shape); run it with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; there is no CPU path to time")
+
+    from fast_memory_amd import Memory, fit_projection, ops, synth, update_out_and_lse
+    from fast_memory_amd import _lib
+    _lib.load()
+    cfg = synth.CONFIGS[args.config]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    H, G, d, N, C, Z, S = cfg.H, cfg.G, cfg.d, cfg.N, cfg.C, cfg.Z, cfg.S
+    Sq = G * S
+    e = 2 if cfg.dtype == torch.bfloat16 else 4
+    sm_scale = d ** -0.5
+    ws_bytes = int(args.workspace_gib * (1 << 30))
+
+    t0 = time.time()
+    wl = synth.make_workload(cfg, dev)
+    torch.cuda.synchronize()
+    log(f"[bench] {cfg.name}: inputs generated in {time.time() - t0:.1f}s "
+        f"(keys {tuple(wl.keys.shape)} {wl.keys.dtype})")
+
+    # ---- A by spherical K-means, index build (both timed, outside the step) ----
+    km_ms, A = timed(lambda: fit_projection(wl.keys, C, iters=cfg.kmeans_iters), reps=1, warm=0)
+    log(f"[bench] K-means ({cfg.kmeans_iters} iterations): {km_ms:.1f} ms")
+    build_ms, mem = timed(lambda: Memory.build(wl.keys, wl.values, A, Z, workspace_bytes=ws_bytes), reps=2, warm=1)
+    keys_per_s = H * N / (build_ms * 1e-3)
+    log(f"[bench] index build: {build_ms:.1f} ms  ({keys_per_s / 1e6:.1f} M keys/s)")
+
+    # component kernels of the build on one chunk of rows
+    rows = min(C, max(1, min(512, ws_bytes // (N * 4))))
+    Asub = A[:1, :rows].contiguous()
+    proj_ms, Y = timed(lambda: ops.project(Asub, wl.keys[:1]), reps=3, warm=1)
+    sel_ms, _ = timed(lambda: ops.argtopz(Y, Z), reps=3, warm=1)
+    proj_flops = 2.0 * rows * N * d
+    proj_bytes = rows * N * 4 + (rows + N) * d * e
+    sel_bytes = rows * N * 4 + rows * min(Z, N) * 4
+    del Y
+    build_parts = {
+        "chunk_rows": rows,
+        "project": {"ms": proj_ms, "tflops": proj_flops / proj_ms / 1e9,
+                    "mfma_frac": proj_flops / proj_ms / 1e9 / BF16_MFMA_PEAK_TFLOPS,
+                    "hbm_gbs": proj_bytes / proj_ms / 1e6, "hbm_frac": proj_bytes / proj_ms / 1e6 / HBM_PEAK_GBS},
+        "argtopz": {"ms": sel_ms, "hbm_gbs": sel_bytes / sel_ms / 1e6,
+                    "hbm_frac": sel_bytes / sel_ms / 1e6 / HBM_PEAK_GBS},
+    }
+    log(f"[bench] project {rows}x{N}: {proj_ms:.2f} ms, {build_parts['project']['tflops']:.1f} TFLOP/s, "
+        f"{build_parts['project']['hbm_gbs']:.0f} GB/s; argtopz: {sel_ms:.2f} ms, "
+        f"{build_parts['argtopz']['hbm_gbs']:.0f} GB/s (algorithmic)")
+
+    q = wl.queries
+    has_local = wl.k_local is not None
+    attn_events = []
+    part_events = {"qhash": [], "group": [], "local": [], "merge": []}
+
+    def step(record=True):
+        e0, e1 = ev_pair()
+        e0.record()
+        qh = mem.hash(q)
+        e1.record()
+        g0, g1 = ev_pair()
+        groups = ops.group_queries(qh, C)
+        g1.record()
+        a0, a1 = ev_pair()
+        a0.record()
+        mo, ml = ops.hash_attn_fwd(q, mem.keys, mem.values, mem.bucket_idx.reshape(-1), mem.bucket_off,
+                                   mem.bucket_cnt, groups, sm_scale)
+        a1.record()
+        if has_local:
+            l1, m1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            lo, ll = ops.local_attn_fwd(q.reshape(H * G, S, d), wl.k_local, wl.v_local, sm_scale, True)
+            l1.record()
+            out, lse = update_out_and_lse(None, None, lo.reshape(H, Sq, d), ll.reshape(H, Sq))
+            out, lse = update_out_and_lse(out, lse, mo, ml)
+            m1.record()
+        else:
+            out, lse = mo, ml
+        if record:
+            attn_events.append((a0, a1))
+            part_events["qhash"].append((e0, e1))
+            part_events["group"].append((e1, g1))
+            if has_local:
+                part_events["local"].append((a1, l1))
+                part_events["merge"].append((l1, m1))
+        return out, lse, qh, groups, mo, ml
+
+    for _ in range(args.warmup):
+        step(record=False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        res = step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    qheads = H * Sq
+    value = qheads / (ms_per_step * 1e-3)
+    out, lse, qh, groups, mo, ml = res
+
+    attn_ms = sum(a.elapsed_time(b) for a, b in attn_events) / len(attn_events)
+    parts_ms = {k: (sum(a.elapsed_time(b) for a, b in v) / len(v) if v else None) for k, v in part_events.items()}
+    # algorithmic bytes of the gather-attention launch: every hit bucket once + q, out, lse
+    hit = int((groups.bin_count > 0).sum().item())
+    alg_bytes = hit * Z * (2 * d * e + 4) + qheads * (2 * d * e + 4)
+    alg_flops = 4.0 * d * Z * qheads
+    achieved = alg_bytes / attn_ms / 1e6
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(f"hash_attn_mfma_kernel/{cfg.name}")
+        except Exception:
+            traffic = None
+    roofline = {"kernel": "hash_attn_mfma_kernel" if (d == 128 and e == 2) else "hash_attn_generic_kernel",
+                "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms,
+                "hit_buckets": hit, "mfma_tflops": alg_flops / attn_ms / 1e9}
+    log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M query-heads/s; attention kernel "
+        f"{attn_ms:.2f} ms = {achieved:.0f} GB/s algorithmic ({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak); "
+        f"parts {parts_ms}")
+
+    # ---- CPU baseline on a bounded sample (head 0), also used as a parity spot check ----
+    cpu = None
+    parity = None
+    if not args.no_cpu_baseline:
+        from oracle import cpu_path
+        threads = min(16, os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        K0, V0, A0 = wl.keys[0].cpu(), wl.values[0].cpu(), A[0].cpu()
+        lists0 = mem.bucket_idx[0].cpu().long()
+        q0 = q[0].cpu()
+        kl0 = wl.k_local[0].cpu() if has_local else None
+        vl0 = wl.v_local[0].cpu() if has_local else None
+        n = min(32, Sq)
+        pick = lambda m: torch.linspace(0, Sq - 1, m).long()        # spread over heads and positions
+        sel = pick(n)
+        t_probe = cpu_path.time_query_path(q0[sel], K0, V0, A0, lists0, sm_scale, kl0, vl0, sel % S, S)
+        n = int(max(n, min(Sq, n * args.cpu_seconds / max(t_probe, 1e-3))))
+        sel = pick(n)
+        t_cpu = cpu_path.time_query_path(q0[sel], K0, V0, A0, lists0, sm_scale, kl0, vl0, sel % S, S)
+        # index-build sample: a few rows of A against all keys of head 0
+        r = 2 if N > 200000 else 16
+        tb0 = time.perf_counter()
+        cpu_lists = cpu_path.build_rows(A0[:r], K0, Z)
+        t_build = time.perf_counter() - tb0
+        cpu = {"value": n / t_cpu, "unit": "query-heads/s", "cores": threads, "kind": "port",
+               "sample": f"KV head 0, {n} of its {Sq} query-heads evenly spaced, full N={N}, C={C}, Z={Z}; hash + per-bucket "
+                         f"gathered softmax attention" + (" + causal local attention + merge" if has_local else "")
+                         + f"; {t_cpu:.2f} s",
+               "index_build_rows_per_s": r / t_build,
+               "index_build_keys_per_s_extrapolated": N / (C * t_build / r),
+               "index_build_sample": f"{r} of {C} bucket rows of head 0 against all {N} keys, {t_build:.2f} s"}
+        # parity spot check of the GPU results on the same sample
+        co, cl, ch = cpu_path.hashed_attention(q0[sel], K0, V0, A0, lists0, sm_scale)
+        gh = qh[0].cpu().long()[sel]
+        same = gh == ch
+        go, gl = mo[0].float().cpu()[sel], ml[0].cpu()[sel]
+        parity = {"hash_agree_frac": same.float().mean().item(),
+                  "out_max_abs_err": (go[same] - co[same]).abs().max().item(),
+                  "lse_max_abs_err": (gl[same] - cl[same]).abs().max().item(),
+                  "bucket_rows_bit_exact_vs_cpu_stable_sort_of_gpu_Y": None}
+        Yg = ops.project(A[:1, :r].contiguous(), wl.keys[:1])[0].cpu()
+        ref_lists = torch.sort(Yg + 0.0, dim=-1, descending=True, stable=True)[1][:, :min(Z, N)]
+        parity["bucket_rows_bit_exact_vs_cpu_stable_sort_of_gpu_Y"] = bool(
+            torch.equal(ref_lists, mem.bucket_idx[0, :r].cpu().long()))
+        log(f"[bench] cpu baseline: {cpu['value']:.1f} query-heads/s on {threads} threads; parity {parity}")
+
+    line = {
+        "metric": "hashed-attn query-heads/s",
+        "value": value, "unit": "query-heads/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if e == 2 else "f32", "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: H={H} KV heads, G={G}, d={d}, N={N} keys/head, C={C}, Z={Z}, "
+                               f"S={S} tokens/q-head ({qheads} query-heads)"
+                               + (f", {wl.k_local.shape[1]} local keys causal + LSE merge" if has_local else ""),
+                   "step": "qhash + group + gather attention" + (" + local attention + merge" if has_local else "")},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "index_build": {"keys_per_s": keys_per_s, "ms": build_ms, "keys": H * N, "parts": build_parts,
+                        "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters},
+        "step_parts_ms": {"attention": attn_ms, **parts_ms},
+        "parity_spot_check": parity,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -60,6 +60,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--workspace-gib", type=float, default=8.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch copy_probe_kernel over 1 GiB (the known-size kernel profiler "
+                         "HBM counters are scaled against)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures one GPU (one MI355X holds a whole memory at its real "
@@ -170,12 +173,12 @@ def main():
     alg_flops = 4.0 * d * Z * qheads
     achieved = alg_bytes / attn_ms / 1e6
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    # measured offline with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) and kept as text under profiles/
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
     if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get(f"hash_attn_mfma_kernel/{cfg.name}")
-        except Exception:
-            traffic = None
+        for ln in open(tpath):
+            if ln.strip().startswith(f"hash_attn_mfma_kernel/{cfg.name}") and "=" in ln:
+                traffic = float(ln.split("=")[1])
     roofline = {"kernel": "hash_attn_mfma_kernel" if (d == 128 and e == 2) else "hash_attn_generic_kernel",
                 "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
@@ -184,6 +187,15 @@ def main():
     log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M query-heads/s; attention kernel "
         f"{attn_ms:.2f} ms = {achieved:.0f} GB/s algorithmic ({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak); "
         f"parts {parts_ms}")
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(_lib.load().fm_debug_copy(dst.data_ptr(), src.data_ptr(), src.numel(),
+                                                 torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- CPU baseline on a bounded sample (head 0), also used as a parity spot check ----
     cpu = None

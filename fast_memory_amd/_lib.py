@@ -47,6 +47,7 @@ SIGNATURES = {
     "fm_topk_mean": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_segment_mean": (c_int, [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_debug_force_generic": (None, [c_int]),
+    "fm_debug_copy": (c_int, [P, P, c_int64, P]),
 }
 
 _lib = None

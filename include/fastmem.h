@@ -172,6 +172,10 @@ int fm_segment_mean(const void* X, const int32_t* perm, const int32_t* seg_off,
  * (used by tests to compare the two implementations), 0 restores dispatch. */
 void fm_debug_force_generic(int on);
 
+/* Diagnostic: streaming copy of nbytes (multiple of 16) device to device; the
+ * known-size kernel that profiler HBM counters are calibrated against. */
+int fm_debug_copy(void* dst, const void* src, int64_t nbytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -28,6 +28,8 @@ SIGNATURES = {
     "fm_argtopz_f32": (c_int, [P, c_int64, c_int, c_int64, c_int, P, P, c_size_t, P]),
     "fm_build_index_workspace": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int64]),
     "fm_build_index": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P]),
+    "fm_build_index_fused_workspace": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "fm_build_index_fused": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P, P]),
     "fm_qhash": (c_int, [P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_window_filter_workspace": (c_size_t, [c_int64]),
     "fm_window_filter": (c_int, [P, c_int64, c_int, c_int64, c_int64, P, P, P, P, c_size_t, P]),

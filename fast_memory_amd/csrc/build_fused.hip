@@ -1,0 +1,396 @@
+// Fused index build (memory.py:260-278 on one device) that never writes the
+// projection Y = A.K^T to memory.
+//
+//   phase 0  per-row threshold.  Y is computed for a strided sample of the keys
+//            (every `stride`-th key, 32 Ki - 64 Ki of them) with the ordinary
+//            projection kernel, and the `rank`-th largest sampled value of every
+//            (head, bucket) row becomes that row's threshold tau; `rank` sits six
+//            standard deviations above Z*ns/N, so with overwhelming probability
+//            at least Z keys of the full row reach tau and not many more.
+//   phase 1  fused_filter_kernel: bf16 MFMA GEMM over all keys with an epilogue
+//            that keeps only elements >= tau.  Keys are the M side of the MFMA
+//            tile and buckets the N side, so in the accumulator layout one lane
+//            owns one bucket column: its threshold, its write cursor and its
+//            private segment of the row's candidate buffer live in registers and
+//            survivors are appended with plain stores -- no atomics.
+//   phase 2  cand_select_kernel: exact top-Z (value desc, index asc) of each
+//            row's candidates: radix select + in-LDS bitonic sort, the same code
+//            as the dense arg-top-Z kernel, reading ~1.2 Z candidates instead of
+//            the N-element row.
+//   phase 3  repair.  A row whose candidate count fell short of Z or overflowed
+//            a segment is listed by phase 2; its Y row is recomputed (same MFMA
+//            instruction and contraction order) into a small buffer and handed to
+//            the dense arg-top-Z kernel.  Up to kMaxRepair rows are repaired on
+//            the device; status_dev reports how many were, and how many were left
+//            (the caller then falls back to the unfused build).
+//
+// Results are bit-identical to fm_project + fm_argtopz_f32: both compute every Y
+// element with v_mfma_f32_32x32x16_bf16 in ascending 16-element steps with keys
+// on the A operand.
+//
+// Roofline of phase 1: MFMA, 2*d flops per (key, bucket) pair; K is re-read once
+// per 512-bucket slab from L2.  Phases 0, 2, 3 are HBM/L2-bound and small.
+#include "mfma_tile.hpp"
+#include "select.hpp"
+
+namespace fm {
+
+int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out,
+                   const int32_t* row_map, const int32_t* n_rows_dev, hipStream_t st);
+
+constexpr int kFD = 128;          // head dimension the fused kernels are built for
+constexpr int kFThreads = 512;    // 8 waves
+constexpr int kFKeys = 64;        // keys per iteration of a workgroup
+constexpr int kFSlab = 512;       // buckets per workgroup (64 per wave)
+constexpr int kFLd = kFD + 8;     // LDS row stride in bf16 elements
+constexpr int kMaxRepair = 64;
+
+struct FusedPlan {
+  int ns, stride, rank, n_splits, slabs, n_writers, cap_w;
+  int64_t ld_s, ldy;
+  size_t off_Ks, off_Ys, off_tau, off_cand, off_cnt, off_fail, off_nfail, off_Yf, total;
+};
+
+static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& p) {
+  if (dtype != FM_BF16 || d != kFD) return false;
+  if (N < 65536 || int64_t(Z) * 8 > N || Z > FM_MAX_Z || Z < 64) return false;
+  p.stride = N / 32768;
+  p.ns = N / p.stride;
+  const double mu = double(Z) * p.ns / N;
+  p.rank = int(mu + 6.0 * sqrt(mu) + 3.0);
+  if (p.rank * 4 > p.ns) return false;
+  const double m_exp = double(p.rank) * N / p.ns;
+  p.slabs = int(ceil_div(C, kFSlab));
+  const int64_t ntiles = ceil_div(N, kFKeys);
+  int64_t s = ceil_div(256, int64_t(H) * p.slabs);
+  s = std::max<int64_t>(1, std::min<int64_t>(32, std::min(s, ntiles)));
+  p.n_splits = int(s);
+  p.n_writers = 2 * p.n_splits;
+  p.cap_w = int(1.35 * m_exp / p.n_writers) + 64;
+  p.ld_s = (int64_t(p.ns) + 3) / 4 * 4;
+  p.ldy = (int64_t(N) + 3) / 4 * 4;
+  size_t o = 0;
+  auto take = [&](size_t bytes) {
+    size_t r = o;
+    o = align_up(o + bytes, 256);
+    return r;
+  };
+  const size_t rows = size_t(H) * C;
+  p.off_Ks = take(size_t(H) * p.ns * d * sizeof(bf16_t));
+  p.off_Ys = take(rows * p.ld_s * sizeof(float));
+  p.off_tau = take(rows * sizeof(float));
+  p.off_cand = take(rows * p.n_writers * size_t(p.cap_w) * sizeof(uint2));
+  p.off_cnt = take(rows * p.n_writers * sizeof(int32_t));
+  p.off_fail = take(kMaxRepair * sizeof(int32_t));
+  p.off_nfail = take(4 * sizeof(int32_t));
+  p.off_Yf = take(size_t(kMaxRepair) * p.ldy * sizeof(float));
+  p.total = o;
+  return true;
+}
+
+// ---- phase 0 ---------------------------------------------------------------
+__global__ __launch_bounds__(256) void gather_sample_kernel(const bf16_t* __restrict__ K,
+                                                            bf16_t* __restrict__ Ks, int N, int ns,
+                                                            int stride) {
+  const int h = blockIdx.y;
+  const int64_t e = int64_t(blockIdx.x) * 256 + threadIdx.x;  // 16-byte chunk id
+  if (e >= int64_t(ns) * (kFD / 8)) return;
+  const int i = int(e / (kFD / 8)), ch = int(e % (kFD / 8));
+  const uint4* src = reinterpret_cast<const uint4*>(K + (int64_t(h) * N + int64_t(i) * stride) * kFD) + ch;
+  reinterpret_cast<uint4*>(Ks + (int64_t(h) * ns + i) * kFD)[ch] = *src;
+}
+
+// tau[row] = a lower bound of the rank-th largest value of the sampled row that
+// at least `rank` sampled values reach (value bits only: 12+10+10).
+__global__ __launch_bounds__(kSelThreads) void row_threshold_kernel(const float* __restrict__ Ys,
+                                                                    int ns, int64_t ld, int rank,
+                                                                    float* __restrict__ tau,
+                                                                    int32_t* __restrict__ n_fail) {
+  __shared__ SelectShared sh;
+  if (blockIdx.x == 0 && threadIdx.x < 4) n_fail[threadIdx.x] = 0;
+  DenseRow src{Ys + int64_t(blockIdx.x) * ld, ns};
+  const uint64_t cut = radix_select_cut(src, rank, 3, sh);
+  if (threadIdx.x == 0) tau[blockIdx.x] = key_to_float(uint32_t(cut >> 32));
+}
+
+// ---- phase 1 ---------------------------------------------------------------
+// grid (n_splits, slabs, H); workgroup (sk, slab, h) takes key tiles sk, sk+n_splits, ...
+__global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const float* __restrict__ tau,
+    uint2* __restrict__ cand, int32_t* __restrict__ cnt, int C, int N, int n_splits, int cap_w) {
+  __shared__ __attribute__((aligned(16))) bf16_t sK[2][kFKeys * kFLd];
+  const int sk = blockIdx.x, slab = blockIdx.y, h = blockIdx.z;
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+  const int n_writers = 2 * n_splits;
+  const int cb = slab * kFSlab + w * 64;  // this wave's first bucket
+  const bf16_t* Ah = A + int64_t(h) * C * kFD;
+  const bf16_t* Kh = K + int64_t(h) * N * kFD;
+
+  // resident B fragments (bucket rows of A), thresholds, candidate segments
+  bf16x8 bfrag[2][8];
+  float th[2];
+  uint2* seg[2];
+  int cur[2] = {0, 0};
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int row = cb + ni * 32 + (l & 31);
+    const bool ok = row < C;
+    const uint4* pa = reinterpret_cast<const uint4*>(Ah + int64_t(ok ? row : 0) * kFD + (l >> 5) * 8);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      uint4 v = ok ? pa[2 * ks] : make_uint4(0, 0, 0, 0);
+      union {
+        uint4 u;
+        bf16x8 b;
+      } cvt;
+      cvt.u = v;
+      bfrag[ni][ks] = cvt.b;
+    }
+    const int64_t grow = int64_t(h) * C + (ok ? row : 0);
+    th[ni] = ok ? tau[grow] : INFINITY;
+    seg[ni] = cand + (grow * n_writers + sk * 2 + (l >> 5)) * int64_t(cap_w);
+  }
+
+  const int ntiles = (N + kFKeys - 1) / kFKeys;
+  // staging: 64 rows x 16 chunks of 16 B = 1024 chunks, two per thread
+  auto fetch = [&](int t, uint4 (&st)[2]) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int e = tid + u * kFThreads;
+      const int r = e >> 4, ch = e & 15;
+      const int key = t * kFKeys + r;
+      st[u] = key < N ? reinterpret_cast<const uint4*>(Kh + int64_t(key) * kFD)[ch]
+                      : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stash = [&](int buf, const uint4 (&st)[2]) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int e = tid + u * kFThreads;
+      const int r = e >> 4, ch = e & 15;
+      *reinterpret_cast<uint4*>(&sK[buf][r * kFLd + ch * 8]) = st[u];
+    }
+  };
+
+  uint4 st[2];
+  int t = sk;
+  if (t < ntiles) {
+    fetch(t, st);
+    stash(0, st);
+  }
+  __syncthreads();
+  int buf = 0;
+  for (; t < ntiles; t += n_splits) {
+    const int tn = t + n_splits;
+    if (tn < ntiles) fetch(tn, st);
+    if (cb < C) {
+      f32x16 acc[2][2];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+      const bf16_t* pa = &sK[buf][(l & 31) * kFLd + (l >> 5) * 8];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        bf16x8 a0 = *reinterpret_cast<const bf16x8*>(pa + ks * 16);
+        bf16x8 a1 = *reinterpret_cast<const bf16x8*>(pa + 32 * kFLd + ks * 16);
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) {
+          acc[0][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, bfrag[ni][ks], acc[0][ni], 0, 0, 0);
+          acc[1][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, bfrag[ni][ks], acc[1][ni], 0, 0, 0);
+        }
+      }
+      const int kbase = t * kFKeys;
+      const bool tail = kbase + kFKeys > N;
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float y = acc[mi][ni][r];
+            if (!(y < th[ni])) {
+              const int key = kbase + mi * 32 + acc_row_32(r, l);
+              if (!tail || key < N) {
+                if (cur[ni] < cap_w) seg[ni][cur[ni]] = make_uint2(__float_as_uint(y), uint32_t(key));
+                ++cur[ni];
+              }
+            }
+          }
+    }
+    if (tn < ntiles) stash(buf ^ 1, st);
+    __syncthreads();
+    buf ^= 1;
+  }
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int row = cb + ni * 32 + (l & 31);
+    if (row < C) cnt[(int64_t(h) * C + row) * n_writers + sk * 2 + (l >> 5)] = cur[ni];
+  }
+}
+
+// ---- phase 2 ---------------------------------------------------------------
+struct CandRow {
+  const uint2* base;  // [n_writers][cap_w]
+  const int* counts;  // LDS, clamped to cap_w
+  int n_writers, cap_w, maxc;
+  template <typename F>
+  __device__ __forceinline__ void operator()(F f) const {
+    for (int j = threadIdx.x; j < maxc; j += kSelThreads) {
+      for (int w0 = 0; w0 < n_writers; w0 += 8) {
+        uint2 e[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int w = w0 + u;
+          if (w < n_writers && j < counts[w]) e[u] = base[int64_t(w) * cap_w + j];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int w = w0 + u;
+          if (w < n_writers && j < counts[w]) f(__uint_as_float(e[u].x), e[u].y);
+        }
+      }
+    }
+  }
+};
+
+__global__ __launch_bounds__(kSelThreads) void cand_select_kernel(
+    const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, int n_writers, int cap_w,
+    int Zc, int P, int32_t* __restrict__ idx_out, int32_t* __restrict__ fail_rows,
+    int32_t* __restrict__ n_fail) {
+  extern __shared__ uint64_t buf[];
+  __shared__ SelectShared sh;
+  __shared__ int s_counts[64];
+  __shared__ int s_total, s_over, s_max;
+  const int64_t row = blockIdx.x;
+  if (threadIdx.x == 0) {
+    int total = 0, over = 0, mx = 0;
+    for (int w = 0; w < n_writers; ++w) {
+      int c = cnt[row * n_writers + w];
+      over |= (c > cap_w);
+      c = min(c, cap_w);
+      s_counts[w] = c;
+      total += c;
+      mx = max(mx, c);
+    }
+    s_total = total;
+    s_over = over;
+    s_max = mx;
+  }
+  __syncthreads();
+  if (s_over || s_total < Zc) {  // threshold missed for this row: queue it for repair
+    if (threadIdx.x == 0) {
+      int pos = atomicAdd(n_fail, 1);
+      if (pos < kMaxRepair) fail_rows[pos] = int32_t(row);
+    }
+    return;
+  }
+  CandRow src{cand + row * n_writers * int64_t(cap_w), s_counts, n_writers, cap_w, s_max};
+  const uint64_t cut = radix_select_cut(src, Zc, 6, sh);
+  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + row * Zc);
+}
+
+// ---- phase 3 ---------------------------------------------------------------
+// Y of the listed (head, bucket) rows, one output column per workgroup row-slot.
+// grid (ceil(N/128), kMaxRepair); 4 waves x 32 keys.
+__global__ __launch_bounds__(256) void project_listed_rows_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const int32_t* __restrict__ fail_rows,
+    const int32_t* __restrict__ n_fail, float* __restrict__ Yf, int C, int N, int64_t ldy) {
+  const int slot = blockIdx.y;
+  if (slot >= min(*n_fail, kMaxRepair)) return;
+  const int row = fail_rows[slot];
+  const int h = row / C;
+  const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int key = blockIdx.x * 128 + w * 32 + (l & 31);
+  const uint4* pk = reinterpret_cast<const uint4*>(K + (int64_t(h) * N + min(key, N - 1)) * kFD + (l >> 5) * 8);
+  const uint4* pa = reinterpret_cast<const uint4*>(A + int64_t(row) * kFD + (l >> 5) * 8);
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    union {
+      uint4 u;
+      bf16x8 b;
+    } a, b;
+    a.u = key < N ? pk[2 * ks] : make_uint4(0, 0, 0, 0);
+    b.u = (l & 31) == 0 ? pa[2 * ks] : make_uint4(0, 0, 0, 0);  // only column 0 carries the row
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b, b.b, acc, 0, 0, 0);
+  }
+  if ((l & 31) == 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int n = blockIdx.x * 128 + w * 32 + acc_row_32(r, l);
+      if (n < N) Yf[int64_t(slot) * ldy + n] = acc[r];
+    }
+  }
+}
+
+__global__ void fused_status_kernel(const int32_t* __restrict__ n_fail, int32_t* __restrict__ status) {
+  const int f = *n_fail;
+  status[0] = min(f, kMaxRepair);
+  status[1] = max(0, f - kMaxRepair);
+}
+
+}  // namespace fm
+
+extern "C" size_t fm_build_index_fused_workspace(int H, int C, int N, int d, int Z, int dtype) {
+  fm::FusedPlan p;
+  if (H < 1 || C < 1 || N < 1 || !fm::fused_plan(H, C, N, d, Z, dtype, p)) return 0;
+  return p.total;
+}
+
+extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_out, int H, int C,
+                                    int N, int d, int Z, int dtype, void* ws, size_t ws_bytes,
+                                    int32_t* status_dev, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && Z >= 1, FM_ERR_ARG, "fm_build_index_fused: H=%d C=%d N=%d Z=%d",
+             H, C, N, Z);
+  FM_REQUIRE(A && K && idx_out && ws && status_dev, FM_ERR_ARG, "fm_build_index_fused: null pointer");
+  FusedPlan p;
+  FM_REQUIRE(fused_plan(H, C, N, d, Z, dtype, p), FM_ERR_UNSUPPORTED,
+             "fm_build_index_fused: shape not eligible (needs bf16, d=128, N >= 65536, 64 <= Z <= N/8)");
+  FM_REQUIRE(ws_bytes >= p.total, FM_ERR_WORKSPACE, "fm_build_index_fused: workspace %zu < %zu", ws_bytes,
+             p.total);
+  FM_REQUIRE(H <= 65535 && int64_t(H) * C <= 0x7fffffffLL, FM_ERR_UNSUPPORTED,
+             "fm_build_index_fused: too many rows");
+  hipStream_t st = as_stream(stream);
+  char* base = static_cast<char*>(ws);
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(base + p.off_Ks);
+  float* Ys = reinterpret_cast<float*>(base + p.off_Ys);
+  float* tau = reinterpret_cast<float*>(base + p.off_tau);
+  uint2* cand = reinterpret_cast<uint2*>(base + p.off_cand);
+  int32_t* cnt = reinterpret_cast<int32_t*>(base + p.off_cnt);
+  int32_t* fail_rows = reinterpret_cast<int32_t*>(base + p.off_fail);
+  int32_t* n_fail = reinterpret_cast<int32_t*>(base + p.off_nfail);
+  float* Yf = reinterpret_cast<float*>(base + p.off_Yf);
+  const int64_t rows = int64_t(H) * C;
+  const int Zc = Z;  // Z <= N/8 here
+
+  // phase 0
+  hipLaunchKernelGGL(gather_sample_kernel, dim3(unsigned(ceil_div(int64_t(p.ns) * (kFD / 8), 256)), unsigned(H)),
+                     dim3(256), 0, st, (const bf16_t*)K, Ks, N, p.ns, p.stride);
+  int rc = fm_project(A, Ks, Ys, H, C, p.ns, d, p.ld_s, dtype, stream);
+  if (rc) return rc;
+  hipLaunchKernelGGL(row_threshold_kernel, dim3(unsigned(rows)), dim3(kSelThreads), 0, st, Ys, p.ns,
+                     p.ld_s, p.rank, tau, n_fail);
+  // phase 1
+  hipLaunchKernelGGL(fused_filter_kernel, dim3(unsigned(p.n_splits), unsigned(p.slabs), unsigned(H)),
+                     dim3(kFThreads), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N,
+                     p.n_splits, p.cap_w);
+  // phase 2
+  const int P = next_pow2(Zc);
+  FM_ALLOW_LDS(cand_select_kernel, FM_MAX_Z * sizeof(uint64_t), "fm_build_index_fused: lds");
+  hipLaunchKernelGGL(cand_select_kernel, dim3(unsigned(rows)), dim3(kSelThreads),
+                     size_t(P) * sizeof(uint64_t), st, cand, cnt, p.n_writers, p.cap_w, Zc, P, idx_out,
+                     fail_rows, n_fail);
+  // phase 3
+  hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(ceil_div(N, 128)), kMaxRepair), dim3(256), 0,
+                     st, (const bf16_t*)A, (const bf16_t*)K, fail_rows, n_fail, Yf, C, N, p.ldy);
+  rc = launch_argtopz(Yf, kMaxRepair, N, p.ldy, Zc, idx_out, fail_rows, n_fail, st);
+  if (rc) return rc;
+  hipLaunchKernelGGL(fused_status_kernel, dim3(1), dim3(1), 0, st, n_fail, status_dev);
+  return launch_status("fm_build_index_fused");
+}

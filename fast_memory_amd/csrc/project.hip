@@ -6,44 +6,70 @@
 namespace fm {
 
 // ---------------------------------------------------------------------------
-// bf16 projection on MFMA: one workgroup = 128 buckets x 128 keys, the whole
+// bf16 projection on MFMA: one workgroup = 128 keys x 128 buckets, the whole
 // contraction (d <= 256) staged once in LDS, four waves in a 2x2 grid of 64x64
-// sub-tiles, each 2x2 MFMA 32x32x16 tiles.  Lanes run along the key axis in
-// the accumulator layout, so stores are 128-byte segments of a Y row.
-// Bound: HBM write of Y (4 B per multiply-add column of 2*d flops).
+// sub-tiles, each 2x2 v_mfma_f32_32x32x16_bf16 with keys on the A operand and
+// ascending contraction steps (the fused index build computes Y the same way,
+// so both give bit-equal values).  The accumulators are transposed through LDS
+// so that every Y row segment leaves as 512 contiguous bytes.
+// Bound: HBM write of Y (4 B per 2*d flops).
 // ---------------------------------------------------------------------------
+constexpr int kProjYLd = 132;  // floats per staged output row (128 + 4 pad)
+
 __global__ __launch_bounds__(256) void project_bf16_kernel(const bf16_t* __restrict__ A,
                                                            const bf16_t* __restrict__ K,
                                                            float* __restrict__ Y, int C, int N,
                                                            int d, int64_t ldy) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lds_ld = d + 8;  // bf16 elements per staged row (16 B pad: conflict-free b128 reads)
-  bf16_t* sA = reinterpret_cast<bf16_t*>(smem);
-  bf16_t* sB = sA + 128 * lds_ld;
+  bf16_t* sK = reinterpret_cast<bf16_t*>(smem);
+  bf16_t* sA = sK + 128 * lds_ld;
+  float* sY = reinterpret_cast<float*>(smem);  // reused after the MFMA phase: [128 buckets][132]
   const int h = blockIdx.z;
   const int c0 = blockIdx.y * 128;
   const int n0 = blockIdx.x * 128;
   const bf16_t* Ah = A + int64_t(h) * C * d;
   const bf16_t* Kh = K + int64_t(h) * N * d;
+  stage_rows_bf16(sK, lds_ld, Kh, n0, N, d, 128);
   stage_rows_bf16(sA, lds_ld, Ah, c0, C, d, 128);
-  stage_rows_bf16(sB, lds_ld, Kh, n0, N, d, 128);
   __syncthreads();
   const int w = threadIdx.x >> 6, l = lane_id();
-  const int wm = w >> 1, wn = w & 1;
+  const int wm = w >> 1, wn = w & 1;  // wm: key half, wn: bucket half
   f32x16 acc[2][2];
-  mfma_tile_64x64(sA + (wm * 64) * lds_ld, sB + (wn * 64) * lds_ld, lds_ld, d, acc);
-  float* Yh = Y + int64_t(h) * C * ldy;
+  mfma_tile_64x64(sK + (wm * 64) * lds_ld, sA + (wn * 64) * lds_ld, lds_ld, d, acc);
+  __syncthreads();  // operands consumed; the same LDS now takes the output tile
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
     for (int ni = 0; ni < 2; ++ni) {
-      int n = n0 + wn * 64 + ni * 32 + (l & 31);
+      const int bc = wn * 64 + ni * 32 + (l & 31);          // bucket column of this lane
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        int c = c0 + wm * 64 + mi * 32 + acc_row_32(r, l);
-        if (c < C && n < N) Yh[int64_t(c) * ldy + n] = acc[mi][ni][r];
+      for (int q4 = 0; q4 < 4; ++q4) {                      // rows 8*q4 + 4*(l/32) + 0..3
+        const int kr = wm * 64 + mi * 32 + 8 * q4 + ((l >> 5) << 2);
+        float4 v = make_float4(acc[mi][ni][4 * q4], acc[mi][ni][4 * q4 + 1], acc[mi][ni][4 * q4 + 2],
+                               acc[mi][ni][4 * q4 + 3]);
+        *reinterpret_cast<float4*>(&sY[bc * kProjYLd + kr]) = v;
       }
     }
+  __syncthreads();
+  float* Yh = Y + int64_t(h) * C * ldy;
+  const bool vec_ok = ((ldy & 3) == 0) && ((reinterpret_cast<uintptr_t>(Y) & 15) == 0) && (n0 + 128 <= N);
+  // 32 threads per row (512 B), 8 rows per pass
+  for (int r = threadIdx.x >> 5; r < 128; r += 8) {
+    const int c = c0 + r;
+    if (c >= C) break;
+    const int k4 = (threadIdx.x & 31) * 4;
+    const float4 v = *reinterpret_cast<const float4*>(&sY[r * kProjYLd + k4]);
+    float* dst = Yh + int64_t(c) * ldy + n0 + k4;
+    if (vec_ok) {
+      *reinterpret_cast<float4*>(dst) = v;
+    } else {
+      if (n0 + k4 < N) dst[0] = v.x;
+      if (n0 + k4 + 1 < N) dst[1] = v.y;
+      if (n0 + k4 + 2 < N) dst[2] = v.z;
+      if (n0 + k4 + 3 < N) dst[3] = v.w;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -143,7 +169,7 @@ __global__ __launch_bounds__(256) void qhash_generic_kernel(const T* __restrict_
 // bucket tiles of 128 staged in LDS; accumulator layout puts one query per lane
 // column, so the running (max, first index) is kept per lane without shuffles
 // and combined across the two lane halves and the two bucket-side waves at the
-// end.  Scores are the same MFMA sums fm_project would produce for these rows.
+// end.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void qhash_bf16_kernel(const bf16_t* __restrict__ A,
                                                          const bf16_t* __restrict__ q,
@@ -230,7 +256,7 @@ extern "C" int fm_project(const void* A, const void* K, float* Y, int H, int C, 
   hipStream_t st = as_stream(stream);
   if (dtype == FM_BF16 && d % 16 == 0) {
     FM_REQUIRE(ceil_div(C, 128) <= 65535, FM_ERR_UNSUPPORTED, "fm_project: C too large");
-    size_t lds = size_t(2) * 128 * (d + 8) * sizeof(bf16_t);
+    size_t lds = std::max(size_t(2) * 128 * (d + 8) * sizeof(bf16_t), size_t(128) * kProjYLd * sizeof(float));
     FM_ALLOW_LDS(project_bf16_kernel, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_project: lds");
     dim3 grid = dim3(unsigned(ceil_div(N, 128)), unsigned(ceil_div(C, 128)), unsigned(H));
     hipLaunchKernelGGL(project_bf16_kernel, grid, dim3(256), lds, st, (const bf16_t*)A,

@@ -1,0 +1,172 @@
+// Exact top-Z selection shared by the dense arg-top-Z kernel and the fused
+// index build: radix select over unique 64-bit composites, collection of the
+// survivors into LDS and an in-LDS bitonic sort.
+//
+// composite(y, i) = (float_key(y) << 32) | (2^32-1 - i): descending composite
+// order is "value descending, index ascending", and composites are unique, so
+// ties never need a special case.
+//
+// A `Source` is any callable  src(f)  that calls  f(float value, uint32 index)
+// once for every candidate element, from all threads of the workgroup
+// together (each element exactly once).
+#pragma once
+#include "common.hpp"
+
+namespace fm {
+
+constexpr int kSelThreads = 1024;
+constexpr int kSelMaxBins = 4096;
+
+__device__ __forceinline__ uint64_t composite(float y, uint32_t i) {
+  return (uint64_t(float_key(y)) << 32) | uint64_t(0xffffffffu - i);
+}
+
+// inverse of float_key (any 32-bit pattern maps back to some float bit pattern)
+__device__ __forceinline__ float key_to_float(uint32_t key) {
+  uint32_t u = (key & 0x80000000u) ? (key ^ 0x80000000u) : ~key;
+  return __uint_as_float(u);
+}
+
+struct SelectShared {
+  uint32_t hist[kSelMaxBins];
+  int scan_tmp[17];
+  uint64_t prefix;
+  int need, hit, cnt;
+};
+
+// Finds a cut such that exactly `need0` composites of the source are >= cut,
+// looking at no more than `max_passes` digits (12,10,10 value bits, then
+// 11,11,10 index bits).  With all 6 passes the cut is exact; with fewer it is a
+// lower bound of the need0-th largest composite (at least need0 are >= cut).
+// Every thread of the workgroup must call this; returns the same cut to all.
+template <typename Source>
+__device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int max_passes,
+                                                     SelectShared& sh) {
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    sh.prefix = 0;
+    sh.need = need0;
+    sh.hit = 0;
+  }
+  const int kBits[6] = {12, 10, 10, 11, 11, 10};
+  int top = 64;  // bits [top,64) of the cut are known and equal sh.prefix
+  for (int pass = 0; pass < max_passes; ++pass) {
+    const int bits = kBits[pass];
+    const int shift = top - bits;
+    const int nb = 1 << bits;
+    for (int i = tid; i < nb; i += kSelThreads) sh.hist[i] = 0;
+    __syncthreads();
+    const uint64_t prefix = sh.prefix;
+    const int need = sh.need;
+    const bool first = (top == 64);
+    src([&](float y, uint32_t i) {
+      uint64_t c = composite(y, i);
+      if (first || (c >> top) == prefix) atomicAdd(&sh.hist[(c >> shift) & uint64_t(nb - 1)], 1u);
+    });
+    __syncthreads();
+    // thread t owns `per` bins, walking digits from the largest down
+    const int per = nb >> 10;
+    int local = 0;
+    for (int j = 0; j < per; ++j) local += int(sh.hist[nb - 1 - (tid * per + j)]);
+    int total;
+    int running = block_excl_scan(local, sh.scan_tmp, &total);
+    for (int j = 0; j < per; ++j) {
+      int b = nb - 1 - (tid * per + j);
+      int h = int(sh.hist[b]);
+      if (running < need && need <= running + h) {
+        sh.prefix = (prefix << bits) | uint64_t(b);
+        sh.need = need - running;
+        sh.hit = (h == need - running);
+      }
+      running += h;
+    }
+    __syncthreads();
+    top = shift;
+    if (sh.hit || top == 0) break;
+  }
+  const uint64_t cut = sh.prefix << top;
+  __syncthreads();
+  return cut;
+}
+
+// Collects the composites >= cut (at most P) into buf, pads to P with zeros,
+// sorts descending and writes the first Zc indices to out.
+template <typename Source>
+__device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, int Zc, int P,
+                                                   uint64_t* buf, SelectShared& sh,
+                                                   int32_t* __restrict__ out) {
+  const int tid = threadIdx.x;
+  if (tid == 0) sh.cnt = 0;
+  __syncthreads();
+  src([&](float y, uint32_t i) {
+    uint64_t c = composite(y, i);
+    if (c >= cut) {
+      int pos = atomicAdd(&sh.cnt, 1);
+      if (pos < P) buf[pos] = c;
+    }
+  });
+  for (int i = Zc + tid; i < P; i += kSelThreads) buf[i] = 0;
+  __syncthreads();
+  for (int k = 2; k <= P; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = tid; t < (P >> 1); t += kSelThreads) {
+        int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+        int p = i | j;
+        uint64_t a = buf[i], b = buf[p];
+        bool desc = (i & k) == 0;
+        if (desc ? (a < b) : (a > b)) {
+          buf[i] = b;
+          buf[p] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = tid; i < Zc; i += kSelThreads) out[i] = int32_t(0xffffffffu - uint32_t(buf[i]));
+}
+
+// Dense fp32 row as a source; 128-bit loads on the aligned body, kUnroll of
+// them in flight per thread.
+struct DenseRow {
+  const float* row;
+  int N;
+  static constexpr int kUnroll = 8;
+  template <typename F>
+  __device__ __forceinline__ void operator()(F f) const {
+    const int tid = threadIdx.x;
+    int head = int((4 - ((reinterpret_cast<uintptr_t>(row) >> 2) & 3)) & 3);
+    if (head > N) head = N;
+    if (tid < head) f(row[tid], uint32_t(tid));
+    const int nvec = (N - head) >> 2;
+    const float4* v = reinterpret_cast<const float4*>(row + head);
+    for (int i0 = tid; i0 < nvec; i0 += kSelThreads * kUnroll) {
+      float4 x[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        int i = i0 + u * kSelThreads;
+        if (i < nvec) x[u] = v[i];
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        int i = i0 + u * kSelThreads;
+        if (i < nvec) {
+          uint32_t b = uint32_t(head + 4 * i);
+          f(x[u].x, b);
+          f(x[u].y, b + 1);
+          f(x[u].z, b + 2);
+          f(x[u].w, b + 3);
+        }
+      }
+    }
+    const int tail0 = head + 4 * nvec;
+    if (tail0 + tid < N) f(row[tail0 + tid], uint32_t(tail0 + tid));
+  }
+};
+
+static inline int next_pow2(int x) {
+  int p = 1;
+  while (p < x) p <<= 1;
+  return p;
+}
+
+}  // namespace fm

@@ -63,17 +63,40 @@ def argtopz(Y: torch.Tensor, Z: int) -> torch.Tensor:
     return out
 
 
-def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int = 8 << 30) -> torch.Tensor:
-    """Bucket lists [H,C,min(Z,N)] int32 (memory.py:260-278 on one device)."""
+last_build_info = {}
+
+
+def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int = 8 << 30,
+                fused: Optional[bool] = None) -> torch.Tensor:
+    """Bucket lists [H,C,min(Z,N)] int32 (memory.py:260-278 on one device).
+
+    ``fused=None`` takes the fused build (no Y in memory) where the shape is
+    eligible and the unfused one otherwise; both give identical lists.  The
+    fused build reports through a two-int status whether any row could not be
+    resolved on the device, in which case the unfused build runs instead."""
     _dev(A, K)
     H, C, d = A.shape
     _, N, _ = K.shape
     assert K.shape[0] == H and K.shape[2] == d and A.dtype == K.dtype
     lib = _lib.load()
+    out = torch.empty((H, C, min(int(Z), N)), dtype=torch.int32, device=A.device)
+    fws = lib.fm_build_index_fused_workspace(H, C, N, d, int(Z), _dt(A)) if fused is not False else 0
+    if fused and not fws:
+        raise ValueError("fused index build: shape not eligible (bf16, d=128, N>=65536, 64<=Z<=N/8)")
+    if fws:
+        ws = _ws(fws, A)
+        status = torch.empty(2, dtype=torch.int32, device=A.device)
+        check(lib.fm_build_index_fused(_p(A), _p(K), _p(out), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(),
+                                       _p(status), _stream(A)))
+        repaired, unresolved = status.tolist()          # one 8-byte read-back per build
+        last_build_info.update(path="fused", rows_repaired=repaired, rows_unresolved=unresolved)
+        del ws
+        if unresolved == 0:
+            return out
+    last_build_info.update(path="unfused")
     full = lib.fm_build_index_workspace(H, C, N, d, int(Z), C)
     one = lib.fm_build_index_workspace(H, C, N, d, int(Z), 1)
     ws = _ws(max(one, min(full, int(workspace_bytes))), A)
-    out = torch.empty((H, C, min(int(Z), N)), dtype=torch.int32, device=A.device)
     check(lib.fm_build_index(_p(A), _p(K), _p(out), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(), _stream(A)))
     return out
 

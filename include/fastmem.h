@@ -77,6 +77,20 @@ size_t fm_build_index_workspace(int H, int C, int N, int d, int Z, int64_t rows_
 int fm_build_index(const void* A, const void* K, int32_t* idx_out, int H, int C, int N, int d,
                    int Z, int dtype, void* ws, size_t ws_bytes, void* stream);
 
+/* ---- a1+a2 fused: the same lists without ever writing Y to memory ------------
+ * (memory.py:260-278; the selection sees exactly the fp32 values fm_project
+ * would produce, so the lists are bit-identical to fm_build_index).  Built for
+ * bf16, d = 128, N >= 65536, 64 <= Z <= N/8; fm_build_index_fused_workspace
+ * returns 0 for any other shape.  A per-row threshold taken from a sample of the
+ * keys filters the MFMA output; rows whose threshold missed are recomputed
+ * exactly on the device (up to 64 of them).  status_dev (device, 2 ints)
+ * receives {rows repaired, rows left unresolved}; if the second is non-zero the
+ * caller must rebuild with fm_build_index. */
+size_t fm_build_index_fused_workspace(int H, int C, int N, int d, int Z, int dtype);
+int fm_build_index_fused(const void* A, const void* K, int32_t* idx_out, int H, int C, int N, int d,
+                         int Z, int dtype, void* ws, size_t ws_bytes, int32_t* status_dev,
+                         void* stream);
+
 /* ---- a3: query hash  h_q = argmax_c A[h,c,:].q  (first maximum wins) ---------
  * replaces einsum+argmax at memory.py:281-283 / triton_kernel.py:280-281.
  * hash_out [H,Sq] int32.  scores_out is optional ([H,Sq,C] fp32, may be NULL):

@@ -406,3 +406,63 @@ def test_ring_attention_masked_forward_windows(ops):
         ro, rl = O.ring_attention_masked_forward(kh, qh, q, k, v, 0.125, rank)
         assert out.shape == (1, H * G, S, d) and lse.shape == (1, H * G, S)
         assert_attn_close(out[0], lse[0], ro[0], rl[0], torch.bfloat16, f"ring rank {rank}")
+
+
+# ------------------------------------------------------------------ a1+a2 fused build
+def _clustered_keys(g, H, N, d, n_clusters=64, spread=0.5):
+    cen = torch.randn(H, n_clusters, d, generator=g)
+    comp = torch.randint(0, n_clusters, (H, N), generator=g)
+    x = torch.gather(cen, 1, comp[..., None].expand(-1, -1, d)) + spread * torch.randn(H, N, d, generator=g)
+    return x.to(torch.bfloat16)
+
+
+def test_fused_build_bit_identical_to_unfused(ops):
+    g = gen(900)
+    H, C, N, d, Z = 2, 70, 70001, 128, 512                # ragged C (one partial wave) and a key tail
+    K = _clustered_keys(g, H, N, d)
+    A = torch.randn(H, C, d, generator=g).to(torch.bfloat16)
+    Ad, Kd = dev(A, K)
+    assert _libmod().load().fm_build_index_fused_workspace(H, C, N, d, Z, 1) > 0
+    fused = ops.build_index(Ad, Kd, Z, fused=True)
+    assert ops.last_build_info["path"] == "fused" and ops.last_build_info["rows_unresolved"] == 0
+    unfused = ops.build_index(Ad, Kd, Z, fused=False)
+    assert torch.equal(fused, unfused)
+    Y = ops.project(Ad, Kd).cpu()
+    assert torch.equal(fused.cpu().long(), O.argtopz(Y, Z))
+
+
+def test_fused_build_repairs_rows_whose_sampled_threshold_missed(ops):
+    g = gen(901)
+    H, C, N, d, Z = 1, 40, 131072, 128, 1024               # sample stride 4: keys 0,4,8,... are sampled
+    K = (0.3 * torch.randn(H, N, d, generator=g))
+    A = torch.randn(H, C, d, generator=g)
+    A = A / A.norm(dim=-1, keepdim=True)
+    samp = torch.arange(0, N, 4)
+    off = torch.arange(1, N, 4)
+    K[0, off[:20000]] += 3.0 * A[0, 3]                      # row 3: many large values the sample never sees
+    K[0, samp[:600]] += 3.0 * A[0, 7]                       # row 7: the sample over-represents the large values
+    K, A = K.to(torch.bfloat16), A.to(torch.bfloat16)
+    Ad, Kd = dev(A, K)
+    fused = ops.build_index(Ad, Kd, Z, fused=True)
+    info = dict(ops.last_build_info)
+    assert info["path"] == "fused" and info["rows_unresolved"] == 0 and info["rows_repaired"] >= 2, info
+    assert torch.equal(fused, ops.build_index(Ad, Kd, Z, fused=False))
+
+
+def test_fused_build_falls_back_when_too_many_rows_miss(ops):
+    g = gen(902)
+    H, C, N, d, Z = 1, 100, 65536, 128, 256                # stride 2: even keys sampled
+    A = torch.randn(H, C, d, generator=g)
+    K = 0.1 * torch.randn(H, N, d, generator=g)
+    K[0, 1::2] += 2.0 * A[0].sum(0) / 10                    # every row's large values sit on unsampled keys
+    K, A = K.to(torch.bfloat16), A.to(torch.bfloat16)
+    Ad, Kd = dev(A, K)
+    lists = ops.build_index(Ad, Kd, Z)
+    assert torch.equal(lists, ops.build_index(Ad, Kd, Z, fused=False))
+    Y = ops.project(Ad, Kd).cpu()
+    assert torch.equal(lists.cpu().long(), O.argtopz(Y, Z))
+
+
+def _libmod():
+    from fast_memory_amd import _lib
+    return _lib

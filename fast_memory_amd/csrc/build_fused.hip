@@ -39,7 +39,8 @@ int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int
                    const int32_t* row_map, const int32_t* n_rows_dev, hipStream_t st);
 
 constexpr int kFD = 128;          // head dimension the fused kernels are built for
-constexpr int kFThreads = 512;    // 8 waves
+constexpr int kFWaves = 8;        // compute waves per workgroup
+constexpr int kFThreads = 576;    // + one producer wave
 constexpr int kFKeys = 64;        // keys per iteration of a workgroup
 constexpr int kFSlab = 512;       // buckets per workgroup (64 per wave)
 constexpr int kFLd = kFD + 8;     // LDS row stride in bf16 elements
@@ -66,7 +67,7 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   s = std::max<int64_t>(1, std::min<int64_t>(32, std::min(s, ntiles)));
   p.n_splits = int(s);
   p.n_writers = 2 * p.n_splits;
-  p.cap_w = int(1.35 * m_exp / p.n_writers) + 64;
+  p.cap_w = int(1.35 * m_exp / p.n_writers) + 64;  // > 16: the overflow guard keeps 16 slots free
   p.ld_s = (int64_t(p.ns) + 3) / 4 * 4;
   p.ldy = (int64_t(N) + 3) / 4 * 4;
   size_t o = 0;
@@ -115,22 +116,85 @@ __global__ __launch_bounds__(kSelThreads) void row_threshold_kernel(const float*
 
 // ---- phase 1 ---------------------------------------------------------------
 // grid (n_splits, slabs, H); workgroup (sk, slab, h) takes key tiles sk, sk+n_splits, ...
+// Candidates are (value bits, key index) pairs in segments [row][writer][cap_w]; a
+// writer is one (key split, lane half) pair, i.e. exactly one lane of one wave, so
+// cursors are registers and appends need no atomics.
+//
+// Nine waves.  Wave 8 is the producer: it streams the 64-key tiles from global
+// memory into a double-buffered LDS tile, two tiles ahead, and is the only wave
+// that ever waits on vector-memory loads.  Waves 0..7 own 64 buckets each (their A
+// rows stay in registers as MFMA B fragments) and per 32-key half-tile do
+//   * 16 MFMAs (32 keys x 64 buckets x d=128),
+//   * the threshold test: per accumulator register one v_cmp and one v_addc that
+//     shifts the outcome into a per-lane bit mask -- no exec-mask changes and no
+//     memory traffic -- while the accumulators are dumped to a wave-private LDS area,
+//   * emission rounds: every lane that still has mask bits pops one, reads that
+//     value back from its LDS dump and appends (value, key) to its segment.
+// The compute waves issue stores only, so they never stall on a memory counter;
+// the two waves that share a SIMD overlap one's MFMAs with the other's VALU work.
 __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const float* __restrict__ tau,
     uint2* __restrict__ cand, int32_t* __restrict__ cnt, int C, int N, int n_splits, int cap_w) {
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][kFKeys * kFLd];
+  __shared__ __attribute__((aligned(16))) float sDump[kFWaves][2 * 4 * 64 * 4];  // [wave][ni][q][lane][4]
   const int sk = blockIdx.x, slab = blockIdx.y, h = blockIdx.z;
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   const int n_writers = 2 * n_splits;
-  const int cb = slab * kFSlab + w * 64;  // this wave's first bucket
-  const bf16_t* Ah = A + int64_t(h) * C * kFD;
   const bf16_t* Kh = K + int64_t(h) * N * kFD;
+  const int ntiles = (N + kFKeys - 1) / kFKeys;
+  const int my_tiles = sk < ntiles ? (ntiles - sk + n_splits - 1) / n_splits : 0;  // tiles sk + i*n_splits
 
-  // resident B fragments (bucket rows of A), thresholds, candidate segments
+  if (w == kFWaves) {
+    // ------------------------------ producer wave ------------------------------
+    // chunk e = u*64 + l of a tile: row 4u + l/16, 16-byte column l%16 (4 whole rows per instruction)
+    uint4 st[2][16];
+    auto fetch = [&](int i, uint4 (&r)[16]) {
+      const int64_t key0 = (int64_t(sk) + int64_t(i) * n_splits) * kFKeys + (l >> 4);
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int64_t key = key0 + 4 * u;
+        r[u] = key < N ? reinterpret_cast<const uint4*>(Kh + key * kFD)[l & 15] : make_uint4(0, 0, 0, 0);
+      }
+    };
+    auto stash = [&](int buf, const uint4 (&r)[16]) {
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        *reinterpret_cast<uint4*>(&sK[buf][(4 * u + (l >> 4)) * kFLd + (l & 15) * 8]) = r[u];
+    };
+    if (my_tiles > 0) {
+      fetch(0, st[0]);
+      stash(0, st[0]);
+    }
+    if (my_tiles > 1) fetch(1, st[1]);
+    if (my_tiles > 2) fetch(2, st[0]);
+    __syncthreads();
+    for (int i = 0; i < my_tiles; i += 2) {
+      // iteration i: tile i+1 (set 1) -> buffer 1, then tile i+3 into set 1
+      if (i + 1 < my_tiles) stash(1, st[1]);
+      if (i + 3 < my_tiles) fetch(i + 3, st[1]);
+      __syncthreads();
+      if (i + 1 >= my_tiles) break;
+      // iteration i+1: tile i+2 (set 0) -> buffer 0, then tile i+4 into set 0
+      if (i + 2 < my_tiles) stash(0, st[0]);
+      if (i + 4 < my_tiles) fetch(i + 4, st[0]);
+      __syncthreads();
+    }
+    return;
+  }
+
+  // ------------------------------ compute waves ------------------------------
+  const int cb = slab * kFSlab + w * 64;  // this wave's first bucket
+  const bool active = cb < C;
+  const bf16_t* Ah = A + int64_t(h) * C * kFD;
+  // segments of this workgroup's 512 bucket rows; lane offsets below are bytes from here
+  const int64_t wg_row0 = int64_t(h) * C + int64_t(slab) * kFSlab;
+  char* cbase = reinterpret_cast<char*>(cand + wg_row0 * n_writers * int64_t(cap_w));
+  float* dump = sDump[w];
+
   bf16x8 bfrag[2][8];
   float th[2];
-  uint2* seg[2];
-  int cur[2] = {0, 0};
+  uint32_t off[2], start[2], lim[2];
+  int ovf[2] = {0, 0};
 #pragma unroll
   for (int ni = 0; ni < 2; ++ni) {
     const int row = cb + ni * 32 + (l & 31);
@@ -138,102 +202,113 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     const uint4* pa = reinterpret_cast<const uint4*>(Ah + int64_t(ok ? row : 0) * kFD + (l >> 5) * 8);
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      uint4 v = ok ? pa[2 * ks] : make_uint4(0, 0, 0, 0);
       union {
         uint4 u;
         bf16x8 b;
       } cvt;
-      cvt.u = v;
+      cvt.u = ok ? pa[2 * ks] : make_uint4(0, 0, 0, 0);
       bfrag[ni][ks] = cvt.b;
     }
-    const int64_t grow = int64_t(h) * C + (ok ? row : 0);
-    th[ni] = ok ? tau[grow] : INFINITY;
-    seg[ni] = cand + (grow * n_writers + sk * 2 + (l >> 5)) * int64_t(cap_w);
+    th[ni] = ok ? tau[int64_t(h) * C + row] : INFINITY;
+    const uint32_t rl = uint32_t(w * 64 + ni * 32 + (l & 31));  // row inside the slab
+    start[ni] = ((rl * uint32_t(n_writers) + uint32_t(sk * 2 + (l >> 5))) * uint32_t(cap_w)) * 8u;
+    off[ni] = start[ni];
+    lim[ni] = start[ni] + uint32_t(cap_w - 16) * 8u;
   }
-
-  const int ntiles = (N + kFKeys - 1) / kFKeys;
-  // staging: 64 rows x 16 chunks of 16 B = 1024 chunks, two per thread
-  auto fetch = [&](int t, uint4 (&st)[2]) {
+  // make the resident operands "used" here so that the wait for their loads sits before the loop
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int e = tid + u * kFThreads;
-      const int r = e >> 4, ch = e & 15;
-      const int key = t * kFKeys + r;
-      st[u] = key < N ? reinterpret_cast<const uint4*>(Kh + int64_t(key) * kFD)[ch]
-                      : make_uint4(0, 0, 0, 0);
+  for (int ni = 0; ni < 2; ++ni) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) asm volatile("" ::"v"(bfrag[ni][ks]));
+    asm volatile("" ::"v"(th[ni]));
+  }
+  const int lane_key = (l >> 5) << 2;
+  uint32_t msk[2];
+
+  // threshold test of four accumulator registers: mask = 2*mask + (y >= th); and their dump
+  auto test_dump4 = [&](const f32x16& a, int ni, int q) {
+    // The dump comes first: it is the compiler-visible read of freshly written MFMA results, so the
+    // wait states an MFMA result needs before it can be read are inserted there; the asm below
+    // (whose operands the hazard logic does not look into) then only ever reads settled registers.
+    *reinterpret_cast<float4*>(&dump[((ni * 4 + q) * 64 + l) * 4]) =
+        make_float4(a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      asm volatile("v_cmp_nlt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
+                   : "+v"(msk[ni])
+                   : "v"(a[4 * q + j]), "v"(th[ni])
+                   : "vcc", "memory");
+  };
+  // One emission round for column ni: lanes with a mask bit pop the highest one (= earliest test).
+  // Bit 15-r of the mask belongs to accumulator register r = key row 8*(r/4) + 4*(l/32) + r%4.
+  auto emit_round = [&](int ni, int keyl, bool check_n) {
+    if (msk[ni] != 0) {
+      const int b = 31 - __clz(int(msk[ni]));
+      msk[ni] ^= (1u << b);
+      const int r = 15 - b;
+      const float y = dump[((ni * 4 + (r >> 2)) * 64 + l) * 4 + (r & 3)];
+      const int key = keyl + 8 * (r >> 2) + (r & 3);
+      if (!check_n || key < N) {
+        *reinterpret_cast<uint2*>(cbase + off[ni]) = make_uint2(__float_as_uint(y), uint32_t(key));
+        off[ni] += 8u;
+      }
     }
   };
-  auto stash = [&](int buf, const uint4 (&st)[2]) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int e = tid + u * kFThreads;
-      const int r = e >> 4, ch = e & 15;
-      *reinterpret_cast<uint4*>(&sK[buf][r * kFLd + ch * 8]) = st[u];
-    }
-  };
 
-  uint4 st[2];
-  int t = sk;
-  if (t < ntiles) {
-    fetch(t, st);
-    stash(0, st);
-  }
-  __syncthreads();
-  int buf = 0;
-  for (; t < ntiles; t += n_splits) {
-    const int tn = t + n_splits;
-    if (tn < ntiles) fetch(tn, st);
-    if (cb < C) {
-      f32x16 acc[2][2];
+  __syncthreads();  // first tile staged
+  for (int i = 0; i < my_tiles; ++i) {
+    if (active) {
+      const int kbase = (sk + i * n_splits) * kFKeys;
+      const bool check_n = kbase + kFKeys > N;
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
+      for (int half = 0; half < 2; ++half) {
+        const bf16_t* pa = &sK[i & 1][(half * 32 + (l & 31)) * kFLd + (l >> 5) * 8];
+        bf16x8 a[8];
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) a[ks] = *reinterpret_cast<const bf16x8*>(pa + ks * 16);
+        f32x16 acc[2];
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
-      const bf16_t* pa = &sK[buf][(l & 31) * kFLd + (l >> 5) * 8];
+          for (int r = 0; r < 16; ++r) acc[ni][r] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 a0 = *reinterpret_cast<const bf16x8*>(pa + ks * 16);
-        bf16x8 a1 = *reinterpret_cast<const bf16x8*>(pa + 32 * kFLd + ks * 16);
+        for (int ks = 0; ks < 8; ++ks) {
+          acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], bfrag[0][ks], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], bfrag[1][ks], acc[1], 0, 0, 0);
+        }
+        msk[0] = msk[1] = 0;
+        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // all 16 accumulator passes retired
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
-          acc[0][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, bfrag[ni][ks], acc[0][ni], 0, 0, 0);
-          acc[1][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, bfrag[ni][ks], acc[1][ni], 0, 0, 0);
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) test_dump4(acc[ni], ni, q);
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+          if (off[ni] > lim[ni]) {  // fewer than 16 free slots: wrap and mark the row for repair
+            off[ni] = start[ni];
+            ovf[ni] = 1;
+          }
+        const int keyl = kbase + half * 32 + lane_key;
+        while (__ballot((msk[0] | msk[1]) != 0)) {
+          emit_round(0, keyl, check_n);
+          emit_round(1, keyl, check_n);
         }
       }
-      const int kbase = t * kFKeys;
-      const bool tail = kbase + kFKeys > N;
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float y = acc[mi][ni][r];
-            if (!(y < th[ni])) {
-              const int key = kbase + mi * 32 + acc_row_32(r, l);
-              if (!tail || key < N) {
-                if (cur[ni] < cap_w) seg[ni][cur[ni]] = make_uint2(__float_as_uint(y), uint32_t(key));
-                ++cur[ni];
-              }
-            }
-          }
     }
-    if (tn < ntiles) stash(buf ^ 1, st);
     __syncthreads();
-    buf ^= 1;
   }
 #pragma unroll
   for (int ni = 0; ni < 2; ++ni) {
     const int row = cb + ni * 32 + (l & 31);
-    if (row < C) cnt[(int64_t(h) * C + row) * n_writers + sk * 2 + (l >> 5)] = cur[ni];
+    if (row < C)
+      cnt[(int64_t(h) * C + row) * n_writers + sk * 2 + (l >> 5)] =
+          ovf[ni] ? cap_w + 1 : int32_t((off[ni] - start[ni]) >> 3);
   }
 }
 
 // ---- phase 2 ---------------------------------------------------------------
 struct CandRow {
-  const uint2* base;  // [n_writers][cap_w]
+  const uint2* base;  // [n_writers][cap_w] (value bits, key index)
   const int* counts;  // LDS, clamped to cap_w
   int n_writers, cap_w, maxc;
   template <typename F>

@@ -33,7 +33,8 @@ def _hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", src, "-o", obj]
+    extra = os.environ.get("FM_EXTRA_HIPCC_FLAGS", "").split()   # for experiments, e.g. -DSOMETHING
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

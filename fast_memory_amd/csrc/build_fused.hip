@@ -239,17 +239,32 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
                    : "v"(a[4 * q + j]), "v"(th[ni])
                    : "vcc", "memory");
   };
-  // One emission round for column ni: lanes with a mask bit pop the highest one (= earliest test).
-  // Bit 15-r of the mask belongs to accumulator register r = key row 8*(r/4) + 4*(l/32) + r%4.
-  auto emit_round = [&](int ni, int keyl, bool check_n) {
-    if (msk[ni] != 0) {
-      const int b = 31 - __clz(int(msk[ni]));
-      msk[ni] ^= (1u << b);
-      const int r = 15 - b;
-      const float y = dump[((ni * 4 + (r >> 2)) * 64 + l) * 4 + (r & 3)];
-      const int key = keyl + 8 * (r >> 2) + (r & 3);
-      if (!check_n || key < N) {
-        *reinterpret_cast<uint2*>(cbase + off[ni]) = make_uint2(__float_as_uint(y), uint32_t(key));
+  // Emission: every lane pops up to two mask bits per column (highest bit = earliest test first),
+  // reads those accumulator values back from its LDS dump (all four reads in flight together) and
+  // appends (value, key).  Bit 15-r of a mask belongs to accumulator register r, i.e. key row
+  // 8*(r/4) + 4*(l/32) + r%4 of the half-tile.  A lane without bits pops a harmless r = 15.
+  auto emit = [&](int keyl, bool check_n) {
+    bool has[4];
+    int r[4];
+    float y[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      uint32_t& m = msk[p >> 1];
+      has[p] = m != 0;
+      const int b = 31 - __clz(int(m | 1u));
+      m &= ~(1u << b);
+      r[p] = 15 - b;
+    }
+#pragma unroll
+    for (int p = 0; p < 4; ++p) y[p] = dump[(((p >> 1) * 4 + (r[p] >> 2)) * 64 + l) * 4 + (r[p] & 3)];
+    // keep the four reads together ahead of the predicated stores (one LDS round trip, not four)
+    asm volatile("" : "+v"(y[0]), "+v"(y[1]), "+v"(y[2]), "+v"(y[3]));
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int ni = p >> 1;
+      const int key = keyl + 8 * (r[p] >> 2) + (r[p] & 3);
+      if (has[p] && (!check_n || key < N)) {
+        *reinterpret_cast<uint2*>(cbase + off[ni]) = make_uint2(__float_as_uint(y[p]), uint32_t(key));
         off[ni] += 8u;
       }
     }
@@ -289,10 +304,9 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
             ovf[ni] = 1;
           }
         const int keyl = kbase + half * 32 + lane_key;
-        while (__ballot((msk[0] | msk[1]) != 0)) {
-          emit_round(0, keyl, check_n);
-          emit_round(1, keyl, check_n);
-        }
+        do {
+          emit(keyl, check_n);
+        } while (__ballot((msk[0] | msk[1]) != 0));
       }
     }
     __syncthreads();

@@ -466,3 +466,53 @@ def test_fused_build_falls_back_when_too_many_rows_miss(ops):
 def _libmod():
     from fast_memory_amd import _lib
     return _lib
+
+
+# ------------------------------------------------------------------ MFMA kernels vs generic kernels
+def test_mfma_and_generic_attention_agree(ops):
+    q, k, v, kh, cnt, qh = make_attn_case(30, 3, 500, 8192, 40, 700, 128, torch.bfloat16, window="all", std=1.0)
+    qh[1, :200] = 7
+    args = dev(q, k, v, kh.int(), cnt.int(), qh.int())
+    o1, l1 = ops.attention_hash_varlen_i32(*args, 128 ** -0.5)
+    ops.force_generic_kernels(True)
+    try:
+        o2, l2 = ops.attention_hash_varlen_i32(*args, 128 ** -0.5)
+    finally:
+        ops.force_generic_kernels(False)
+    assert torch.allclose(o1.float(), o2.float(), atol=2e-2, rtol=1e-2)
+    assert (l1 - l2).abs().max().item() < 1e-3
+
+
+# ------------------------------------------------------------------ reduced copies of the benchmark workloads
+@pytest.mark.parametrize("name,N,S,H,C,Z", [
+    ("c2", 4096, 64, 2, 32, 256),            # unfused build (N < 65536)
+    ("c5", 65536, 16, 1, 64, 1024),          # fused build, local keys + merge
+])
+def test_reduced_benchmark_workloads_end_to_end(ops, name, N, S, H, C, Z):
+    from fast_memory_amd import Memory, fit_projection, synth
+    cfg = synth.CONFIGS[name]
+    wl = synth.make_workload(cfg, "cpu", N=N, S=S, H=H)
+    keys, vals, q = dev(wl.keys, wl.values, wl.queries)
+    A = fit_projection(keys, C, iters=cfg.kmeans_iters)
+    mem = Memory.build(keys, vals, A, Z)
+    Y = ops.project(A, keys).cpu()
+    assert torch.equal(mem.bucket_idx.cpu().long(), O.argtopz(Y, Z))
+    qh, sc = ops.qhash(A, q, return_scores=True)
+    assert torch.equal(qh.cpu().long(), O.argmax_first(sc.cpu()))
+    scale = cfg.d ** -0.5
+    out, lse = mem.attend(q, scale, q_hash=qh)
+    cnt = torch.full((H, C), Z)
+    ro, rl = O.hashed_attention_gather(wl.queries, wl.keys, wl.values, mem.bucket_idx.cpu().long().reshape(-1),
+                                       cnt, qh.cpu().long(), scale)
+    assert_attn_close(out, lse, ro, rl, cfg.dtype, name)
+    if wl.k_local is not None:
+        G = cfg.G
+        L = wl.k_local.shape[1]
+        kl, vl = wl.k_local[:, L - S:], wl.v_local[:, L - S:]          # S local keys, causal against S tokens
+        mo, ml = mem.attend_with_local(q, dev(kl.contiguous()), dev(vl.contiguous()), scale, n_groups=G, causal=True)
+        lo, ll = O.local_attention(wl.queries.reshape(1, H * G, S, cfg.d), kl.reshape(1, H, S, cfg.d),
+                                   vl.reshape(1, H, S, cfg.d), scale, True)
+        eo, el = O.lse_merge_closed_form(lo[0].reshape(H, G * S, cfg.d).float(), ll[0].reshape(H, G * S),
+                                         ro.float(), rl)
+        assert torch.allclose(mo.cpu().double(), eo, atol=2e-2, rtol=1e-2)
+        assert (ml.cpu().double() - el).abs().max().item() < 2e-3

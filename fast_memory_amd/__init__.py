@@ -6,9 +6,9 @@ All compute runs in hand-written HIP kernels reached through the C ABI of
 streams.  There is no CPU path.
 """
 from .hash_attention import attention_hash, attention_hash_varlen  # noqa: F401
-from .memory import (Memory, compute_centroids, fit_projection, init_centroids, kmeans_spherical,  # noqa: F401
+from .memory import (Memory, MemoryBatch, compute_centroids, fit_projection, init_centroids, kmeans_spherical,  # noqa: F401
                      merge, ring_attention_masked_forward, update_out_and_lse)
 
-__all__ = ["attention_hash", "attention_hash_varlen", "Memory", "compute_centroids", "fit_projection",
+__all__ = ["attention_hash", "attention_hash_varlen", "Memory", "MemoryBatch", "compute_centroids", "fit_projection",
            "init_centroids", "kmeans_spherical", "merge", "ring_attention_masked_forward",
            "update_out_and_lse"]

@@ -42,6 +42,7 @@ SIGNATURES = {
     "fm_attention_hash_varlen_workspace": (c_size_t, [c_int, c_int, c_int]),
     "fm_attention_hash_varlen": (c_int, [P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int,
                                          c_float, c_int, P, c_size_t, P]),
+    "fm_decode_hash_attn": (c_int, [P, P, P, P, P, P, c_int, c_int, c_int, c_float, P, P, P, P, c_int, P]),
     "fm_local_attn_fwd": (c_int, [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                   c_int, P]),
     "fm_lse_merge": (c_int, [P, P, P, P, c_int64, c_int, c_int, P]),

@@ -20,6 +20,10 @@ bool local_attn_mfma_supported(int d, int dtype);
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
                     int S, int L, int d, float sm_scale, int causal, hipStream_t st);
 
+int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
+                     const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, float sm_scale,
+                     void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st);
+
 // 0 = automatic, 1 = force the generic kernels (used by tests to compare paths)
 static int g_force_generic = 0;
 }  // namespace fm
@@ -122,4 +126,19 @@ extern "C" int fm_local_attn_fwd(const void* q, const void* k, const void* v, vo
   if (!g_force_generic && local_attn_mfma_supported(d, dtype))
     return local_attn_mfma(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, st);
   return local_attn_generic(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, dtype, st);
+}
+
+extern "C" int fm_decode_hash_attn(const void* q, const void* A_all, const void* K_all,
+                                   const void* V_all, const int32_t* idx_all, const fm_rowdesc* desc,
+                                   int rows, int G, int d, float sm_scale, void* out, float* lse,
+                                   int32_t* hash_out, float* scores_out, int dtype, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(rows >= 0 && G >= 1 && G <= 16, FM_ERR_ARG, "fm_decode_hash_attn: rows=%d G=%d", rows, G);
+  FM_REQUIRE(dtype == FM_BF16 && d == 128, FM_ERR_UNSUPPORTED,
+             "fm_decode_hash_attn: built for bf16, d=128 (got dtype=%d d=%d)", dtype, d);
+  if (rows == 0) return FM_OK;
+  FM_REQUIRE(q && A_all && K_all && V_all && idx_all && desc && out && lse && hash_out, FM_ERR_ARG,
+             "fm_decode_hash_attn: null pointer");
+  return decode_hash_attn(q, A_all, K_all, V_all, idx_all, desc, rows, G, sm_scale, out, lse, hash_out,
+                          scores_out, as_stream(stream));
 }

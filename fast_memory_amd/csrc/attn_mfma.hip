@@ -323,7 +323,134 @@ __global__ __launch_bounds__(256) void local_attn_mfma_kernel(
                     nullptr, cnt, L, vis0, scale2, out + qbase * kD, lse + qbase, red);
 }
 
+// Decode batch over memories of different sizes: one workgroup per row (one KV head
+// of one sequence) with its G <= 16 queries.  The workgroup hashes its queries
+// against the row's own A (first maximum wins), then attends each distinct bucket
+// once with the queries that chose it.  Rows are described by fm_rowdesc; A, K, V
+// and the bucket lists of all rows are packed back to back.
+__global__ __launch_bounds__(256) void decode_hash_attn_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ A_all, const bf16_t* __restrict__ K_all,
+    const bf16_t* __restrict__ V_all, const int32_t* __restrict__ idx_all,
+    const fm_rowdesc* __restrict__ desc, int G, float scale2, bf16_t* __restrict__ out,
+    float* __restrict__ lse, int32_t* __restrict__ hash_out, float* __restrict__ scores_out) {
+  extern __shared__ __attribute__((aligned(16))) float red[];
+  __shared__ float sq[16 * kD];
+  __shared__ float s_best[4][16];
+  __shared__ int s_besti[4][16];
+  __shared__ int s_hash[16];
+  __shared__ int q_rows[FM_QTILE];
+  const int row = blockIdx.x;
+  const fm_rowdesc ds = desc[row];
+  const int tid = threadIdx.x, l = tid & 63, w = tid >> 6;
+  const bf16_t* qb = q + int64_t(row) * G * kD;
+  for (int e = tid; e < G * kD; e += 256) sq[e] = bf16_to_f32(qb[e]);
+  __syncthreads();
+  // ---- hash: thread scans buckets tid, tid+256, ...; fp32 FMA chain over d ----
+  float best[16];
+  int besti[16];
+#pragma unroll
+  for (int g = 0; g < 16; ++g) {
+    best[g] = -INFINITY;
+    besti[g] = 0x7fffffff;
+  }
+  const int C = ds.n_buckets;
+  for (int c = tid; c < C; c += 256) {
+    const uint4* ar = reinterpret_cast<const uint4*>(A_all + (ds.a_off + c) * kD);
+    float acc[16];
+#pragma unroll
+    for (int g = 0; g < 16; ++g) acc[g] = 0.f;
+    for (int ch = 0; ch < kD / 8; ++ch) {
+      const uint4 u = ar[ch];
+      const uint32_t wv[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float a = bf16_to_f32(bf16_t(e & 1 ? wv[e >> 1] >> 16 : wv[e >> 1] & 0xffffu));
+#pragma unroll
+        for (int g = 0; g < 16; ++g)
+          if (g < G) acc[g] = fmaf(a, sq[g * kD + ch * 8 + e], acc[g]);
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < 16; ++g)
+      if (g < G) {
+        if (scores_out) scores_out[(ds.a_off + c) * G + g] = acc[g];
+        if (besti[g] == 0x7fffffff || acc[g] > best[g]) {  // buckets ascend per thread
+          best[g] = acc[g];
+          besti[g] = c;
+        }
+      }
+  }
+  // wave then workgroup reduction: larger score wins, equal scores keep the lower bucket
+#pragma unroll
+  for (int g = 0; g < 16; ++g)
+    if (g < G) {
+      float b = best[g];
+      int bi = besti[g];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(b, o);
+        const int oi = __shfl_xor(bi, o);
+        if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > b || (ob == b && oi < bi))) {
+          b = ob;
+          bi = oi;
+        }
+      }
+      if (l == 0) {
+        s_best[w][g] = b;
+        s_besti[w][g] = bi;
+      }
+    }
+  __syncthreads();
+  if (tid < G) {
+    float b = s_best[0][tid];
+    int bi = s_besti[0][tid];
+    for (int ww = 1; ww < 4; ++ww) {
+      const float ob = s_best[ww][tid];
+      const int oi = s_besti[ww][tid];
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > b || (ob == b && oi < bi))) {
+        b = ob;
+        bi = oi;
+      }
+    }
+    s_hash[tid] = bi;
+    hash_out[int64_t(row) * G + tid] = bi;
+  }
+  __syncthreads();
+  // ---- one attention item per distinct bucket among the G queries ----
+  const bf16_t* Kb = K_all + ds.k_off * kD;
+  const bf16_t* Vb = V_all + ds.k_off * kD;
+  for (int g0 = 0; g0 < G; ++g0) {
+    const int bkt = s_hash[g0];
+    bool first = true;
+    for (int g = 0; g < g0; ++g) first = first && (s_hash[g] != bkt);
+    if (!first) continue;  // uniform: every thread reads the same s_hash
+    __syncthreads();
+    if (tid == 0) {
+      int n = 0;
+      for (int g = g0; g < G; ++g)
+        if (s_hash[g] == bkt) q_rows[n++] = g;
+      q_rows[FM_QTILE - 1] = n;
+    }
+    __syncthreads();
+    const int n_q = q_rows[FM_QTILE - 1];
+    attend_item<false>(qb, q_rows, n_q, Kb, Vb, idx_all + ds.idx_off + int64_t(bkt) * ds.bucket_size,
+                       ds.bucket_size, ds.n_keys, 0, scale2, out + int64_t(row) * G * kD,
+                       lse + int64_t(row) * G, red);
+  }
+}
+
 bool hash_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_BF16; }
+
+int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
+                     const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, float sm_scale,
+                     void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st) {
+  FM_ALLOW_LDS(decode_hash_attn_kernel, kRedFloats * sizeof(float), "fm_decode_hash_attn: lds");
+  hipLaunchKernelGGL(decode_hash_attn_kernel, dim3(unsigned(rows)), dim3(256), kRedFloats * sizeof(float),
+                     st, (const bf16_t*)q, (const bf16_t*)A_all, (const bf16_t*)K_all,
+                     (const bf16_t*)V_all, idx_all, desc, G, sm_scale * kLog2e, (bf16_t*)out, lse, hash_out,
+                     scores_out);
+  return launch_status("fm_decode_hash_attn");
+}
 bool local_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_BF16; }
 
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,

@@ -177,6 +177,58 @@ class Memory:
         return out, lse.squeeze(-1)
 
 
+class MemoryBatch:
+    """A decode batch of memories with different N, C and Z (one per sequence).
+
+    All rows (sequence, KV head) are packed back to back so that one launch
+    hashes every query and attends its bucket: ``attend(q)`` with
+    ``q [n_seq, H, G, d]`` (one token per query head) returns ``(out
+    [n_seq,H,G,d], lse [n_seq,H,G] fp32, hashes [n_seq,H,G])``.  bf16, d=128.
+    """
+
+    def __init__(self, memories):
+        mems = list(memories)
+        assert mems and all(m.keys.dtype == torch.bfloat16 and m.keys.shape[2] == 128 for m in mems)
+        self.n_seq, self.H = len(mems), mems[0].keys.shape[0]
+        dev = mems[0].keys.device
+        # row order (sequence, head)
+        self.A_all = torch.cat([m.A.reshape(-1, 128) for m in mems])
+        self.K_all = torch.cat([m.keys.reshape(-1, 128) for m in mems])
+        self.V_all = torch.cat([m.values.reshape(-1, 128) for m in mems])
+        self.idx_all = torch.cat([m.bucket_idx.reshape(-1) for m in mems])
+        rows = []
+        a = k = i = 0
+        for m in mems:
+            H, C, Z = m.bucket_idx.shape
+            N = m.keys.shape[1]
+            for _ in range(H):
+                rows.append([a, k, i, N | (C << 32), Z])
+                a, k, i = a + C, k + N, i + C * Z
+        self.desc = torch.tensor(rows, dtype=torch.int64, device=dev)
+        self.shapes = [(m.keys.shape[1], m.bucket_idx.shape[1], m.bucket_idx.shape[2]) for m in mems]
+
+    def attend(self, q: torch.Tensor, sm_scale: float, return_scores: bool = False):
+        n_seq, H, G, d = q.shape
+        assert n_seq == self.n_seq and H == self.H
+        res = ops.decode_hash_attn(q.reshape(n_seq * H, G, d).contiguous(), self.A_all, self.K_all, self.V_all,
+                                   self.idx_all, self.desc, sm_scale, return_scores)
+        out, lse, h = res[0].reshape(n_seq, H, G, d), res[1].reshape(n_seq, H, G), res[2].reshape(n_seq, H, G)
+        return (out, lse, h, res[3]) if return_scores else (out, lse, h)
+
+    def attend_with_local(self, q, k_local, v_local, sm_scale: float):
+        """Merged with dense attention over each sequence's local keys ``[n_seq,H,L,d]`` (the single
+        query token sees all of them).  Returns fp32 ``(out [n_seq,H,G,d], lse [n_seq,H,G])``."""
+        n_seq, H, G, d = q.shape
+        L = k_local.shape[2]
+        mo, ml, _ = self.attend(q, sm_scale)
+        lo, ll = ops.local_attn_fwd(q.reshape(n_seq * H * G, 1, d).contiguous(),
+                                    k_local.reshape(n_seq * H, L, d).contiguous(),
+                                    v_local.reshape(n_seq * H, L, d).contiguous(), sm_scale, True)
+        out, lse = update_out_and_lse(None, None, lo.reshape(n_seq, H, G, d), ll.reshape(n_seq, H, G))
+        out, lse = update_out_and_lse(out.contiguous(), lse.contiguous(), mo, ml)
+        return out, lse.squeeze(-1)
+
+
 def merge(out_a, lse_a, out_b, lse_b):
     """Functional LSE merge of two partial attentions (memory.py:54-71)."""
     out, lse = update_out_and_lse(None, None, out_a, lse_a)

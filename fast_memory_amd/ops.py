@@ -206,6 +206,23 @@ def attention_hash_varlen_i32(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: floa
     return out, lse
 
 
+def decode_hash_attn(q, A_all, K_all, V_all, idx_all, desc, sm_scale: float, return_scores: bool = False):
+    """Hash + gathered attention for a decode batch of rows with different memories.
+    q [rows,G,d]; A_all [sum C,d]; K_all,V_all [sum N,d]; idx_all flat int32; desc [rows,5] int64
+    viewed as fm_rowdesc (a_off, k_off, idx_off, (n_keys | n_buckets<<32), (bucket_size))."""
+    _dev(q, A_all, K_all, V_all, idx_all, desc)
+    rows, G, d = q.shape
+    assert desc.dtype == torch.int64 and desc.shape == (rows, 5) and idx_all.dtype == torch.int32
+    out = torch.empty_like(q)
+    lse = torch.empty((rows, G), dtype=torch.float32, device=q.device)
+    h = torch.empty((rows, G), dtype=torch.int32, device=q.device)
+    scores = torch.empty((A_all.shape[0], G), dtype=torch.float32, device=q.device) if return_scores else None
+    check(_lib.load().fm_decode_hash_attn(_p(q), _p(A_all), _p(K_all), _p(V_all), _p(idx_all), _p(desc), rows, G, d,
+                                          float(sm_scale), _p(out), _p(lse), _p(h), _p(scores), _dt(q),
+                                          _stream(q)))
+    return (out, lse, h, scores) if return_scores else (out, lse, h)
+
+
 # --------------------------------------------------------------------- a11
 def local_attn_fwd(q, k, v, sm_scale: float, causal: bool = True):
     """Dense GQA attention with LSE (call site memory.py:302).  q [H*G,S,d], k,v [H,L,d]."""

@@ -152,6 +152,26 @@ int fm_attention_hash_varlen(const void* q, const void* k, const void* v, const 
                              float* lse, int H, int Sq, int N, int d, int C, float sm_scale,
                              int dtype, void* ws, size_t ws_bytes, void* stream);
 
+/* ---- decode batch over memories of different sizes ---------------------------
+ * The same path (query hash memory.py:281-283 + gathered attention
+ * triton_kernel.py:137-272) for a batch of rows whose memories differ in N, C
+ * and Z -- one row = one KV head of one sequence, G <= 16 queries per row (the
+ * G query heads of that KV head, one token each).  A, K, V of all rows are
+ * packed back to back ([sum C, d], [sum N, d]); the bucket lists likewise, each
+ * row holding C*Z indices local to its own keys.  bf16, d = 128 only.
+ *   q [rows,G,d] -> out [rows,G,d], lse [rows,G] fp32, hash_out [rows,G] int32;
+ *   scores_out (optional, [sum C, G] fp32): the scores the hashes were taken over. */
+typedef struct {
+  int64_t a_off;        /* first row of this row's A in A_all            */
+  int64_t k_off;        /* first key row in K_all / V_all                */
+  int64_t idx_off;      /* first element of its bucket lists in idx_all  */
+  int32_t n_keys, n_buckets, bucket_size, reserved;
+} fm_rowdesc;
+int fm_decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
+                        const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, int d,
+                        float sm_scale, void* out, float* lse, int32_t* hash_out, float* scores_out,
+                        int dtype, void* stream);
+
 /* ---- a11: dense local attention with LSE ------------------------------------
  * the attention_forward(q,k_self,v_self,sm_scale,True) call at memory.py:302
  * (the reference ships no definition).  q [H*G,S,d], k,v [H,L,d]; causal is

@@ -516,3 +516,43 @@ def test_reduced_benchmark_workloads_end_to_end(ops, name, N, S, H, C, Z):
                                          ro.float(), rl)
         assert torch.allclose(mo.cpu().double(), eo, atol=2e-2, rtol=1e-2)
         assert (ml.cpu().double() - el).abs().max().item() < 2e-3
+
+
+# ------------------------------------------------------------------ varlen decode batch (config 3 shape)
+def test_decode_batch_of_different_memories(ops):
+    from fast_memory_amd import Memory, MemoryBatch
+    g = gen(950)
+    H, G, d = 2, 4, 128
+    shapes = [(3000, 55, 219), (5000, 71, 283), (4096, 64, 256), (700, 26, 106)]       # (N, C~sqrt N, Z~4 sqrt N)
+    mems, cpu = [], []
+    for N, C, Z in shapes:
+        K = torch.randn(H, N, d, generator=g).to(torch.bfloat16)
+        V = torch.randn(H, N, d, generator=g).to(torch.bfloat16)
+        A = torch.randn(H, C, d, generator=g)
+        A = (A / A.norm(dim=-1, keepdim=True)).to(torch.bfloat16)
+        mems.append(Memory.build(*dev(K, V, A), Z))
+        cpu.append((K, V, A))
+    batch = MemoryBatch(mems)
+    q = (torch.randn(len(shapes), H, G, d, generator=g) * 2).to(torch.bfloat16)
+    q[1, 0, 2] = q[1, 0, 0]                                          # two queries of a row share a bucket
+    out, lse, h, scores = batch.attend(dev(q), 128 ** -0.5, return_scores=True)
+    out, lse, h, scores = out.cpu(), lse.cpu(), h.cpu().long(), scores.cpu()
+    a_off = 0
+    for s, ((N, C, Z), (K, V, A), mem) in enumerate(zip(shapes, cpu, mems)):
+        for hh in range(H):
+            sc = scores[a_off:a_off + C].T                           # [G, C]
+            assert torch.equal(h[s, hh], O.argmax_first(sc)), "hash is not the first argmax of the scores"
+            assert torch.allclose(sc, O.qhash_scores(A[hh:hh + 1], q[s, hh:hh + 1])[0], atol=2e-3, rtol=1e-5)
+            a_off += C
+        lists = mem.bucket_idx.cpu().long()
+        ro, rl = O.hashed_attention_gather(q[s], K, V, lists.reshape(-1), torch.full((H, C), Z), h[s], 128 ** -0.5)
+        assert_attn_close(out[s], lse[s], ro, rl, torch.bfloat16, f"decode batch seq {s}")
+    # merged with 512 local keys per sequence
+    kl = torch.randn(len(shapes), H, 512, d, generator=g).to(torch.bfloat16)
+    vl = torch.randn(len(shapes), H, 512, d, generator=g).to(torch.bfloat16)
+    mo, ml = batch.attend_with_local(dev(q), dev(kl), dev(vl), 128 ** -0.5)
+    for s, ((N, C, Z), (K, V, A), mem) in enumerate(zip(shapes, cpu, mems)):
+        lo, ll = O.local_attention(q[s].reshape(1, H * G, 1, d), kl[s:s + 1], vl[s:s + 1], 128 ** -0.5, True)
+        eo, el = O.lse_merge_closed_form(lo.reshape(H, G, d).float(), ll.reshape(H, G), out[s].float(), lse[s])
+        assert torch.allclose(mo[s].cpu().double(), eo, atol=2e-2, rtol=1e-2)
+        assert (ml[s].cpu().double() - el).abs().max().item() < 2e-3

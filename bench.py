@@ -51,12 +51,117 @@ def timed(fn, reps=1, warm=1):
     return a.elapsed_time(b) / reps, r
 
 
+def fused_phase_times(run):
+    """Milliseconds of the phases of the fused index build, from HIP events the library records on
+    its stream between them."""
+    import ctypes
+    from fast_memory_amd import _lib
+    lib = _lib.load()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(5)]
+    for e in evs:
+        e.record()                      # instantiates the underlying hipEvent_t
+    torch.cuda.synchronize()
+    arr = (ctypes.c_void_p * 5)(*[e.cuda_event for e in evs])
+    lib.fm_debug_set_phase_events(arr, 5)
+    try:
+        run()
+        torch.cuda.synchronize()
+    finally:
+        lib.fm_debug_set_phase_events(None, 0)
+    names = ["thresholds_ms", "mfma_filter_ms", "select_ms", "repair_ms"]
+    return {n: evs[i].elapsed_time(evs[i + 1]) for i, n in enumerate(names)}
+
+
+def bench_decode_batch(args):
+    """Config 3: decode batch of 64 sequences with memories of 8192..131072 keys, 8 KV heads x 4 query
+    heads, one token each, merged with dense attention over 512 local keys per sequence."""
+    from fast_memory_amd import Memory, MemoryBatch, fit_projection, ops, synth
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    base = synth.CONFIGS["c2"]
+    H, G, d = base.H, base.G, base.d
+    lens = synth.decode_lengths()
+    sm_scale = d ** -0.5
+    t0 = time.time()
+    mems, qs, kls, vls = [], [], [], []
+    build_ms = 0.0
+    for s, (N, C, Z) in enumerate(lens):
+        cfg = synth.Config(f"c3-seq{s}", base.dtype, H, G, d, N, C, Z, 1, 256, 20.0, 2, 512, 1003 + s)
+        wl = synth.make_workload(cfg, dev)
+        A = fit_projection(wl.keys, C, iters=2)
+        ms, mem = timed(lambda: Memory.build(wl.keys, wl.values, A, Z), reps=1, warm=0)
+        build_ms += ms
+        mems.append(mem)
+        qs.append(wl.queries.reshape(H, G, d))
+        kls.append(wl.k_local)
+        vls.append(wl.v_local)
+    batch = MemoryBatch(mems)
+    q = torch.stack(qs)
+    kl, vl = torch.stack(kls), torch.stack(vls)
+    n_seq = len(lens)
+    total_keys = sum(n for n, _, _ in lens) * H
+    torch.cuda.synchronize()
+    log(f"[bench] c3: {n_seq} memories built in {time.time() - t0:.1f}s wall, index builds {build_ms:.1f} ms "
+        f"for {total_keys} keys")
+    evs = []
+
+    def step(record=True):
+        a, b = ev_pair()
+        a.record()
+        mo, ml, h = batch.attend(q, sm_scale)
+        b.record()
+        L = kl.shape[2]
+        lo, ll = ops.local_attn_fwd(q.reshape(n_seq * H * G, 1, d), kl.reshape(n_seq * H, L, d),
+                                    vl.reshape(n_seq * H, L, d), sm_scale, True)
+        from fast_memory_amd import update_out_and_lse
+        out, lse = update_out_and_lse(None, None, lo.reshape(n_seq, H, G, d), ll.reshape(n_seq, H, G))
+        out, lse = update_out_and_lse(out.contiguous(), lse.contiguous(), mo, ml)
+        if record:
+            evs.append((a, b))
+        return out, lse, h
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out, lse, h = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    qheads = n_seq * H * G
+    attn_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    hc = h.cpu()
+    alg_bytes = 0
+    for s, (N, C, Z) in enumerate(lens):
+        for hh in range(H):
+            alg_bytes += len(set(hc[s, hh].tolist())) * Z * (2 * d * 2 + 4) + C * d * 2
+    alg_bytes += qheads * (2 * d * 2 + 4)
+    achieved = alg_bytes / attn_ms / 1e6
+    line = {
+        "metric": "hashed-attn query-heads/s", "value": qheads / (ms_per_step * 1e-3), "unit": "query-heads/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"c3-varlen-decode-bf16: {n_seq} sequences, memory lengths {min(l[0] for l in lens)}.."
+                               f"{max(l[0] for l in lens)} keys, H={H}, G={G}, d={d}, C=round(sqrt N), "
+                               f"Z=round(4 sqrt N), 1 token per query head ({qheads} query-heads), 512 local keys",
+                   "step": "batched hash + gather attention (one launch) + local attention + merge"},
+        "roofline": {"kernel": "decode_hash_attn_kernel", "bound": "hbm", "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms},
+        "cpu_baseline": None,
+        "index_build": {"keys_per_s": total_keys / (build_ms * 1e-3), "ms": build_ms, "keys": total_keys},
+    }
+    log(f"[bench] c3 step {ms_per_step:.3f} ms -> {line['value'] / 1e6:.2f} M query-heads/s; decode kernel "
+        f"{attn_ms:.3f} ms = {achieved:.0f} GB/s algorithmic")
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="c5", choices=["c1", "c2", "c4", "c5"])
+    ap.add_argument("--config", default="c5", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--workspace-gib", type=float, default=8.0)
@@ -73,6 +178,8 @@ def main():
     from fast_memory_amd import Memory, fit_projection, ops, synth, update_out_and_lse
     from fast_memory_amd import _lib
     _lib.load()
+    if args.config == "c3":
+        return bench_decode_batch(args)
     cfg = synth.CONFIGS[args.config]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -95,7 +202,16 @@ def main():
     keys_per_s = H * N / (build_ms * 1e-3)
     log(f"[bench] index build: {build_ms:.1f} ms  ({keys_per_s / 1e6:.1f} M keys/s)")
 
-    # component kernels of the build on one chunk of rows
+    build_path = dict(ops.last_build_info)
+    fused_phases = None
+    if build_path.get("path") == "fused":
+        fused_phases = fused_phase_times(lambda: ops.build_index(A, wl.keys, Z, ws_bytes))
+        gemm_flops = 2.0 * H * C * N * d
+        fused_phases["filter_tflops"] = gemm_flops / fused_phases["mfma_filter_ms"] / 1e9
+        fused_phases["filter_mfma_frac"] = fused_phases["filter_tflops"] / BF16_MFMA_PEAK_TFLOPS
+        log(f"[bench] fused build phases (ms): {fused_phases}")
+
+    # component kernels of the unfused build on one chunk of rows
     rows = min(C, max(1, min(512, ws_bytes // (N * 4))))
     Asub = A[:1, :rows].contiguous()
     proj_ms, Y = timed(lambda: ops.project(Asub, wl.keys[:1]), reps=3, warm=1)
@@ -164,6 +280,16 @@ def main():
     qheads = H * Sq
     value = qheads / (ms_per_step * 1e-3)
     out, lse, qh, groups, mo, ml = res
+    query_path = {"ms_per_step": ms_per_step, "query_heads_per_s": value}
+    if args.config == "c4":
+        # index-build-heavy configuration: a step is one index build over all H*N keys
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            ops.build_index(A, wl.keys, Z, ws_bytes)
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+        value = H * N / (ms_per_step * 1e-3)
 
     attn_ms = sum(a.elapsed_time(b) for a, b in attn_events) / len(attn_events)
     parts_ms = {k: (sum(a.elapsed_time(b) for a, b in v) / len(v) if v else None) for k, v in part_events.items()}
@@ -243,19 +369,28 @@ def main():
             torch.equal(ref_lists, mem.bucket_idx[0, :r].cpu().long()))
         log(f"[bench] cpu baseline: {cpu['value']:.1f} query-heads/s on {threads} threads; parity {parity}")
 
+    if args.config == "c4" and fused_phases:
+        roofline = {"kernel": "fused_filter_kernel", "bound": "mfma", "achieved": fused_phases["filter_tflops"],
+                    "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": fused_phases["filter_mfma_frac"],
+                    "traffic": None, "algorithmic_flops_per_launch": 2.0 * H * C * N * d,
+                    "avg_launch_ms": fused_phases["mfma_filter_ms"]}
     line = {
-        "metric": "hashed-attn query-heads/s",
-        "value": value, "unit": "query-heads/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": "index-build keys/s" if args.config == "c4" else "hashed-attn query-heads/s",
+        "value": value, "unit": "keys/s" if args.config == "c4" else "query-heads/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if e == 2 else "f32", "data": "synthetic",
         "config": {"workload": f"{cfg.name}: H={H} KV heads, G={G}, d={d}, N={N} keys/head, C={C}, Z={Z}, "
                                f"S={S} tokens/q-head ({qheads} query-heads)"
                                + (f", {wl.k_local.shape[1]} local keys causal + LSE merge" if has_local else ""),
-                   "step": "qhash + group + gather attention" + (" + local attention + merge" if has_local else "")},
+                   "step": ("index build (sampled thresholds + fused MFMA filter + selection) over all keys"
+                            if args.config == "c4" else
+                            "qhash + group + gather attention" + (" + local attention + merge" if has_local else ""))},
         "roofline": roofline,
         "cpu_baseline": cpu,
-        "index_build": {"keys_per_s": keys_per_s, "ms": build_ms, "keys": H * N, "parts": build_parts,
+        "index_build": {"keys_per_s": keys_per_s, "ms": build_ms, "keys": H * N, "path": build_path,
+                        "fused_phases_ms": fused_phases, "unfused_parts": build_parts,
                         "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters},
+        "query_path": query_path,
         "step_parts_ms": {"attention": attn_ms, **parts_ms},
         "parity_spot_check": parity,
     }

@@ -423,7 +423,19 @@ __global__ void fused_status_kernel(const int32_t* __restrict__ n_fail, int32_t*
   status[1] = max(0, f - kMaxRepair);
 }
 
+// optional phase markers for profiling: events recorded after phases 0, 1, 2, 3
+static hipEvent_t* g_phase_events = nullptr;
+static int g_n_phase_events = 0;
+static inline void mark_phase(int i, hipStream_t st) {
+  if (g_phase_events && i < g_n_phase_events) (void)hipEventRecord(g_phase_events[i], st);
+}
+
 }  // namespace fm
+
+extern "C" void fm_debug_set_phase_events(void** events, int n) {
+  fm::g_phase_events = reinterpret_cast<hipEvent_t*>(events);
+  fm::g_n_phase_events = events ? n : 0;
+}
 
 extern "C" size_t fm_build_index_fused_workspace(int H, int C, int N, int d, int Z, int dtype) {
   fm::FusedPlan p;
@@ -459,6 +471,7 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   const int Zc = Z;  // Z <= N/8 here
 
   // phase 0
+  mark_phase(0, st);
   hipLaunchKernelGGL(gather_sample_kernel, dim3(unsigned(ceil_div(int64_t(p.ns) * (kFD / 8), 256)), unsigned(H)),
                      dim3(256), 0, st, (const bf16_t*)K, Ks, N, p.ns, p.stride);
   int rc = fm_project(A, Ks, Ys, H, C, p.ns, d, p.ld_s, dtype, stream);
@@ -466,20 +479,24 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   hipLaunchKernelGGL(row_threshold_kernel, dim3(unsigned(rows)), dim3(kSelThreads), 0, st, Ys, p.ns,
                      p.ld_s, p.rank, tau, n_fail);
   // phase 1
+  mark_phase(1, st);
   hipLaunchKernelGGL(fused_filter_kernel, dim3(unsigned(p.n_splits), unsigned(p.slabs), unsigned(H)),
                      dim3(kFThreads), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N,
                      p.n_splits, p.cap_w);
   // phase 2
+  mark_phase(2, st);
   const int P = next_pow2(Zc);
   FM_ALLOW_LDS(cand_select_kernel, FM_MAX_Z * sizeof(uint64_t), "fm_build_index_fused: lds");
   hipLaunchKernelGGL(cand_select_kernel, dim3(unsigned(rows)), dim3(kSelThreads),
                      size_t(P) * sizeof(uint64_t), st, cand, cnt, p.n_writers, p.cap_w, Zc, P, idx_out,
                      fail_rows, n_fail);
   // phase 3
+  mark_phase(3, st);
   hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(ceil_div(N, 128)), kMaxRepair), dim3(256), 0,
                      st, (const bf16_t*)A, (const bf16_t*)K, fail_rows, n_fail, Yf, C, N, p.ldy);
   rc = launch_argtopz(Yf, kMaxRepair, N, p.ldy, Zc, idx_out, fail_rows, n_fail, st);
   if (rc) return rc;
   hipLaunchKernelGGL(fused_status_kernel, dim3(1), dim3(1), 0, st, n_fail, status_dev);
+  mark_phase(4, st);
   return launch_status("fm_build_index_fused");
 }

@@ -206,6 +206,11 @@ int fm_segment_mean(const void* X, const int32_t* perm, const int32_t* seg_off,
  * (used by tests to compare the two implementations), 0 restores dispatch. */
 void fm_debug_force_generic(int on);
 
+/* Diagnostic: hand the fused index build up to 5 hipEvent_t (host array that
+ * must stay valid; NULL clears) which it records on its stream before phase 0
+ * (thresholds), 1 (MFMA filter), 2 (selection), 3 (repair) and at the end. */
+void fm_debug_set_phase_events(void** events, int n);
+
 /* Diagnostic: streaming copy of nbytes (multiple of 16) device to device; the
  * known-size kernel that profiler HBM counters are calibrated against. */
 int fm_debug_copy(void* dst, const void* src, int64_t nbytes, void* stream);

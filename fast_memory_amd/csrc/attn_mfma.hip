@@ -81,7 +81,8 @@ __device__ __forceinline__ void load_block(KVRegs& r, const bf16_t* __restrict__
 
 // CAUSAL = false: gathered bucket (rows come from an index list).
 // CAUSAL = true : contiguous keys [0, cnt) with per-query visibility limit.
-template <bool CAUSAL>
+// NQ = number of 16-query tiles the instantiation carries (register footprint grows with it).
+template <bool CAUSAL, int NQ>
 __device__ __forceinline__ void attend_item(
     const bf16_t* __restrict__ Qb,   // query rows of this item's row/head: [*, 128]
     const int* __restrict__ q_rows,  // LDS: row index (into Qb / out) of the item's queries
@@ -94,9 +95,9 @@ __device__ __forceinline__ void attend_item(
   const int nqt = (n_q + 15) >> 4;
 
   // ---- Q^T fragments -------------------------------------------------------
-  uint4 qf[kNQT][4];
+  uint4 qf[NQ][4];
 #pragma unroll
-  for (int qt = 0; qt < kNQT; ++qt) {
+  for (int qt = 0; qt < NQ; ++qt) {
     const int j = qt * 16 + c;
     const bool ok = (qt < nqt) && (j < n_q);
     const uint4* pq = reinterpret_cast<const uint4*>(Qb + int64_t(ok ? q_rows[j] : 0) * kD + 8 * g);
@@ -104,10 +105,10 @@ __device__ __forceinline__ void attend_item(
     for (int s = 0; s < 4; ++s) qf[qt][s] = ok ? pq[4 * s] : make_uint4(0, 0, 0, 0);
   }
 
-  f32x4 O[kNQT][8];
-  float m[kNQT], lsum[kNQT];
+  f32x4 O[NQ][8];
+  float m[NQ], lsum[NQ];
 #pragma unroll
-  for (int qt = 0; qt < kNQT; ++qt) {
+  for (int qt = 0; qt < NQ; ++qt) {
     m[qt] = -INFINITY;
     lsum[qt] = 0.f;
 #pragma unroll
@@ -146,7 +147,7 @@ __device__ __forceinline__ void attend_item(
     }
     const bool tail = CAUSAL || (kp0 + kBlk > cnt);
 #pragma unroll
-    for (int qt = 0; qt < kNQT; ++qt) {
+    for (int qt = 0; qt < NQ; ++qt) {
       if (qt < nqt) {
         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -226,7 +227,7 @@ __device__ __forceinline__ void attend_item(
   float* redL = red + 4 * kNQT * 8 * 4 * 64;
   float* redM = redL + 4 * kNQT * 64;
 #pragma unroll
-  for (int qt = 0; qt < kNQT; ++qt) {
+  for (int qt = 0; qt < NQ; ++qt) {
     if (qt < nqt) {
 #pragma unroll
       for (int t = 0; t < 8; ++t)
@@ -238,7 +239,7 @@ __device__ __forceinline__ void attend_item(
   }
   __syncthreads();
 #pragma unroll
-  for (int qt = 0; qt < kNQT; ++qt) {
+  for (int qt = 0; qt < NQ; ++qt) {
     if (qt < nqt) {
       float mw[4], mstar = -INFINITY;
 #pragma unroll
@@ -295,9 +296,11 @@ __global__ __launch_bounds__(256) void hash_attn_mfma_kernel(
   if (threadIdx.x < it.n_q) q_rows[threadIdx.x] = q_perm[it.q_start + threadIdx.x];
   __syncthreads();
   const int64_t qbase = int64_t(it.row) * Sq;
-  attend_item<false>(q + qbase * kD, q_rows, it.n_q, k + int64_t(it.row) * N * kD,
-                     v + int64_t(it.row) * N * kD, k_idx + bucket_off[bkt], cnt, N, 0, scale2,
-                     out + qbase * kD, lse + qbase, red);
+  const bf16_t* Kb = k + int64_t(it.row) * N * kD;
+  const bf16_t* Vb = v + int64_t(it.row) * N * kD;
+  const int32_t* idx = k_idx + bucket_off[bkt];
+  attend_item<false, kNQT>(q + qbase * kD, q_rows, it.n_q, Kb, Vb, idx, cnt, N, 0, scale2, out + qbase * kD,
+                           lse + qbase, red);
 }
 
 // Dense local attention: one workgroup per (query head, tile of 64 consecutive queries).
@@ -319,8 +322,8 @@ __global__ __launch_bounds__(256) void local_attn_mfma_kernel(
     vis0 = i0 + (L - S);                       // query j of the tile sees keys < vis0 + j + 1
     cnt = min(L, max(0, vis0 + n_q));
   }
-  attend_item<true>(q + qbase * kD, q_rows, n_q, k + int64_t(hk) * L * kD, v + int64_t(hk) * L * kD,
-                    nullptr, cnt, L, vis0, scale2, out + qbase * kD, lse + qbase, red);
+  attend_item<true, 4>(q + qbase * kD, q_rows, n_q, k + int64_t(hk) * L * kD, v + int64_t(hk) * L * kD,
+                       nullptr, cnt, L, vis0, scale2, out + qbase * kD, lse + qbase, red);
 }
 
 // Decode batch over memories of different sizes: one workgroup per row (one KV head
@@ -433,9 +436,9 @@ __global__ __launch_bounds__(256) void decode_hash_attn_kernel(
     }
     __syncthreads();
     const int n_q = q_rows[FM_QTILE - 1];
-    attend_item<false>(qb, q_rows, n_q, Kb, Vb, idx_all + ds.idx_off + int64_t(bkt) * ds.bucket_size,
-                       ds.bucket_size, ds.n_keys, 0, scale2, out + int64_t(row) * G * kD,
-                       lse + int64_t(row) * G, red);
+    attend_item<false, 1>(qb, q_rows, n_q, Kb, Vb, idx_all + ds.idx_off + int64_t(bkt) * ds.bucket_size,
+                          ds.bucket_size, ds.n_keys, 0, scale2, out + int64_t(row) * G * kD,
+                          lse + int64_t(row) * G, red);
   }
 }
 

@@ -486,9 +486,9 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   // phase 2
   mark_phase(2, st);
   const int P = next_pow2(Zc);
-  FM_ALLOW_LDS(cand_select_kernel, FM_MAX_Z * sizeof(uint64_t), "fm_build_index_fused: lds");
+  FM_ALLOW_LDS(cand_select_kernel, sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");
   hipLaunchKernelGGL(cand_select_kernel, dim3(unsigned(rows)), dim3(kSelThreads),
-                     size_t(P) * sizeof(uint64_t), st, cand, cnt, p.n_writers, p.cap_w, Zc, P, idx_out,
+                     sort_lds_bytes(P), st, cand, cnt, p.n_writers, p.cap_w, Zc, P, idx_out,
                      fail_rows, n_fail);
   // phase 3
   mark_phase(3, st);

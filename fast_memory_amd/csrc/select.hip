@@ -30,9 +30,9 @@ __global__ __launch_bounds__(kSelThreads) void argtopz_kernel(
 int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out,
                    const int32_t* row_map, const int32_t* n_rows_dev, hipStream_t st) {
   const int P = next_pow2(Zc);
-  FM_ALLOW_LDS(argtopz_kernel, FM_MAX_Z * sizeof(uint64_t), "argtopz: lds");
+  FM_ALLOW_LDS(argtopz_kernel, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
   hipLaunchKernelGGL(argtopz_kernel, dim3(unsigned(rows)), dim3(kSelThreads),
-                     size_t(P) * sizeof(uint64_t), st, Y, N, ldy, Zc, P, idx_out, row_map, n_rows_dev);
+                     sort_lds_bytes(P), st, Y, N, ldy, Zc, P, idx_out, row_map, n_rows_dev);
   return launch_status("argtopz");
 }
 

@@ -1,6 +1,6 @@
 // Exact top-Z selection shared by the dense arg-top-Z kernel and the fused
 // index build: radix select over unique 64-bit composites, collection of the
-// survivors into LDS and an in-LDS bitonic sort.
+// survivors into LDS and a register-blocked in-LDS bitonic sort.
 //
 // composite(y, i) = (float_key(y) << 32) | (2^32-1 - i): descending composite
 // order is "value descending, index ascending", and composites are unique, so
@@ -89,8 +89,99 @@ __device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int
   return cut;
 }
 
+// ---- in-LDS bitonic sort, descending, register-blocked -------------------------
+// The P = 2^logP keys live in LDS at phys(e) = e + e/16 (one pad slot per 16 keeps
+// every access pattern below spread over the banks).  A thread owns 16 keys whose
+// indices differ in four consecutive bits [p, p+4); all compare-exchange stages
+// whose distance bit falls in that window run in registers, so a pass over LDS
+// (load 16, up to four stages, store 16) replaces up to four passes of the plain
+// network: 29 passes instead of 105 at P = 16384.
+__device__ __forceinline__ int sort_phys(int e) { return e + (e >> 4); }
+static inline size_t sort_lds_bytes(int P) { return size_t(P + (P >> 4) + 1) * sizeof(uint64_t); }
+
+// One compare-exchange stage at register distance 2^D.  Key i of a thread sorts descending when
+// bit L of its index is 0; that bit is either a thread bit (tdesc, the same for all 16 keys) or,
+// when ib >= 0, bit ib of the register number i (uniform per unrolled i).  Keys are unique (or equal
+// padding), so "a > b" is "!(a < b)".
+template <int D>
+__device__ __forceinline__ void sort_stage_regs(uint64_t (&r)[16], bool tdesc, int ib) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    if (i & (1 << D)) continue;
+    const int j = i | (1 << D);
+    const bool flip = ib >= 0 && ((i >> ib) & 1);
+    const uint64_t a = r[i], b = r[j];
+    const bool sw = (a < b) == (tdesc != flip);
+    r[i] = sw ? b : a;
+    r[j] = sw ? a : b;
+  }
+}
+
+__device__ __forceinline__ void bitonic_sort_desc(uint64_t* buf, int logP) {
+  const int tid = threadIdx.x;
+  if (logP < 6) {  // tiny: plain network, one key pair per thread step
+    const int P = 1 << logP;
+    for (int k = 2; k <= P; k <<= 1)
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        for (int t = tid; t < (P >> 1); t += kSelThreads) {
+          const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+          const int q = i | j;
+          const uint64_t a = buf[sort_phys(i)], b = buf[sort_phys(q)];
+          const bool desc = (i & k) == 0;
+          if (desc ? (a < b) : (a > b)) {
+            buf[sort_phys(i)] = b;
+            buf[sort_phys(q)] = a;
+          }
+        }
+        __syncthreads();
+      }
+    return;
+  }
+  const bool active = tid < (1 << (logP - 4));
+  uint64_t r[16];
+  auto pass = [&](int p, int L, int s_hi, int s_lo, int L_first, int L_last) {
+    // one LDS round trip; either the stages s_hi..s_lo of level L, or (L_first > 0) all stages of
+    // the levels L_first..L_last, which must all lie in the window [p, p+4)
+    if (active) {
+      const int base = (tid & ((1 << p) - 1)) | ((tid >> p) << (p + 4));
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[i] = buf[sort_phys(base | (i << p))];
+      auto run = [&](int lev, int hi, int lo) {
+        const int ib = (lev >= p && lev < p + 4) ? lev - p : -1;  // level bit inside the register window?
+        const bool tdesc = ib >= 0 ? true : (((base >> lev) & 1) == 0);
+        for (int s = hi; s >= lo; --s) {
+          switch (s - p) {
+            case 0: sort_stage_regs<0>(r, tdesc, ib); break;
+            case 1: sort_stage_regs<1>(r, tdesc, ib); break;
+            case 2: sort_stage_regs<2>(r, tdesc, ib); break;
+            default: sort_stage_regs<3>(r, tdesc, ib); break;
+          }
+        }
+      };
+      if (L_first > 0)
+        for (int lev = L_first; lev <= L_last; ++lev) run(lev, lev - 1, 0);
+      else
+        run(L, s_hi, s_lo);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) buf[sort_phys(base | (i << p))] = r[i];
+    }
+    __syncthreads();
+  };
+  pass(0, 0, 0, 0, 1, 4);  // levels 1..4 entirely in registers
+  for (int L = 5; L <= logP; ++L) {
+    int s = L - 1;
+    while (s >= 0) {
+      const int lo = s - 3 > 0 ? s - 3 : 0;
+      const int p = lo < logP - 4 ? lo : logP - 4;
+      pass(p, L, s, lo, 0, 0);
+      s = lo - 1;
+    }
+  }
+}
+
 // Collects the composites >= cut (at most P) into buf, pads to P with zeros,
-// sorts descending and writes the first Zc indices to out.
+// sorts descending and writes the first Zc indices to out.  buf holds
+// sort_lds_bytes(P) bytes.
 template <typename Source>
 __device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, int Zc, int P,
                                                    uint64_t* buf, SelectShared& sh,
@@ -102,27 +193,13 @@ __device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, in
     uint64_t c = composite(y, i);
     if (c >= cut) {
       int pos = atomicAdd(&sh.cnt, 1);
-      if (pos < P) buf[pos] = c;
+      if (pos < P) buf[sort_phys(pos)] = c;
     }
   });
-  for (int i = Zc + tid; i < P; i += kSelThreads) buf[i] = 0;
+  for (int i = Zc + tid; i < P; i += kSelThreads) buf[sort_phys(i)] = 0;
   __syncthreads();
-  for (int k = 2; k <= P; k <<= 1) {
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      for (int t = tid; t < (P >> 1); t += kSelThreads) {
-        int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
-        int p = i | j;
-        uint64_t a = buf[i], b = buf[p];
-        bool desc = (i & k) == 0;
-        if (desc ? (a < b) : (a > b)) {
-          buf[i] = b;
-          buf[p] = a;
-        }
-      }
-      __syncthreads();
-    }
-  }
-  for (int i = tid; i < Zc; i += kSelThreads) out[i] = int32_t(0xffffffffu - uint32_t(buf[i]));
+  bitonic_sort_desc(buf, 31 - __clz(P));
+  for (int i = tid; i < Zc; i += kSelThreads) out[i] = int32_t(0xffffffffu - uint32_t(buf[sort_phys(i)]));
 }
 
 // Dense fp32 row as a source; 128-bit loads on the aligned body, kUnroll of

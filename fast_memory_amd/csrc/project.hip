@@ -241,6 +241,151 @@ __global__ __launch_bounds__(256) void qhash_bf16_kernel(const bf16_t* __restric
   }
 }
 
+// ---------------------------------------------------------------------------
+// bf16 query hash, d = 128, streaming form (no scores written): a workgroup of 8
+// waves holds 512 queries as resident MFMA B fragments (64 per wave) and streams
+// the bucket rows of A through a double-buffered LDS tile of 64 rows.  One query
+// per lane column: the running maximum and its position are per-lane registers,
+// updated with three VALU instructions per accumulator register (compare, select
+// value, select the row number as an inline constant); buckets arrive in
+// ascending order, so "strictly greater" keeps the first maximum.  The scores are
+// the same MFMA sums as in qhash_bf16_kernel (same instruction, operand roles and
+// contraction order), so both kernels return identical hashes.
+// Roofline: MFMA, 2*C*d flops per query.
+// ---------------------------------------------------------------------------
+constexpr int kQsLd = 128 + 8;
+
+template <int K>
+__device__ __forceinline__ void argmax_step(float& best, int& pos, float s) {
+  asm volatile("v_cmp_gt_f32 vcc, %2, %0\n\tv_cndmask_b32_e32 %0, %0, %2, vcc\n\tv_cndmask_b32_e64 %1, %1, %3, vcc"
+               : "+v"(best), "+v"(pos)
+               : "v"(s), "n"(K)
+               : "vcc");
+}
+
+template <int MI, int R>
+__device__ __forceinline__ void argmax_tile(float& best, int& pos, const f32x16& acc) {
+  if constexpr (R < 16) {
+    argmax_step<MI * 32 + 8 * (R >> 2) + (R & 3)>(best, pos, acc[R]);
+    argmax_tile<MI, R + 1>(best, pos, acc);
+  }
+}
+
+__global__ __launch_bounds__(512) void qhash_stream_kernel(const bf16_t* __restrict__ A,
+                                                           const bf16_t* __restrict__ q,
+                                                           int32_t* __restrict__ hash_out, int C, int Sq) {
+  __shared__ __attribute__((aligned(16))) bf16_t sA[2][64 * kQsLd];
+  const int h = blockIdx.y;
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+  const bf16_t* Ah = A + int64_t(h) * C * 128;
+  const bf16_t* qh = q + int64_t(h) * Sq * 128;
+  const int i0 = blockIdx.x * 512 + w * 64;
+
+  bf16x8 bfrag[2][8];
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int i = i0 + ni * 32 + (l & 31);
+    const bool ok = i < Sq;
+    const uint4* pq = reinterpret_cast<const uint4*>(qh + int64_t(ok ? i : 0) * 128 + (l >> 5) * 8);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      union {
+        uint4 u;
+        bf16x8 b;
+      } cvt;
+      cvt.u = ok ? pq[2 * ks] : make_uint4(0, 0, 0, 0);
+      bfrag[ni][ks] = cvt.b;
+    }
+  }
+  float best[2] = {-INFINITY, -INFINITY};
+  int pos[2] = {0, 0}, btile[2] = {0, 0};
+
+  const int ntiles = (C + 63) / 64;
+  auto fetch = [&](int t, uint4 (&st)[2]) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int e = tid + u * 512;
+      const int r = t * 64 + (e >> 4);
+      st[u] = r < C ? reinterpret_cast<const uint4*>(Ah + int64_t(r) * 128)[e & 15] : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stash = [&](int buf, const uint4 (&st)[2]) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int e = tid + u * 512;
+      *reinterpret_cast<uint4*>(&sA[buf][(e >> 4) * kQsLd + (e & 15) * 8]) = st[u];
+    }
+  };
+  uint4 st[2];
+  fetch(0, st);
+  stash(0, st);
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const int buf = t & 1;
+    if (t + 1 < ntiles) fetch(t + 1, st);
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+    const bf16_t* pa = &sA[buf][(l & 31) * kQsLd + (l >> 5) * 8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(pa + ks * 16);
+      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(pa + 32 * kQsLd + ks * 16);
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        acc[0][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, bfrag[ni][ks], acc[0][ni], 0, 0, 0);
+        acc[1][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, bfrag[ni][ks], acc[1][ni], 0, 0, 0);
+      }
+    }
+    if (t * 64 + 64 <= C) {
+      // the asm reads accumulators the hazard logic cannot see into: let the MFMA pipeline drain
+      asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        const float before = best[ni];
+        argmax_tile<0, 0>(best[ni], pos[ni], acc[0][ni]);
+        argmax_tile<1, 0>(best[ni], pos[ni], acc[1][ni]);
+        if (best[ni] != before) btile[ni] = t;
+      }
+    } else {  // last, partial tile: rows past C are padding
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kk = mi * 32 + 8 * (r >> 2) + (r & 3);
+            const float sv = acc[mi][ni][r];
+            if (t * 64 + kk + 4 * (l >> 5) < C && sv > best[ni]) {
+              best[ni] = sv;
+              pos[ni] = kk;
+              btile[ni] = t;
+            }
+          }
+    }
+    if (t + 1 < ntiles) stash(buf ^ 1, st);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    int idx = btile[ni] * 64 + pos[ni] + 4 * (l >> 5);
+    float b = best[ni];
+    if (b == -INFINITY) idx = 0x7fffffff;  // nothing seen (only NaN or -inf scores): handled below
+    const float ob = __shfl_xor(b, 32);
+    const int oi = __shfl_xor(idx, 32);
+    if (oi != 0x7fffffff && (idx == 0x7fffffff || ob > b || (ob == b && oi < idx))) {
+      b = ob;
+      idx = oi;
+    }
+    const int i = i0 + ni * 32 + (l & 31);
+    if (l < 32 && i < Sq) hash_out[int64_t(h) * Sq + i] = idx == 0x7fffffff ? 0 : idx;
+  }
+}
+
 }  // namespace fm
 
 extern "C" int fm_project(const void* A, const void* K, float* Y, int H, int C, int N, int d,
@@ -286,7 +431,11 @@ extern "C" int fm_qhash(const void* A, const void* q, int32_t* hash_out, float* 
   FM_REQUIRE(A && q && hash_out, FM_ERR_ARG, "fm_qhash: null pointer");
   FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_qhash: H=%d > 65535", H);
   hipStream_t st = as_stream(stream);
-  if (dtype == FM_BF16 && d % 16 == 0) {
+  if (dtype == FM_BF16 && d == 128 && !scores_out) {
+    dim3 grid = dim3(unsigned(ceil_div(Sq, 512)), unsigned(H));
+    hipLaunchKernelGGL(qhash_stream_kernel, grid, dim3(512), 0, st, (const bf16_t*)A, (const bf16_t*)q,
+                       hash_out, C, Sq);
+  } else if (dtype == FM_BF16 && d % 16 == 0) {
     size_t lds = size_t(2) * 128 * (d + 8) * sizeof(bf16_t);
     FM_ALLOW_LDS(qhash_bf16_kernel, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_qhash: lds");
     dim3 grid = dim3(unsigned(ceil_div(Sq, 128)), unsigned(H));

@@ -342,8 +342,14 @@ def main():
         n = int(max(n, min(Sq, n * args.cpu_seconds / max(t_probe, 1e-3))))
         sel = pick(n)
         t_cpu = cpu_path.time_query_path(q0[sel], K0, V0, A0, lists0, sm_scale, kl0, vl0, sel % S, S)
+        if t_cpu < 0.6 * args.cpu_seconds and n < Sq:
+            # queries that share a bucket share its gather, so the cost per query falls as the
+            # sample grows: size it once more from the larger run
+            n = int(min(Sq, n * args.cpu_seconds / max(t_cpu, 1e-3)))
+            sel = pick(n)
+            t_cpu = cpu_path.time_query_path(q0[sel], K0, V0, A0, lists0, sm_scale, kl0, vl0, sel % S, S)
         # index-build sample: a few rows of A against all keys of head 0
-        r = 2 if N > 200000 else 16
+        r = min(C, 32 if N > 200000 else 64)
         tb0 = time.perf_counter()
         cpu_lists = cpu_path.build_rows(A0[:r], K0, Z)
         t_build = time.perf_counter() - tb0

@@ -51,6 +51,7 @@ SIGNATURES = {
     "fm_segment_mean": (c_int, [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_debug_force_generic": (None, [c_int]),
     "fm_debug_copy": (c_int, [P, P, c_int64, P]),
+    "fm_debug_read": (c_int, [P, c_int64, P, P]),
     "fm_debug_set_phase_events": (None, [P, c_int]),
 }
 

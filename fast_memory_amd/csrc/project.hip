@@ -248,7 +248,11 @@ __global__ __launch_bounds__(256) void qhash_bf16_kernel(const bf16_t* __restric
 // per lane column: the running maximum and its position are per-lane registers,
 // updated with three VALU instructions per accumulator register (compare, select
 // value, select the row number as an inline constant); buckets arrive in
-// ascending order, so "strictly greater" keeps the first maximum.  The scores are
+// ascending order, so "strictly greater" keeps the first maximum.  The loop is
+// software-pipelined in half tiles: while the MFMAs of one 32-row sub-tile run,
+// the finished sub-tile before it is scanned and the A fragments of the next are
+// read from LDS.  On this hardware VALU and MFMA time of a SIMD add up rather
+// than overlap, so the scan costs about as much as the products.  The scores are
 // the same MFMA sums as in qhash_bf16_kernel (same instruction, operand roles and
 // contraction order), so both kernels return identical hashes.
 // Roofline: MFMA, 2*C*d flops per query.
@@ -263,11 +267,51 @@ __device__ __forceinline__ void argmax_step(float& best, int& pos, float s) {
                : "vcc");
 }
 
-template <int MI, int R>
-__device__ __forceinline__ void argmax_tile(float& best, int& pos, const f32x16& acc) {
-  if constexpr (R < 16) {
-    argmax_step<MI * 32 + 8 * (R >> 2) + (R & 3)>(best, pos, acc[R]);
-    argmax_tile<MI, R + 1>(best, pos, acc);
+// position of accumulator register R of the 32-row sub-tile MI inside the 64-row tile, for
+// lanes 0..31 (lanes 32..63 hold the rows 4 further down)
+constexpr int qs_row(int MI, int R) { return MI * 32 + 8 * (R >> 2) + (R & 3); }
+
+// Elements E and E+1 (of 32: query column half E/16, register E%16) of a finished sub-tile.
+// Register 0 of each half goes through plain C++ so that the compiler, which cannot see into the
+// asm, places the wait states a read of a fresh MFMA result needs; the MFMA that produced a half
+// was issued before those of anything read later.
+template <int MI, int E>
+__device__ __forceinline__ void argmax_pair(float (&best)[2], int (&pos)[2], const f32x16 (&acc)[2]) {
+  constexpr int NI = E >> 4, R = E & 15;
+  if constexpr (R == 0) {
+    const bool gt = acc[NI][0] > best[NI];
+    best[NI] = gt ? acc[NI][0] : best[NI];
+    pos[NI] = gt ? qs_row(MI, 0) : pos[NI];
+  } else {
+    argmax_step<qs_row(MI, R)>(best[NI], pos[NI], acc[NI][R]);
+  }
+  argmax_step<qs_row(MI, R + 1)>(best[NI], pos[NI], acc[NI][R + 1]);
+}
+
+// One half step of the pipeline: the 16 MFMAs of sub-tile (MM) of one tile, with the running
+// argmax over the finished sub-tile (ME) of the tile before it and the LDS reads of the next
+// half step's A fragments spread between them.  sched_barrier pins the interleaving: an MFMA
+// keeps the matrix pipe busy for 32 cycles, the six VALU instructions behind it take 24.
+template <int ME, bool MFMA, bool PREFETCH, int I>
+__device__ __forceinline__ void qs_half_step(f32x16 (&accM)[2], const f32x16 (&accE)[2], const bf16x8 (&af)[8],
+                                             bf16x8 (&af_next)[8], const bf16_t* next_lds,
+                                             const bf16x8 (&bfrag)[2][8], float (&best)[2], int (&pos)[2]) {
+  if constexpr (I < 16) {
+    constexpr int ks = I >> 1, ni = I & 1;
+    if constexpr (MFMA) {
+      if constexpr (ks == 0) {
+        f32x16 z;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+        accM[ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks], bfrag[ni][ks], z, 0, 0, 0);
+      } else {
+        accM[ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks], bfrag[ni][ks], accM[ni], 0, 0, 0);
+      }
+    }
+    if constexpr (PREFETCH && ni == 0) af_next[ks] = *reinterpret_cast<const bf16x8*>(next_lds + ks * 16);
+    argmax_pair<ME, 2 * I>(best, pos, accE);
+    __builtin_amdgcn_sched_barrier(0);
+    qs_half_step<ME, MFMA, PREFETCH, I + 1>(accM, accE, af, af_next, next_lds, bfrag, best, pos);
   }
 }
 
@@ -301,73 +345,66 @@ __global__ __launch_bounds__(512) void qhash_stream_kernel(const bf16_t* __restr
   int pos[2] = {0, 0}, btile[2] = {0, 0};
 
   const int ntiles = (C + 63) / 64;
-  auto fetch = [&](int t, uint4 (&st)[2]) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int e = tid + u * 512;
-      const int r = t * 64 + (e >> 4);
-      st[u] = r < C ? reinterpret_cast<const uint4*>(Ah + int64_t(r) * 128)[e & 15] : make_uint4(0, 0, 0, 0);
-    }
+  // rows past C repeat row 0: an equal score later in the order never replaces the running maximum
+  uint4 st0, st1;  // a tile on its way from global memory to LDS: rows tid/16 and 32 + tid/16
+  auto fetch = [&](int t) {
+    const int r0 = t * 64 + (tid >> 4), r1 = r0 + 32;
+    st0 = reinterpret_cast<const uint4*>(Ah + int64_t(r0 < C ? r0 : 0) * 128)[tid & 15];
+    st1 = reinterpret_cast<const uint4*>(Ah + int64_t(r1 < C ? r1 : 0) * 128)[tid & 15];
   };
-  auto stash = [&](int buf, const uint4 (&st)[2]) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int e = tid + u * 512;
-      *reinterpret_cast<uint4*>(&sA[buf][(e >> 4) * kQsLd + (e & 15) * 8]) = st[u];
-    }
+  auto stash = [&](int buf) {
+    *reinterpret_cast<uint4*>(&sA[buf][(tid >> 4) * kQsLd + (tid & 15) * 8]) = st0;
+    *reinterpret_cast<uint4*>(&sA[buf][(32 + (tid >> 4)) * kQsLd + (tid & 15) * 8]) = st1;
   };
-  uint4 st[2];
-  fetch(0, st);
-  stash(0, st);
+  // LDS address of this lane's A fragment 0 of sub-tile mi of the tile in buffer buf
+  auto frag_ptr = [&](int buf, int mi) -> const bf16_t* {
+    return &sA[buf][(mi * 32 + (l & 31)) * kQsLd + (l >> 5) * 8];
+  };
+  fetch(0);
+  stash(0);
+  if (ntiles > 1) {
+    fetch(1);
+    stash(1);
+  }
   __syncthreads();
+
+  // Pipeline over half steps: sub-tile 0 of tile t+1 is multiplied while sub-tile 1 of tile t
+  // is scanned, and the other way round; tile t+2 travels global -> registers -> LDS meanwhile.
+  f32x16 acc[2][2];
+  bf16x8 af0[8], af1[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) af0[ks] = *reinterpret_cast<const bf16x8*>(frag_ptr(0, 0) + ks * 16);
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    f32x16 z;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) z[r] = 0.f;
+    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af0[ks], bfrag[0][ks], ks ? acc[0][0] : z, 0, 0, 0);
+    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af0[ks], bfrag[1][ks], ks ? acc[0][1] : z, 0, 0, 0);
+    af1[ks] = *reinterpret_cast<const bf16x8*>(frag_ptr(0, 1) + ks * 16);
+  }
   for (int t = 0; t < ntiles; ++t) {
-    const int buf = t & 1;
-    if (t + 1 < ntiles) fetch(t + 1, st);
-    f32x16 acc[2][2];
-#pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
-    const bf16_t* pa = &sA[buf][(l & 31) * kQsLd + (l >> 5) * 8];
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(pa + ks * 16);
-      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(pa + 32 * kQsLd + ks * 16);
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni) {
-        acc[0][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, bfrag[ni][ks], acc[0][ni], 0, 0, 0);
-        acc[1][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, bfrag[ni][ks], acc[1][ni], 0, 0, 0);
-      }
+    const bool more = t + 1 < ntiles;
+    if (t + 2 < ntiles) fetch(t + 2);
+    {
+      const float b0 = best[0], b1 = best[1];
+      if (more)
+        qs_half_step<0, true, true, 0>(acc[1], acc[0], af1, af0, frag_ptr((t + 1) & 1, 0), bfrag, best, pos);
+      else
+        qs_half_step<0, true, false, 0>(acc[1], acc[0], af1, af0, nullptr, bfrag, best, pos);
+      if (best[0] != b0) btile[0] = t;
+      if (best[1] != b1) btile[1] = t;
     }
-    if (t * 64 + 64 <= C) {
-      // the asm reads accumulators the hazard logic cannot see into: let the MFMA pipeline drain
-      asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni) {
-        const float before = best[ni];
-        argmax_tile<0, 0>(best[ni], pos[ni], acc[0][ni]);
-        argmax_tile<1, 0>(best[ni], pos[ni], acc[1][ni]);
-        if (best[ni] != before) btile[ni] = t;
-      }
-    } else {  // last, partial tile: rows past C are padding
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int kk = mi * 32 + 8 * (r >> 2) + (r & 3);
-            const float sv = acc[mi][ni][r];
-            if (t * 64 + kk + 4 * (l >> 5) < C && sv > best[ni]) {
-              best[ni] = sv;
-              pos[ni] = kk;
-              btile[ni] = t;
-            }
-          }
+    {
+      const float b0 = best[0], b1 = best[1];
+      if (more)
+        qs_half_step<1, true, true, 0>(acc[0], acc[1], af0, af1, frag_ptr((t + 1) & 1, 1), bfrag, best, pos);
+      else
+        qs_half_step<1, false, false, 0>(acc[0], acc[1], af0, af1, nullptr, bfrag, best, pos);
+      if (best[0] != b0) btile[0] = t;
+      if (best[1] != b1) btile[1] = t;
     }
-    if (t + 1 < ntiles) stash(buf ^ 1, st);
+    if (t + 2 < ntiles) stash(t & 1);  // the buffer of tile t: its last reads were a tile ago
     __syncthreads();
   }
 #pragma unroll

@@ -215,6 +215,11 @@ void fm_debug_set_phase_events(void** events, int n);
  * known-size kernel that profiler HBM counters are calibrated against. */
 int fm_debug_copy(void* dst, const void* src, int64_t nbytes, void* stream);
 
+/* Diagnostic: read-only stream over nbytes (multiple of 32768) of device memory;
+ * nothing is written (sink: 4 bytes of device memory, left untouched).  Times the
+ * read bandwidth a kernel reaches on the device. */
+int fm_debug_read(const void* src, int64_t nbytes, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,251 @@
+// Dense local attention for bf16, head dimension 128 (gfx950): the attention over
+// the most recent keys that the memory's output is merged with (call site
+// memory.py:302; the reference leaves `attention_forward` undefined, the contract
+// here is softmax(q.k^T * scale) v with a causal mask aligned bottom-right, output
+// plus natural-log LSE).
+//
+// One workgroup (4 waves) per 128 consecutive queries of one query head, 32 queries
+// per wave.  K and V tiles of 64 keys go global -> registers -> LDS, double buffered;
+// V is transposed on the way ( Vt[d][key] ) because both MFMA operands want the
+// contraction index contiguous per lane.
+//   S^T = K.Q^T    v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q^T fragments
+//                  resident in registers.  Lane (query l%32, half l/32) ends up with
+//                  the scores of keys 8*(r/4) + 4*(l/32) + r%4 of each 32-key block:
+//                  one query per lane column, so the softmax statistics are per-lane
+//                  registers and need one cross-half shuffle per tile.
+//   O^T += Vt.P^T  same instruction; registers 8s..8s+7 of a score block are exactly
+//                  the B operand of contraction step s if the 16 keys of the step are
+//                  taken in the order [0..3, 8..11 | 4..7, 12..15]; Vt is stored in LDS
+//                  with its key columns in that order, so neither P nor V is shuffled.
+// Softmax as in the gather kernel (triton_kernel.py:248-263): base 2 with
+// sm_scale*log2(e), fp32 running max and denominator, denominator from unrounded p,
+// p rounded to bf16 before P.V.
+//
+// Roofline: MFMA (4*d flops per visible query-key pair); the per-element softmax
+// VALU work is of the same order as the MFMA time and does not overlap with it.
+#include "common.hpp"
+
+namespace fm {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+
+constexpr int kLD = 128;    // head dimension
+constexpr int kLQ = 128;    // queries per workgroup
+constexpr int kLK = 64;     // keys per tile
+constexpr int kLKld = 136;  // K tile row stride in LDS (elements)
+constexpr int kLVld = 72;   // Vt row stride in LDS (elements): 64 keys + 8
+
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+  f32x2 x = {lo, hi};
+  bf16x2 y = __builtin_convertvector(x, bf16x2);  // v_cvt_pk_bf16_f32, round to nearest even
+  return *reinterpret_cast<uint32_t*>(&y);
+}
+
+__device__ __forceinline__ bf16x8 u4_as_bf16x8(uint4 u) {
+  union {
+    uint4 u;
+    bf16x8 b;
+  } x;
+  x.u = u;
+  return x.b;
+}
+
+struct LocalTileRegs {
+  uint4 k[4];  // K rows tid/16 + 16u, 16-byte chunk tid%16
+  uint4 v[4];  // V rows 4j..4j+3 (j = lane/4), chunk c = 4*wave + lane%4
+};
+
+__global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    bf16_t* __restrict__ out, float* __restrict__ lse, int G, int S, int L, float scale2, int causal) {
+  __shared__ __attribute__((aligned(16))) bf16_t sK[2][kLK * kLKld];
+  __shared__ __attribute__((aligned(16))) bf16_t sVt[2][kLD * kLVld];
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+  const int col = l & 31, hb = l >> 5;
+  const int hq = blockIdx.y, hk = hq / G;
+  const int qb = int(gridDim.x) - 1 - int(blockIdx.x);  // late query blocks see most keys: start them first
+  const int i0 = qb * kLQ;
+  const bf16_t* Kh = k + int64_t(hk) * L * kLD;
+  const bf16_t* Vh = v + int64_t(hk) * L * kLD;
+  const int64_t qrow0 = int64_t(hq) * S;
+
+  // visible keys: query i sees keys [0, lim(i))
+  auto lim_of = [&](int i) { return causal ? min(L, max(0, i + (L - S) + 1)) : L; };
+  const int i_last = min(S, i0 + kLQ) - 1;
+  const int wg_lim = lim_of(i_last);
+  const int ntiles = (wg_lim + kLK - 1) / kLK;
+
+  const int iq = i0 + w * 32 + col;  // this lane's query
+  const bool q_ok = iq < S;
+  const int my_lim = q_ok ? lim_of(iq) : 0;
+  const int wave_lim_hi = lim_of(min(S - 1, i0 + w * 32 + 31));  // most keys any query of the wave sees
+  const int wave_lim_lo = (i0 + w * 32 + 31 < S) ? lim_of(i0 + w * 32) : 0;  // fewest
+
+  bf16x8 qf[8];
+  {
+    const uint4* pq = reinterpret_cast<const uint4*>(q + (qrow0 + (q_ok ? iq : 0)) * kLD + hb * 8);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = u4_as_bf16x8(q_ok ? pq[2 * ks] : make_uint4(0, 0, 0, 0));
+  }
+  f32x16 O[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) O[dt][r] = 0.f;
+  float m = -INFINITY, lsum = 0.f;
+
+  LocalTileRegs tr;
+  const int vj = l >> 2, vc = 4 * w + (l & 3);
+  auto load_tile = [&](int t) {
+    const int kp0 = t * kLK;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int row = kp0 + (tid >> 4) + 16 * u;
+      tr.k[u] = row < L ? reinterpret_cast<const uint4*>(Kh + int64_t(row) * kLD)[tid & 15] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int row = kp0 + 4 * vj + kk;
+      tr.v[kk] = row < L ? reinterpret_cast<const uint4*>(Vh + int64_t(row) * kLD)[vc] : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stash_tile = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      *reinterpret_cast<uint4*>(&sK[buf][((tid >> 4) + 16 * u) * kLKld + (tid & 15) * 8]) = tr.k[u];
+    // keys 4j..4j+3 of the tile keep their order; the groups of four inside each 16 are
+    // stored in the order 0, 2, 1, 3
+    const int a = vj >> 2, g4 = vj & 3;
+    const int pos0 = 16 * a + 4 * ((g4 & 1) * 2 + (g4 >> 1));
+    const uint32_t w0[4] = {tr.v[0].x, tr.v[0].y, tr.v[0].z, tr.v[0].w};
+    const uint32_t w1[4] = {tr.v[1].x, tr.v[1].y, tr.v[1].z, tr.v[1].w};
+    const uint32_t w2[4] = {tr.v[2].x, tr.v[2].y, tr.v[2].z, tr.v[2].w};
+    const uint32_t w3[4] = {tr.v[3].x, tr.v[3].y, tr.v[3].z, tr.v[3].w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int wi = e >> 1;
+      uint2 o;
+      if (e & 1) {
+        o.x = (w0[wi] >> 16) | (w1[wi] & 0xffff0000u);
+        o.y = (w2[wi] >> 16) | (w3[wi] & 0xffff0000u);
+      } else {
+        o.x = (w0[wi] & 0xffffu) | (w1[wi] << 16);
+        o.y = (w2[wi] & 0xffffu) | (w3[wi] << 16);
+      }
+      *reinterpret_cast<uint2*>(&sVt[buf][(8 * vc + e) * kLVld + pos0]) = o;
+    }
+  };
+
+  auto compute_tile = [&](int t, int buf) {
+    const int kp0 = t * kLK;
+    if (kp0 >= wave_lim_hi) return;  // no query of this wave sees the tile
+    // ---- S^T for the two 32-key blocks ----
+    f32x16 s[2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[sb][r] = 0.f;
+      const bf16_t* pa = &sK[buf][(sb * 32 + col) * kLKld + hb * 8];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks)
+        s[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(pa + ks * 16), qf[ks],
+                                                        s[sb], 0, 0, 0);
+    }
+    // ---- mask (only tiles that reach past what some query of the wave sees) ----
+    if (kp0 + kLK > wave_lim_lo) {
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kp0 + sb * 32 + 8 * (r >> 2) + 4 * hb + (r & 3);
+          if (key >= my_lim) s[sb][r] = -INFINITY;
+        }
+    }
+    // ---- online softmax, one query per lane column ----
+    float mx = s[0][0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[0][r]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[1][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32)) * scale2;  // scale2 > 0: scaling commutes with the maximum
+    const float m_new = fmaxf(m, mx);
+    const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;  // a query that sees no key yet
+    if (__any(m_new != m)) {
+      const float alpha = __builtin_amdgcn_exp2f(m - m_sub);
+      lsum *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) O[dt][r] *= alpha;
+      m = m_new;
+    }
+    bf16x8 pf[2][2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float p[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        p[r] = __builtin_amdgcn_exp2f(fmaf(s[sb][r], scale2, -m_sub));
+        lsum += p[r];
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+        pf[sb][st] = u4_as_bf16x8(make_uint4(cvt_pk_bf16(p[8 * st + 0], p[8 * st + 1]), cvt_pk_bf16(p[8 * st + 2], p[8 * st + 3]),
+                                             cvt_pk_bf16(p[8 * st + 4], p[8 * st + 5]), cvt_pk_bf16(p[8 * st + 6], p[8 * st + 7])));
+    }
+    // ---- O^T += Vt.P^T ----
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      const bf16_t* pv = &sVt[buf][(dt * 32 + col) * kLVld + hb * 8];
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+          O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(pv + sb * 32 + st * 16),
+                                                          pf[sb][st], O[dt], 0, 0, 0);
+    }
+  };
+
+  if (ntiles > 0) {
+    load_tile(0);
+    stash_tile(0);
+  }
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    if (t + 1 < ntiles) load_tile(t + 1);
+    compute_tile(t, t & 1);
+    if (t + 1 < ntiles) stash_tile((t + 1) & 1);  // last read one tile ago, behind the barrier below
+    __syncthreads();
+  }
+
+  // ---- finish: lane (query, half) holds d = 32*dt + 8*(r/4) + 4*half + r%4 ----
+  const float ltot = lsum + __shfl_xor(lsum, 32);
+  const bool empty = (m == -INFINITY);
+  const float inv = empty ? 0.f : 1.f / ltot;
+  if (q_ok) {
+    bf16_t* po = out + (qrow0 + iq) * kLD;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        uint2 o;
+        o.x = cvt_pk_bf16(O[dt][4 * rq + 0] * inv, O[dt][4 * rq + 1] * inv);
+        o.y = cvt_pk_bf16(O[dt][4 * rq + 2] * inv, O[dt][4 * rq + 3] * inv);
+        *reinterpret_cast<uint2*>(po + dt * 32 + 8 * rq + 4 * hb) = o;
+      }
+    if (hb == 0) lse[qrow0 + iq] = empty ? -FLT_MAX : (m + __builtin_amdgcn_logf(ltot)) * kLn2;
+  }
+}
+
+int local_attn_dense(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G, int S,
+                     int L, float sm_scale, int causal, hipStream_t st) {
+  dim3 grid = dim3(unsigned(ceil_div(S, kLQ)), unsigned(H * G));
+  hipLaunchKernelGGL(local_attn_dense_kernel, grid, dim3(256), 0, st, (const bf16_t*)q, (const bf16_t*)k,
+                     (const bf16_t*)v, (bf16_t*)out, lse, G, S, L, sm_scale * kLog2e, causal);
+  return launch_status("fm_local_attn_fwd(dense)");
+}
+
+}  // namespace fm

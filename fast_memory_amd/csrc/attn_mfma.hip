@@ -1,6 +1,5 @@
-// bf16 attention on MFMA for head dimension 128 (gfx950): the bucket-gathered
-// forward (triton_kernel.py:137-272) and the dense local attention it is merged
-// with (call site memory.py:302).
+// bf16 bucket-gathered attention forward on MFMA for head dimension 128 (gfx950)
+// (triton_kernel.py:137-272), for grouped work items and for decode batches.
 //
 // Work decomposition.  One workgroup (4 waves) per work item = up to 64 queries
 // that hashed to the same (row, bucket).  The bucket's key list is cut into
@@ -55,8 +54,13 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint4 u) {
   return x.b;
 }
 
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+  f32x2 x = {lo, hi};
+  bf16x2 y = __builtin_convertvector(x, bf16x2);  // v_cvt_pk_bf16_f32, round to nearest even
+  return *reinterpret_cast<uint32_t*>(&y);
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -79,17 +83,14 @@ __device__ __forceinline__ void load_block(KVRegs& r, const bf16_t* __restrict__
   }
 }
 
-// CAUSAL = false: gathered bucket (rows come from an index list).
-// CAUSAL = true : contiguous keys [0, cnt) with per-query visibility limit.
 // NQ = number of 16-query tiles the instantiation carries (register footprint grows with it).
-template <bool CAUSAL, int NQ>
+template <int NQ>
 __device__ __forceinline__ void attend_item(
     const bf16_t* __restrict__ Qb,   // query rows of this item's row/head: [*, 128]
     const int* __restrict__ q_rows,  // LDS: row index (into Qb / out) of the item's queries
     int n_q, const bf16_t* __restrict__ Kb, const bf16_t* __restrict__ Vb,
-    const int32_t* __restrict__ idx,  // bucket list (nullptr when CAUSAL)
-    int cnt, int N, int vis0,         // CAUSAL: query j of the item sees keys < vis0 + j + 1
-    float scale2, bf16_t* __restrict__ Ob, float* __restrict__ Lb, float* __restrict__ red) {
+    const int32_t* __restrict__ idx,  // bucket list
+    int cnt, int N, float scale2, bf16_t* __restrict__ Ob, float* __restrict__ Lb, float* __restrict__ red) {
   const int l = lane_id(), w = threadIdx.x >> 6;
   const int g = l >> 4, c = l & 15;
   const int nqt = (n_q + 15) >> 4;
@@ -119,7 +120,7 @@ __device__ __forceinline__ void attend_item(
   auto rows_of = [&](int b) -> int {
     const int kp = b * kBlk + (l & 31);
     int r = 0;
-    if (kp < cnt) r = CAUSAL ? kp : idx[kp];
+    if (kp < cnt) r = idx[kp];
     return min(max(r, 0), N - 1);
   };
 
@@ -145,7 +146,7 @@ __device__ __forceinline__ void attend_item(
                        : ((a[2 * e] & 0xffffu) | (a[2 * e + 1] << 16));
       vf[t] = make_uint4(o[0], o[1], o[2], o[3]);
     }
-    const bool tail = CAUSAL || (kp0 + kBlk > cnt);
+    const bool tail = kp0 + kBlk > cnt;
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
       if (qt < nqt) {
@@ -162,8 +163,7 @@ __device__ __forceinline__ void attend_item(
           x[4 + r] = s1[r] * scale2;
         }
         if (tail) {
-          int lim = cnt;
-          if (CAUSAL) lim = min(cnt, vis0 + qt * 16 + c + 1);
+          const int lim = cnt;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             if (kp0 + 4 * g + r >= lim) x[r] = -INFINITY;
@@ -177,26 +177,32 @@ __device__ __forceinline__ void attend_item(
         const float m_new = fmaxf(m[qt], mx);
         // a query that sees no key yet keeps m = -inf; subtract 0 instead of -inf
         const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m[qt] - m_sub);
-        m[qt] = m_new;
+        // bucket lists are sorted by descending projection, so after the first blocks the
+        // running maximum rarely moves: rescale only when it moved for some query of the tile
+        if (__any(m_new != m[qt])) {
+          const float alpha = fast_exp2(m[qt] - m_sub);
+          lsum[qt] *= alpha;
+#pragma unroll
+          for (int t = 0; t < 8; ++t) {
+            O[qt][t][0] *= alpha;
+            O[qt][t][1] *= alpha;
+            O[qt][t][2] *= alpha;
+            O[qt][t][3] *= alpha;
+          }
+          m[qt] = m_new;
+        }
         float p[8], ps = 0.f;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
           p[r] = fast_exp2(x[r] - m_sub);
           ps += p[r];
         }
-        lsum[qt] = lsum[qt] * alpha + ps;
+        lsum[qt] += ps;
         const uint4 pf = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]),
                                     pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          f32x4 o = O[qt][t];
-          o[0] *= alpha;
-          o[1] *= alpha;
-          o[2] *= alpha;
-          o[3] *= alpha;
-          O[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[t]), as_bf16x8(pf), o, 0, 0, 0);
-        }
+        for (int t = 0; t < 8; ++t)
+          O[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[t]), as_bf16x8(pf), O[qt][t], 0, 0, 0);
       }
     }
   };
@@ -299,31 +305,8 @@ __global__ __launch_bounds__(256) void hash_attn_mfma_kernel(
   const bf16_t* Kb = k + int64_t(it.row) * N * kD;
   const bf16_t* Vb = v + int64_t(it.row) * N * kD;
   const int32_t* idx = k_idx + bucket_off[bkt];
-  attend_item<false, kNQT>(q + qbase * kD, q_rows, it.n_q, Kb, Vb, idx, cnt, N, 0, scale2, out + qbase * kD,
-                           lse + qbase, red);
-}
-
-// Dense local attention: one workgroup per (query head, tile of 64 consecutive queries).
-__global__ __launch_bounds__(256) void local_attn_mfma_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
-    bf16_t* __restrict__ out, float* __restrict__ lse, int G, int S, int L, float scale2,
-    int causal) {
-  extern __shared__ __attribute__((aligned(16))) float red[];
-  __shared__ int q_rows[FM_QTILE];
-  const int hq = blockIdx.y, hk = hq / G;
-  const int i0 = blockIdx.x * FM_QTILE;
-  const int n_q = min(FM_QTILE, S - i0);
-  if (threadIdx.x < FM_QTILE) q_rows[threadIdx.x] = i0 + threadIdx.x;
-  __syncthreads();
-  const int64_t qbase = int64_t(hq) * S;
-  // keys any query of the tile can see; per-query limit applied inside
-  int cnt = L, vis0 = L;  // non-causal: every query sees all L keys
-  if (causal) {
-    vis0 = i0 + (L - S);                       // query j of the tile sees keys < vis0 + j + 1
-    cnt = min(L, max(0, vis0 + n_q));
-  }
-  attend_item<true, 4>(q + qbase * kD, q_rows, n_q, k + int64_t(hk) * L * kD, v + int64_t(hk) * L * kD,
-                       nullptr, cnt, L, vis0, scale2, out + qbase * kD, lse + qbase, red);
+  attend_item<kNQT>(q + qbase * kD, q_rows, it.n_q, Kb, Vb, idx, cnt, N, scale2, out + qbase * kD,
+                     lse + qbase, red);
 }
 
 // Decode batch over memories of different sizes: one workgroup per row (one KV head
@@ -436,9 +419,8 @@ __global__ __launch_bounds__(256) void decode_hash_attn_kernel(
     }
     __syncthreads();
     const int n_q = q_rows[FM_QTILE - 1];
-    attend_item<false, 1>(qb, q_rows, n_q, Kb, Vb, idx_all + ds.idx_off + int64_t(bkt) * ds.bucket_size,
-                          ds.bucket_size, ds.n_keys, 0, scale2, out + int64_t(row) * G * kD,
-                          lse + int64_t(row) * G, red);
+    attend_item<1>(qb, q_rows, n_q, Kb, Vb, idx_all + ds.idx_off + int64_t(bkt) * ds.bucket_size, ds.bucket_size,
+                   ds.n_keys, scale2, out + int64_t(row) * G * kD, lse + int64_t(row) * G, red);
   }
 }
 
@@ -469,15 +451,13 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
   return launch_status("fm_hash_attn_fwd(mfma)");
 }
 
+int local_attn_dense(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G, int S,
+                     int L, float sm_scale, int causal, hipStream_t st);
+
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
                     int S, int L, int d, float sm_scale, int causal, hipStream_t st) {
   (void)d;
-  FM_ALLOW_LDS(local_attn_mfma_kernel, kRedFloats * sizeof(float), "fm_local_attn_fwd: lds");
-  dim3 grid = dim3(unsigned(ceil_div(S, FM_QTILE)), unsigned(H * G));
-  hipLaunchKernelGGL(local_attn_mfma_kernel, grid, dim3(256), kRedFloats * sizeof(float), st,
-                     (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)out, lse, G, S,
-                     L, sm_scale * kLog2e, causal);
-  return launch_status("fm_local_attn_fwd(mfma)");
+  return local_attn_dense(q, k, v, out, lse, H, G, S, L, sm_scale, causal, st);
 }
 
 }  // namespace fm

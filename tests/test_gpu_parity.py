@@ -288,6 +288,10 @@ def test_lse_merge(ops):
     (torch.bfloat16, 2, 4, 1, 512, 128, True),          # decode: one query sees all local keys
     (torch.float32, 1, 1, 16, 80, 32, True),            # rectangular, bottom-right aligned
     (torch.bfloat16, 1, 2, 70, 130, 128, False),
+    (torch.bfloat16, 1, 2, 300, 1000, 128, True),       # several query blocks, ragged tiles
+    (torch.bfloat16, 1, 1, 260, 100, 128, True),        # more queries than keys: the first 160 see nothing
+    (torch.bfloat16, 1, 1, 128, 64, 128, False),        # exactly one tile
+    (torch.bfloat16, 2, 2, 129, 257, 128, True),
 ])
 def test_local_attention(ops, dtype, H, G, S, L, d, causal):
     g = gen(600)

@@ -13,10 +13,12 @@
 //            owns one bucket column: its threshold, its write cursor and its
 //            private segment of the row's candidate buffer live in registers and
 //            survivors are appended with plain stores -- no atomics.
-//   phase 2  cand_select_kernel: exact top-Z (value desc, index asc) of each
-//            row's candidates: radix select + in-LDS bitonic sort, the same code
-//            as the dense arg-top-Z kernel, reading ~1.2 Z candidates instead of
-//            the N-element row.
+//   phase 2  exact top-Z (value desc, index asc) of each row's candidates, the
+//            same code as the dense arg-top-Z kernel reading ~1.2 Z candidates
+//            instead of the N-element row, in two kernels of very different
+//            shape: cand_cut_kernel (radix select of the cut; small workgroups,
+//            many per compute unit) and cand_sort_kernel (collect + in-LDS
+//            bitonic sort; one workgroup fills a compute unit's LDS).
 //   phase 3  repair.  A row whose candidate count fell short of Z or overflowed
 //            a segment is listed by phase 2; its Y row is recomputed (same MFMA
 //            instruction and contraction order) into a small buffer and handed to
@@ -49,7 +51,7 @@ constexpr int kMaxRepair = 64;
 struct FusedPlan {
   int ns, stride, rank, n_splits, slabs, n_writers, cap_w;
   int64_t ld_s, ldy;
-  size_t off_Ks, off_Ys, off_tau, off_cand, off_cnt, off_fail, off_nfail, off_Yf, total;
+  size_t off_Ks, off_Ys, off_tau, off_cand, off_cnt, off_cut, off_ok, off_fail, off_nfail, off_Yf, total;
 };
 
 static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& p) {
@@ -82,6 +84,8 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   p.off_tau = take(rows * sizeof(float));
   p.off_cand = take(rows * p.n_writers * size_t(p.cap_w) * sizeof(uint2));
   p.off_cnt = take(rows * p.n_writers * sizeof(int32_t));
+  p.off_cut = take(rows * sizeof(uint64_t));
+  p.off_ok = take(rows * sizeof(int32_t));
   p.off_fail = take(kMaxRepair * sizeof(int32_t));
   p.off_nfail = take(4 * sizeof(int32_t));
   p.off_Yf = take(size_t(kMaxRepair) * p.ldy * sizeof(float));
@@ -321,13 +325,14 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
 }
 
 // ---- phase 2 ---------------------------------------------------------------
+template <int NT>
 struct CandRow {
   const uint2* base;  // [n_writers][cap_w] (value bits, key index)
   const int* counts;  // LDS, clamped to cap_w
   int n_writers, cap_w, maxc;
   template <typename F>
   __device__ __forceinline__ void operator()(F f) const {
-    for (int j = threadIdx.x; j < maxc; j += kSelThreads) {
+    for (int j = threadIdx.x; j < maxc; j += NT) {
       for (int w0 = 0; w0 < n_writers; w0 += 8) {
         uint2 e[8];
 #pragma unroll
@@ -345,40 +350,74 @@ struct CandRow {
   }
 };
 
-__global__ __launch_bounds__(kSelThreads) void cand_select_kernel(
-    const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, int n_writers, int cap_w,
-    int Zc, int P, int32_t* __restrict__ idx_out, int32_t* __restrict__ fail_rows,
-    int32_t* __restrict__ n_fail) {
-  extern __shared__ uint64_t buf[];
-  __shared__ SelectShared sh;
-  __shared__ int s_counts[64];
-  __shared__ int s_total, s_over, s_max;
-  const int64_t row = blockIdx.x;
-  if (threadIdx.x == 0) {
-    int total = 0, over = 0, mx = 0;
-    for (int w = 0; w < n_writers; ++w) {
-      int c = cnt[row * n_writers + w];
-      over |= (c > cap_w);
-      c = min(c, cap_w);
-      s_counts[w] = c;
-      total += c;
-      mx = max(mx, c);
+// Loads the per-writer counts of a row into LDS; returns false (to all threads) if a segment
+// overflowed or the row has fewer than Zc candidates, i.e. the sampled threshold failed.
+struct CandCounts {
+  int counts[64];
+  int total, over, maxc;
+};
+__device__ __forceinline__ bool load_cand_counts(const int32_t* __restrict__ cnt, int64_t row, int n_writers,
+                                                 int cap_w, int Zc, CandCounts& cc) {
+  if (threadIdx.x < 64) {
+    int c = threadIdx.x < n_writers ? cnt[row * n_writers + threadIdx.x] : 0;
+    const int over = __any(c > cap_w);
+    c = min(c, cap_w);
+    cc.counts[threadIdx.x] = c;
+    int total = c, mx = c;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      total += __shfl_xor(total, o);
+      mx = max(mx, __shfl_xor(mx, o));
     }
-    s_total = total;
-    s_over = over;
-    s_max = mx;
+    if (threadIdx.x == 0) {
+      cc.total = total;
+      cc.over = over;
+      cc.maxc = mx;
+    }
   }
   __syncthreads();
-  if (s_over || s_total < Zc) {  // threshold missed for this row: queue it for repair
+  return !(cc.over || cc.total < Zc);
+}
+
+// Phase 2a: the exact cut (Zc-th largest composite) of every row's candidates.  Small workgroups
+// with a small LDS footprint, so that eight rows per compute unit hide each other's round trips
+// (a pass over ~1.2 Zc candidates is short and latency-bound).
+constexpr int kCutThreads = 256;
+__global__ __launch_bounds__(kCutThreads) void cand_cut_kernel(
+    const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, int n_writers, int cap_w, int Zc,
+    uint64_t* __restrict__ cut_out, int32_t* __restrict__ row_ok, int32_t* __restrict__ fail_rows,
+    int32_t* __restrict__ n_fail) {
+  __shared__ SelectShared sh;
+  __shared__ CandCounts cc;
+  const int64_t row = blockIdx.x;
+  if (!load_cand_counts(cnt, row, n_writers, cap_w, Zc, cc)) {  // queue the row for repair
     if (threadIdx.x == 0) {
+      row_ok[row] = 0;
       int pos = atomicAdd(n_fail, 1);
       if (pos < kMaxRepair) fail_rows[pos] = int32_t(row);
     }
     return;
   }
-  CandRow src{cand + row * n_writers * int64_t(cap_w), s_counts, n_writers, cap_w, s_max};
-  const uint64_t cut = radix_select_cut(src, Zc, 6, sh);
-  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + row * Zc);
+  CandRow<kCutThreads> src{cand + row * n_writers * int64_t(cap_w), cc.counts, n_writers, cap_w, cc.maxc};
+  const uint64_t cut = radix_select_cut<kCutThreads>(src, Zc, 6, sh);
+  if (threadIdx.x == 0) {
+    cut_out[row] = cut;
+    row_ok[row] = 1;
+  }
+}
+
+// Phase 2b: the Zc candidates at or above the cut, sorted in LDS, indices out.
+__global__ __launch_bounds__(kSelThreads) void cand_sort_kernel(
+    const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, const uint64_t* __restrict__ cut_in,
+    const int32_t* __restrict__ row_ok, int n_writers, int cap_w, int Zc, int P, int32_t* __restrict__ idx_out) {
+  extern __shared__ uint64_t buf[];
+  __shared__ SelectShared sh;
+  __shared__ CandCounts cc;
+  const int64_t row = blockIdx.x;
+  if (!row_ok[row]) return;
+  load_cand_counts(cnt, row, n_writers, cap_w, Zc, cc);
+  CandRow<kSelThreads> src{cand + row * n_writers * int64_t(cap_w), cc.counts, n_writers, cap_w, cc.maxc};
+  collect_sort_write(src, cut_in[row], Zc, P, buf, sh, idx_out + row * Zc);
 }
 
 // ---- phase 3 ---------------------------------------------------------------
@@ -464,6 +503,8 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   float* tau = reinterpret_cast<float*>(base + p.off_tau);
   uint2* cand = reinterpret_cast<uint2*>(base + p.off_cand);
   int32_t* cnt = reinterpret_cast<int32_t*>(base + p.off_cnt);
+  uint64_t* cut = reinterpret_cast<uint64_t*>(base + p.off_cut);
+  int32_t* row_ok = reinterpret_cast<int32_t*>(base + p.off_ok);
   int32_t* fail_rows = reinterpret_cast<int32_t*>(base + p.off_fail);
   int32_t* n_fail = reinterpret_cast<int32_t*>(base + p.off_nfail);
   float* Yf = reinterpret_cast<float*>(base + p.off_Yf);
@@ -486,10 +527,11 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   // phase 2
   mark_phase(2, st);
   const int P = next_pow2(Zc);
-  FM_ALLOW_LDS(cand_select_kernel, sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");
-  hipLaunchKernelGGL(cand_select_kernel, dim3(unsigned(rows)), dim3(kSelThreads),
-                     sort_lds_bytes(P), st, cand, cnt, p.n_writers, p.cap_w, Zc, P, idx_out,
-                     fail_rows, n_fail);
+  hipLaunchKernelGGL(cand_cut_kernel, dim3(unsigned(rows)), dim3(kCutThreads), 0, st, cand, cnt, p.n_writers,
+                     p.cap_w, Zc, cut, row_ok, fail_rows, n_fail);
+  FM_ALLOW_LDS(cand_sort_kernel, sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");
+  hipLaunchKernelGGL(cand_sort_kernel, dim3(unsigned(rows)), dim3(kSelThreads), sort_lds_bytes(P), st, cand, cnt,
+                     cut, row_ok, p.n_writers, p.cap_w, Zc, P, idx_out);
   // phase 3
   mark_phase(3, st);
   hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(ceil_div(N, 128)), kMaxRepair), dim3(256), 0,

@@ -38,8 +38,9 @@ struct SelectShared {
 // looking at no more than `max_passes` digits (12,10,10 value bits, then
 // 11,11,10 index bits).  With all 6 passes the cut is exact; with fewer it is a
 // lower bound of the need0-th largest composite (at least need0 are >= cut).
-// Every thread of the workgroup must call this; returns the same cut to all.
-template <typename Source>
+// Every thread of the workgroup (NT threads, a power of two between 64 and 1024) must call
+// this; returns the same cut to all.
+template <int NT = kSelThreads, typename Source>
 __device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int max_passes,
                                                      SelectShared& sh) {
   const int tid = threadIdx.x;
@@ -54,7 +55,7 @@ __device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int
     const int bits = kBits[pass];
     const int shift = top - bits;
     const int nb = 1 << bits;
-    for (int i = tid; i < nb; i += kSelThreads) sh.hist[i] = 0;
+    for (int i = tid; i < nb; i += NT) sh.hist[i] = 0;
     __syncthreads();
     const uint64_t prefix = sh.prefix;
     const int need = sh.need;
@@ -65,7 +66,7 @@ __device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int
     });
     __syncthreads();
     // thread t owns `per` bins, walking digits from the largest down
-    const int per = nb >> 10;
+    const int per = nb / NT;
     int local = 0;
     for (int j = 0; j < per; ++j) local += int(sh.hist[nb - 1 - (tid * per + j)]);
     int total;

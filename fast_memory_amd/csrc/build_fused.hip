@@ -32,6 +32,8 @@
 //
 // Roofline of phase 1: MFMA, 2*d flops per (key, bucket) pair; K is re-read once
 // per 512-bucket slab from L2.  Phases 0, 2, 3 are HBM/L2-bound and small.
+#include <type_traits>
+
 #include "mfma_tile.hpp"
 #include "select.hpp"
 
@@ -93,6 +95,12 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   return true;
 }
 
+// The filter stores a candidate's key as a code: first key of its 32-key half-tile (a multiple of
+// 32) + 16*(lane half) + accumulator register r; that register holds key row 8*(r/4) + 4*half + r%4.
+__device__ __forceinline__ uint32_t fused_key_of_code(uint32_t code) {
+  return (code & ~31u) + ((code & 12u) << 1) + ((code & 16u) >> 2) + (code & 3u);
+}
+
 // ---- phase 0 ---------------------------------------------------------------
 __global__ __launch_bounds__(256) void gather_sample_kernel(const bf16_t* __restrict__ K,
                                                             bf16_t* __restrict__ Ks, int N, int ns,
@@ -139,8 +147,13 @@ __global__ __launch_bounds__(kSelThreads) void row_threshold_kernel(const float*
 __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const float* __restrict__ tau,
     uint2* __restrict__ cand, int32_t* __restrict__ cnt, int C, int N, int n_splits, int cap_w) {
-  __shared__ __attribute__((aligned(16))) bf16_t sK[2][kFKeys * kFLd];
-  __shared__ __attribute__((aligned(16))) float sDump[kFWaves][2 * 4 * 64 * 4];  // [wave][ni][q][lane][4]
+  // one object, so that the dump area is preceded by the key tiles: a lane without candidates
+  // reads 256 bytes below its dump column, which must stay inside the allocation
+  __shared__ __attribute__((aligned(16))) struct {
+    bf16_t keys[2][kFKeys * kFLd];
+    float dump[kFWaves][2 * 16 * 64];  // [wave][column half ni][accumulator register][lane]
+  } sm;
+  bf16_t(&sK)[2][kFKeys * kFLd] = sm.keys;
   const int sk = blockIdx.x, slab = blockIdx.y, h = blockIdx.z;
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   const int n_writers = 2 * n_splits;
@@ -193,7 +206,7 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
   // segments of this workgroup's 512 bucket rows; lane offsets below are bytes from here
   const int64_t wg_row0 = int64_t(h) * C + int64_t(slab) * kFSlab;
   char* cbase = reinterpret_cast<char*>(cand + wg_row0 * n_writers * int64_t(cap_w));
-  float* dump = sDump[w];
+  float* dump = sm.dump[w];
 
   bf16x8 bfrag[2][8];
   float th[2];
@@ -226,28 +239,27 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     for (int ks = 0; ks < 8; ++ks) asm volatile("" ::"v"(bfrag[ni][ks]));
     asm volatile("" ::"v"(th[ni]));
   }
-  const int lane_key = (l >> 5) << 2;
+  const int lane_code = (l >> 5) << 4;
   uint32_t msk[2];
 
-  // threshold test of four accumulator registers: mask = 2*mask + (y >= th); and their dump
-  auto test_dump4 = [&](const f32x16& a, int ni, int q) {
-    // The dump comes first: it is the compiler-visible read of freshly written MFMA results, so the
-    // wait states an MFMA result needs before it can be read are inserted there; the asm below
-    // (whose operands the hazard logic does not look into) then only ever reads settled registers.
-    *reinterpret_cast<float4*>(&dump[((ni * 4 + q) * 64 + l) * 4]) =
-        make_float4(a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      asm volatile("v_cmp_nlt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
-                   : "+v"(msk[ni])
-                   : "v"(a[4 * q + j]), "v"(th[ni])
-                   : "vcc", "memory");
+  // Threshold test of one accumulator register: mask = 2*mask + (y >= th), and its dump.  The
+  // registers of a column half are tested from 15 down to 0, so bit r of the mask belongs to
+  // register r.  The dump comes first: it is the compiler-visible read of freshly written MFMA
+  // results, so the wait states an MFMA result needs before it can be read are inserted there; the
+  // asm (whose operands the hazard logic does not look into) then only ever reads settled registers.
+  auto test_dump = [&](const f32x16& a, int ni, int r) {
+    dump[(ni * 16 + r) * 64 + l] = a[r];
+    asm volatile("v_cmp_nlt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
+                 : "+v"(msk[ni])
+                 : "v"(a[r]), "v"(th[ni])
+                 : "vcc", "memory");
   };
-  // Emission: every lane pops up to two mask bits per column (highest bit = earliest test first),
-  // reads those accumulator values back from its LDS dump (all four reads in flight together) and
-  // appends (value, key).  Bit 15-r of a mask belongs to accumulator register r, i.e. key row
-  // 8*(r/4) + 4*(l/32) + r%4 of the half-tile.  A lane without bits pops a harmless r = 15.
-  auto emit = [&](int keyl, bool check_n) {
+  // Emission: every lane pops up to two mask bits per column half (lowest register first), reads
+  // those values back from its LDS dump (all four reads in flight together) and appends
+  // (value bits, key code) to its segment.  The key code is  first key of the half-tile + 16*(l/32)
+  // + register; fused_key_of_code() turns it into the key index.  A lane without bits reads a
+  // harmless word below its column and stores nothing.
+  auto emit = [&](auto check_n, uint32_t code0) {
     bool has[4];
     int r[4];
     float y[4];
@@ -255,20 +267,21 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     for (int p = 0; p < 4; ++p) {
       uint32_t& m = msk[p >> 1];
       has[p] = m != 0;
-      const int b = 31 - __clz(int(m | 1u));
-      m &= ~(1u << b);
-      r[p] = 15 - b;
+      r[p] = __builtin_ffs(int(m)) - 1;
+      m &= m - 1u;
     }
 #pragma unroll
-    for (int p = 0; p < 4; ++p) y[p] = dump[(((p >> 1) * 4 + (r[p] >> 2)) * 64 + l) * 4 + (r[p] & 3)];
+    for (int p = 0; p < 4; ++p) y[p] = dump[((p >> 1) * 16 + r[p]) * 64 + l];
     // keep the four reads together ahead of the predicated stores (one LDS round trip, not four)
     asm volatile("" : "+v"(y[0]), "+v"(y[1]), "+v"(y[2]), "+v"(y[3]));
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const int ni = p >> 1;
-      const int key = keyl + 8 * (r[p] >> 2) + (r[p] & 3);
-      if (has[p] && (!check_n || key < N)) {
-        *reinterpret_cast<uint2*>(cbase + off[ni]) = make_uint2(__float_as_uint(y[p]), uint32_t(key));
+      const uint32_t code = code0 + uint32_t(r[p]);
+      bool ok = has[p];
+      if constexpr (decltype(check_n)::value) ok = ok && fused_key_of_code(code) < uint32_t(N);
+      if (ok) {
+        *reinterpret_cast<uint2*>(cbase + off[ni]) = make_uint2(__float_as_uint(y[p]), code);
         off[ni] += 8u;
       }
     }
@@ -300,17 +313,23 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) test_dump4(acc[ni], ni, q);
+          for (int r = 15; r >= 0; --r) test_dump(acc[ni], ni, r);
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
           if (off[ni] > lim[ni]) {  // fewer than 16 free slots: wrap and mark the row for repair
             off[ni] = start[ni];
             ovf[ni] = 1;
           }
-        const int keyl = kbase + half * 32 + lane_key;
-        do {
-          emit(keyl, check_n);
-        } while (__ballot((msk[0] | msk[1]) != 0));
+        const uint32_t code0 = uint32_t(kbase + half * 32 + lane_code);
+        if (check_n) {
+          do {
+            emit(std::true_type{}, code0);
+          } while (__ballot((msk[0] | msk[1]) != 0));
+        } else {
+          do {
+            emit(std::false_type{}, code0);
+          } while (__ballot((msk[0] | msk[1]) != 0));
+        }
       }
     }
     __syncthreads();
@@ -327,7 +346,7 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
 // ---- phase 2 ---------------------------------------------------------------
 template <int NT>
 struct CandRow {
-  const uint2* base;  // [n_writers][cap_w] (value bits, key index)
+  const uint2* base;  // [n_writers][cap_w] (value bits, key code)
   const int* counts;  // LDS, clamped to cap_w
   int n_writers, cap_w, maxc;
   template <typename F>
@@ -343,7 +362,7 @@ struct CandRow {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const int w = w0 + u;
-          if (w < n_writers && j < counts[w]) f(__uint_as_float(e[u].x), e[u].y);
+          if (w < n_writers && j < counts[w]) f(__uint_as_float(e[u].x), fused_key_of_code(e[u].y));
         }
       }
     }

@@ -12,6 +12,7 @@
 #pragma once
 #include "common.hpp"
 
+
 namespace fm {
 
 constexpr int kSelThreads = 1024;
@@ -92,7 +93,8 @@ __device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int
 
 // ---- in-LDS bitonic sort, descending, register-blocked -------------------------
 // The P = 2^logP keys live in LDS at phys(e) = e + e/16 (one pad slot per 16 keeps
-// every access pattern below spread over the banks).  A thread owns 16 keys whose
+// every access pattern below spread over the banks; an XOR swizzle of the low index bits that
+// looks conflict-free on paper measured slower).  A thread owns 16 keys whose
 // indices differ in four consecutive bits [p, p+4); all compare-exchange stages
 // whose distance bit falls in that window run in registers, so a pass over LDS
 // (load 16, up to four stages, store 16) replaces up to four passes of the plain
@@ -140,9 +142,20 @@ __device__ __forceinline__ void bitonic_sort_desc(uint64_t* buf, int logP) {
   }
   const bool active = tid < (1 << (logP - 4));
   uint64_t r[16];
+  // A pass whose window lies below bit 10 only moves keys inside aligned groups of 1024, and a
+  // group of 1024 is exactly what one wave owns in such a pass (64 threads x 16 keys).  Between
+  // two such passes the waves need no workgroup barrier, only program order inside the wave (the
+  // LDS serves one wave's requests in order); they drift apart and one wave's LDS traffic overlaps
+  // another's compare-exchanges.  A barrier stands only around the passes with a window above bit 6.
+  int prev_p = 31;
   auto pass = [&](int p, int L, int s_hi, int s_lo, int L_first, int L_last) {
     // one LDS round trip; either the stages s_hi..s_lo of level L, or (L_first > 0) all stages of
     // the levels L_first..L_last, which must all lie in the window [p, p+4)
+    if (p > 6 || prev_p > 6)
+      __syncthreads();
+    else
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    prev_p = p;
     if (active) {
       const int base = (tid & ((1 << p) - 1)) | ((tid >> p) << (p + 4));
 #pragma unroll
@@ -166,7 +179,6 @@ __device__ __forceinline__ void bitonic_sort_desc(uint64_t* buf, int logP) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) buf[sort_phys(base | (i << p))] = r[i];
     }
-    __syncthreads();
   };
   pass(0, 0, 0, 0, 1, 4);  // levels 1..4 entirely in registers
   for (int L = 5; L <= logP; ++L) {
@@ -178,6 +190,7 @@ __device__ __forceinline__ void bitonic_sort_desc(uint64_t* buf, int logP) {
       s = lo - 1;
     }
   }
+  __syncthreads();
 }
 
 // Collects the composites >= cut (at most P) into buf, pads to P with zeros,

@@ -13,6 +13,7 @@
 #include "common.hpp"
 
 
+
 namespace fm {
 
 constexpr int kSelThreads = 1024;
@@ -102,21 +103,54 @@ __device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int
 __device__ __forceinline__ int sort_phys(int e) { return e + (e >> 4); }
 static inline size_t sort_lds_bytes(int P) { return size_t(P + (P >> 4) + 1) * sizeof(uint64_t); }
 
-// One compare-exchange stage at register distance 2^D.  Key i of a thread sorts descending when
-// bit L of its index is 0; that bit is either a thread bit (tdesc, the same for all 16 keys) or,
-// when ib >= 0, bit ib of the register number i (uniform per unrolled i).  Keys are unique (or equal
-// padding), so "a > b" is "!(a < b)".
-template <int D>
-__device__ __forceinline__ void sort_stage_regs(uint64_t (&r)[16], bool tdesc, int ib) {
+// The 16 keys of a thread as separate low and high words: the compare-exchange below works on
+// 32-bit registers.
+struct SortKeys {
+  uint32_t lo[16], hi[16];
+};
+
+// Compare-exchange, larger key to slot i.  A 64-bit subtract (two full-rate instructions) leaves
+// "key i < key j" in the carry, which selects the four output words; the quarter-rate 64-bit
+// compare is avoided.
+__device__ __forceinline__ void sort_ce(SortKeys& k, int i, int j) {
+  uint32_t t, nil, nih, njl, njh;
+  asm("v_sub_co_u32 %0, vcc, %5, %7\n\t"
+      "v_subb_co_u32 %0, vcc, %6, %8, vcc\n\t"
+      "v_cndmask_b32 %1, %5, %7, vcc\n\t"
+      "v_cndmask_b32 %2, %6, %8, vcc\n\t"
+      "v_cndmask_b32 %3, %7, %5, vcc\n\t"
+      "v_cndmask_b32 %4, %8, %6, vcc"
+      : "=&v"(t), "=&v"(nil), "=&v"(nih), "=&v"(njl), "=&v"(njh)
+      : "v"(k.lo[i]), "v"(k.hi[i]), "v"(k.lo[j]), "v"(k.hi[j])
+      : "vcc");
+  k.lo[i] = nil;
+  k.hi[i] = nih;
+  k.lo[j] = njl;
+  k.hi[j] = njh;
+}
+
+// One stage at register distance 2^D, descending, except that pairs whose register number has
+// bit FLIP set (FLIP >= 0) sort ascending.  A direction that depends on the thread is not a case
+// here: such keys are held bit-inverted (see bitonic_sort_desc), which turns it into descending.
+template <int D, int FLIP>
+__device__ __forceinline__ void sort_stage_regs(SortKeys& k) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     if (i & (1 << D)) continue;
     const int j = i | (1 << D);
-    const bool flip = ib >= 0 && ((i >> ib) & 1);
-    const uint64_t a = r[i], b = r[j];
-    const bool sw = (a < b) == (tdesc != flip);
-    r[i] = sw ? b : a;
-    r[j] = sw ? a : b;
+    if (FLIP >= 0 && ((i >> (FLIP >= 0 ? FLIP : 0)) & 1))
+      sort_ce(k, j, i);
+    else
+      sort_ce(k, i, j);
+  }
+}
+
+__device__ __forceinline__ void sort_xor_keys(SortKeys& k, uint32_t m_low_half, uint32_t m_high_half) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const uint32_t m = i < 8 ? m_low_half : m_high_half;
+    k.lo[i] ^= m;
+    k.hi[i] ^= m;
   }
 }
 
@@ -141,16 +175,22 @@ __device__ __forceinline__ void bitonic_sort_desc(uint64_t* buf, int logP) {
     return;
   }
   const bool active = tid < (1 << (logP - 4));
-  uint64_t r[16];
-  // A pass whose window lies below bit 10 only moves keys inside aligned groups of 1024, and a
-  // group of 1024 is exactly what one wave owns in such a pass (64 threads x 16 keys).  Between
-  // two such passes the waves need no workgroup barrier, only program order inside the wave (the
-  // LDS serves one wave's requests in order); they drift apart and one wave's LDS traffic overlaps
-  // another's compare-exchanges.  A barrier stands only around the passes with a window above bit 6.
+  SortKeys k;
+  // Direction.  In level L a key sorts ascending if bit L of its index is set.  Instead of a
+  // per-thread direction in every compare-exchange, keys of ascending positions are held
+  // bit-inverted while level L runs (in registers and in LDS), so that every compare-exchange is
+  // "descending".  The pattern moves from bit L-1 to bit L in the first pass of level L, where
+  // bit L-1 is bit 3 of the register number and bit L a bit of the thread; in the last level bit L
+  // is zero for every index and the keys come out plain.
+  //
+  // Barriers.  A pass whose window lies below bit 10 only moves keys inside aligned groups of 1024,
+  // and a group of 1024 is exactly what one wave owns in such a pass (64 threads x 16 keys).
+  // Between two such passes the waves need no workgroup barrier, only program order inside the
+  // wave (the LDS serves one wave's requests in order); they drift apart and one wave's LDS traffic
+  // overlaps another's compare-exchanges.  A barrier stands only around passes with a window above
+  // bit 6.
   int prev_p = 31;
-  auto pass = [&](int p, int L, int s_hi, int s_lo, int L_first, int L_last) {
-    // one LDS round trip; either the stages s_hi..s_lo of level L, or (L_first > 0) all stages of
-    // the levels L_first..L_last, which must all lie in the window [p, p+4)
+  auto pass = [&](int p, int L, int n_stages, bool first_of_level) {
     if (p > 6 || prev_p > 6)
       __syncthreads();
     else
@@ -158,35 +198,68 @@ __device__ __forceinline__ void bitonic_sort_desc(uint64_t* buf, int logP) {
     prev_p = p;
     if (active) {
       const int base = (tid & ((1 << p) - 1)) | ((tid >> p) << (p + 4));
+      // base and i << p share no bit, so phys(base | i << p) = phys(base) + phys(i << p); the second
+      // term is the same for all threads and stays in scalar registers
+      uint64_t* pb = buf + sort_phys(base);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) r[i] = buf[sort_phys(base | (i << p))];
-      auto run = [&](int lev, int hi, int lo) {
-        const int ib = (lev >= p && lev < p + 4) ? lev - p : -1;  // level bit inside the register window?
-        const bool tdesc = ib >= 0 ? true : (((base >> lev) & 1) == 0);
-        for (int s = hi; s >= lo; --s) {
-          switch (s - p) {
-            case 0: sort_stage_regs<0>(r, tdesc, ib); break;
-            case 1: sort_stage_regs<1>(r, tdesc, ib); break;
-            case 2: sort_stage_regs<2>(r, tdesc, ib); break;
-            default: sort_stage_regs<3>(r, tdesc, ib); break;
-          }
+      for (int i = 0; i < 16; ++i) {
+        const uint64_t v = pb[sort_phys(i << p)];
+        k.lo[i] = uint32_t(v);
+        k.hi[i] = uint32_t(v >> 32);
+      }
+      // Stage sequences are spelled out at compile time: a loop over stages makes the compiler
+      // copy the 16 keys back to fixed registers after every stage.
+      if (L == 0) {
+        // levels 1..4 in the window [0,4): for levels 1..3 the level bit is a bit of the register
+        // number; level 4 takes its direction from bit 4 of the index, a thread bit
+        sort_stage_regs<0, 1>(k);
+        sort_stage_regs<1, 2>(k);
+        sort_stage_regs<0, 2>(k);
+        sort_stage_regs<2, 3>(k);
+        sort_stage_regs<1, 3>(k);
+        sort_stage_regs<0, 3>(k);
+        const uint32_t m = 0u - uint32_t((base >> 4) & 1);
+        sort_xor_keys(k, m, m);
+        sort_stage_regs<3, -1>(k);
+        sort_stage_regs<2, -1>(k);
+        sort_stage_regs<1, -1>(k);
+        sort_stage_regs<0, -1>(k);
+      } else {
+        if (first_of_level) {  // window [L-4, L): pattern from bit L-1 (bit 3 of i) to bit L (thread)
+          const uint32_t m = 0u - uint32_t((base >> L) & 1);
+          sort_xor_keys(k, m, ~m);
         }
-      };
-      if (L_first > 0)
-        for (int lev = L_first; lev <= L_last; ++lev) run(lev, lev - 1, 0);
-      else
-        run(L, s_hi, s_lo);
+        switch (n_stages) {
+          case 4:
+            sort_stage_regs<3, -1>(k);
+            sort_stage_regs<2, -1>(k);
+            sort_stage_regs<1, -1>(k);
+            sort_stage_regs<0, -1>(k);
+            break;
+          case 3:
+            sort_stage_regs<2, -1>(k);
+            sort_stage_regs<1, -1>(k);
+            sort_stage_regs<0, -1>(k);
+            break;
+          case 2:
+            sort_stage_regs<1, -1>(k);
+            sort_stage_regs<0, -1>(k);
+            break;
+          default:
+            sort_stage_regs<0, -1>(k);
+            break;
+        }
+      }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) buf[sort_phys(base | (i << p))] = r[i];
+      for (int i = 0; i < 16; ++i) pb[sort_phys(i << p)] = (uint64_t(k.hi[i]) << 32) | k.lo[i];
     }
   };
-  pass(0, 0, 0, 0, 1, 4);  // levels 1..4 entirely in registers
+  pass(0, 0, 4, true);  // levels 1..4 entirely in registers
   for (int L = 5; L <= logP; ++L) {
     int s = L - 1;
     while (s >= 0) {
-      const int lo = s - 3 > 0 ? s - 3 : 0;
-      const int p = lo < logP - 4 ? lo : logP - 4;
-      pass(p, L, s, lo, 0, 0);
+      const int lo = s - 3 > 0 ? s - 3 : 0;  // lo <= logP - 4: the window [lo, lo+4) fits
+      pass(lo, L, s - lo + 1, s == L - 1);
       s = lo - 1;
     }
   }

@@ -34,6 +34,56 @@ __global__ __launch_bounds__(256) void l2_normalize_kernel(const T* __restrict__
   for (int k = lane_id(); k < d; k += kWave) Elem<T>::store(Xn + r * d + k, Elem<T>::load(x + k) * inv);
 }
 
+// bf16, d = 128: a row is 16 lanes x 16 bytes, four rows per wave and load instruction, four such
+// loads in flight per thread.  HBM-bound: 2*d*2 bytes per row.
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 cbf16x2;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float cf32x2;
+__device__ __forceinline__ uint32_t cent_pack_bf16(float lo, float hi) {
+  cf32x2 x = {lo, hi};
+  cbf16x2 y = __builtin_convertvector(x, cbf16x2);  // round to nearest even
+  return *reinterpret_cast<uint32_t*>(&y);
+}
+__device__ __forceinline__ void cent_unpack8(uint4 u, float (&f)[8]) {
+  const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(w[i] << 16);
+    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+__global__ __launch_bounds__(256) void l2_normalize_bf16_d128_kernel(const bf16_t* __restrict__ X,
+                                                                     bf16_t* __restrict__ Xn, int64_t rows,
+                                                                     float eps) {
+  constexpr int U = 4;
+  const int c = threadIdx.x & 15;
+  const int64_t stride = int64_t(gridDim.x) * 16;
+  for (int64_t r0 = int64_t(blockIdx.x) * 16 + (threadIdx.x >> 4); r0 < rows; r0 += stride * U) {
+    uint4 u[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const int64_t r = r0 + k * stride;
+      u[k] = r < rows ? reinterpret_cast<const uint4*>(X + r * 128)[c] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const int64_t r = r0 + k * stride;
+      float f[8];
+      cent_unpack8(u[k], f);
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+#pragma unroll
+      for (int o = 1; o < 16; o <<= 1) ss += __shfl_xor(ss, o);
+      const float inv = 1.f / fmaxf(sqrtf(ss), eps);
+      if (r < rows)
+        reinterpret_cast<uint4*>(Xn + r * 128)[c] =
+            make_uint4(cent_pack_bf16(f[0] * inv, f[1] * inv), cent_pack_bf16(f[2] * inv, f[3] * inv),
+                       cent_pack_bf16(f[4] * inv, f[5] * inv), cent_pack_bf16(f[6] * inv, f[7] * inv));
+    }
+  }
+}
+
 // A[c,h,:] = normalise( mean over g<G, j<k of Xn[h*G+g, top_idx[c,h*G+g,j], :] )
 // one workgroup per (c,h); thread = dimension (d <= 256)
 template <typename T>
@@ -91,6 +141,60 @@ __global__ __launch_bounds__(256) void segment_mean_kernel(
   }
 }
 
+
+// bf16, d = 128: sixteen groups of 16 lanes walk the member list in turn (member j goes to group
+// j % 16), each lane adding its 8 dimensions of the gathered rows, four rows in flight per group;
+// the sixteen partial sums are then added in group order, so the result does not depend on
+// scheduling.  HBM-bound on the gathered rows (256 bytes per member).
+__global__ __launch_bounds__(256) void segment_mean_bf16_d128_kernel(
+    const bf16_t* __restrict__ X, const int32_t* __restrict__ perm, const int32_t* __restrict__ seg_off,
+    const int32_t* __restrict__ seg_cnt, const bf16_t* __restrict__ prev, bf16_t* __restrict__ out, int C,
+    int N) {
+  __shared__ float red[16][128];
+  __shared__ float sh[4];
+  const int c = blockIdx.x, h = blockIdx.y, t = threadIdx.x;
+  const int g = t >> 4, ch = t & 15;
+  const int64_t hc = int64_t(h) * C + c;
+  const int cnt = seg_cnt[hc];
+  const int32_t* mem = perm + seg_off[hc];
+  const uint4* xb = reinterpret_cast<const uint4*>(X + int64_t(h) * N * 128);
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  constexpr int U = 4;
+  for (int j0 = g; j0 < cnt; j0 += 16 * U) {
+    uint4 u[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const int j = j0 + 16 * k;
+      const int row = j < cnt ? min(max(mem[j], 0), N - 1) : 0;
+      u[k] = j < cnt ? xb[int64_t(row) * 16 + ch] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      float f[8];
+      cent_unpack8(u[k], f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += f[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) red[g][ch * 8 + i] = acc[i];
+  __syncthreads();
+  float v = 0.f;
+  if (t < 128) {
+#pragma unroll
+    for (int gg = 0; gg < 16; ++gg) v += red[gg][t];
+    if (cnt > 0) v /= float(cnt);
+  }
+  const float ss = block_sum_256(t < 128 ? v * v : 0.f, sh);
+  const float nrm = sqrtf(ss);
+  if (t < 128) {
+    if (cnt == 0 || nrm < 1e-12f)
+      out[hc * 128 + t] = prev[hc * 128 + t];
+    else
+      out[hc * 128 + t] = f32_to_bf16(v / nrm);
+  }
+}
+
 }  // namespace fm
 
 extern "C" int fm_l2_normalize(const void* X, void* Xn, int64_t rows, int d, float eps, int dtype,
@@ -102,7 +206,11 @@ extern "C" int fm_l2_normalize(const void* X, void* Xn, int64_t rows, int d, flo
   FM_REQUIRE(X && Xn, FM_ERR_ARG, "fm_l2_normalize: null pointer");
   FM_REQUIRE(ceil_div(rows, 4) <= 0x7fffffffLL, FM_ERR_UNSUPPORTED, "fm_l2_normalize: too many rows");
   dim3 grid = dim3(unsigned(ceil_div(rows, 4)));
-  if (dtype == FM_F32)
+  if (dtype == FM_BF16 && d == 128) {
+    const unsigned wgs = unsigned(std::min<int64_t>(ceil_div(rows, 16 * 4), 256 * 64));
+    hipLaunchKernelGGL(l2_normalize_bf16_d128_kernel, dim3(wgs), dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)X, (bf16_t*)Xn, rows, eps);
+  } else if (dtype == FM_F32)
     hipLaunchKernelGGL(l2_normalize_kernel<float>, grid, dim3(256), 0, as_stream(stream),
                        (const float*)X, (float*)Xn, rows, d, eps);
   else
@@ -140,7 +248,10 @@ extern "C" int fm_segment_mean(const void* X, const int32_t* perm, const int32_t
              "fm_segment_mean: null pointer");
   FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_segment_mean: H > 65535");
   dim3 grid = dim3(unsigned(C), unsigned(H));
-  if (dtype == FM_F32)
+  if (dtype == FM_BF16 && d == 128)
+    hipLaunchKernelGGL(segment_mean_bf16_d128_kernel, grid, dim3(256), 0, as_stream(stream), (const bf16_t*)X,
+                       perm, seg_off, seg_cnt, (const bf16_t*)prev, (bf16_t*)cent_out, C, N);
+  else if (dtype == FM_F32)
     hipLaunchKernelGGL(segment_mean_kernel<float>, grid, dim3(256), 0, as_stream(stream),
                        (const float*)X, perm, seg_off, seg_cnt, (const float*)prev,
                        (float*)cent_out, C, N, d);

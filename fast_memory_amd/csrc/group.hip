@@ -71,11 +71,23 @@ __global__ void group_colscan_kernel(int32_t* __restrict__ block_hist, int H, in
   int64_t g = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (g >= int64_t(H) * C) return;
   int h = int(g / C), c = int(g - int64_t(h) * C);
+  // sixteen independent loads in flight per thread; the prefix itself runs in registers
+  int32_t* col = block_hist + int64_t(h) * NB * C + c;
   int run = 0;
-  for (int blk = 0; blk < NB; ++blk) {
-    int64_t a = (int64_t(h) * NB + blk) * C + c;
-    int v = block_hist[a];
-    block_hist[a] = run;
+  int blk = 0;
+  for (; blk + 16 <= NB; blk += 16) {
+    int v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = col[int64_t(blk + u) * C];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      col[int64_t(blk + u) * C] = run;
+      run += v[u];
+    }
+  }
+  for (; blk < NB; ++blk) {
+    const int v = col[int64_t(blk) * C];
+    col[int64_t(blk) * C] = run;
     run += v;
   }
   bin_count[g] = run;

@@ -372,6 +372,27 @@ def test_l2_normalize(ops):
     assert (got[3] == 0).all()
 
 
+def test_l2_normalize_and_segment_mean_bf16_d128(ops):
+    # the vectorised bf16 / d = 128 kernels against the oracle on the same (bf16-rounded) inputs
+    from fast_memory_amd import kmeans_spherical
+    g = gen(703)
+    H, N, d, C = 2, 5000, 128, 37
+    X = torch.randn(H, N, d, generator=g).to(torch.bfloat16)
+    X[0, 7] = 0
+    got = ops.l2_normalize(dev(X)).float().cpu()
+    ref = O.l2_normalize(X.float())
+    assert torch.allclose(got, ref, atol=4e-3, rtol=8e-3)           # one bf16 rounding of the result
+    assert (got[0, 7] == 0).all()
+    Xn = ref.to(torch.bfloat16)
+    init = O.l2_normalize(O.init_centroids(C, d)).to(torch.bfloat16).unsqueeze(0).expand(H, -1, -1).contiguous()
+    cent, labels = kmeans_spherical(dev(Xn), dev(init), 1)
+    for h in range(H):
+        # the centroid update on the labels the GPU assigned: mean of the members, normalised
+        lab = labels[h].cpu().long()
+        rc = O.kmeans_update(Xn[h].float(), lab, init[h].float())
+        assert torch.allclose(cent[h].float().cpu().double(), rc.double(), atol=4e-3, rtol=8e-3)
+
+
 # ------------------------------------------------------------------ a15 composite, config c1
 def test_config1_toy_end_to_end(ops):
     from fast_memory_amd import Memory, fit_projection

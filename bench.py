@@ -196,7 +196,7 @@ def main():
         f"(keys {tuple(wl.keys.shape)} {wl.keys.dtype})")
 
     # ---- A by spherical K-means, index build (both timed, outside the step) ----
-    km_ms, A = timed(lambda: fit_projection(wl.keys, C, iters=cfg.kmeans_iters), reps=1, warm=0)
+    km_ms, A = timed(lambda: fit_projection(wl.keys, C, iters=cfg.kmeans_iters), reps=1, warm=1)
     log(f"[bench] K-means ({cfg.kmeans_iters} iterations): {km_ms:.1f} ms")
     build_ms, mem = timed(lambda: Memory.build(wl.keys, wl.values, A, Z, workspace_bytes=ws_bytes), reps=2, warm=1)
     keys_per_s = H * N / (build_ms * 1e-3)
@@ -348,22 +348,11 @@ def main():
         q0 = q[0].cpu()
         kl0 = wl.k_local[0].cpu() if has_local else None
         vl0 = wl.v_local[0].cpu() if has_local else None
-        n = min(32, Sq)
         pick = lambda m: torch.linspace(0, Sq - 1, m).long()        # spread over heads and positions
-        sel = pick(n)
-        t_probe = cpu_path.time_query_path(q0[sel], K0, V0, A0, lists0, sm_scale, kl0, vl0, sel % S, S)
-        n = int(max(n, min(Sq, n * args.cpu_seconds / max(t_probe, 1e-3))))
-        sel = pick(n)
-        t_cpu = cpu_path.time_query_path(q0[sel], K0, V0, A0, lists0, sm_scale, kl0, vl0, sel % S, S)
-        if t_cpu < 0.6 * args.cpu_seconds and n < Sq:
-            # queries that share a bucket share its gather, so the cost per query falls as the
-            # sample grows: size it once more from the larger run
-            n = int(min(Sq, n * args.cpu_seconds / max(t_cpu, 1e-3)))
-            sel = pick(n)
-            t_cpu = cpu_path.time_query_path(q0[sel], K0, V0, A0, lists0, sm_scale, kl0, vl0, sel % S, S)
-        n_total, t_total, heads_used = n, t_cpu, 1
-        while n == Sq and t_total < 0.6 * args.cpu_seconds and heads_used < H:
-            # a whole head costs less than the time budget: add whole heads
+        # whole KV heads, one after the other, until the time budget is used: the cost is per bucket
+        # gathered, not per query, so a subsample of a head's queries costs almost as much as all
+        n_total, t_total, heads_used = 0, 0.0, 0
+        while heads_used < H and t_total < args.cpu_seconds:
             hh = heads_used
             t_total += cpu_path.time_query_path(
                 q[hh].cpu(), wl.keys[hh].cpu(), wl.values[hh].cpu(), A[hh].cpu(), mem.bucket_idx[hh].cpu().long(),
@@ -371,13 +360,13 @@ def main():
                 torch.arange(Sq) % S, S)
             n_total += Sq
             heads_used += 1
+        sel = pick(min(Sq, 4096))                                      # parity spot-check sample of head 0
         # index-build sample: a few rows of A against all keys of head 0
         r = min(C, 32 if N > 200000 else 64)
         tb0 = time.perf_counter()
         cpu_lists = cpu_path.build_rows(A0[:r], K0, Z)
         t_build = time.perf_counter() - tb0
-        what = (f"KV head 0, {n} of its {Sq} query-heads evenly spaced" if heads_used == 1 else
-                f"KV heads 0..{heads_used - 1} of {H}, all {Sq} query-heads of each")
+        what = f"KV heads 0..{heads_used - 1} of {H}, all {Sq} query-heads of each"
         cpu = {"value": n_total / t_total, "unit": "query-heads/s", "cores": threads, "kind": "port",
                "sample": f"{what}, full N={N}, C={C}, Z={Z}; hash + per-bucket "
                          f"gathered softmax attention" + (" + causal local attention + merge" if has_local else "")
@@ -401,9 +390,14 @@ def main():
         log(f"[bench] cpu baseline: {cpu['value']:.1f} query-heads/s on {threads} threads; parity {parity}")
 
     if args.config == "c4" and fused_phases:
+        filter_traffic = None
+        if os.path.exists(tpath):
+            for ln in open(tpath):
+                if ln.strip().startswith(f"fused_filter_kernel/{cfg.name}") and "=" in ln:
+                    filter_traffic = float(ln.split("=")[1])
         roofline = {"kernel": "fused_filter_kernel", "bound": "mfma", "achieved": fused_phases["filter_tflops"],
                     "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": fused_phases["filter_mfma_frac"],
-                    "traffic": None, "algorithmic_flops_per_launch": 2.0 * H * C * N * d,
+                    "traffic": filter_traffic, "algorithmic_flops_per_launch": 2.0 * H * C * N * d,
                     "avg_launch_ms": fused_phases["mfma_filter_ms"]}
     line = {
         "metric": "index-build keys/s" if args.config == "c4" else "hashed-attn query-heads/s",

@@ -4,21 +4,19 @@
 //   phase 0  per-row threshold.  Y is computed for a strided sample of the keys
 //            (every `stride`-th key, 32 Ki - 64 Ki of them) with the ordinary
 //            projection kernel, and the `rank`-th largest sampled value of every
-//            (head, bucket) row becomes that row's threshold tau; `rank` sits six
-//            standard deviations above Z*ns/N, so with overwhelming probability
-//            at least Z keys of the full row reach tau and not many more.
+//            (head, bucket) row becomes that row's threshold tau; `rank` sits four
+//            standard deviations above Z*ns/N, so all but about one row in 30000
+//            have at least Z keys reaching tau, and not many more than Z.
 //   phase 1  fused_filter_kernel: bf16 MFMA GEMM over all keys with an epilogue
 //            that keeps only elements >= tau.  Keys are the M side of the MFMA
 //            tile and buckets the N side, so in the accumulator layout one lane
 //            owns one bucket column: its threshold, its write cursor and its
 //            private segment of the row's candidate buffer live in registers and
 //            survivors are appended with plain stores -- no atomics.
-//   phase 2  exact top-Z (value desc, index asc) of each row's candidates, the
-//            same code as the dense arg-top-Z kernel reading ~1.2 Z candidates
-//            instead of the N-element row, in two kernels of very different
-//            shape: cand_cut_kernel (radix select of the cut; small workgroups,
-//            many per compute unit) and cand_sort_kernel (collect + in-LDS
-//            bitonic sort; one workgroup fills a compute unit's LDS).
+//   phase 2  cand_select_kernel: exact top-Z (value desc, index asc) of each
+//            row's candidates: radix select + in-LDS bitonic sort, the same code
+//            as the dense arg-top-Z kernel, on ~1.2 Z candidates that are read
+//            once and then held in registers, instead of the N-element row.
 //   phase 3  repair.  A row whose candidate count fell short of Z or overflowed
 //            a segment is listed by phase 2; its Y row is recomputed (same MFMA
 //            instruction and contraction order) into a small buffer and handed to
@@ -49,11 +47,15 @@ constexpr int kFKeys = 64;        // keys per iteration of a workgroup
 constexpr int kFSlab = 512;       // buckets per workgroup (64 per wave)
 constexpr int kFLd = kFD + 8;     // LDS row stride in bf16 elements
 constexpr int kMaxRepair = 64;
+// The sampled threshold is the value of rank mu + kRankSigmas*sqrt(mu) + 3 of the sample (mu = Z*ns/N).
+// Four standard deviations: a row misses with probability ~3e-5, i.e. about one repaired row in two
+// builds of 16384 rows, and ~18 % more candidates than Z are kept at mu = 512 (six would keep 27 %).
+constexpr double kRankSigmas = 4.0;
 
 struct FusedPlan {
   int ns, stride, rank, n_splits, slabs, n_writers, cap_w;
   int64_t ld_s, ldy;
-  size_t off_Ks, off_Ys, off_tau, off_cand, off_cnt, off_cut, off_ok, off_fail, off_nfail, off_Yf, total;
+  size_t off_Ks, off_Ys, off_tau, off_cand, off_cnt, off_fail, off_nfail, off_Yf, total;
 };
 
 static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& p) {
@@ -62,7 +64,7 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   p.stride = N / 32768;
   p.ns = N / p.stride;
   const double mu = double(Z) * p.ns / N;
-  p.rank = int(mu + 6.0 * sqrt(mu) + 3.0);
+  p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
   if (p.rank * 4 > p.ns) return false;
   const double m_exp = double(p.rank) * N / p.ns;
   p.slabs = int(ceil_div(C, kFSlab));
@@ -86,8 +88,6 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   p.off_tau = take(rows * sizeof(float));
   p.off_cand = take(rows * p.n_writers * size_t(p.cap_w) * sizeof(uint2));
   p.off_cnt = take(rows * p.n_writers * sizeof(int32_t));
-  p.off_cut = take(rows * sizeof(uint64_t));
-  p.off_ok = take(rows * sizeof(int32_t));
   p.off_fail = take(kMaxRepair * sizeof(int32_t));
   p.off_nfail = take(4 * sizeof(int32_t));
   p.off_Yf = take(size_t(kMaxRepair) * p.ldy * sizeof(float));
@@ -344,32 +344,7 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
 }
 
 // ---- phase 2 ---------------------------------------------------------------
-template <int NT>
-struct CandRow {
-  const uint2* base;  // [n_writers][cap_w] (value bits, key code)
-  const int* counts;  // LDS, clamped to cap_w
-  int n_writers, cap_w, maxc;
-  template <typename F>
-  __device__ __forceinline__ void operator()(F f) const {
-    for (int j = threadIdx.x; j < maxc; j += NT) {
-      for (int w0 = 0; w0 < n_writers; w0 += 8) {
-        uint2 e[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int w = w0 + u;
-          if (w < n_writers && j < counts[w]) e[u] = base[int64_t(w) * cap_w + j];
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int w = w0 + u;
-          if (w < n_writers && j < counts[w]) f(__uint_as_float(e[u].x), fused_key_of_code(e[u].y));
-        }
-      }
-    }
-  }
-};
-
-// Loads the per-writer counts of a row into LDS; returns false (to all threads) if a segment
+// Per-writer candidate counts of a row in LDS; returns false (to all threads) if a segment
 // overflowed or the row has fewer than Zc candidates, i.e. the sampled threshold failed.
 struct CandCounts {
   int counts[64];
@@ -398,45 +373,52 @@ __device__ __forceinline__ bool load_cand_counts(const int32_t* __restrict__ cnt
   return !(cc.over || cc.total < Zc);
 }
 
-// Phase 2a: the exact cut (Zc-th largest composite) of every row's candidates.  Small workgroups
-// with a small LDS footprint, so that eight rows per compute unit hide each other's round trips
-// (a pass over ~1.2 Zc candidates is short and latency-bound).
-constexpr int kCutThreads = 256;
-__global__ __launch_bounds__(kCutThreads) void cand_cut_kernel(
-    const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, int n_writers, int cap_w, int Zc,
-    uint64_t* __restrict__ cut_out, int32_t* __restrict__ row_ok, int32_t* __restrict__ fail_rows,
-    int32_t* __restrict__ n_fail) {
+// A row's candidates held in registers: the 1024 threads are dealt to the writers' segments in
+// groups of 1024 / n_writers, and a thread keeps elements t, t + T, t + 2T, ... of its segment
+// (at most kCandRegs of them).  The candidates are read from memory once; the radix passes of
+// the selection and the collection into the sort buffer then run from registers.
+constexpr int kCandRegs = 24;
+struct CandRegs {
+  uint2 e[kCandRegs];  // (value bits, key code)
+  int n;               // valid entries of this thread
+  template <typename F>
+  __device__ __forceinline__ void operator()(F f) const {
+#pragma unroll
+    for (int r = 0; r < kCandRegs; ++r)
+      if (r < n) f(__uint_as_float(e[r].x), fused_key_of_code(e[r].y));
+  }
+};
+
+// Exact top-Z (value desc, index asc) of every row's candidates: radix select of the cut,
+// collection of the Zc survivors into LDS, bitonic sort, indices out -- the code of the dense
+// arg-top-Z kernel, on ~1.2 Zc register-resident candidates instead of the N-element row.
+__global__ __launch_bounds__(kSelThreads) void cand_select_kernel(
+    const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, int n_writers, int cap_w, int Zc, int P,
+    int32_t* __restrict__ idx_out, int32_t* __restrict__ fail_rows, int32_t* __restrict__ n_fail) {
+  extern __shared__ uint64_t buf[];
   __shared__ SelectShared sh;
   __shared__ CandCounts cc;
   const int64_t row = blockIdx.x;
-  if (!load_cand_counts(cnt, row, n_writers, cap_w, Zc, cc)) {  // queue the row for repair
+  const int T = kSelThreads / n_writers;  // threads per segment
+  bool ok = load_cand_counts(cnt, row, n_writers, cap_w, Zc, cc);
+  ok = ok && cc.maxc <= T * kCandRegs;
+  if (!ok) {  // threshold missed (or a segment too long to hold): queue the row for repair
     if (threadIdx.x == 0) {
-      row_ok[row] = 0;
       int pos = atomicAdd(n_fail, 1);
       if (pos < kMaxRepair) fail_rows[pos] = int32_t(row);
     }
     return;
   }
-  CandRow<kCutThreads> src{cand + row * n_writers * int64_t(cap_w), cc.counts, n_writers, cap_w, cc.maxc};
-  const uint64_t cut = radix_select_cut<kCutThreads>(src, Zc, 6, sh);
-  if (threadIdx.x == 0) {
-    cut_out[row] = cut;
-    row_ok[row] = 1;
-  }
-}
-
-// Phase 2b: the Zc candidates at or above the cut, sorted in LDS, indices out.
-__global__ __launch_bounds__(kSelThreads) void cand_sort_kernel(
-    const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, const uint64_t* __restrict__ cut_in,
-    const int32_t* __restrict__ row_ok, int n_writers, int cap_w, int Zc, int P, int32_t* __restrict__ idx_out) {
-  extern __shared__ uint64_t buf[];
-  __shared__ SelectShared sh;
-  __shared__ CandCounts cc;
-  const int64_t row = blockIdx.x;
-  if (!row_ok[row]) return;
-  load_cand_counts(cnt, row, n_writers, cap_w, Zc, cc);
-  CandRow<kSelThreads> src{cand + row * n_writers * int64_t(cap_w), cc.counts, n_writers, cap_w, cc.maxc};
-  collect_sort_write(src, cut_in[row], Zc, P, buf, sh, idx_out + row * Zc);
+  CandRegs src;
+  const int w = threadIdx.x / T, t = threadIdx.x - w * T;
+  const int cw = w < n_writers ? cc.counts[w] : 0;
+  const uint2* seg = cand + (row * n_writers + min(w, n_writers - 1)) * int64_t(cap_w);
+  src.n = cw > t ? (cw - t + T - 1) / T : 0;
+#pragma unroll
+  for (int r = 0; r < kCandRegs; ++r)
+    if (r < src.n) src.e[r] = seg[t + r * T];
+  const uint64_t cut = radix_select_cut(src, Zc, 6, sh);
+  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + row * Zc);
 }
 
 // ---- phase 3 ---------------------------------------------------------------
@@ -522,8 +504,6 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   float* tau = reinterpret_cast<float*>(base + p.off_tau);
   uint2* cand = reinterpret_cast<uint2*>(base + p.off_cand);
   int32_t* cnt = reinterpret_cast<int32_t*>(base + p.off_cnt);
-  uint64_t* cut = reinterpret_cast<uint64_t*>(base + p.off_cut);
-  int32_t* row_ok = reinterpret_cast<int32_t*>(base + p.off_ok);
   int32_t* fail_rows = reinterpret_cast<int32_t*>(base + p.off_fail);
   int32_t* n_fail = reinterpret_cast<int32_t*>(base + p.off_nfail);
   float* Yf = reinterpret_cast<float*>(base + p.off_Yf);
@@ -546,11 +526,9 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   // phase 2
   mark_phase(2, st);
   const int P = next_pow2(Zc);
-  hipLaunchKernelGGL(cand_cut_kernel, dim3(unsigned(rows)), dim3(kCutThreads), 0, st, cand, cnt, p.n_writers,
-                     p.cap_w, Zc, cut, row_ok, fail_rows, n_fail);
-  FM_ALLOW_LDS(cand_sort_kernel, sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");
-  hipLaunchKernelGGL(cand_sort_kernel, dim3(unsigned(rows)), dim3(kSelThreads), sort_lds_bytes(P), st, cand, cnt,
-                     cut, row_ok, p.n_writers, p.cap_w, Zc, P, idx_out);
+  FM_ALLOW_LDS(cand_select_kernel, sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");
+  hipLaunchKernelGGL(cand_select_kernel, dim3(unsigned(rows)), dim3(kSelThreads), sort_lds_bytes(P), st, cand, cnt,
+                     p.n_writers, p.cap_w, Zc, P, idx_out, fail_rows, n_fail);
   // phase 3
   mark_phase(3, st);
   hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(ceil_div(N, 128)), kMaxRepair), dim3(256), 0,

@@ -46,6 +46,7 @@ constexpr int kFThreads = 576;    // + one producer wave
 constexpr int kFKeys = 64;        // keys per iteration of a workgroup
 constexpr int kFSlab = 512;       // buckets per workgroup (64 per wave)
 constexpr int kFLd = kFD + 8;     // LDS row stride in bf16 elements
+constexpr int kFDumpLd = 20;      // floats per lane in the dump: 16 registers + 4 (16-byte stores spread over banks)
 constexpr int kMaxRepair = 64;
 // The sampled threshold is the value of rank mu + kRankSigmas*sqrt(mu) + 3 of the sample (mu = Z*ns/N).
 // Four standard deviations: a row misses with probability ~3e-5, i.e. about one repaired row in two
@@ -148,10 +149,10 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const float* __restrict__ tau,
     uint2* __restrict__ cand, int32_t* __restrict__ cnt, int C, int N, int n_splits, int cap_w) {
   // one object, so that the dump area is preceded by the key tiles: a lane without candidates
-  // reads 256 bytes below its dump column, which must stay inside the allocation
+  // reads the word below its dump row, which must stay inside the allocation
   __shared__ __attribute__((aligned(16))) struct {
     bf16_t keys[2][kFKeys * kFLd];
-    float dump[kFWaves][2 * 16 * 64];  // [wave][column half ni][accumulator register][lane]
+    float dump[kFWaves][2 * 64 * kFDumpLd];  // [wave][column half ni][lane][accumulator register, padded]
   } sm;
   bf16_t(&sK)[2][kFKeys * kFLd] = sm.keys;
   const int sk = blockIdx.x, slab = blockIdx.y, h = blockIdx.z;
@@ -242,17 +243,20 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
   const int lane_code = (l >> 5) << 4;
   uint32_t msk[2];
 
-  // Threshold test of one accumulator register: mask = 2*mask + (y >= th), and its dump.  The
-  // registers of a column half are tested from 15 down to 0, so bit r of the mask belongs to
-  // register r.  The dump comes first: it is the compiler-visible read of freshly written MFMA
+  // Threshold test of four accumulator registers: mask = 2*mask + (y >= th) for each, and their
+  // dump.  The registers of a column half are tested from 15 down to 0, so bit r of the mask
+  // belongs to register r.  The dump comes first: it is the compiler-visible read of freshly written MFMA
   // results, so the wait states an MFMA result needs before it can be read are inserted there; the
   // asm (whose operands the hazard logic does not look into) then only ever reads settled registers.
-  auto test_dump = [&](const f32x16& a, int ni, int r) {
-    dump[(ni * 16 + r) * 64 + l] = a[r];
-    asm volatile("v_cmp_nlt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
-                 : "+v"(msk[ni])
-                 : "v"(a[r]), "v"(th[ni])
-                 : "vcc", "memory");
+  auto test_dump4 = [&](const f32x16& a, int ni, int q) {
+    *reinterpret_cast<float4*>(&dump[(ni * 64 + l) * kFDumpLd + 4 * q]) =
+        make_float4(a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]);
+#pragma unroll
+    for (int j = 3; j >= 0; --j)
+      asm volatile("v_cmp_nlt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
+                   : "+v"(msk[ni])
+                   : "v"(a[4 * q + j]), "v"(th[ni])
+                   : "vcc", "memory");
   };
   // Emission: every lane pops up to two mask bits per column half (lowest register first), reads
   // those values back from its LDS dump (all four reads in flight together) and appends
@@ -271,7 +275,7 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
       m &= m - 1u;
     }
 #pragma unroll
-    for (int p = 0; p < 4; ++p) y[p] = dump[((p >> 1) * 16 + r[p]) * 64 + l];
+    for (int p = 0; p < 4; ++p) y[p] = dump[((p >> 1) * 64 + l) * kFDumpLd + r[p]];
     // keep the four reads together ahead of the predicated stores (one LDS round trip, not four)
     asm volatile("" : "+v"(y[0]), "+v"(y[1]), "+v"(y[2]), "+v"(y[3]));
 #pragma unroll
@@ -292,12 +296,17 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     if (active) {
       const int kbase = (sk + i * n_splits) * kFKeys;
       const bool check_n = kbase + kFKeys > N;
+      bf16x8 a_pre[4];  // fragments 0..3 of the second half, read while the first half is emitted
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         const bf16_t* pa = &sK[i & 1][(half * 32 + (l & 31)) * kFLd + (l >> 5) * 8];
         bf16x8 a[8];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) a[ks] = *reinterpret_cast<const bf16x8*>(pa + ks * 16);
+        for (int ks = 0; ks < 8; ++ks)
+          if (half == 0 || ks >= 4)
+            a[ks] = *reinterpret_cast<const bf16x8*>(pa + ks * 16);
+          else
+            a[ks] = a_pre[ks];
         f32x16 acc[2];
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
@@ -308,12 +317,16 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
           acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], bfrag[0][ks], acc[0], 0, 0, 0);
           acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], bfrag[1][ks], acc[1], 0, 0, 0);
         }
+        if (half == 0) {
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) a_pre[ks] = *reinterpret_cast<const bf16x8*>(pa + 32 * kFLd + ks * 16);
+        }
         msk[0] = msk[1] = 0;
         asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // all 16 accumulator passes retired
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-          for (int r = 15; r >= 0; --r) test_dump(acc[ni], ni, r);
+          for (int q = 3; q >= 0; --q) test_dump4(acc[ni], ni, q);
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
           if (off[ni] > lim[ni]) {  // fewer than 16 free slots: wrap and mark the row for repair

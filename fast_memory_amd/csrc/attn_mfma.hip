@@ -89,7 +89,7 @@ __device__ __forceinline__ void attend_item(
     const bf16_t* __restrict__ Qb,   // query rows of this item's row/head: [*, 128]
     const int* __restrict__ q_rows,  // LDS: row index (into Qb / out) of the item's queries
     int n_q, const bf16_t* __restrict__ Kb, const bf16_t* __restrict__ Vb,
-    const int32_t* __restrict__ idx,  // bucket list
+    const int32_t* __restrict__ idx,  // bucket list; nullptr = keys 0..cnt-1
     int cnt, int N, float scale2, bf16_t* __restrict__ Ob, float* __restrict__ Lb, float* __restrict__ red) {
   const int l = lane_id(), w = threadIdx.x >> 6;
   const int g = l >> 4, c = l & 15;
@@ -120,7 +120,7 @@ __device__ __forceinline__ void attend_item(
   auto rows_of = [&](int b) -> int {
     const int kp = b * kBlk + (l & 31);
     int r = 0;
-    if (kp < cnt) r = idx[kp];
+    if (kp < cnt) r = idx ? idx[kp] : kp;
     return min(max(r, 0), N - 1);
   };
 
@@ -228,19 +228,19 @@ __device__ __forceinline__ void attend_item(
 
   // ---- merge the four waves ---------------------------------------------------
   // red layout (floats): O part [wave][qt][t][r][lane], then l [wave][qt][lane],
-  // then m [wave][qt][16]
+  // then m [wave][qt][16], with NQ query tiles: red_floats(NQ) floats
   float* redO = red;
-  float* redL = red + 4 * kNQT * 8 * 4 * 64;
-  float* redM = redL + 4 * kNQT * 64;
+  float* redL = red + 4 * NQ * 8 * 4 * 64;
+  float* redM = redL + 4 * NQ * 64;
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
     if (qt < nqt) {
 #pragma unroll
       for (int t = 0; t < 8; ++t)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) redO[(((w * kNQT + qt) * 8 + t) * 4 + r) * 64 + l] = O[qt][t][r];
-      redL[(w * kNQT + qt) * 64 + l] = lsum[qt];
-      if (g == 0) redM[(w * kNQT + qt) * 16 + c] = m[qt];
+        for (int r = 0; r < 4; ++r) redO[(((w * NQ + qt) * 8 + t) * 4 + r) * 64 + l] = O[qt][t][r];
+      redL[(w * NQ + qt) * 64 + l] = lsum[qt];
+      if (g == 0) redM[(w * NQ + qt) * 16 + c] = m[qt];
     }
   }
   __syncthreads();
@@ -250,7 +250,7 @@ __device__ __forceinline__ void attend_item(
       float mw[4], mstar = -INFINITY;
 #pragma unroll
       for (int ww = 0; ww < 4; ++ww) {
-        mw[ww] = redM[(ww * kNQT + qt) * 16 + c];
+        mw[ww] = redM[(ww * NQ + qt) * 16 + c];
         mstar = fmaxf(mstar, mw[ww]);
       }
       const int j = qt * 16 + c;
@@ -260,7 +260,7 @@ __device__ __forceinline__ void attend_item(
         f[ww] = (mw[ww] == -INFINITY) ? 0.f : fast_exp2(mw[ww] - mstar);
         float lw = 0.f;
 #pragma unroll
-        for (int gg = 0; gg < 4; ++gg) lw += redL[(ww * kNQT + qt) * 64 + gg * 16 + c];
+        for (int gg = 0; gg < 4; ++gg) lw += redL[(ww * NQ + qt) * 64 + gg * 16 + c];
         lstar += f[ww] * lw;
       }
       const bool empty = (mstar == -INFINITY);  // the query saw no key at all
@@ -271,7 +271,7 @@ __device__ __forceinline__ void attend_item(
       for (int t = 0; t < 8; ++t) {
         float a = 0.f;
 #pragma unroll
-        for (int ww = 0; ww < 4; ++ww) a += f[ww] * redO[(((ww * kNQT + qt) * 8 + t) * 4 + w) * 64 + l];
+        for (int ww = 0; ww < 4; ++ww) a += f[ww] * redO[(((ww * NQ + qt) * 8 + t) * 4 + w) * 64 + l];
         o[t] = a * inv;
       }
       if (j < n_q) {
@@ -285,7 +285,9 @@ __device__ __forceinline__ void attend_item(
   }
 }
 
-constexpr int kRedFloats = 4 * kNQT * 8 * 4 * 64 + 4 * kNQT * 64 + 4 * kNQT * 16;
+// floats of LDS the merge of the four waves needs for NQ query tiles
+constexpr int red_floats(int nq) { return 4 * nq * 8 * 4 * 64 + 4 * nq * 64 + 4 * nq * 16; }
+constexpr int kRedFloats = red_floats(kNQT);
 
 __global__ __launch_bounds__(256) void hash_attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
@@ -309,10 +311,12 @@ __global__ __launch_bounds__(256) void hash_attn_mfma_kernel(
                      lse + qbase, red);
 }
 
-// Decode batch over memories of different sizes: one workgroup per row (one KV head
-// of one sequence) with its G <= 16 queries.  The workgroup hashes its queries
-// against the row's own A (first maximum wins), then attends each distinct bucket
-// once with the queries that chose it.  Rows are described by fm_rowdesc; A, K, V
+// Decode batch over memories of different sizes: G workgroups per row (one KV head
+// of one sequence) with its G <= 16 queries.  Every workgroup of a row hashes the
+// row's queries against the row's own A (first maximum wins; cheap, and it keeps the
+// launch free of any host-side grouping); workgroup s then attends the s-th distinct
+// bucket among the G hashes with the queries that chose it, or exits if there are
+// fewer distinct buckets.  Each bucket is read once, and a row's buckets in parallel.  Rows are described by fm_rowdesc; A, K, V
 // and the bucket lists of all rows are packed back to back.
 __global__ __launch_bounds__(256) void decode_hash_attn_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ A_all, const bf16_t* __restrict__ K_all,
@@ -320,72 +324,67 @@ __global__ __launch_bounds__(256) void decode_hash_attn_kernel(
     const fm_rowdesc* __restrict__ desc, int G, float scale2, bf16_t* __restrict__ out,
     float* __restrict__ lse, int32_t* __restrict__ hash_out, float* __restrict__ scores_out) {
   extern __shared__ __attribute__((aligned(16))) float red[];
-  __shared__ float sq[16 * kD];
   __shared__ float s_best[4][16];
   __shared__ int s_besti[4][16];
   __shared__ int s_hash[16];
   __shared__ int q_rows[FM_QTILE];
-  const int row = blockIdx.x;
+  const int row = blockIdx.x, slot = blockIdx.y;
   const fm_rowdesc ds = desc[row];
   const int tid = threadIdx.x, l = tid & 63, w = tid >> 6;
   const bf16_t* qb = q + int64_t(row) * G * kD;
-  for (int e = tid; e < G * kD; e += 256) sq[e] = bf16_to_f32(qb[e]);
-  __syncthreads();
-  // ---- hash: thread scans buckets tid, tid+256, ...; fp32 FMA chain over d ----
-  float best[16];
-  int besti[16];
-#pragma unroll
-  for (int g = 0; g < 16; ++g) {
-    best[g] = -INFINITY;
-    besti[g] = 0x7fffffff;
-  }
+  // ---- hash on MFMA: 32 buckets x (G queries padded to 32) per v_mfma_f32_32x32x16_bf16 chain,
+  //      buckets on the A operand and ascending contraction steps: the sums of the other hash
+  //      kernels.  Wave w takes bucket chunks w, w+4, ...; lane (column l%32, half l/32) sees the
+  //      scores of its query for 16 buckets of a chunk in ascending order.
+  typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
   const int C = ds.n_buckets;
-  for (int c = tid; c < C; c += 256) {
-    const uint4* ar = reinterpret_cast<const uint4*>(A_all + (ds.a_off + c) * kD);
-    float acc[16];
+  const int col = l & 31, hb = l >> 5;
+  bf16x8 bq[8];
+  {
+    const uint4* pq = reinterpret_cast<const uint4*>(qb + int64_t(col < G ? col : 0) * kD + hb * 8);
 #pragma unroll
-    for (int g = 0; g < 16; ++g) acc[g] = 0.f;
-    for (int ch = 0; ch < kD / 8; ++ch) {
-      const uint4 u = ar[ch];
-      const uint32_t wv[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float a = bf16_to_f32(bf16_t(e & 1 ? wv[e >> 1] >> 16 : wv[e >> 1] & 0xffffu));
-#pragma unroll
-        for (int g = 0; g < 16; ++g)
-          if (g < G) acc[g] = fmaf(a, sq[g * kD + ch * 8 + e], acc[g]);
-      }
-    }
-#pragma unroll
-    for (int g = 0; g < 16; ++g)
-      if (g < G) {
-        if (scores_out) scores_out[(ds.a_off + c) * G + g] = acc[g];
-        if (besti[g] == 0x7fffffff || acc[g] > best[g]) {  // buckets ascend per thread
-          best[g] = acc[g];
-          besti[g] = c;
-        }
-      }
+    for (int ks = 0; ks < 8; ++ks) bq[ks] = as_bf16x8(col < G ? pq[2 * ks] : make_uint4(0, 0, 0, 0));
   }
-  // wave then workgroup reduction: larger score wins, equal scores keep the lower bucket
+  float best = -INFINITY;
+  int besti = 0x7fffffff;
+  for (int c0 = 32 * w; c0 < C; c0 += 128) {
+    const int cr = min(c0 + col, C - 1);
+    const uint4* pa = reinterpret_cast<const uint4*>(A_all + (ds.a_off + cr) * kD + hb * 8);
+    uint4 au[8];
 #pragma unroll
-  for (int g = 0; g < 16; ++g)
-    if (g < G) {
-      float b = best[g];
-      int bi = besti[g];
+    for (int ks = 0; ks < 8; ++ks) au[ks] = pa[2 * ks];
+    f32x16 acc;
 #pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        const float ob = __shfl_xor(b, o);
-        const int oi = __shfl_xor(bi, o);
-        if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > b || (ob == b && oi < bi))) {
-          b = ob;
-          bi = oi;
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(au[ks]), bq[ks], acc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int c = c0 + 8 * (r >> 2) + 4 * hb + (r & 3);
+      if (c < C && col < G) {
+        if (scores_out && slot == 0) scores_out[(ds.a_off + c) * G + col] = acc[r];
+        if (besti == 0x7fffffff || acc[r] > best) {  // buckets ascend per lane
+          best = acc[r];
+          besti = c;
         }
       }
-      if (l == 0) {
-        s_best[w][g] = b;
-        s_besti[w][g] = bi;
-      }
     }
+  }
+  // the two lane halves of a column, then the four waves: larger score wins, equal scores keep the
+  // lower bucket
+  {
+    const float ob = __shfl_xor(best, 32);
+    const int oi = __shfl_xor(besti, 32);
+    if (oi != 0x7fffffff && (besti == 0x7fffffff || ob > best || (ob == best && oi < besti))) {
+      best = ob;
+      besti = oi;
+    }
+    if (l < G) {
+      s_best[w][l] = best;
+      s_besti[w][l] = besti;
+    }
+  }
   __syncthreads();
   if (tid < G) {
     float b = s_best[0][tid];
@@ -399,29 +398,56 @@ __global__ __launch_bounds__(256) void decode_hash_attn_kernel(
       }
     }
     s_hash[tid] = bi;
-    hash_out[int64_t(row) * G + tid] = bi;
+    if (slot == 0) hash_out[int64_t(row) * G + tid] = bi;
   }
   __syncthreads();
-  // ---- one attention item per distinct bucket among the G queries ----
+  // ---- this workgroup's bucket: the slot-th distinct one among the G hashes ----
   const bf16_t* Kb = K_all + ds.k_off * kD;
   const bf16_t* Vb = V_all + ds.k_off * kD;
-  for (int g0 = 0; g0 < G; ++g0) {
-    const int bkt = s_hash[g0];
+  int seen = 0, bkt = -1;
+  for (int g0 = 0; g0 < G; ++g0) {  // uniform: every thread reads the same s_hash
     bool first = true;
-    for (int g = 0; g < g0; ++g) first = first && (s_hash[g] != bkt);
-    if (!first) continue;  // uniform: every thread reads the same s_hash
-    __syncthreads();
-    if (tid == 0) {
-      int n = 0;
-      for (int g = g0; g < G; ++g)
-        if (s_hash[g] == bkt) q_rows[n++] = g;
-      q_rows[FM_QTILE - 1] = n;
-    }
-    __syncthreads();
-    const int n_q = q_rows[FM_QTILE - 1];
-    attend_item<1>(qb, q_rows, n_q, Kb, Vb, idx_all + ds.idx_off + int64_t(bkt) * ds.bucket_size, ds.bucket_size,
-                   ds.n_keys, scale2, out + int64_t(row) * G * kD, lse + int64_t(row) * G, red);
+    for (int g = 0; g < g0; ++g) first = first && (s_hash[g] != s_hash[g0]);
+    if (!first) continue;
+    if (seen == slot) bkt = s_hash[g0];
+    ++seen;
   }
+  if (bkt < 0) return;
+  if (tid == 0) {
+    int n = 0;
+    for (int g = 0; g < G; ++g)
+      if (s_hash[g] == bkt) q_rows[n++] = g;
+    q_rows[FM_QTILE - 1] = n;
+  }
+  __syncthreads();
+  const int n_q = q_rows[FM_QTILE - 1];
+  attend_item<1>(qb, q_rows, n_q, Kb, Vb, idx_all + ds.idx_off + int64_t(bkt) * ds.bucket_size, ds.bucket_size,
+                 ds.n_keys, scale2, out + int64_t(row) * G * kD, lse + int64_t(row) * G, red);
+}
+
+// Dense attention of one token per query head over L local keys (decode): one workgroup per KV
+// head with its G <= 16 query heads; the four waves take the 32-key blocks in turn, as for a
+// gathered bucket, so four blocks of loads are in flight per workgroup.  With one query per head a
+// causal mask aligned bottom-right hides nothing.
+__global__ __launch_bounds__(256) void local_attn_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    bf16_t* __restrict__ out, float* __restrict__ lse, int G, int L, float scale2) {
+  extern __shared__ __attribute__((aligned(16))) float red[];
+  __shared__ int q_rows[FM_QTILE];
+  const int hk = blockIdx.x;
+  if (threadIdx.x < FM_QTILE) q_rows[threadIdx.x] = threadIdx.x;
+  __syncthreads();
+  const int64_t qbase = int64_t(hk) * G;
+  attend_item<1>(q + qbase * kD, q_rows, G, k + int64_t(hk) * L * kD, v + int64_t(hk) * L * kD, nullptr, L, L,
+                 scale2, out + qbase * kD, lse + qbase, red);
+}
+
+int local_attn_decode(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G, int L,
+                      float sm_scale, hipStream_t st) {
+  hipLaunchKernelGGL(local_attn_decode_kernel, dim3(unsigned(H)), dim3(256), red_floats(1) * sizeof(float), st,
+                     (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)out, lse, G, L,
+                     sm_scale * kLog2e);
+  return launch_status("fm_local_attn_fwd(decode)");
 }
 
 bool hash_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_BF16; }
@@ -429,8 +455,7 @@ bool hash_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_
 int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
                      const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, float sm_scale,
                      void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st) {
-  FM_ALLOW_LDS(decode_hash_attn_kernel, kRedFloats * sizeof(float), "fm_decode_hash_attn: lds");
-  hipLaunchKernelGGL(decode_hash_attn_kernel, dim3(unsigned(rows)), dim3(256), kRedFloats * sizeof(float),
+  hipLaunchKernelGGL(decode_hash_attn_kernel, dim3(unsigned(rows), unsigned(G)), dim3(256), red_floats(1) * sizeof(float),
                      st, (const bf16_t*)q, (const bf16_t*)A_all, (const bf16_t*)K_all,
                      (const bf16_t*)V_all, idx_all, desc, G, sm_scale * kLog2e, (bf16_t*)out, lse, hash_out,
                      scores_out);
@@ -457,6 +482,7 @@ int local_attn_dense(const void* q, const void* k, const void* v, void* out, flo
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
                     int S, int L, int d, float sm_scale, int causal, hipStream_t st) {
   (void)d;
+  if (S == 1 && G <= 16 && L >= 1) return local_attn_decode(q, k, v, out, lse, H, G, L, sm_scale, st);
   return local_attn_dense(q, k, v, out, lse, H, G, S, L, sm_scale, causal, st);
 }
 

@@ -83,3 +83,30 @@ def attention_hash(q, k, v, centroids, bucket_size, sm_scale, window=None):
         flat, counts, _ = ops.window_filter(k_hashes, lo, hi)
         flat = flat + lo if lo else flat
     return ops.attention_hash_varlen_i32(q, k, v, flat, counts, q_hashes, sm_scale)
+
+
+def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                                   out: torch.Tensor, lse: torch.Tensor, k_hashes: torch.Tensor,
+                                   k_hash_counts: torch.Tensor, q_hashes: torch.Tensor, sm_scale: float
+                                   ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Gradients of :func:`attention_hash_varlen` w.r.t. ``q``, ``k`` and ``v``.
+
+    The reference registers no gradient for its operator (triton_kernel.py:44-48) and falls back to a
+    dense ``[S, N]`` evaluation (memory.py:166-206); this visits only each query's bucket.  ``out`` and
+    ``lse`` are the forward's results (fp32 natural-log LSE) or the ones merged with further keys, in
+    which case the gradients are the gathered keys' share.
+
+    :return: ``(dq [batch, q_seq_len, d_head], dk, dv [batch, kv_seq_len, d_head])``; ``dq`` in q's dtype,
+        ``dk`` / ``dv`` in fp32 (sums over every bucket a key belongs to).
+    """
+    batch_size, q_seq_len, d_head = q.shape
+    assert d_out.shape == q.shape and out.shape == q.shape and lse.shape == (batch_size, q_seq_len)
+    assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    n_buckets = k_hash_counts.shape[1]
+    counts = _as_i32(k_hash_counts).contiguous()
+    hashes = _as_i32(q_hashes).contiguous()
+    off = ops.bucket_offsets(counts)
+    groups = ops.group_queries(hashes, n_buckets)
+    return ops.hash_attn_bwd(q, k, v, _as_i32(k_hashes).contiguous(), off, counts, groups, out.contiguous(),
+                             lse.float().contiguous(), d_out.contiguous(), sm_scale)
+

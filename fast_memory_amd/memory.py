@@ -121,6 +121,29 @@ def ring_attention_masked_forward(k_hashes, q_hashes, q, k, v, sm_scale, rank,
 
 
 # --------------------------------------------------------------------------
+def ring_attention_masked_backward(k_hashes, q_hashes, h_idx, d_out, q, k, v, out, softmax_lse, sm_scale, rank):
+    """Drop-in for ``ring_attention_masked_backward`` (memory.py:166-206) on one window of keys.
+
+    Same arguments and layouts as the reference (``h_idx`` is accepted and unused: the head index is
+    implied by the layout); ``out`` / ``softmax_lse`` are the final (merged) results.  The reference
+    materialises the dense ``[S, N]`` probabilities; here every query only visits its bucket's keys.
+
+    :return: ``(dQ [1,n_heads,seq_len,d], dK, dV [1,k_heads,context_len,d])`` in q's dtype.
+    """
+    from .hash_attention import attention_hash_varlen_backward
+    batch_size, n_heads, seq_len, d_head = q.shape
+    _, k_heads, context_len, _ = k.shape
+    assert batch_size == 1 and n_heads % k_heads == 0
+    kh = k_hashes.permute(1, 0, 2).to(torch.int32).contiguous()     # H C Z
+    flat, counts, _ = ops.window_filter(kh, rank * context_len, (rank + 1) * context_len)
+    dq, dk, dv = attention_hash_varlen_backward(
+        d_out.reshape(k_heads, -1, d_head).contiguous(), q.reshape(k_heads, -1, d_head).contiguous(),
+        k.reshape(k_heads, -1, d_head), v.reshape(k_heads, -1, d_head), out.reshape(k_heads, -1, d_head),
+        softmax_lse.reshape(k_heads, -1).float(), flat, counts, q_hashes.reshape(k_heads, -1), sm_scale)
+    return (dq.reshape(q.shape), dk.to(k.dtype).reshape(k.shape), dv.to(v.dtype).reshape(v.shape))
+
+
+# --------------------------------------------------------------------------
 class Memory:
     """Indexed memory over one sequence's past keys (README.md:5-7).
 

@@ -189,6 +189,31 @@ def hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, s
     return out, lse
 
 
+def hash_attn_bwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, out, lse, dout, sm_scale: float,
+                  dk: Optional[torch.Tensor] = None, dv: Optional[torch.Tensor] = None):
+    """Backward of :func:`hash_attn_fwd` (memory.py:166-206 on the gathered pairs).  ``out`` / ``lse`` are
+    the forward's result or the merged one; ``dout [H,Sq,d]``.  Returns ``dq`` (dtype of q) and the fp32
+    ``dk``, ``dv [H,N,d]``; when ``dk`` / ``dv`` are given the gradients are added into them."""
+    _dev(q, k, v, k_idx, bucket_off, bucket_cnt, out, lse, dout)
+    H, Sq, d = q.shape
+    _, N, _ = k.shape
+    C = bucket_cnt.shape[-1]
+    assert k.shape == v.shape and out.shape == q.shape and dout.shape == q.shape and lse.shape == (H, Sq)
+    assert q.dtype == k.dtype == v.dtype == out.dtype == dout.dtype and lse.dtype == torch.float32
+    assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and bucket_off.dtype == torch.int64
+    dq = torch.empty_like(q)
+    if dk is None:
+        dk = torch.zeros((H, N, d), dtype=torch.float32, device=q.device)
+    if dv is None:
+        dv = torch.zeros((H, N, d), dtype=torch.float32, device=q.device)
+    assert dk.dtype == dv.dtype == torch.float32 and dk.shape == dv.shape == (H, N, d)
+    check(_lib.load().fm_hash_attn_bwd(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
+                                       _p(groups.q_perm), _p(groups.items), _p(groups.n_items), groups.max_items,
+                                       _p(out), _p(lse), _p(dout), _p(dq), _p(dk), _p(dv), H, Sq, N, d, C,
+                                       float(sm_scale), _dt(q), _stream(q)))
+    return dq, dk, dv
+
+
 def attention_hash_varlen_i32(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: float):
     """The reference operator in one C call (triton_kernel.py:51-119) on int32 index tensors."""
     _dev(q, k, v, k_idx, bucket_cnt, q_hash)

@@ -143,6 +143,27 @@ int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t*
                      float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype,
                      void* stream);
 
+/* ---- f1: backward of the bucket-gathered attention --------------------------
+ * replaces ring_attention_masked_backward (memory.py:166-206), which forms the
+ * dense [S, N] probability matrix; here only a query's bucket is visited.
+ *   q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items
+ *                                      as for fm_hash_attn_fwd
+ *   out [H,Sq,d], lse [H,Sq] fp32      the forward's result, or the result merged
+ *                                      with further keys (the gradients are then
+ *                                      the gathered keys' share)
+ *   dout [H,Sq,d]                      gradient of the loss w.r.t. out
+ *   dq [H,Sq,d] (dtype of q)           written; a query whose bucket is empty gets 0
+ *   dk, dv [H,N,d] fp32                ACCUMULATED into (atomic adds): zero them
+ *                                      before the first call; several calls
+ *                                      (key windows) may add into the same buffers.
+ * The order of the atomic adds depends on scheduling, so the last bits of dk and
+ * dv can differ between runs. */
+int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                     const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                     const fm_item* items, const int32_t* n_items, int64_t max_items, const void* out,
+                     const float* lse, const void* dout, void* dq, float* dk, float* dv, int H, int Sq, int N,
+                     int d, int C, float sm_scale, int dtype, void* stream);
+
 /* ---- the reference operator in one call -------------------------------------
  * attention_hash_varlen(q,k,v,k_hashes,k_hash_counts,q_hashes,sm_scale)
  * (triton_kernel.py:51-119): bucket offsets + grouping + attention. */

@@ -21,6 +21,10 @@ How each function is pinned (tests/test_oracle_*.py):
                         reference's dense-masked procedure) against each other,
                         C=1,Z=N == full softmax (torch.logsumexp / SDPA),
                         Z=1 == V[idx]; invariants on the LSE
+  *_backward_*       -- torch autograd (fp64) through an independent dense
+                        softmax over the same visible pairs, alone and as part
+                        of a larger softmax (merged out / lse); the two
+                        formulations (dense-masked, gather) against each other
   update_out_and_lse -- closed form logaddexp / convex combination, split test
   local_attention    -- torch SDPA (math path) + torch.logsumexp.
                         PARITY UNPINNED against the reference: the reference
@@ -353,6 +357,70 @@ def ring_attention_masked_forward(k_hashes_zhj, q_hashes_hgi, q, k, v, sm_scale,
                                        flat, counts, q_hashes_hgi.reshape(H, -1), sm_scale,
                                        lse_dtype=lse_dtype)
     return out.reshape(bs, n_heads, S, d), lse.reshape(bs, n_heads, S)
+
+
+# --------------------------------------------------------------------------
+# f1  backward of the gathered attention                       mem:166-206
+# --------------------------------------------------------------------------
+def ring_attention_masked_backward_ref(k_hashes_zhj, q_hashes_hgi, d_out, q, k, v, out, softmax_lse, sm_scale,
+                                       rank):
+    """mem:166-206 restated in fp64 (dense, masked): with ``P = exp(s - lse)`` on
+    the visible (query, key) pairs, ``dV = P^T dO``, ``dP = dO V^T``, ``D =
+    rowsum(dO * O)``, ``dS = P * (dP - D)``, ``dQ = scale * dS K``, ``dK =
+    scale * dS^T Q``.  ``out`` / ``softmax_lse`` may be those of a larger
+    softmax the gathered keys are only a part of (the merged result).  Layouts
+    as in :func:`ring_attention_masked_forward_ref`; returns ``(dQ [1,H*G,S,d],
+    dK [1,H,N,d], dV [1,H,N,d])`` in fp64."""
+    bs, n_heads, S, d = q.shape
+    _, H, N, _ = k.shape
+    G = n_heads // H
+    h_idx = torch.arange(H)
+    mask = torch.zeros((bs, H, G, S, N + 1), dtype=torch.bool)
+    k_idx = k_hashes_zhj[q_hashes_hgi, h_idx[:, None, None]]         # H G S Z
+    m = torch.logical_and(rank * N <= k_idx, k_idx < (rank + 1) * N)
+    k_idx = (k_idx - rank * N) * m + (N * ~m)
+    mask.scatter_(-1, k_idx.unsqueeze(0), m.unsqueeze(0))
+    mask = mask[..., :-1]
+    shape = (bs, H, G, S, d)
+    qd, dod, od = q.double().view(shape), d_out.double().view(shape), out.double().view(shape)
+    kd, vd = k.double(), v.double()
+    scores = torch.einsum('bhgid,bhjd->bhgij', qd, kd) * sm_scale
+    P = torch.exp(scores - softmax_lse.double().view(bs, H, G, S, 1)).masked_fill(~mask, 0.0)
+    dV = torch.einsum('bhgij,bhgid->bhjd', P, dod)
+    dP = torch.einsum('bhgid,bhjd->bhgij', dod, vd)
+    D = (dod * od).sum(-1, keepdim=True)
+    dS = P * (dP - D)
+    dQ = torch.einsum('bhgij,bhjd->bhgid', dS, kd) * sm_scale
+    dK = torch.einsum('bhgij,bhgid->bhjd', dS, qd) * sm_scale
+    return dQ.reshape(bs, n_heads, S, d), dK, dV
+
+
+def hashed_attention_backward_gather(q, k, v, k_hashes, k_hash_counts, q_hashes, out, lse, d_out, sm_scale):
+    """The same gradients on the gather formulation (the layouts of
+    :func:`hashed_attention_gather`: ``q,out,d_out [H,Sq,d]``, ``k,v [H,N,d]``,
+    flat bucket lists): per query only its bucket's keys are visited.  fp64."""
+    H, Sq, d = q.shape
+    N = k.shape[1]
+    off = bucket_offsets(k_hash_counts)
+    dq = torch.zeros((H, Sq, d), dtype=torch.float64)
+    dk = torch.zeros((H, N, d), dtype=torch.float64)
+    dv = torch.zeros((H, N, d), dtype=torch.float64)
+    for h in range(H):
+        for i in range(Sq):
+            b = int(q_hashes[h, i])
+            c = int(k_hash_counts[h, b])
+            if c == 0:
+                continue
+            idx = k_hashes[int(off[h, b]):int(off[h, b]) + c].long()
+            kk, vv = k[h, idx].double(), v[h, idx].double()
+            qi, doi = q[h, i].double(), d_out[h, i].double()
+            p = torch.exp(kk @ qi * sm_scale - float(lse[h, i]))
+            dp = vv @ doi
+            ds = p * (dp - float((doi * out[h, i].double()).sum()))
+            dq[h, i] = sm_scale * (ds @ kk)
+            dk[h].index_add_(0, idx, sm_scale * ds[:, None] * qi[None, :])
+            dv[h].index_add_(0, idx, p[:, None] * doi[None, :])
+    return dq, dk, dv
 
 
 # --------------------------------------------------------------------------

@@ -433,6 +433,86 @@ def test_ring_attention_masked_forward_windows(ops):
         assert_attn_close(out[0], lse[0], ro[0], rl[0], torch.bfloat16, f"ring rank {rank}")
 
 
+# ------------------------------------------------------------------ f1 backward of the gathered attention
+def _assert_grad_close(got, ref, dtype, what):
+    got, ref = got.float().cpu().double(), ref.double()
+    if dtype == torch.float32:
+        ok = torch.allclose(got, ref, atol=1e-4, rtol=1e-4)
+    else:
+        # bf16 inputs: products of bf16-rounded operands, gradients summed over up to hundreds of terms
+        ok = torch.allclose(got, ref, atol=2e-2 * max(1.0, ref.abs().max().item()), rtol=2e-2)
+    assert ok, f"{what}: max err {(got - ref).abs().max().item():.3e} (ref max {ref.abs().max().item():.3e})"
+
+
+@pytest.mark.parametrize("dtype,B,S,N,C,Z,d", [
+    (torch.float32, 2, 70, 300, 6, 40, 64),
+    (torch.float32, 1, 24, 1024, 8, 16, 16),             # the reference's small test shape (tk:500)
+    (torch.bfloat16, 2, 200, 2000, 12, 150, 128),
+    (torch.bfloat16, 1, 130, 700, 3, 333, 128),          # more than 64 queries per bucket: several items
+])
+def test_hash_attention_backward(ops, dtype, B, S, N, C, Z, d):
+    from fast_memory_amd import attention_hash_varlen, attention_hash_varlen_backward
+    q, k, v, kh, cnt, qh = make_attn_case(1200 + S, B, S, N, C, Z, d, dtype, window="ref", std=0.7)
+    dout = (torch.randn(B, S, d, generator=gen(1300 + S)) * 0.5).to(dtype)
+    sm = d ** -0.5
+    args = dev(q, k, v, kh, cnt, qh)
+    out, lse = attention_hash_varlen(*args, sm)
+    dq, dk, dv = attention_hash_varlen_backward(dev(dout), args[0], args[1], args[2], out, lse, args[3], args[4],
+                                                args[5], sm)
+    assert dq.dtype == dtype and dk.dtype == torch.float32 and dk.shape == k.shape
+    # oracle on the same (rounded) inputs and on the GPU's own out / lse
+    rq, rk, rv = O.hashed_attention_backward_gather(q.float(), k.float(), v.float(), kh, cnt, qh, out.float().cpu(),
+                                                    lse.cpu(), dout.float(), sm)
+    _assert_grad_close(dq, rq, dtype, "dq")
+    _assert_grad_close(dk, rk, dtype, "dk")
+    _assert_grad_close(dv, rv, dtype, "dv")
+    empty = lse.cpu() < -1e30
+    assert (dq.float().cpu()[empty] == 0).all()
+
+
+def test_ring_attention_masked_backward_with_merged_result(ops):
+    # memory part of a merged attention: out / lse passed to the backward are those of the softmax over
+    # bucket keys and local keys together; checked against autograd through a dense fp64 evaluation
+    from fast_memory_amd import ring_attention_masked_backward, ring_attention_masked_forward, update_out_and_lse
+    g = gen(1400)
+    C, H, G, S, N, Z, d, L = 5, 2, 2, 12, 200, 30, 64, 9
+    sm = 0.125
+    q = torch.randn(1, H * G, S, d, generator=g)
+    k = torch.randn(1, H, N, d, generator=g)
+    v = torch.randn(1, H, N, d, generator=g)
+    kl = torch.randn(1, H, L, d, generator=g)
+    vl = torch.randn(1, H, L, d, generator=g)
+    w = torch.randn(1, H * G, S, d, generator=g)
+    kh = torch.stack([torch.stack([torch.randperm(N, generator=g)[:Z] for _ in range(H)]) for _ in range(C)])
+    qh = torch.randint(0, C, (H, G, S), generator=g)
+    # dense fp64 forward of the union softmax with autograd
+    qd, kd, vd = (t.double().clone().requires_grad_(True) for t in (q, k, v))
+    vis = torch.zeros(H, G, S, N, dtype=torch.bool)
+    for h in range(H):
+        for gg in range(G):
+            for i in range(S):
+                vis[h, gg, i, kh[qh[h, gg, i], h]] = True
+    s_m = (torch.einsum('hgid,hjd->hgij', qd[0].view(H, G, S, d), kd[0]) * sm).masked_fill(~vis, -float("inf"))
+    s_l = torch.einsum('hgid,hjd->hgij', qd[0].view(H, G, S, d), kl[0].double()) * sm
+    P = torch.softmax(torch.cat([s_m, s_l], -1), -1)
+    o = torch.einsum('hgij,hjd->hgid', P[..., :N], vd[0]) + torch.einsum('hgij,hjd->hgid', P[..., N:], vl[0].double())
+    (o.reshape(1, H * G, S, d) * w.double()).sum().backward()
+    # GPU: forward of both parts, merge, backward of the memory part with the merged result
+    mo, ml = ring_attention_masked_forward(*dev(kh, qh, q, k, v), sm, 0)
+    lo, ll = ops.local_attn_fwd(dev(q[0]), dev(kl[0]), dev(vl[0]), sm, False)
+    out, lse = update_out_and_lse(None, None, lo.unsqueeze(0), ll.unsqueeze(0))
+    out, lse = update_out_and_lse(out.contiguous(), lse.contiguous(), mo, ml)
+    assert torch.allclose(out.cpu().double(), o.detach().reshape(1, H * G, S, d), atol=1e-4)
+    dq, dk, dv = ring_attention_masked_backward(*dev(kh, qh), torch.arange(H), dev(w), dev(q), dev(k), dev(v),
+                                                out.to(q.dtype), lse.squeeze(-1), sm, 0)
+    assert torch.allclose(dk.cpu().double(), kd.grad, atol=2e-4, rtol=1e-4)
+    assert torch.allclose(dv.cpu().double(), vd.grad, atol=2e-4, rtol=1e-4)
+    rq, _, _ = O.ring_attention_masked_backward_ref(kh, qh, w, q, k, v, o.detach().reshape(q.shape),
+                                                    torch.logsumexp(torch.cat([s_m, s_l], -1), -1).detach().reshape(1, H * G, S),
+                                                    sm, 0)
+    assert torch.allclose(dq.cpu().double(), rq, atol=2e-4, rtol=1e-4)
+
+
 # ------------------------------------------------------------------ a1+a2 fused build
 def _clustered_keys(g, H, N, d, n_clusters=64, spread=0.5):
     cen = torch.randn(H, n_clusters, d, generator=g)

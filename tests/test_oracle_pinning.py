@@ -255,6 +255,85 @@ def test_ring_masked_forward_matches_ref_formulation():
 
 
 # ------------------------------------------------------------------ a10
+def _bwd_case(seed, H=2, G=2, S=5, N=40, d=8, C=4, Z=7, extra=0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(1, H * G, S, d, generator=g, dtype=torch.float64)
+    k = torch.randn(1, H, N, d, generator=g, dtype=torch.float64)
+    v = torch.randn(1, H, N, d, generator=g, dtype=torch.float64)
+    kh = torch.stack([torch.stack([torch.randperm(N, generator=g)[:Z] for _ in range(H)]) for _ in range(C)])  # C H Z
+    qh = torch.randint(0, C, (H, G, S), generator=g)
+    w = torch.randn(1, H * G, S, d, generator=g, dtype=torch.float64)
+    ke = torch.randn(1, H, extra, d, generator=g, dtype=torch.float64) if extra else None
+    ve = torch.randn(1, H, extra, d, generator=g, dtype=torch.float64) if extra else None
+    return q, k, v, kh, qh, w, ke, ve
+
+
+def _dense_forward(q, k, v, kh, qh, sm_scale, ke=None, ve=None):
+    """Independent dense forward for autograd: softmax over the bucket's keys (and, if given, over
+    extra keys every query sees), plain torch ops."""
+    bs, HG, S, d = q.shape
+    H, N = k.shape[1], k.shape[2]
+    G = HG // H
+    vis = torch.zeros(H, G, S, N, dtype=torch.bool)
+    for h in range(H):
+        for gg in range(G):
+            for i in range(S):
+                vis[h, gg, i, kh[qh[h, gg, i], h]] = True
+    s = torch.einsum('hgid,hjd->hgij', q[0].view(H, G, S, d), k[0]) * sm_scale
+    s = s.masked_fill(~vis, -math.inf)
+    vv = v[0][:, None, None].expand(H, G, S, N, d)
+    if ke is not None:
+        se = torch.einsum('hgid,hjd->hgij', q[0].view(H, G, S, d), ke[0]) * sm_scale
+        s = torch.cat([s, se], -1)
+    lse = torch.logsumexp(s, -1)
+    P = torch.exp(s - lse[..., None])
+    out = torch.einsum('hgij,hjd->hgid', P[..., :N], v[0])
+    if ke is not None:
+        out = out + torch.einsum('hgij,hjd->hgid', P[..., N:], ve[0])
+    return out.reshape(1, HG, S, d), lse.reshape(1, HG, S)
+
+
+@pytest.mark.parametrize("extra", [0, 6])
+def test_backward_matches_autograd(extra):
+    # extra = 0: the gathered softmax alone.  extra > 0: the gathered keys are part of a larger softmax
+    # (the merged result); out and lse passed to the backward are the merged ones, and the gradients of
+    # the memory's k, v and the memory part of dq must be those autograd finds.
+    q, k, v, kh, qh, w, ke, ve = _bwd_case(77 + extra, extra=extra)
+    sm = 0.37
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    out, lse = _dense_forward(leaves[0], leaves[1], leaves[2], kh, qh, sm, ke, ve)
+    (out * w).sum().backward()
+    dq_ref, dk_ref, dv_ref = O.ring_attention_masked_backward_ref(kh, qh, w, q, k, v, out.detach(), lse.detach(), sm, 0)
+    assert torch.allclose(dk_ref, leaves[1].grad, atol=1e-10)
+    assert torch.allclose(dv_ref, leaves[2].grad, atol=1e-10)
+    if extra == 0:
+        assert torch.allclose(dq_ref, leaves[0].grad, atol=1e-10)
+    else:
+        # the rest of dq comes from the extra keys: the same formula with those keys all visible
+        H, G, S, d = k.shape[1], q.shape[1] // k.shape[1], q.shape[2], q.shape[3]
+        qd = q.view(1, H, G, S, d)
+        P = torch.exp(torch.einsum('bhgid,bhjd->bhgij', qd, ke) * sm - lse.detach().view(1, H, G, S, 1))
+        dP = torch.einsum('bhgid,bhjd->bhgij', w.view(1, H, G, S, d), ve)
+        D = (w * out.detach()).sum(-1).view(1, H, G, S, 1)
+        dq_e = torch.einsum('bhgij,bhjd->bhgid', P * (dP - D), ke) * sm
+        assert torch.allclose(dq_ref + dq_e.reshape(q.shape), leaves[0].grad, atol=1e-10)
+
+
+def test_backward_gather_and_dense_formulations_agree():
+    q, k, v, kh, qh, w, _, _ = _bwd_case(91, H=2, G=3, S=6, N=50, d=8, C=5, Z=9)
+    sm = 0.21
+    out, lse = O.ring_attention_masked_forward_ref(kh, qh, q, k, v, sm, 0)
+    dq1, dk1, dv1 = O.ring_attention_masked_backward_ref(kh, qh, w, q, k, v, out, lse, sm, 0)
+    H, Z = k.shape[1], kh.shape[2]
+    flat = kh.permute(1, 0, 2).reshape(-1)
+    counts = torch.full((H, kh.shape[0]), Z)
+    dq2, dk2, dv2 = O.hashed_attention_backward_gather(
+        q.reshape(H, -1, 8), k[0], v[0], flat, counts, qh.reshape(H, -1), out.reshape(H, -1, 8),
+        lse.reshape(H, -1), w.reshape(H, -1, 8), sm)
+    assert torch.allclose(dq1.reshape(H, -1, 8), dq2, atol=1e-9)
+    assert torch.allclose(dk1[0], dk2, atol=1e-9) and torch.allclose(dv1[0], dv2, atol=1e-9)
+
+
 def test_merge_closed_form_and_first_call():
     gen = g(30)
     oa, ob = torch.randn(3, 5, 8, generator=gen), torch.randn(3, 5, 8, generator=gen)

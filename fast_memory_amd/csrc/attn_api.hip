@@ -25,7 +25,7 @@ int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const 
                      void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st);
 
 // 0 = automatic, 1 = force the generic kernels (used by tests to compare paths)
-static int g_force_generic = 0;
+int g_force_generic = 0;
 }  // namespace fm
 
 extern "C" void fm_debug_force_generic(int on) { fm::g_force_generic = on; }

@@ -65,8 +65,8 @@ __device__ __forceinline__ void backward_one_query(const T* __restrict__ qrow, c
         const int k = l + 64 * r;
         if (k < d) {
           dq[r] = fmaf(dst, Elem<T>::load(kr + k), dq[r]);
-          atomicAdd(dKb + int64_t(rt) * d + k, dst * qv[r]);
-          atomicAdd(dVb + int64_t(rt) * d + k, pt * dov[r]);
+          unsafeAtomicAdd(dKb + int64_t(rt) * d + k, dst * qv[r]);
+          unsafeAtomicAdd(dVb + int64_t(rt) * d + k, pt * dov[r]);
         }
       }
     }
@@ -97,6 +97,13 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_generic_kernel(
   }
 }
 
+extern int g_force_generic;
+bool hash_attn_bwd_mfma_supported(int d, int dtype);
+int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
+                       const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                       int64_t max_items, const void* out, const float* lse, const void* dout, void* dq, float* dk,
+                       float* dv, int Sq, int N, int C, float sm_scale, hipStream_t st);
+
 }  // namespace fm
 
 extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
@@ -114,6 +121,9 @@ extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, con
   FM_REQUIRE(max_items >= 1 && max_items <= 0x7fffffffLL, FM_ERR_ARG, "fm_hash_attn_bwd: max_items=%lld",
              (long long)max_items);
   hipStream_t st = as_stream(stream);
+  if (!g_force_generic && hash_attn_bwd_mfma_supported(d, dtype))
+    return hash_attn_bwd_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse,
+                              dout, dq, dk, dv, Sq, N, C, sm_scale, st);
   if (dtype == FM_F32)
     hipLaunchKernelGGL(hash_attn_bwd_generic_kernel<float>, dim3(unsigned(max_items)), dim3(256), 0, st,
                        (const float*)q, (const float*)k, (const float*)v, k_idx, bucket_off, bucket_cnt, q_perm, items,

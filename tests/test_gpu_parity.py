@@ -470,6 +470,27 @@ def test_hash_attention_backward(ops, dtype, B, S, N, C, Z, d):
     assert (dq.float().cpu()[empty] == 0).all()
 
 
+def test_backward_mfma_and_generic_agree(ops):
+    from fast_memory_amd import attention_hash_varlen, attention_hash_varlen_backward
+    q, k, v, kh, cnt, qh = make_attn_case(1500, 2, 300, 3000, 9, 500, 128, torch.bfloat16, window="ref", std=0.7)
+    qh[0, :150] = 2                                             # a bucket with several 16-query tiles and items
+    dout = (torch.randn(2, 300, 128, generator=gen(1501)) * 0.5).to(torch.bfloat16)
+    args = dev(q, k, v, kh, cnt, qh)
+    out, lse = attention_hash_varlen(*args, 128 ** -0.5)
+    call = lambda: attention_hash_varlen_backward(dev(dout), args[0], args[1], args[2], out, lse, args[3], args[4],
+                                                  args[5], 128 ** -0.5)
+    dq1, dk1, dv1 = call()
+    ops.force_generic_kernels(True)
+    try:
+        dq2, dk2, dv2 = call()
+    finally:
+        ops.force_generic_kernels(False)
+    for a, b, name in ((dq1, dq2, "dq"), (dk1, dk2, "dk"), (dv1, dv2, "dv")):
+        a, b = a.float(), b.float()
+        assert torch.allclose(a, b, atol=2e-2 * max(1.0, b.abs().max().item()), rtol=2e-2), \
+            f"{name}: {(a - b).abs().max().item():.3e} vs max {b.abs().max().item():.3e}"
+
+
 def test_ring_attention_masked_backward_with_merged_result(ops):
     # memory part of a merged attention: out / lse passed to the backward are those of the softmax over
     # bucket keys and local keys together; checked against autograd through a dense fp64 evaluation

@@ -163,6 +163,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c5", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-backward", action="store_true", help="skip timing the backward of the gathered attention")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--workspace-gib", type=float, default=8.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -291,6 +292,24 @@ def main():
         ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
         value = H * N / (ms_per_step * 1e-3)
 
+    # ---- backward of the gathered attention (training use), timed beside the forward ----
+    backward = None
+    if not args.no_backward:
+        dout = torch.randn_like(mo)
+        dkb = torch.zeros(mem.keys.shape, dtype=torch.float32, device=dev)
+        dvb = torch.zeros_like(dkb)
+        run_bwd = lambda: ops.hash_attn_bwd(q, mem.keys, mem.values, mem.bucket_idx.reshape(-1), mem.bucket_off,
+                                            mem.bucket_cnt, groups, mo, ml, dout, sm_scale, dkb, dvb)
+        bwd_ms, _ = timed(run_bwd, reps=2, warm=1)
+        n_tiles = int(((groups.bin_count + 15) // 16).sum().item())       # 16-query tiles, each sweeps its bucket
+        atomic_bytes = n_tiles * Z * 2 * d * 4
+        backward = {"ms": bwd_ms, "query_heads_per_s": qheads / (bwd_ms * 1e-3),
+                    "kernel": "hash_attn_bwd_mfma_kernel" if (d == 128 and e == 2) else "hash_attn_bwd_generic_kernel",
+                    "atomic_bytes_per_launch": atomic_bytes, "atomic_gbs": atomic_bytes / bwd_ms / 1e6}
+        del dout, dkb, dvb
+        log(f"[bench] backward of the gathered attention: {bwd_ms:.2f} ms ({backward['atomic_gbs']:.0f} GB/s of "
+            f"atomic adds)")
+
     attn_ms = sum(a.elapsed_time(b) for a, b in attn_events) / len(attn_events)
     parts_ms = {k: (sum(a.elapsed_time(b) for a, b in v) / len(v) if v else None) for k, v in part_events.items()}
     # algorithmic bytes of the gather-attention launch: every hit bucket once + q, out, lse
@@ -417,6 +436,7 @@ def main():
                         "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters},
         "query_path": query_path,
         "step_parts_ms": {"attention": attn_ms, **parts_ms},
+        "backward": backward,
         "parity_spot_check": parity,
     }
     print(json.dumps(line), flush=True)

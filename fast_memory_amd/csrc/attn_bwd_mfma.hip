@@ -13,12 +13,13 @@
 //     (contraction over keys; K^T comes from coalesced loads repacked per lane,
 //     as V does in the forward kernel);
 //   queries on accumulator rows (S = Q.K^T, dP = dO.V^T): lane (g,c) holds key
-//     c, queries 4g+r -- exactly the B operand of  dV^T = dO^T . P  and
-//     dK^T = Q^T . dS  (v_mfma_f32_16x16x16_bf16, contraction over the 16
-//     queries; dO^T and Q^T fragments are loaded once per tile).
+//     c, queries 4g+r -- exactly the A operand of  dV = P^T . dO  and
+//     dK = dS^T . Q  (v_mfma_f32_16x16x16_bf16, contraction over the 16
+//     queries; dO^T and Q^T fragments, the B operands, are loaded once per tile).
 // dQ partial sums of the four waves are added through LDS and written once.  dK
-// and dV tiles leave the wave as fp32 atomic adds into the key's rows (a key
-// belongs to many buckets), four consecutive floats per lane.
+// and dV tiles (keys on rows, d on columns) leave the wave as fp32 atomic adds
+// into the keys' rows (a key belongs to many buckets): per instruction and lane
+// group 16 consecutive floats of one row.
 //
 // Roofline: the atomic traffic, 2 * d * 4 bytes per gathered (item tile, key)
 // pair, on top of the forward's gather traffic.
@@ -234,22 +235,29 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
         pr[r] = key_ok ? __builtin_amdgcn_exp2f(fmaf(sN[r], scale2, -lse2q[r])) : 0.f;
         dsr[r] = pr[r] * (pN[r] - Dq[r]) * sm_scale;
       }
-      const bf16x4s pB = b_as_bf16x4(make_uint2(b_pack(pr[0], pr[1]), b_pack(pr[2], pr[3])));
-      const bf16x4s dsB = b_as_bf16x4(make_uint2(b_pack(dsr[0], dsr[1]), b_pack(dsr[2], dsr[3])));
-      float* dvrow = dVb + int64_t(kv.rk[kt]) * kBD + 4 * g;
-      float* dkrow = dKb + int64_t(kv.rk[kt]) * kBD + 4 * g;
+      // P and dS as the A operand (lane (g,c): row = key c, contraction = queries 4g..4g+3), dO^T and
+      // Q^T fragments as B: the output tile has keys on rows and d on columns, so that one atomic
+      // instruction covers, per lane group, 16 consecutive floats (a 64-byte line) of one key's row
+      const bf16x4s pA = b_as_bf16x4(make_uint2(b_pack(pr[0], pr[1]), b_pack(pr[2], pr[3])));
+      const bf16x4s dsA = b_as_bf16x4(make_uint2(b_pack(dsr[0], dsr[1]), b_pack(dsr[2], dsr[3])));
+      int64_t rowoff[4];
+      bool rok[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        rowoff[r] = int64_t(__shfl(kv.rk[kt], 4 * g + r)) * kBD + c;
+        rok[r] = kp0 + 16 * kt + 4 * g + r < cnt;
+      }
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        const f32x4 tv = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(b_as_bf16x4(doT[t]), pB, z, 0, 0, 0);
-        const f32x4 tk = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(b_as_bf16x4(qT[t]), dsB, z, 0, 0, 0);
-        if (key_ok) {
+        const f32x4 tv = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pA, b_as_bf16x4(doT[t]), z, 0, 0, 0);
+        const f32x4 tk = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(dsA, b_as_bf16x4(qT[t]), z, 0, 0, 0);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            unsafeAtomicAdd(dvrow + 16 * t + r, tv[r]);
-            unsafeAtomicAdd(dkrow + 16 * t + r, tk[r]);
+        for (int r = 0; r < 4; ++r)
+          if (rok[r]) {
+            unsafeAtomicAdd(dVb + rowoff[r] + 16 * t, tv[r]);
+            unsafeAtomicAdd(dKb + rowoff[r] + 16 * t, tk[r]);
           }
-        }
       }
     }
   };

@@ -6,9 +6,9 @@ All compute runs in hand-written HIP kernels reached through the C ABI of
 streams.  There is no CPU path.
 """
 from .hash_attention import attention_hash, attention_hash_varlen, attention_hash_varlen_backward  # noqa: F401
-from .memory import (Memory, MemoryBatch, compute_centroids, fit_projection, init_centroids, kmeans_spherical,  # noqa: F401
+from .memory import (Memory, MemoryBatch, calc_ref_centroids, compute_centroids, fit_projection, init_centroids, kmeans_spherical, learn_emb_proj,  # noqa: F401
                      merge, ring_attention_masked_backward, ring_attention_masked_forward, update_out_and_lse)
 
-__all__ = ["attention_hash", "attention_hash_varlen", "attention_hash_varlen_backward", "Memory", "MemoryBatch", "compute_centroids", "fit_projection",
-           "init_centroids", "kmeans_spherical", "merge", "ring_attention_masked_backward", "ring_attention_masked_forward",
+__all__ = ["attention_hash", "attention_hash_varlen", "attention_hash_varlen_backward", "Memory", "MemoryBatch", "calc_ref_centroids", "compute_centroids", "fit_projection",
+           "init_centroids", "kmeans_spherical", "learn_emb_proj", "merge", "ring_attention_masked_backward", "ring_attention_masked_forward",
            "update_out_and_lse"]

@@ -51,6 +51,7 @@ SIGNATURES = {
     "fm_l2_normalize": (c_int, [P, P, c_int64, c_int, c_float, c_int, P]),
     "fm_topk_mean": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_segment_mean": (c_int, [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
+    "fm_segment_sum": (c_int, [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_debug_force_generic": (None, [c_int]),
     "fm_debug_copy": (c_int, [P, P, c_int64, P]),
     "fm_debug_read": (c_int, [P, c_int64, P, P]),

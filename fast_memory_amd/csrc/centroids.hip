@@ -195,7 +195,47 @@ __global__ __launch_bounds__(256) void segment_mean_bf16_d128_kernel(
   }
 }
 
+
+// out[h,c,:] = sum of X[h, perm[...], :] over the segment's members, fp32, member order; empty -> 0.
+// One workgroup per (c, h); 16 groups of 16 lanes when a row is 16 chunks of 8 elements (bf16, d = 128),
+// else thread = dimension.
+template <typename T>
+__global__ __launch_bounds__(256) void segment_sum_kernel(const T* __restrict__ X, const int32_t* __restrict__ perm,
+                                                          const int32_t* __restrict__ seg_off,
+                                                          const int32_t* __restrict__ seg_cnt,
+                                                          float* __restrict__ out, int C, int N, int d) {
+  const int c = blockIdx.x, h = blockIdx.y, t = threadIdx.x;
+  const int64_t hc = int64_t(h) * C + c;
+  const int cnt = seg_cnt[hc];
+  const int32_t* mem = perm + seg_off[hc];
+  const T* xb = X + int64_t(h) * N * d;
+  float acc = 0.f;
+  for (int j = 0; j < cnt; ++j) {
+    const int row = min(max(mem[j], 0), N - 1);
+    if (t < d) acc += Elem<T>::load(xb + int64_t(row) * d + t);
+  }
+  if (t < d) out[hc * d + t] = acc;
+}
+
 }  // namespace fm
+
+extern "C" int fm_segment_sum(const void* X, const int32_t* perm, const int32_t* seg_off, const int32_t* seg_cnt,
+                              float* sum_out, int H, int C, int N, int d, int dtype, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG, "fm_segment_sum: H=%d C=%d N=%d d=%d",
+             H, C, N, d);
+  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_segment_sum: dtype=%d", dtype);
+  FM_REQUIRE(X && perm && seg_off && seg_cnt && sum_out, FM_ERR_ARG, "fm_segment_sum: null pointer");
+  FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_segment_sum: H > 65535");
+  dim3 grid = dim3(unsigned(C), unsigned(H));
+  if (dtype == FM_F32)
+    hipLaunchKernelGGL(segment_sum_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)X, perm,
+                       seg_off, seg_cnt, sum_out, C, N, d);
+  else
+    hipLaunchKernelGGL(segment_sum_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream), (const bf16_t*)X, perm,
+                       seg_off, seg_cnt, sum_out, C, N, d);
+  return launch_status("fm_segment_sum");
+}
 
 extern "C" int fm_l2_normalize(const void* X, void* Xn, int64_t rows, int d, float eps, int dtype,
                                void* stream) {

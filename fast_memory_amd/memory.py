@@ -121,6 +121,62 @@ def ring_attention_masked_forward(k_hashes, q_hashes, q, k, v, sm_scale, rank,
 
 
 # --------------------------------------------------------------------------
+@torch.no_grad()
+def calc_ref_centroids(q_self: torch.Tensor, k: torch.Tensor, topk: int = 128,
+                       workspace_bytes: int = 2 << 30) -> torch.Tensor:
+    """Drop-in for ``calc_ref_centroids`` (memory.py:428-456): the target of the learned projection.
+
+    For every query the ``topk`` keys with the largest scores ``q.k`` are found (value descending, key
+    index ascending; the reference's ``torch.topk`` leaves ties unspecified and ranks scores rounded to
+    q's dtype, here the fp32 scores are ranked); every key's centroid is the sum of the queries that
+    selected it, divided by ``topk`` and by its norm clamped at 1e-6.
+
+    :param q_self: ``[batch, n_heads, seq_len, d]``
+    :param k: ``[batch, k_heads, context_len, d]``
+    :return: ``[batch, k_heads, n_groups, context_len, d]`` in q's dtype
+    """
+    batch_size, n_heads, seq_len, d_qkv = q_self.shape
+    _, k_heads, context_len, _ = k.shape
+    n_groups = n_heads // k_heads
+    _topk = min(topk, context_len)
+    rows = batch_size * k_heads
+    qa = q_self.reshape(rows, n_groups * seq_len, d_qkv).contiguous()
+    top = ops.build_index(qa, k.reshape(rows, context_len, d_qkv).contiguous(), _topk)   # [rows, G*S, topk]
+    labels = top.reshape(rows * n_groups, seq_len * _topk)
+    X = q_self.reshape(rows * n_groups, seq_len, d_qkv).contiguous()
+    sums = torch.empty((rows * n_groups, context_len, d_qkv), dtype=torch.float32, device=q_self.device)
+    # the grouping's table is (blocks of 256 entries) x context_len ints per row: bound it
+    per_row = ((seq_len * _topk + 255) // 256) * context_len * 4
+    step = max(1, workspace_bytes // max(per_row, 1))
+    for r0 in range(0, rows * n_groups, step):
+        r1 = min(rows * n_groups, r0 + step)
+        g = ops.group_queries(labels[r0:r1].contiguous(), context_len)
+        members = torch.div(g.q_perm, _topk, rounding_mode="floor").to(torch.int32)   # entry -> its query
+        sums[r0:r1] = ops.segment_sum(X[r0:r1].contiguous(), members, g.bin_off, g.bin_count)
+    cent = sums / _topk
+    cent = cent / cent.norm(p=2, dim=-1, keepdim=True).clamp(min=1e-6)
+    return cent.to(q_self.dtype).reshape(batch_size, k_heads, n_groups, context_len, d_qkv)
+
+
+def learn_emb_proj(kq: torch.Tensor, q_self: torch.Tensor, k: torch.Tensor):
+    """Drop-in for ``learn_emb_proj`` (memory.py:459-484) without its logging: normalised ``kq`` and the
+    MSE between it and :func:`calc_ref_centroids`.
+
+    :param kq: ``[batch, context_len, n_heads * d]``
+    :return: ``(kq [batch, n_heads, context_len, d] normalised, loss)``"""
+    batch_size, n_heads, seq_len, d_qkv = q_self.shape
+    _, k_heads, context_len, _ = k.shape
+    n_groups = n_heads // k_heads
+    kq = kq.view(*kq.shape[:2], n_heads, d_qkv).permute(0, 2, 1, 3).contiguous()
+    kq = kq.reshape(batch_size, k_heads, n_groups, -1, d_qkv)
+    kq = kq / torch.norm(kq, p=2, dim=-1, keepdim=True).clamp(min=1e-6)
+    with torch.no_grad():
+        centroids = calc_ref_centroids(q_self, k)
+    assert list(kq.shape) == list(centroids.shape), f'{kq.shape} != {centroids.shape}'
+    return kq.reshape(batch_size, n_heads, -1, d_qkv), torch.nn.functional.mse_loss(kq, centroids)
+
+
+# --------------------------------------------------------------------------
 def ring_attention_masked_backward(k_hashes, q_hashes, h_idx, d_out, q, k, v, out, softmax_lse, sm_scale, rank):
     """Drop-in for ``ring_attention_masked_backward`` (memory.py:166-206) on one window of keys.
 

@@ -308,6 +308,19 @@ def segment_mean(X: torch.Tensor, groups: QueryGroups, prev: torch.Tensor) -> to
     return out
 
 
+def segment_sum(X: torch.Tensor, perm: torch.Tensor, seg_off: torch.Tensor, seg_cnt: torch.Tensor) -> torch.Tensor:
+    """fp32 sums of the rows of X [H,N,d] listed per segment: perm int32 row indices (flat, per h), seg_off /
+    seg_cnt [H,C] int32 -> [H,C,d] fp32 (the segmented form of scatter_add_, memory.py:449-450)."""
+    _dev(X, perm, seg_off, seg_cnt)
+    H, N, d = X.shape
+    C = seg_cnt.shape[-1]
+    assert perm.dtype == seg_off.dtype == seg_cnt.dtype == torch.int32
+    out = torch.empty((H, C, d), dtype=torch.float32, device=X.device)
+    check(_lib.load().fm_segment_sum(_p(X), _p(perm), _p(seg_off), _p(seg_cnt), _p(out), H, C, N, d, _dt(X),
+                                     _stream(X)))
+    return out
+
+
 def force_generic_kernels(on: bool) -> None:
     """Diagnostic switch: route attention through the generic kernels."""
     _lib.load().fm_debug_force_generic(int(on))

@@ -223,6 +223,14 @@ int fm_segment_mean(const void* X, const int32_t* perm, const int32_t* seg_off,
                     const int32_t* seg_cnt, const void* prev, void* cent_out, int H, int C, int N,
                     int d, int dtype, void* stream);
 
+/* ---- f2: scatter-add of rows onto index lists -------------------------------
+ * the segmented form of centroids.scatter_add_(...) in calc_ref_centroids
+ * (memory.py:449-450): sum_out[h,c,:] = sum of X[h, perm[j], :] over the members j
+ * of segment (h,c) (perm/seg_off/seg_cnt from fm_group_queries on the target
+ * indices), fp32, in member order; an empty segment gives zeros. */
+int fm_segment_sum(const void* X, const int32_t* perm, const int32_t* seg_off, const int32_t* seg_cnt,
+                   float* sum_out, int H, int C, int N, int d, int dtype, void* stream);
+
 /* Diagnostic: 1 routes the attention entry points through the generic kernels
  * (used by tests to compare the two implementations), 0 restores dispatch. */
 void fm_debug_force_generic(int on);

@@ -25,6 +25,7 @@ How each function is pinned (tests/test_oracle_*.py):
                         softmax over the same visible pairs, alone and as part
                         of a larger softmax (merged out / lse); the two
                         formulations (dense-masked, gather) against each other
+  calc_ref_centroids -- brute-force loops over (query, rank) on a tiny input
   update_out_and_lse -- closed form logaddexp / convex combination, split test
   local_attention    -- torch SDPA (math path) + torch.logsumexp.
                         PARITY UNPINNED against the reference: the reference
@@ -543,3 +544,28 @@ def kmeans_spherical(X: torch.Tensor, init: torch.Tensor, iters: int):
         labels = kmeans_assign(X, cent)
         cent = kmeans_update(X, labels, cent)
     return cent, labels
+
+
+
+# --------------------------------------------------------------------------
+# f2  target of the learned projection                         mem:428-456
+# --------------------------------------------------------------------------
+def calc_ref_centroids(q_self: torch.Tensor, k: torch.Tensor, topk: int = 128) -> torch.Tensor:
+    """mem:428-456 in fp64: scores ``q.k`` per (batch, kv head, group), the
+    ``min(topk, N)`` best keys per query (ties: lower key index, the rule of
+    :func:`argtopz`; the reference's ``torch.topk`` leaves them open), every
+    query scatter-added onto its keys (mem:449-450), divided by ``topk`` and by
+    the norm clamped at 1e-6.  Returns ``[B, H, G, N, d]`` fp64."""
+    B, n_heads, S, d = q_self.shape
+    _, H, N, _ = k.shape
+    G = n_heads // H
+    _topk = min(topk, N)
+    qa = q_self.double().reshape(B, H, G, S, d)
+    scores = torch.einsum('bhgid,bhjd->bhgij', qa, k.double())
+    best = argtopz(scores.reshape(-1, N), _topk).reshape(B, H, G, S, _topk)
+    cent = torch.zeros((B, H, G, N, d), dtype=torch.float64)
+    idx = best.reshape(B, H, G, S * _topk, 1).expand(-1, -1, -1, -1, d)
+    src = qa.unsqueeze(-2).expand(-1, -1, -1, -1, _topk, -1).reshape(B, H, G, S * _topk, d)
+    cent.scatter_add_(3, idx, src)
+    cent = cent / _topk
+    return cent / cent.norm(p=2, dim=-1, keepdim=True).clamp(min=1e-6)

@@ -534,6 +534,30 @@ def test_ring_attention_masked_backward_with_merged_result(ops):
     assert torch.allclose(dq.cpu().double(), rq, atol=2e-4, rtol=1e-4)
 
 
+# ------------------------------------------------------------------ f2 target of the learned projection
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_calc_ref_centroids(ops, dtype):
+    from fast_memory_amd import calc_ref_centroids, learn_emb_proj
+    g = gen(1600)
+    B, H, G, S, N, d = 1, 2, 2, 50, 700, 128 if dtype == torch.bfloat16 else 32
+    q = torch.randn(B, H * G, S, d, generator=g).to(dtype)
+    k = torch.randn(B, H, N, d, generator=g).to(dtype)
+    got = calc_ref_centroids(dev(q), dev(k), workspace_bytes=1 << 20)      # small table: several row chunks
+    assert got.shape == (B, H, G, N, d) and got.dtype == dtype
+    ref = O.calc_ref_centroids(q.float(), k.float())
+    diff = (got.float().cpu().double() - ref).abs().amax(-1)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    # a key whose score sits at a query's rank-128 boundary can flip on fp32-vs-fp64 rounding of that score
+    assert (diff <= tol).double().mean().item() > 0.995, (diff > tol).sum().item()
+    kq = torch.randn(B, N, H * G * d, generator=g).to(dtype)
+    kqn, loss = learn_emb_proj(dev(kq), dev(q), dev(k))
+    assert kqn.shape == (B, H * G, N, d)
+    kq_ref = kq.float().view(B, N, H * G, d).permute(0, 2, 1, 3).reshape(B, H, G, N, d)
+    kq_ref = kq_ref / kq_ref.norm(dim=-1, keepdim=True).clamp(min=1e-6)
+    ref_loss = torch.nn.functional.mse_loss(kq_ref.double(), ref).item()
+    assert abs(loss.item() - ref_loss) < (1e-5 if dtype == torch.float32 else 2e-3) * max(1.0, ref_loss)
+
+
 # ------------------------------------------------------------------ a1+a2 fused build
 def _clustered_keys(g, H, N, d, n_clusters=64, spread=0.5):
     cen = torch.randn(H, n_clusters, d, generator=g)

@@ -465,3 +465,27 @@ def test_kmeans_update_brute_force_and_empty_cluster():
     m0 = (X[0] + X[1]).double() / 2
     assert torch.allclose(new[0], m0 / m0.norm(), atol=1e-7)
     assert torch.allclose(new[2], prev[2].double())                 # empty cluster keeps its centroid
+
+
+def test_calc_ref_centroids_brute_force():
+    g = torch.Generator().manual_seed(123)
+    B, H, G, S, N, d, topk = 1, 2, 2, 7, 11, 4, 3
+    q = torch.randn(B, H * G, S, d, generator=g, dtype=torch.float64)
+    k = torch.randn(B, H, N, d, generator=g, dtype=torch.float64)
+    got = O.calc_ref_centroids(q, k, topk)
+    ref = torch.zeros(B, H, G, N, d, dtype=torch.float64)
+    for h in range(H):
+        for gg in range(G):
+            for i in range(S):
+                qi = q[0, h * G + gg, i]
+                sc = [(float(k[0, h, j] @ qi), j) for j in range(N)]
+                sc.sort(key=lambda t: (-t[0], t[1]))
+                for _, j in sc[:topk]:
+                    ref[0, h, gg, j] += qi
+    ref = ref / topk
+    nrm = ref.norm(dim=-1, keepdim=True)
+    ref = ref / nrm.clamp(min=1e-6)
+    assert torch.allclose(got, ref, atol=1e-12)
+    untouched = nrm.squeeze(-1) == 0
+    assert untouched.any() and (got[untouched] == 0).all()     # keys nobody selected stay zero
+

@@ -212,6 +212,24 @@ def main():
         fused_phases["filter_mfma_frac"] = fused_phases["filter_tflops"] / BF16_MFMA_PEAK_TFLOPS
         log(f"[bench] fused build phases (ms): {fused_phases}")
 
+    # extending the index by M new keys instead of rebuilding it (same lists as a rebuild over N+M keys)
+    append = None
+    if N >= Z and wl.k_local is not None:
+        idx_v, val_v = ops.build_index(A, wl.keys, Z, ws_bytes, return_values=True)
+        append = {}
+        for M in (1, wl.k_local.shape[1]):       # the local window's keys are the ones a memory takes in next
+            K_new = wl.k_local[:, :M].contiguous()
+            ms_copy, _ = timed(lambda: ops.index_append(A, K_new, N, idx_v, val_v, Z), reps=3, warm=1)
+            i2, v2 = idx_v.clone(), val_v.clone()
+            ops.index_append(A, K_new, N, i2, v2, Z, inplace=True)          # warm, on a copy of its own
+            i2.copy_(idx_v), v2.copy_(val_v)
+            ms_inpl, _ = timed(lambda: ops.index_append(A, K_new, N, i2, v2, Z, inplace=True), reps=1, warm=0)
+            append[f"M={M}"] = {"out_of_place_ms": ms_copy, "in_place_ms": ms_inpl,
+                               "rebuild_over_append": build_ms / ms_inpl}
+            del i2, v2
+        del idx_v, val_v
+        log(f"[bench] index append: {append}")
+
     # component kernels of the unfused build on one chunk of rows
     rows = min(C, max(1, min(512, ws_bytes // (N * 4))))
     Asub = A[:1, :rows].contiguous()
@@ -433,7 +451,7 @@ def main():
         "cpu_baseline": cpu,
         "index_build": {"keys_per_s": keys_per_s, "ms": build_ms, "keys": H * N, "path": build_path,
                         "fused_phases_ms": fused_phases, "unfused_parts": build_parts,
-                        "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters},
+                        "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters, "append": append},
         "query_path": query_path,
         "step_parts_ms": {"attention": attn_ms, **parts_ms},
         "backward": backward,

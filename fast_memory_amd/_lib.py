@@ -25,11 +25,11 @@ SIGNATURES = {
     "fm_last_error": (c_char_p, []),
     "fm_project": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int64, c_int, P]),
     "fm_argtopz_workspace": (c_size_t, [c_int64, c_int, c_int]),
-    "fm_argtopz_f32": (c_int, [P, c_int64, c_int, c_int64, c_int, P, P, c_size_t, P]),
+    "fm_argtopz_f32": (c_int, [P, c_int64, c_int, c_int64, c_int, P, P, P, c_size_t, P]),
     "fm_build_index_workspace": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int64]),
-    "fm_build_index": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P]),
+    "fm_build_index": (c_int, [P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P]),
     "fm_build_index_fused_workspace": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
-    "fm_build_index_fused": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P, P]),
+    "fm_build_index_fused": (c_int, [P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P, P]),
     "fm_qhash": (c_int, [P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_window_filter_workspace": (c_size_t, [c_int64]),
     "fm_window_filter": (c_int, [P, c_int64, c_int, c_int64, c_int64, P, P, P, P, c_size_t, P]),
@@ -51,6 +51,8 @@ SIGNATURES = {
     "fm_l2_normalize": (c_int, [P, P, c_int64, c_int, c_float, c_int, P]),
     "fm_topk_mean": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_segment_mean": (c_int, [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
+    "fm_index_append_workspace": (c_size_t, [c_int, c_int, c_int]),
+    "fm_index_append": (c_int, [P, P, c_int, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P, P]),
     "fm_segment_sum": (c_int, [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_debug_force_generic": (None, [c_int]),
     "fm_debug_copy": (c_int, [P, P, c_int64, P]),

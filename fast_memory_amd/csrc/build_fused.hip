@@ -37,7 +37,7 @@
 
 namespace fm {
 
-int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out,
+int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out, float* val_out,
                    const int32_t* row_map, const int32_t* n_rows_dev, hipStream_t st);
 
 constexpr int kFD = 128;          // head dimension the fused kernels are built for
@@ -407,7 +407,8 @@ struct CandRegs {
 // arg-top-Z kernel, on ~1.2 Zc register-resident candidates instead of the N-element row.
 __global__ __launch_bounds__(kSelThreads) void cand_select_kernel(
     const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, int n_writers, int cap_w, int Zc, int P,
-    int32_t* __restrict__ idx_out, int32_t* __restrict__ fail_rows, int32_t* __restrict__ n_fail) {
+    int32_t* __restrict__ idx_out, float* __restrict__ val_out, int32_t* __restrict__ fail_rows,
+    int32_t* __restrict__ n_fail) {
   extern __shared__ uint64_t buf[];
   __shared__ SelectShared sh;
   __shared__ CandCounts cc;
@@ -431,7 +432,7 @@ __global__ __launch_bounds__(kSelThreads) void cand_select_kernel(
   for (int r = 0; r < kCandRegs; ++r)
     if (r < src.n) src.e[r] = seg[t + r * T];
   const uint64_t cut = radix_select_cut(src, Zc, 6, sh);
-  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + row * Zc);
+  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + row * Zc, val_out ? val_out + row * Zc : nullptr);
 }
 
 // ---- phase 3 ---------------------------------------------------------------
@@ -496,8 +497,8 @@ extern "C" size_t fm_build_index_fused_workspace(int H, int C, int N, int d, int
   return p.total;
 }
 
-extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_out, int H, int C,
-                                    int N, int d, int Z, int dtype, void* ws, size_t ws_bytes,
+extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_out, float* val_out, int H,
+                                    int C, int N, int d, int Z, int dtype, void* ws, size_t ws_bytes,
                                     int32_t* status_dev, void* stream) {
   using namespace fm;
   FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && Z >= 1, FM_ERR_ARG, "fm_build_index_fused: H=%d C=%d N=%d Z=%d",
@@ -541,12 +542,12 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   const int P = next_pow2(Zc);
   FM_ALLOW_LDS(cand_select_kernel, sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");
   hipLaunchKernelGGL(cand_select_kernel, dim3(unsigned(rows)), dim3(kSelThreads), sort_lds_bytes(P), st, cand, cnt,
-                     p.n_writers, p.cap_w, Zc, P, idx_out, fail_rows, n_fail);
+                     p.n_writers, p.cap_w, Zc, P, idx_out, val_out, fail_rows, n_fail);
   // phase 3
   mark_phase(3, st);
   hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(ceil_div(N, 128)), kMaxRepair), dim3(256), 0,
                      st, (const bf16_t*)A, (const bf16_t*)K, fail_rows, n_fail, Yf, C, N, p.ldy);
-  rc = launch_argtopz(Yf, kMaxRepair, N, p.ldy, Zc, idx_out, fail_rows, n_fail, st);
+  rc = launch_argtopz(Yf, kMaxRepair, N, p.ldy, Zc, idx_out, val_out, fail_rows, n_fail, st);
   if (rc) return rc;
   hipLaunchKernelGGL(fused_status_kernel, dim3(1), dim3(1), 0, st, n_fail, status_dev);
   mark_phase(4, st);

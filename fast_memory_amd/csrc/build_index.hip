@@ -14,8 +14,8 @@ extern "C" size_t fm_build_index_workspace(int H, int C, int N, int d, int Z,
   return size_t(rows) * size_t(ldy) * sizeof(float);
 }
 
-extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, int H, int C, int N,
-                              int d, int Z, int dtype, void* ws, size_t ws_bytes, void* stream) {
+extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, float* val_out, int H, int C,
+                              int N, int d, int Z, int dtype, void* ws, size_t ws_bytes, void* stream) {
   using namespace fm;
   FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && d >= 1 && Z >= 1, FM_ERR_ARG,
              "fm_build_index: H=%d C=%d N=%d d=%d Z=%d", H, C, N, d, Z);
@@ -35,7 +35,8 @@ extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, in
       const char* Kh = static_cast<const char*>(K) + int64_t(h) * N * d * esz;
       int rc = fm_project(Ah, Kh, Y, 1, nc, N, d, ldy, dtype, stream);
       if (rc) return rc;
-      rc = fm_argtopz_f32(Y, nc, N, ldy, Z, idx_out + (int64_t(h) * C + c0) * Zc, nullptr, 0, stream);
+      rc = fm_argtopz_f32(Y, nc, N, ldy, Z, idx_out + (int64_t(h) * C + c0) * Zc,
+                          val_out ? val_out + (int64_t(h) * C + c0) * Zc : nullptr, nullptr, 0, stream);
       if (rc) return rc;
       c0 += nc;
     }

@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256) void window_compact_kernel(const int32_t* __re
   }
 }
 
-static int launch_fill(int32_t* p, int64_t n, int32_t v, hipStream_t st) {
+int launch_fill(int32_t* p, int64_t n, int32_t v, hipStream_t st) {
   if (n <= 0) return FM_OK;
   unsigned blocks = unsigned(std::min<int64_t>(ceil_div(n, 256), 4096));
   hipLaunchKernelGGL(fill_i32_kernel, dim3(blocks), dim3(256), 0, st, p, n, v);

@@ -17,22 +17,22 @@ namespace fm {
 // b and writes output row row_map[b], and exits if b >= min(*n_rows_dev, grid).
 __global__ __launch_bounds__(kSelThreads) void argtopz_kernel(
     const float* __restrict__ Y, int N, int64_t ldy, int Zc, int P, int32_t* __restrict__ idx_out,
-    const int32_t* __restrict__ row_map, const int32_t* __restrict__ n_rows_dev) {
+    float* __restrict__ val_out, const int32_t* __restrict__ row_map, const int32_t* __restrict__ n_rows_dev) {
   extern __shared__ uint64_t buf[];  // P composites
   __shared__ SelectShared sh;
   if (n_rows_dev && int(blockIdx.x) >= *n_rows_dev) return;
   const int64_t out_row = row_map ? row_map[blockIdx.x] : int64_t(blockIdx.x);
   DenseRow src{Y + int64_t(blockIdx.x) * ldy, N};
   const uint64_t cut = radix_select_cut(src, Zc, 6, sh);
-  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + out_row * Zc);
+  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + out_row * Zc, val_out ? val_out + out_row * Zc : nullptr);
 }
 
-int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out,
+int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out, float* val_out,
                    const int32_t* row_map, const int32_t* n_rows_dev, hipStream_t st) {
   const int P = next_pow2(Zc);
   FM_ALLOW_LDS(argtopz_kernel, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
   hipLaunchKernelGGL(argtopz_kernel, dim3(unsigned(rows)), dim3(kSelThreads),
-                     sort_lds_bytes(P), st, Y, N, ldy, Zc, P, idx_out, row_map, n_rows_dev);
+                     sort_lds_bytes(P), st, Y, N, ldy, Zc, P, idx_out, val_out, row_map, n_rows_dev);
   return launch_status("argtopz");
 }
 
@@ -41,7 +41,7 @@ int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int
 extern "C" size_t fm_argtopz_workspace(int64_t, int, int) { return 0; }
 
 extern "C" int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, int Z,
-                              int32_t* idx_out, void* ws, size_t ws_bytes, void* stream) {
+                              int32_t* idx_out, float* val_out, void* ws, size_t ws_bytes, void* stream) {
   using namespace fm;
   (void)ws;
   (void)ws_bytes;
@@ -54,5 +54,5 @@ extern "C" int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, 
   const int Zc = Z < N ? Z : N;
   FM_REQUIRE(Zc <= FM_MAX_Z, FM_ERR_UNSUPPORTED, "fm_argtopz_f32: min(Z,N)=%d exceeds FM_MAX_Z=%d",
              Zc, FM_MAX_Z);
-  return launch_argtopz(Y, rows, N, ldy, Zc, idx_out, nullptr, nullptr, as_stream(stream));
+  return launch_argtopz(Y, rows, N, ldy, Zc, idx_out, val_out, nullptr, nullptr, as_stream(stream));
 }

@@ -101,7 +101,7 @@ __device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int
 // (load 16, up to four stages, store 16) replaces up to four passes of the plain
 // network: 29 passes instead of 105 at P = 16384.
 __device__ __forceinline__ int sort_phys(int e) { return e + (e >> 4); }
-static inline size_t sort_lds_bytes(int P) { return size_t(P + (P >> 4) + 1) * sizeof(uint64_t); }
+__host__ __device__ static inline size_t sort_lds_bytes(int P) { return size_t(P + (P >> 4) + 1) * sizeof(uint64_t); }
 
 // The 16 keys of a thread as separate low and high words: the compare-exchange below works on
 // 32-bit registers.
@@ -267,12 +267,13 @@ __device__ __forceinline__ void bitonic_sort_desc(uint64_t* buf, int logP) {
 }
 
 // Collects the composites >= cut (at most P) into buf, pads to P with zeros,
-// sorts descending and writes the first Zc indices to out.  buf holds
-// sort_lds_bytes(P) bytes.
+// sorts descending and writes the first Zc indices to out (and, if val_out is
+// given, their values: -0 reads back as +0).  buf holds sort_lds_bytes(P) bytes.
 template <typename Source>
 __device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, int Zc, int P,
                                                    uint64_t* buf, SelectShared& sh,
-                                                   int32_t* __restrict__ out) {
+                                                   int32_t* __restrict__ out,
+                                                   float* __restrict__ val_out = nullptr) {
   const int tid = threadIdx.x;
   if (tid == 0) sh.cnt = 0;
   __syncthreads();
@@ -286,7 +287,11 @@ __device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, in
   for (int i = Zc + tid; i < P; i += kSelThreads) buf[sort_phys(i)] = 0;
   __syncthreads();
   bitonic_sort_desc(buf, 31 - __clz(P));
-  for (int i = tid; i < Zc; i += kSelThreads) out[i] = int32_t(0xffffffffu - uint32_t(buf[sort_phys(i)]));
+  for (int i = tid; i < Zc; i += kSelThreads) {
+    const uint64_t c = buf[sort_phys(i)];
+    out[i] = int32_t(0xffffffffu - uint32_t(c));
+    if (val_out) val_out[i] = key_to_float(uint32_t(c >> 32));
+  }
 }
 
 // Dense fp32 row as a source; 128-bit loads on the aligned body, kUnroll of

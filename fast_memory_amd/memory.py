@@ -209,18 +209,66 @@ class Memory:
     (``merge`` / ``update_out_and_lse``).
     """
 
-    def __init__(self, keys: torch.Tensor, values: torch.Tensor, A: torch.Tensor, bucket_idx: torch.Tensor):
-        self.keys, self.values, self.A, self.bucket_idx = keys, values, A, bucket_idx
-        H, C, Z = bucket_idx.shape
-        self.bucket_cnt = torch.full((H, C), Z, dtype=torch.int32, device=keys.device)
-        self.bucket_off = (torch.arange(H * C, dtype=torch.int64, device=keys.device) * Z).reshape(H, C)
+    def __init__(self, keys: torch.Tensor, values: torch.Tensor, A: torch.Tensor, bucket_idx: torch.Tensor,
+                 bucket_val: Optional[torch.Tensor] = None, Z: Optional[int] = None):
+        self.keys, self.values, self.A = keys, values, A
+        self.Z = int(Z) if Z is not None else bucket_idx.shape[2]       # capacity; lists are shorter while N < Z
+        self._set_lists(bucket_idx, bucket_val)
+
+    def _set_lists(self, bucket_idx: torch.Tensor, bucket_val: Optional[torch.Tensor]):
+        self.bucket_idx, self.bucket_val = bucket_idx, bucket_val
+        H, C, L = bucket_idx.shape
+        dev = bucket_idx.device
+        self.bucket_cnt = torch.full((H, C), L, dtype=torch.int32, device=dev)
+        self.bucket_off = (torch.arange(H * C, dtype=torch.int64, device=dev) * L).reshape(H, C)
 
     @classmethod
     def build(cls, keys: torch.Tensor, values: torch.Tensor, A: torch.Tensor, Z: int,
-              workspace_bytes: int = 8 << 30) -> "Memory":
+              workspace_bytes: int = 8 << 30, keep_values: bool = False) -> "Memory":
+        """``keep_values`` also stores the projections of the listed keys (4 bytes per list entry), which
+        :meth:`append` needs."""
         keys, values, A = keys.contiguous(), values.contiguous(), A.contiguous()
         assert keys.shape == values.shape and A.shape[0] == keys.shape[0] and A.shape[2] == keys.shape[2]
-        return cls(keys, values, A, ops.build_index(A, keys, Z, workspace_bytes))
+        if keep_values:
+            idx, val = ops.build_index(A, keys, Z, workspace_bytes, return_values=True)
+            return cls(keys, values, A, idx, val, Z)
+        return cls(keys, values, A, ops.build_index(A, keys, Z, workspace_bytes), None, Z)
+
+    def append(self, new_keys: torch.Tensor, new_values: torch.Tensor, workspace_bytes: int = 8 << 30) -> "Memory":
+        """Add keys/values ``[H,M,d]`` at the end of the memory and bring the bucket lists to what a rebuild
+        over all keys would give, without projecting the old keys again (the reference rebuilds on every
+        forward, memory.py:252-278).  Needs ``build(..., keep_values=True)``.  Returns ``self``."""
+        assert self.bucket_val is not None, "Memory.build(..., keep_values=True) is needed to append"
+        new_keys, new_values = new_keys.contiguous(), new_values.contiguous()
+        H, M, d = new_keys.shape
+        assert new_values.shape == new_keys.shape and H == self.keys.shape[0] and d == self.keys.shape[2]
+        n_old = self.keys.shape[1]
+        full = n_old >= self.Z        # full lists are updated in place: buckets that take no new key stay untouched
+        res = ops.index_append(self.A, new_keys, n_old, self.bucket_idx, self.bucket_val, self.Z, inplace=full)
+        self.keys = torch.cat([self.keys, new_keys], dim=1)
+        self.values = torch.cat([self.values, new_values], dim=1)
+        if res is None:       # a bucket took more new keys than the merge holds: rebuild
+            res = ops.build_index(self.A, self.keys, self.Z, workspace_bytes, return_values=True)
+        if res[0] is not self.bucket_idx:
+            self._set_lists(*res)
+        return self
+
+    def save(self, path: str) -> None:
+        """Write the memory (keys, values, A, lists and, if kept, their values) as a safetensors file."""
+        from safetensors.torch import save_file
+        t = {"keys": self.keys, "values": self.values, "A": self.A, "bucket_idx": self.bucket_idx}
+        if self.bucket_val is not None:
+            t["bucket_val"] = self.bucket_val
+        save_file({k: v.contiguous().cpu() for k, v in t.items()}, path, metadata={"Z": str(self.Z), "format": "1"})
+
+    @classmethod
+    def load(cls, path: str, device="cuda") -> "Memory":
+        """Read a memory written by :meth:`save`; no index is rebuilt."""
+        from safetensors import safe_open
+        with safe_open(path, framework="pt", device="cpu") as f:
+            meta = f.metadata() or {}
+            t = {k: f.get_tensor(k).to(device) for k in f.keys()}
+        return cls(t["keys"], t["values"], t["A"], t["bucket_idx"], t.get("bucket_val"), int(meta.get("Z", 0)) or None)
 
     @property
     def n_buckets(self) -> int:

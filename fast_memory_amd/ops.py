@@ -51,24 +51,27 @@ def project(A: torch.Tensor, K: torch.Tensor) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------- a2
-def argtopz(Y: torch.Tensor, Z: int) -> torch.Tensor:
-    """Indices of the min(Z,N) largest entries per row: value desc, index asc (memory.py:273)."""
+def argtopz(Y: torch.Tensor, Z: int, return_values: bool = False):
+    """Indices of the min(Z,N) largest entries per row: value desc, index asc (memory.py:273);
+    with ``return_values`` also the values in that order."""
     _dev(Y)
     assert Y.dtype == torch.float32
     N = Y.shape[-1]
     rows = Y.numel() // N if N else 0
     Zc = min(int(Z), N)
     out = torch.empty((*Y.shape[:-1], Zc), dtype=torch.int32, device=Y.device)
-    check(_lib.load().fm_argtopz_f32(_p(Y), rows, N, N, int(Z), _p(out), None, 0, _stream(Y)))
-    return out
+    vals = torch.empty(out.shape, dtype=torch.float32, device=Y.device) if return_values else None
+    check(_lib.load().fm_argtopz_f32(_p(Y), rows, N, N, int(Z), _p(out), _p(vals), None, 0, _stream(Y)))
+    return (out, vals) if return_values else out
 
 
 last_build_info = {}
 
 
 def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int = 8 << 30,
-                fused: Optional[bool] = None) -> torch.Tensor:
-    """Bucket lists [H,C,min(Z,N)] int32 (memory.py:260-278 on one device).
+                fused: Optional[bool] = None, return_values: bool = False):
+    """Bucket lists [H,C,min(Z,N)] int32 (memory.py:260-278 on one device); with ``return_values`` also
+    the fp32 projections of the listed keys (what an index needs to be extended later).
 
     ``fused=None`` takes the fused build (no Y in memory) where the shape is
     eligible and the unfused one otherwise; both give identical lists.  The
@@ -80,25 +83,59 @@ def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int =
     assert K.shape[0] == H and K.shape[2] == d and A.dtype == K.dtype
     lib = _lib.load()
     out = torch.empty((H, C, min(int(Z), N)), dtype=torch.int32, device=A.device)
+    vals = torch.empty(out.shape, dtype=torch.float32, device=A.device) if return_values else None
+    done = lambda: (out, vals) if return_values else out
     fws = lib.fm_build_index_fused_workspace(H, C, N, d, int(Z), _dt(A)) if fused is not False else 0
     if fused and not fws:
         raise ValueError("fused index build: shape not eligible (bf16, d=128, N>=65536, 64<=Z<=N/8)")
     if fws:
         ws = _ws(fws, A)
         status = torch.empty(2, dtype=torch.int32, device=A.device)
-        check(lib.fm_build_index_fused(_p(A), _p(K), _p(out), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(),
+        check(lib.fm_build_index_fused(_p(A), _p(K), _p(out), _p(vals), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(),
                                        _p(status), _stream(A)))
         repaired, unresolved = status.tolist()          # one 8-byte read-back per build
         last_build_info.update(path="fused", rows_repaired=repaired, rows_unresolved=unresolved)
         del ws
         if unresolved == 0:
-            return out
+            return done()
     last_build_info.update(path="unfused")
     full = lib.fm_build_index_workspace(H, C, N, d, int(Z), C)
     one = lib.fm_build_index_workspace(H, C, N, d, int(Z), 1)
     ws = _ws(max(one, min(full, int(workspace_bytes))), A)
-    check(lib.fm_build_index(_p(A), _p(K), _p(out), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(), _stream(A)))
-    return out
+    check(lib.fm_build_index(_p(A), _p(K), _p(out), _p(vals), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(),
+                             _stream(A)))
+    return done()
+
+
+def index_append(A: torch.Tensor, K_new: torch.Tensor, n_old: int, idx: torch.Tensor, val: torch.Tensor, Z: int,
+                 inplace: bool = False):
+    """Merge M new keys (global indices n_old..n_old+M-1) into bucket lists ``idx`` / ``val``
+    [H,C,min(Z,n_old)]: the lists a rebuild over all keys would give (memory.py:252-278 rebuilds).
+    Returns ``(idx, val)`` [H,C,min(Z,n_old+M)], or ``None`` when a bucket took more new keys than the
+    merge buffers hold (rebuild then).  ``inplace`` (full lists only) updates ``idx`` / ``val`` themselves
+    and touches only the buckets that take a new key; after ``None`` they are damaged."""
+    _dev(A, K_new, idx, val)
+    H, C, d = A.shape
+    _, M, _ = K_new.shape
+    assert K_new.shape[0] == H and K_new.shape[2] == d and A.dtype == K_new.dtype
+    L_in = min(int(Z), int(n_old))
+    assert idx.shape == (H, C, L_in) and val.shape == (H, C, L_in)
+    assert idx.dtype == torch.int32 and val.dtype == torch.float32 and idx.is_contiguous() and val.is_contiguous()
+    L_out = min(int(Z), int(n_old) + M)
+    lib = _lib.load()
+    if inplace:
+        assert L_in == L_out, "in place needs full lists (n_old >= Z)"
+        idx2, val2 = idx, val
+    else:
+        idx2 = torch.empty((H, C, L_out), dtype=torch.int32, device=A.device)
+        val2 = torch.empty((H, C, L_out), dtype=torch.float32, device=A.device)
+    ws = _ws(lib.fm_index_append_workspace(H, C, M), A)
+    status = torch.empty(1, dtype=torch.int32, device=A.device)
+    check(lib.fm_index_append(_p(A), _p(K_new.contiguous()), int(n_old), M, _p(idx), _p(val), _p(idx2), _p(val2), H, C,
+                              int(Z), d, _dt(A), _p(ws), ws.numel(), _p(status), _stream(A)))
+    if int(status.item()) != 0:
+        return None
+    return idx2, val2
 
 
 # --------------------------------------------------------------------- a3

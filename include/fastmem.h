@@ -63,19 +63,22 @@ int fm_project(const void* A, const void* K, float* Y, int H, int C, int N, int 
  * replaces torch.topk at memory.py:273 / triton_kernel.py:278.  Output row r =
  * the min(Z,N) indices of the largest entries of Y[r,:], ordered by value
  * descending then index ascending (the first Z entries of a stable descending
- * sort; -0 == +0; NaN is the largest).  idx_out is [rows, min(Z,N)] int32. */
+ * sort; -0 == +0; NaN is the largest).  idx_out is [rows, min(Z,N)] int32;
+ * val_out (may be NULL) receives the selected values in the same order (-0 as
+ * +0): the lists' values are what fm_index_append needs to extend an index. */
 size_t fm_argtopz_workspace(int64_t rows, int N, int Z);
 int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, int Z, int32_t* idx_out,
-                   void* ws, size_t ws_bytes, void* stream);
+                   float* val_out, void* ws, size_t ws_bytes, void* stream);
 
 /* ---- a1+a2: index build without handing Y to the caller ---------------------
- * memory.py:260-278 on one device.  idx_out [H,C,min(Z,N)] int32.  The
+ * memory.py:260-278 on one device.  idx_out [H,C,min(Z,N)] int32, val_out (may
+ * be NULL) the projections of the listed keys, same shape, fp32.  The
  * workspace holds fp32 projection rows for as many (head,bucket) rows as fit;
  * any size from fm_build_index_workspace(...,1) up is accepted and larger ones
  * mean fewer passes. */
 size_t fm_build_index_workspace(int H, int C, int N, int d, int Z, int64_t rows_per_pass);
-int fm_build_index(const void* A, const void* K, int32_t* idx_out, int H, int C, int N, int d,
-                   int Z, int dtype, void* ws, size_t ws_bytes, void* stream);
+int fm_build_index(const void* A, const void* K, int32_t* idx_out, float* val_out, int H, int C, int N,
+                   int d, int Z, int dtype, void* ws, size_t ws_bytes, void* stream);
 
 /* ---- a1+a2 fused: the same lists without ever writing Y to memory ------------
  * (memory.py:260-278; the selection sees exactly the fp32 values fm_project
@@ -87,8 +90,8 @@ int fm_build_index(const void* A, const void* K, int32_t* idx_out, int H, int C,
  * receives {rows repaired, rows left unresolved}; if the second is non-zero the
  * caller must rebuild with fm_build_index. */
 size_t fm_build_index_fused_workspace(int H, int C, int N, int d, int Z, int dtype);
-int fm_build_index_fused(const void* A, const void* K, int32_t* idx_out, int H, int C, int N, int d,
-                         int Z, int dtype, void* ws, size_t ws_bytes, int32_t* status_dev,
+int fm_build_index_fused(const void* A, const void* K, int32_t* idx_out, float* val_out, int H, int C,
+                         int N, int d, int Z, int dtype, void* ws, size_t ws_bytes, int32_t* status_dev,
                          void* stream);
 
 /* ---- a3: query hash  h_q = argmax_c A[h,c,:].q  (first maximum wins) ---------
@@ -222,6 +225,28 @@ int fm_topk_mean(const void* Xn, const int32_t* top_idx, void* A_out, int C, int
 int fm_segment_mean(const void* X, const int32_t* perm, const int32_t* seg_off,
                     const int32_t* seg_cnt, const void* prev, void* cent_out, int H, int C, int N,
                     int d, int dtype, void* stream);
+
+/* ---- f3: extending an index by new keys -----------------------------------
+ * The reference rebuilds the bucket lists from all keys on every forward
+ * (memory.py:252-278); this merges M new keys (global indices n_old ..
+ * n_old+M-1) into existing lists, with the result a rebuild over all n_old+M
+ * keys would give, in O(Z + M) per bucket.
+ *   A [H,C,d], K_new [H,M,d]
+ *   idx_in, val_in  [H,C,min(Z,n_old)]      lists and their projections (val_out of
+ *                                            the build or of an earlier append)
+ *   idx_out, val_out [H,C,min(Z,n_old+M)]   either separate buffers, or exactly
+ *                                            idx_in and val_in (in place; full lists
+ *                                            only, n_old >= Z): a bucket that takes no
+ *                                            new key is then not touched, so a few new
+ *                                            keys cost almost no memory traffic
+ *   status_dev (device, 1 int)               number of rows that accepted more new keys
+ *                                            than the merge holds (8192): if non-zero the lists written are
+ *                                            incomplete (in place: damaged), rebuild.
+ * The workspace holds the fp32 projections of the new keys. */
+size_t fm_index_append_workspace(int H, int C, int M);
+int fm_index_append(const void* A, const void* K_new, int n_old, int M, const int32_t* idx_in,
+                    const float* val_in, int32_t* idx_out, float* val_out, int H, int C, int Z, int d,
+                    int dtype, void* ws, size_t ws_bytes, int32_t* status_dev, void* stream);
 
 /* ---- f2: scatter-add of rows onto index lists -------------------------------
  * the segmented form of centroids.scatter_add_(...) in calc_ref_centroids

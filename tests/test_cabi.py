@@ -36,7 +36,7 @@ def test_version_and_error_string():
 
 def test_argument_errors_are_status_codes():
     lib = _lib.load()
-    assert lib.fm_argtopz_f32(None, 4, 0, 0, 1, None, None, 0, None) == 1        # N = 0
+    assert lib.fm_argtopz_f32(None, 4, 0, 0, 1, None, None, None, 0, None) == 1  # N = 0
     assert b"fm_argtopz_f32" in lib.fm_last_error()
     assert lib.fm_project(None, None, None, 1, 1, 1, 1000, 1, 0, None) == 1      # d > FM_MAX_D
     assert lib.fm_qhash(None, None, None, None, 1, 1, 1, 8, 7, None) == 1        # bad dtype

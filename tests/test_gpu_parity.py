@@ -558,6 +558,68 @@ def test_calc_ref_centroids(ops, dtype):
     assert abs(loss.item() - ref_loss) < (1e-5 if dtype == torch.float32 else 2e-3) * max(1.0, ref_loss)
 
 
+# ------------------------------------------------------------------ f3 persistent memory, incremental append
+@pytest.mark.parametrize("dtype,H,C,N0,M,Z,d", [
+    (torch.float32, 2, 9, 500, 77, 64, 32),
+    (torch.bfloat16, 2, 20, 3000, 1000, 256, 128),
+    (torch.bfloat16, 1, 6, 40, 30, 64, 128),              # the lists are not full yet: they grow, then fill
+    (torch.bfloat16, 1, 4, 2000, 9000, 8192, 128),        # more new keys than old ones, long lists
+])
+def test_append_equals_rebuild(ops, dtype, H, C, N0, M, Z, d, tmp_path):
+    from fast_memory_amd import Memory
+    g = gen(1700 + M)
+    K = torch.randn(H, N0 + 2 * M, d, generator=g).to(dtype)
+    K[:, N0 + 3] = K[:, 5]                                   # a new key that ties with an old one: the old one wins
+    V = torch.randn(H, N0 + 2 * M, d, generator=g).to(dtype)
+    A = torch.randn(H, C, d, generator=g).to(dtype)
+    Kd, Vd, Ad = dev(K, V, A)
+    mem = Memory.build(Kd[:, :N0], Vd[:, :N0], Ad, Z, keep_values=True)
+    Y0 = ops.project(Ad, Kd[:, :N0].contiguous())
+    assert torch.equal(mem.bucket_val, torch.gather(Y0, 2, mem.bucket_idx.long()) + 0.0)   # the values are Y's
+    for step in range(2):                                    # two appends in a row
+        n1 = N0 + (step + 1) * M
+        before = mem.bucket_idx
+        mem.append(Kd[:, n1 - M:n1], Vd[:, n1 - M:n1])
+        assert (mem.bucket_idx is before) == (n1 - M >= Z)      # full lists are updated in place
+        ref = Memory.build(Kd[:, :n1], Vd[:, :n1], Ad, Z, keep_values=True)
+        assert torch.equal(mem.bucket_idx, ref.bucket_idx), f"append {step}: lists differ from a rebuild"
+        assert torch.equal(mem.bucket_val, ref.bucket_val)
+        assert torch.equal(mem.keys, Kd[:, :n1]) and torch.equal(mem.bucket_cnt, ref.bucket_cnt)
+    # and the oracle on the final state
+    Y = ops.project(Ad, Kd).cpu()
+    assert torch.equal(mem.bucket_idx.cpu().long(), O.argtopz(Y, Z))
+    # persistence: a saved and reloaded memory answers queries bit-identically
+    path = str(tmp_path / "mem.safetensors")
+    mem.save(path)
+    mem2 = Memory.load(path, "cuda")
+    assert mem2.Z == Z and torch.equal(mem2.bucket_idx, mem.bucket_idx) and torch.equal(mem2.bucket_val, mem.bucket_val)
+    q = dev(torch.randn(H, 33, d, generator=g).to(dtype))
+    o1, l1 = mem.attend(q, d ** -0.5)
+    o2, l2 = mem2.attend(q, d ** -0.5)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+
+
+def test_append_falls_back_to_rebuild_when_a_bucket_takes_too_many(ops):
+    from fast_memory_amd import Memory
+    g = gen(1750)
+    H, C, N0, M, Z, d = 1, 3, 20000, 12000, 16384, 128
+    K = (torch.randn(H, N0 + M, d, generator=g) * 0.1)
+    A = torch.randn(H, C, d, generator=g)
+    K[0, N0:] += A[0, 1] / A[0, 1].norm() * 3.0            # every new key lands at the top of bucket 1
+    K, A = K.to(torch.bfloat16), A.to(torch.bfloat16)
+    V = torch.zeros_like(K)
+    Kd, Vd, Ad = dev(K, V, A)
+    mem = Memory.build(Kd[:, :N0], Vd[:, :N0], Ad, Z, keep_values=True)
+    assert ops.index_append(Ad, Kd[:, N0:].contiguous(), N0, mem.bucket_idx, mem.bucket_val, Z) is None
+    snap = mem.bucket_idx.clone()
+    mem_b = Memory.build(Kd[:, :N0 - 1], Vd[:, :N0 - 1], Ad, Z, keep_values=True)
+    mem_b.append(Kd[:, N0 - 1:N0], Vd[:, N0 - 1:N0])                 # one key, in place: almost every bucket untouched
+    assert torch.equal(mem_b.bucket_idx, snap) and torch.equal(mem_b.bucket_val, mem.bucket_val)
+    mem.append(Kd[:, N0:], Vd[:, N0:])
+    ref = ops.build_index(Ad, Kd, Z)
+    assert torch.equal(mem.bucket_idx, ref)
+
+
 # ------------------------------------------------------------------ a1+a2 fused build
 def _clustered_keys(g, H, N, d, n_clusters=64, spread=0.5):
     cen = torch.randn(H, n_clusters, d, generator=g)

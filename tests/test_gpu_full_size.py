@@ -1,0 +1,199 @@
+"""The benchmark configurations at their full sizes.  The CPU oracle cannot
+finish these in seconds, so whole results are checked through properties that
+hold at any size (lists: range, uniqueness, order, tie rule, agreement with the
+library's own list values; attention: LSE bounds, equivariance under a
+permutation of the queries, the split test of the merge), and samples of rows
+and queries are checked against the definition: a stable descending sort for the
+bucket lists (bit-exact), the oracle's fp64 gather attention for outputs (the
+tolerances of the parity tests).  Config 2 is small enough for the oracle to
+check every list and every query."""
+import math
+
+import pytest
+import torch
+
+from oracle import fm_oracle as O
+from tests.util import BF16_ATOL, BF16_RTOL, LSE_ATOL, assert_attn_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from fast_memory_amd import ops as _ops
+    from fast_memory_amd import _lib
+    _lib.load()
+    assert torch.cuda.is_available()
+    return _ops
+
+
+def check_lists_whole(idx, val, N):
+    """Properties of every list: indices in range and distinct, values descending, ties by ascending index."""
+    assert idx.dtype == torch.int32 and int(idx.min()) >= 0 and int(idx.max()) < N
+    rows = idx.reshape(-1, idx.shape[-1])
+    srt = torch.sort(rows, dim=1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all()), "an index appears twice in a list"
+    v = val.reshape(rows.shape)
+    assert bool((v[:, 1:] <= v[:, :-1]).all()), "list values are not descending"
+    tie = v[:, 1:] == v[:, :-1]
+    assert bool((rows[:, 1:][tie] > rows[:, :-1][tie]).all()), "equal values are not in ascending index order"
+
+
+def check_lists_sampled(ops, A, keys, idx, val, Z, rows_per_head=4, seed=0):
+    """Sampled (head, bucket) rows against the definition: the first Z entries of a stable descending sort
+    of the row of Y (bit-exact), with the list's values equal to Y at the listed keys; Y itself against
+    fp64 dot products."""
+    H, C, d = A.shape
+    g = torch.Generator().manual_seed(seed)
+    for h in range(H):
+        rows = torch.randperm(C, generator=g)[:rows_per_head].to(A.device)
+        Y = ops.project(A[h:h + 1, rows].contiguous(), keys[h:h + 1].contiguous())[0]          # [r, N] fp32
+        ref = torch.sort(Y, dim=1, descending=True, stable=True)
+        assert torch.equal(idx[h, rows].long(), ref.indices[:, :Z]), f"head {h}: list differs from the stable sort"
+        assert torch.equal(val[h, rows], ref.values[:, :Z] + 0.0)
+        cols = torch.randint(0, keys.shape[1], (64,), generator=g).to(A.device)
+        exact = A[h, rows].double() @ keys[h, cols].double().T
+        assert torch.allclose(Y[:, cols].double(), exact, atol=1e-4, rtol=1e-5)
+
+
+def oracle_on_sample(q_sel, buckets, lists_h, K_h, V_h, scale):
+    """fp64 gather attention of a few queries of one head: the listed keys of each query's bucket are copied
+    out, so the oracle sees a small problem with the same arithmetic (one bucket per sampled query)."""
+    n, Z = q_sel.shape[0], lists_h.shape[1]
+    ids = lists_h[buckets].long()                                   # [n, Z]
+    Ks, Vs = K_h[ids.reshape(-1)].cpu(), V_h[ids.reshape(-1)].cpu()  # [n*Z, d]
+    k_hashes = torch.arange(n * Z)
+    return O.hashed_attention_gather(q_sel.cpu()[None], Ks[None], Vs[None], k_hashes, torch.full((1, n), Z),
+                                     torch.arange(n)[None], scale)
+
+
+def check_attention_sampled(mem, q, qh, out, lse, scale, per_head=12, seed=1):
+    H, Sq, d = q.shape
+    g = torch.Generator().manual_seed(seed)
+    for h in range(H):
+        sel = torch.randperm(Sq, generator=g)[:per_head].to(q.device)
+        ro, rl = oracle_on_sample(q[h, sel], qh[h, sel].long(), mem.bucket_idx[h], mem.keys[h], mem.values[h], scale)
+        assert_attn_close(out[h, sel][None], lse[h, sel][None], ro, rl, q.dtype, f"head {h} sampled queries")
+        # max_j s_j <= lse <= max_j s_j + ln Z
+        ids = mem.bucket_idx[h][qh[h, sel].long()].long()
+        s = torch.einsum("nd,nzd->nz", q[h, sel].double(), mem.keys[h][ids].double()) * scale
+        smax = s.max(dim=1).values
+        l = lse[h, sel].double()
+        assert bool((l >= smax - LSE_ATOL).all()) and bool((l <= smax + math.log(ids.shape[1]) + LSE_ATOL).all())
+
+
+def test_config2_prefill_every_list_and_query_against_the_oracle(ops):
+    from fast_memory_amd import Memory, fit_projection, synth
+    cfg = synth.CONFIGS["c2"]
+    wl = synth.make_workload(cfg, "cuda")
+    A = fit_projection(wl.keys, cfg.C, iters=cfg.kmeans_iters)
+    assert torch.allclose(A.float().norm(dim=-1), torch.ones(cfg.H, cfg.C, device="cuda"), atol=1e-2)
+    mem = Memory.build(wl.keys, wl.values, A, cfg.Z, keep_values=True)
+    check_lists_whole(mem.bucket_idx, mem.bucket_val, cfg.N)
+    Y = ops.project(A, wl.keys).cpu()
+    assert torch.equal(mem.bucket_idx.cpu().long(), O.argtopz(Y, cfg.Z))
+    qh, sc = ops.qhash(A, wl.queries, return_scores=True)
+    assert torch.equal(qh.cpu().long(), O.argmax_first(sc.cpu()))
+    scale = cfg.d ** -0.5
+    out, lse = mem.attend(wl.queries, scale, q_hash=qh)
+    ro, rl = O.hashed_attention_gather(wl.queries.cpu(), wl.keys.cpu(), wl.values.cpu(),
+                                       mem.bucket_idx.cpu().long().reshape(-1), torch.full((cfg.H, cfg.C), cfg.Z),
+                                       qh.cpu().long(), scale)
+    assert_attn_close(out, lse, ro, rl, cfg.dtype, "c2")
+
+
+def test_config4_index_build_full_size(ops):
+    from fast_memory_amd import fit_projection, synth
+    cfg = synth.CONFIGS["c4"]
+    wl = synth.make_workload(cfg, "cuda")
+    A = fit_projection(wl.keys, cfg.C, iters=cfg.kmeans_iters)
+    assert torch.allclose(A.float().norm(dim=-1), torch.ones(cfg.H, cfg.C, device="cuda"), atol=1e-2)
+    idx, val = ops.build_index(A, wl.keys, cfg.Z, return_values=True)
+    assert ops.last_build_info.get("path") == "fused"
+    assert idx.shape == (cfg.H, cfg.C, cfg.Z)
+    check_lists_whole(idx, val, cfg.N)
+    check_lists_sampled(ops, A, wl.keys, idx, val, cfg.Z, rows_per_head=8)
+    idx2 = ops.build_index(A, wl.keys, cfg.Z, fused=False)          # the chunked build: the same lists
+    assert torch.equal(idx, idx2)
+    idx3 = ops.build_index(A, wl.keys, cfg.Z)                        # and the same again: nothing depends on scheduling
+    assert torch.equal(idx, idx3)
+
+
+def test_config5_one_million_keys_full_size(ops):
+    from fast_memory_amd import Memory, fit_projection, synth
+    cfg = synth.CONFIGS["c5"]
+    H, G, S, d, C, Z, N = cfg.H, cfg.G, cfg.S, cfg.d, cfg.C, cfg.Z, cfg.N
+    wl = synth.make_workload(cfg, "cuda")
+    A = fit_projection(wl.keys, C, iters=cfg.kmeans_iters)
+    mem = Memory.build(wl.keys, wl.values, A, Z, keep_values=True)
+    check_lists_whole(mem.bucket_idx, mem.bucket_val, N)
+    check_lists_sampled(ops, A, wl.keys, mem.bucket_idx, mem.bucket_val, Z, rows_per_head=2)
+    q = wl.queries
+    scale = d ** -0.5
+    # hash: the chosen bucket holds the first maximum of the scores (sampled: the score matrix is 2 GB per head)
+    qh = ops.qhash(A, q)
+    sel = torch.arange(0, q.shape[1], 997, device="cuda")
+    qs, sc = ops.qhash(A, q[:, sel].contiguous(), return_scores=True)
+    assert torch.equal(qs, qh[:, sel]) and torch.equal(qs.cpu().long(), O.argmax_first(sc.cpu()))
+    out, lse = mem.attend(q, scale, q_hash=qh)
+    assert bool(torch.isfinite(out.float()).all()) and bool((lse > -1e30).all())      # every bucket is full
+    check_attention_sampled(mem, q, qh, out, lse, scale, per_head=8)
+    # equivariance: the queries in another order give the same rows
+    perm = torch.randperm(q.shape[1], device="cuda")
+    o2, l2 = mem.attend(q[:, perm].contiguous(), scale)
+    assert torch.allclose(o2.float(), out[:, perm].float(), atol=BF16_ATOL, rtol=BF16_RTOL)
+    assert float((l2 - lse[:, perm]).abs().max()) <= LSE_ATOL
+    # with the causal local window: the merged result of sampled queries equals one softmax over both key sets
+    L = wl.k_local.shape[1]
+    mo, ml = mem.attend_with_local(q, wl.k_local, wl.v_local, scale, n_groups=G, causal=True)
+    g = torch.Generator().manual_seed(5)
+    for h in range(0, H, 3):
+        sel = torch.randperm(G * S, generator=g)[:6]
+        for j in sel.tolist():
+            t = j % S                                            # token position: sees local keys 0 .. t + (L - S)
+            ids = mem.bucket_idx[h, qh[h, j].long()].long()
+            Kj = torch.cat([wl.keys[h, ids], wl.k_local[h, :t + 1 + (L - S)]]).double()
+            Vj = torch.cat([wl.values[h, ids], wl.v_local[h, :t + 1 + (L - S)]]).double()
+            s = (Kj @ q[h, j].double()) * scale
+            ref_l = torch.logsumexp(s, 0)
+            ref_o = torch.softmax(s, 0) @ Vj
+            assert abs(float(ml[h, j]) - float(ref_l)) <= 2e-3
+            assert torch.allclose(mo[h, j].double(), ref_o, atol=BF16_ATOL, rtol=BF16_RTOL)
+
+
+def test_config3_decode_batch_full_size(ops):
+    from fast_memory_amd import Memory, MemoryBatch, synth
+    cfg_d, H, G = 128, 8, 4
+    lengths = synth.decode_lengths()
+    g = torch.Generator(device="cuda").manual_seed(1003)
+    mems = []
+    for N, C, Z in lengths:
+        K = torch.randn(H, N, cfg_d, generator=g, device="cuda").to(torch.bfloat16)
+        V = torch.randn(H, N, cfg_d, generator=g, device="cuda").to(torch.bfloat16)
+        A = torch.randn(H, C, cfg_d, generator=g, device="cuda")
+        A = (A / A.norm(dim=-1, keepdim=True)).to(torch.bfloat16)
+        mems.append(Memory.build(K, V, A, Z))
+    batch = MemoryBatch(mems)
+    q = (torch.randn(len(lengths), H, G, cfg_d, generator=g, device="cuda") * 2).to(torch.bfloat16)
+    scale = cfg_d ** -0.5
+    out, lse, h, scores = batch.attend(q, scale, return_scores=True)
+    a_off = 0
+    for s, ((N, C, Z), mem) in enumerate(zip(lengths, mems)):
+        sc = scores[a_off:a_off + H * C].reshape(H, C, G).transpose(1, 2)       # [H, G, C]
+        a_off += H * C
+        assert torch.equal(h[s].cpu().long(), O.argmax_first(sc.cpu())), f"sequence {s}: hash"
+        if s % 8 == 0:                                                          # sampled sequences, all heads
+            for hh in range(H):
+                ro, rl = oracle_on_sample(q[s, hh], h[s, hh].long(), mem.bucket_idx[hh], mem.keys[hh],
+                                          mem.values[hh], scale)
+                assert_attn_close(out[s, hh][None], lse[s, hh][None], ro, rl, torch.bfloat16, f"seq {s} head {hh}")
+    kl = torch.randn(len(lengths), H, 512, cfg_d, generator=g, device="cuda").to(torch.bfloat16)
+    vl = torch.randn(len(lengths), H, 512, cfg_d, generator=g, device="cuda").to(torch.bfloat16)
+    mo, ml = batch.attend_with_local(q, kl, vl, scale)
+    for s in range(0, len(lengths), 8):
+        lo, ll = O.local_attention(q[s].cpu().reshape(1, H * G, 1, cfg_d), kl[s:s + 1].cpu(), vl[s:s + 1].cpu(),
+                                   scale, True)
+        eo, el = O.lse_merge_closed_form(lo.reshape(H, G, cfg_d).float(), ll.reshape(H, G), out[s].cpu().float(),
+                                         lse[s].cpu())
+        assert torch.allclose(mo[s].cpu().double(), eo, atol=BF16_ATOL, rtol=BF16_RTOL)
+        assert float((ml[s].cpu().double() - el).abs().max()) < 2e-3

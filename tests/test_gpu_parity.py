@@ -393,6 +393,31 @@ def test_l2_normalize_and_segment_mean_bf16_d128(ops):
         assert torch.allclose(cent[h].float().cpu().double(), rc.double(), atol=4e-3, rtol=8e-3)
 
 
+# ------------------------------------------------------------------ golden fixture (frozen oracle outputs)
+def test_library_against_the_golden_fixture(ops):
+    import os
+    from fast_memory_amd import (attention_hash_varlen, attention_hash_varlen_backward, update_out_and_lse)
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "small_fp32.npz"))
+    t = {k: torch.from_numpy(gold[k]) for k in gold.files}
+    H, G, d, N, C, Z, S, L = (int(x) for x in gold["dims"])
+    K, V, Q, A = dev(t["K"], t["V"], t["Q"], t["A"])
+    sm = d ** -0.5
+    assert torch.allclose(ops.project(A, K).cpu(), t["Y"], atol=1e-5, rtol=1e-5)
+    assert torch.equal(ops.argtopz(dev(t["Y"]), Z).cpu(), t["lists"])                    # bit-exact on the stored Y
+    assert torch.equal(ops.qhash(A, Q).cpu(), t["qh"])
+    kh, cnt, qh = dev(t["lists"].long().reshape(-1), torch.full((H, C), Z), t["qh"].long())
+    out, lse = attention_hash_varlen(Q, K, V, kh, cnt, qh, sm)
+    assert_attn_close(out, lse, t["out"], t["lse"], torch.float32, "fixture attention")
+    lo, ll = ops.local_attn_fwd(Q.reshape(H * G, S, d), dev(t["KL"]), dev(t["VL"]), sm, True)
+    assert_attn_close(lo.reshape(H, G * S, d), ll.reshape(H, G * S), t["lout"], t["llse"], torch.float32, "fixture local")
+    mo, ml = update_out_and_lse(None, None, lo.reshape(H, G * S, d), ll.reshape(H, G * S))
+    mo, ml = update_out_and_lse(mo, ml, out, lse)
+    assert torch.allclose(mo.cpu(), t["mout"], atol=1e-4) and torch.allclose(ml.squeeze(-1).cpu(), t["mlse"], atol=1e-3)
+    dq, dk, dv = attention_hash_varlen_backward(dev(t["dO"]), Q, K, V, dev(t["out"]), dev(t["lse"]), kh, cnt, qh, sm)
+    for got, name in ((dq, "dq"), (dk, "dk"), (dv, "dv")):
+        assert torch.allclose(got.float().cpu(), t[name], atol=2e-4, rtol=1e-4), name
+
+
 # ------------------------------------------------------------------ a15 composite, config c1
 def test_config1_toy_end_to_end(ops):
     from fast_memory_amd import Memory, fit_projection

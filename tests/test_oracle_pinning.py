@@ -489,3 +489,29 @@ def test_calc_ref_centroids_brute_force():
     untouched = nrm.squeeze(-1) == 0
     assert untouched.any() and (got[untouched] == 0).all()     # keys nobody selected stay zero
 
+
+
+# ---------------------------------------------------------------- frozen outputs of the oracle
+def test_oracle_reproduces_the_golden_fixture():
+    """tests/golden/small_fp32.npz holds the oracle's outputs on seeded inputs, stage by stage; the oracle of
+    today must still give them (integer stages bit for bit)."""
+    import importlib.util
+    import os
+    import numpy as np
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(here, "make_fixtures.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    now = mod.build()
+    gold = np.load(os.path.join(here, "small_fp32.npz"))
+    assert set(now) | {"dims"} == set(gold.files)
+    for name, arr in now.items():
+        if arr.dtype.kind in "iu" or name in ("K", "V", "Q", "A", "KL", "VL", "dO"):
+            assert np.array_equal(arr, gold[name]), name          # inputs (the generator) and integer results
+        else:
+            assert np.allclose(arr, gold[name], rtol=1e-6, atol=1e-6), name
+    # what the fixture was built to contain: exact ties at the list boundary region and a zero row
+    Y, lists = gold["Y"], gold["lists"]
+    assert (Y[0, :, 100] == Y[0, :, 7]).all() and (Y[0, :, 20] == 0).all()
+    both = [(list(r).index(7), list(r).index(100)) for r in lists[0] if 7 in r and 100 in r]
+    assert both and all(a < b for a, b in both), "of two equal values the lower index must come first"

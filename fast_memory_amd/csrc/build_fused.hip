@@ -53,8 +53,11 @@ constexpr int kMaxRepair = 64;
 // builds of 16384 rows, and ~18 % more candidates than Z are kept at mu = 512 (six would keep 27 %).
 constexpr double kRankSigmas = 4.0;
 
+constexpr int kCandRegs = 24;       // candidates a thread of the selection holds, 1024 threads per row
+constexpr int kCandRegsSmall = 32;  // ... with 256 or 512 threads per row
+
 struct FusedPlan {
-  int ns, stride, rank, n_splits, slabs, n_writers, cap_w;
+  int ns, stride, rank, n_splits, slabs, n_writers, cap_w, sel_threads;
   int64_t ld_s, ldy;
   size_t off_Ks, off_Ys, off_tau, off_cand, off_cnt, off_fail, off_nfail, off_Yf, total;
 };
@@ -62,18 +65,42 @@ struct FusedPlan {
 static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& p) {
   if (dtype != FM_BF16 || d != kFD) return false;
   if (N < 65536 || int64_t(Z) * 8 > N || Z > FM_MAX_Z || Z < 64) return false;
-  p.stride = N / 32768;
-  p.ns = N / p.stride;
-  const double mu = double(Z) * p.ns / N;
-  p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
-  if (p.rank * 4 > p.ns) return false;
-  const double m_exp = double(p.rank) * N / p.ns;
   p.slabs = int(ceil_div(C, kFSlab));
   const int64_t ntiles = ceil_div(N, kFKeys);
   int64_t s = ceil_div(256, int64_t(H) * p.slabs);
   s = std::max<int64_t>(1, std::min<int64_t>(32, std::min(s, ntiles)));
   p.n_splits = int(s);
   p.n_writers = 2 * p.n_splits;
+  // Sample size and threads per row of the selection.  A smaller sample makes phase 0 cheaper and the
+  // threshold noisier: a row keeps m = rank*stride +- stride*sqrt(rank) candidates, which the
+  // selection must hold in registers (R per thread, T = NT / n_writers threads per writer segment,
+  // whose share of m spreads by another sqrt).  The sort keeps 16 keys per thread, so P/16 threads
+  // are all it can use; fewer threads per row let several rows share a CU.  Take the smallest
+  // sample, then the fewest threads, that leave five standard deviations of room; failing that, the
+  // large sample with 1024 threads (rows that do not fit are repaired).
+  const int P = next_pow2(Z);
+  bool found = false;
+  double m_exp = 0;
+  for (int ns_try : {16384, 32768}) {
+    p.stride = N / ns_try;
+    p.ns = N / p.stride;
+    const double mu = double(Z) * p.ns / N;
+    p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
+    if (p.rank * 4 > p.ns) continue;
+    m_exp = double(p.rank) * N / p.ns;
+    const double per_w = m_exp / p.n_writers;
+    const double sd_w = sqrt(pow(double(N) / p.ns * sqrt(double(p.rank)) / p.n_writers, 2) + per_w);
+    for (int nt = 256; nt <= kSelThreads && !found; nt *= 2)
+      if (nt * 16 >= P && (nt / p.n_writers) * (nt < kSelThreads ? kCandRegsSmall : kCandRegs) >= per_w + 5.0 * sd_w) {
+        p.sel_threads = nt;
+        found = true;
+      }
+    if (found) break;
+  }
+  if (!found) {
+    if (p.rank * 4 > p.ns) return false;
+    p.sel_threads = kSelThreads;
+  }
   p.cap_w = int(1.35 * m_exp / p.n_writers) + 64;  // > 16: the overflow guard keeps 16 slots free
   p.ld_s = (int64_t(p.ns) + 3) / 4 * 4;
   p.ldy = (int64_t(N) + 3) / 4 * 4;
@@ -386,18 +413,18 @@ __device__ __forceinline__ bool load_cand_counts(const int32_t* __restrict__ cnt
   return !(cc.over || cc.total < Zc);
 }
 
-// A row's candidates held in registers: the 1024 threads are dealt to the writers' segments in
-// groups of 1024 / n_writers, and a thread keeps elements t, t + T, t + 2T, ... of its segment
-// (at most kCandRegs of them).  The candidates are read from memory once; the radix passes of
+// A row's candidates held in registers: the NT threads are dealt to the writers' segments in
+// groups of T = NT / n_writers, and a thread keeps elements t, t + T, t + 2T, ... of its segment
+// (at most R of them).  The candidates are read from memory once; the radix passes of
 // the selection and the collection into the sort buffer then run from registers.
-constexpr int kCandRegs = 24;
+template <int R>
 struct CandRegs {
-  uint2 e[kCandRegs];  // (value bits, key code)
+  uint2 e[R];  // (value bits, key code)
   int n;               // valid entries of this thread
   template <typename F>
   __device__ __forceinline__ void operator()(F f) const {
 #pragma unroll
-    for (int r = 0; r < kCandRegs; ++r)
+    for (int r = 0; r < R; ++r)
       if (r < n) f(__uint_as_float(e[r].x), fused_key_of_code(e[r].y));
   }
 };
@@ -405,7 +432,8 @@ struct CandRegs {
 // Exact top-Z (value desc, index asc) of every row's candidates: radix select of the cut,
 // collection of the Zc survivors into LDS, bitonic sort, indices out -- the code of the dense
 // arg-top-Z kernel, on ~1.2 Zc register-resident candidates instead of the N-element row.
-__global__ __launch_bounds__(kSelThreads) void cand_select_kernel(
+template <int NT, int R>
+__global__ __launch_bounds__(NT) void cand_select_kernel(
     const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, int n_writers, int cap_w, int Zc, int P,
     int32_t* __restrict__ idx_out, float* __restrict__ val_out, int32_t* __restrict__ fail_rows,
     int32_t* __restrict__ n_fail) {
@@ -413,9 +441,9 @@ __global__ __launch_bounds__(kSelThreads) void cand_select_kernel(
   __shared__ SelectShared sh;
   __shared__ CandCounts cc;
   const int64_t row = blockIdx.x;
-  const int T = kSelThreads / n_writers;  // threads per segment
+  const int T = NT / n_writers;  // threads per segment
   bool ok = load_cand_counts(cnt, row, n_writers, cap_w, Zc, cc);
-  ok = ok && cc.maxc <= T * kCandRegs;
+  ok = ok && cc.maxc <= T * R;
   if (!ok) {  // threshold missed (or a segment too long to hold): queue the row for repair
     if (threadIdx.x == 0) {
       int pos = atomicAdd(n_fail, 1);
@@ -423,15 +451,15 @@ __global__ __launch_bounds__(kSelThreads) void cand_select_kernel(
     }
     return;
   }
-  CandRegs src;
+  CandRegs<R> src;
   const int w = threadIdx.x / T, t = threadIdx.x - w * T;
   const int cw = w < n_writers ? cc.counts[w] : 0;
   const uint2* seg = cand + (row * n_writers + min(w, n_writers - 1)) * int64_t(cap_w);
   src.n = cw > t ? (cw - t + T - 1) / T : 0;
 #pragma unroll
-  for (int r = 0; r < kCandRegs; ++r)
+  for (int r = 0; r < R; ++r)
     if (r < src.n) src.e[r] = seg[t + r * T];
-  const uint64_t cut = radix_select_cut(src, Zc, 6, sh);
+  const uint64_t cut = radix_select_cut<NT>(src, Zc, 6, sh);
   collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + row * Zc, val_out ? val_out + row * Zc : nullptr);
 }
 
@@ -540,9 +568,19 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   // phase 2
   mark_phase(2, st);
   const int P = next_pow2(Zc);
-  FM_ALLOW_LDS(cand_select_kernel, sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");
-  hipLaunchKernelGGL(cand_select_kernel, dim3(unsigned(rows)), dim3(kSelThreads), sort_lds_bytes(P), st, cand, cnt,
-                     p.n_writers, p.cap_w, Zc, P, idx_out, val_out, fail_rows, n_fail);
+#define FM_CAND_SELECT(NT, R)                                                                           \
+  do {                                                                                                  \
+    FM_ALLOW_LDS((cand_select_kernel<NT, R>), sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");   \
+    hipLaunchKernelGGL((cand_select_kernel<NT, R>), dim3(unsigned(rows)), dim3(NT), sort_lds_bytes(P), st, cand, cnt, \
+                       p.n_writers, p.cap_w, Zc, P, idx_out, val_out, fail_rows, n_fail);                      \
+  } while (0)
+  if (p.sel_threads == 256)
+    FM_CAND_SELECT(256, kCandRegsSmall);
+  else if (p.sel_threads == 512)
+    FM_CAND_SELECT(512, kCandRegsSmall);
+  else
+    FM_CAND_SELECT(kSelThreads, kCandRegs);
+#undef FM_CAND_SELECT
   // phase 3
   mark_phase(3, st);
   hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(ceil_div(N, 128)), kMaxRepair), dim3(256), 0,

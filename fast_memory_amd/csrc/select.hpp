@@ -160,7 +160,7 @@ __device__ __forceinline__ void bitonic_sort_desc(uint64_t* buf, int logP) {
     const int P = 1 << logP;
     for (int k = 2; k <= P; k <<= 1)
       for (int j = k >> 1; j > 0; j >>= 1) {
-        for (int t = tid; t < (P >> 1); t += kSelThreads) {
+        for (int t = tid; t < (P >> 1); t += int(blockDim.x)) {
           const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
           const int q = i | j;
           const uint64_t a = buf[sort_phys(i)], b = buf[sort_phys(q)];
@@ -284,10 +284,10 @@ __device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, in
       if (pos < P) buf[sort_phys(pos)] = c;
     }
   });
-  for (int i = Zc + tid; i < P; i += kSelThreads) buf[sort_phys(i)] = 0;
+  for (int i = Zc + tid; i < P; i += int(blockDim.x)) buf[sort_phys(i)] = 0;
   __syncthreads();
   bitonic_sort_desc(buf, 31 - __clz(P));
-  for (int i = tid; i < Zc; i += kSelThreads) {
+  for (int i = tid; i < Zc; i += int(blockDim.x)) {
     const uint64_t c = buf[sort_phys(i)];
     out[i] = int32_t(0xffffffffu - uint32_t(c));
     if (val_out) val_out[i] = key_to_float(uint32_t(c >> 32));

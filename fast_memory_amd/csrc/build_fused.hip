@@ -53,7 +53,7 @@ constexpr int kMaxRepair = 64;
 // builds of 16384 rows, and ~18 % more candidates than Z are kept at mu = 512 (six would keep 27 %).
 constexpr double kRankSigmas = 4.0;
 
-constexpr int kCandRegs = 24;       // candidates a thread of the selection holds, 1024 threads per row
+constexpr int kCandRegs = 28;       // candidates a thread of the selection holds, 1024 threads per row
 constexpr int kCandRegsSmall = 32;  // ... with 256 or 512 threads per row
 
 struct FusedPlan {

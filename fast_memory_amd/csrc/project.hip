@@ -73,6 +73,108 @@ __global__ __launch_bounds__(256) void project_bf16_kernel(const bf16_t* __restr
 }
 
 // ---------------------------------------------------------------------------
+// bf16, d = 128: bucket-stationary streaming form of the same product.  The kernel
+// is a fill of Y (4 B written per 256 flops: HBM-write-bound by a wide margin), so
+// it is built to keep stores flowing: a workgroup of four waves holds a slab of
+// buckets as MFMA A-operand fragments in registers for its whole life and walks
+// a range of keys step by step; the keys of a step go through a
+// double-buffered LDS tile (global loads of step i+1 are in flight while step i
+// computes and stores; one barrier per step), and the accumulators are stored
+// straight from registers: with the keys on the B operand a register holds 32
+// consecutive keys of one bucket row across lanes, i.e. every store instruction
+// writes two full 128-byte lines.  Same contraction order per output as the
+// tile kernel above (ascending 16-element steps into one fp32 accumulator).
+// grid (key ranges, slabs, H).
+// ---------------------------------------------------------------------------
+constexpr int kPsLd = 136;  // bf16 elements per staged key row (128 + 8 pad)
+
+// 16-byte chunks of keys key0, key0 + 16, ... (clamped to the last key) into registers.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // (an array of HIP's uint4 structs stays in scratch)
+template <int NCH>
+__device__ __forceinline__ void ps_fetch(u32x4 (&st)[NCH], const bf16_t* __restrict__ kp, int key0, int N) {
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) st[i] = *reinterpret_cast<const u32x4*>(kp + int64_t(min(key0 + 16 * i, N - 1)) * 128);
+}
+
+// BT bucket tiles per wave (the slab of a workgroup is 4 * 32 BT buckets), KT key tiles per step.
+template <int BT, int KT>
+__global__ __launch_bounds__(256) void project_stream_bf16_d128_kernel(const bf16_t* __restrict__ A,
+                                                                       const bf16_t* __restrict__ K,
+                                                                       float* __restrict__ Y, int C, int N,
+                                                                       int64_t ldy, int steps_per_wg) {
+  constexpr int kKeys = 32 * KT, kWaveRows = 32 * BT;
+  __shared__ __attribute__((aligned(16))) bf16_t sK[2][kKeys * kPsLd];
+  const int h = blockIdx.z;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), l = lane_id();
+  const int b0 = blockIdx.y * (4 * kWaveRows) + w * kWaveRows;  // first bucket of this wave
+  const bf16_t* Ah = A + int64_t(h) * C * 128;
+  const bf16_t* Kh = K + int64_t(h) * N * 128;
+  float* Yh = Y + int64_t(h) * C * ldy;
+  const int n_steps_total = (N + kKeys - 1) / kKeys;
+  const int s0 = blockIdx.x * steps_per_wg;
+  const int s1 = min(s0 + steps_per_wg, n_steps_total);
+  if (s0 >= s1) return;
+  // A fragments: bucket tile bt, contraction step ks -> 8 bf16 of row (l % 32) at k = 16 ks + 8 (l / 32)
+  bf16x8 af[BT][8];
+#pragma unroll
+  for (int bt = 0; bt < BT; ++bt) {
+    const int row = min(b0 + bt * 32 + (l & 31), C - 1);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+      af[bt][ks] = *reinterpret_cast<const bf16x8*>(Ah + int64_t(row) * 128 + ks * 16 + (l >> 5) * 8);
+  }
+  // staging: kKeys x 16 chunks of 16 B, 2 KT per thread (thread t: chunk t % 16 of keys t / 16 + 16 i)
+  u32x4 st[2 * KT];
+  const int e_row = threadIdx.x >> 4, e_ch = (threadIdx.x & 15) * 8;
+  const bf16_t* kp = Kh + e_ch;
+  ps_fetch<2 * KT>(st, kp, s0 * kKeys + e_row, N);
+  const bool rows_full = b0 + kWaveRows <= C;
+  const uint32_t lane_off = uint32_t(4 * (l >> 5)) * uint32_t(ldy) + uint32_t(l & 31);
+  for (int step = s0; step < s1; ++step) {
+    bf16_t* buf = sK[(step - s0) & 1];
+#pragma unroll
+    for (int i = 0; i < 2 * KT; ++i) *reinterpret_cast<u32x4*>(buf + (e_row + 16 * i) * kPsLd + e_ch) = st[i];
+    __syncthreads();
+    ps_fetch<2 * KT>(st, kp, min(step + 1, s1 - 1) * kKeys + e_row, N);  // (the last step fetches its own tile again)
+    if (b0 >= C) continue;  // a wave past the last bucket only helps staging
+    f32x16 acc[BT][KT];
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[bt][kt][r] = 0.f;
+    const bf16_t* pb = buf + (l & 31) * kPsLd + (l >> 5) * 8;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      bf16x8 kf[KT];
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) kf[kt] = *reinterpret_cast<const bf16x8*>(pb + kt * 32 * kPsLd + ks * 16);
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+          acc[bt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[bt][ks], kf[kt], acc[bt][kt], 0, 0, 0);
+    }
+    // store: wave-uniform 64-bit base per (tile, register) + one 32-bit lane offset
+    const int n0 = step * kKeys;
+    const bool full = rows_full && n0 + kKeys <= N;
+    float* ubase = Yh + int64_t(b0) * ldy + n0;
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+          const int key = n0 + kt * 32 + (l & 31);
+          float* ur = ubase + int64_t(bt * 32 + 8 * (r >> 2) + (r & 3)) * ldy + kt * 32;
+          const int row = b0 + bt * 32 + acc_row_32(r, l);
+          if (full || (row < C && key < N)) ur[lane_off] = acc[bt][kt][r];
+        }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Generic projection (any d <= 256, fp32 or bf16 storage, fp32 FMA chain over
 // k = 0..d-1).  64 keys staged in LDS per workgroup; lane = key, waves stride
 // over buckets.
@@ -430,13 +532,26 @@ extern "C" int fm_project(const void* A, const void* K, float* Y, int H, int C, 
   using namespace fm;
   FM_REQUIRE(H >= 0 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_project: H=%d C=%d N=%d d=%d", H, C, N, d);
-  FM_REQUIRE(ldy >= N, FM_ERR_ARG, "fm_project: ldy=%lld < N=%d", (long long)ldy, N);
+  FM_REQUIRE(ldy >= N && ldy < (int64_t(1) << 29), FM_ERR_ARG, "fm_project: ldy=%lld, N=%d", (long long)ldy, N);
   FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_project: dtype=%d", dtype);
   if (H == 0) return FM_OK;
   FM_REQUIRE(A && K && Y, FM_ERR_ARG, "fm_project: null pointer");
   FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_project: H=%d > 65535", H);
   hipStream_t st = as_stream(stream);
-  if (dtype == FM_BF16 && d % 16 == 0) {
+  if (dtype == FM_BF16 && d == 128) {
+    constexpr int kBT = 1, kKT = 4;  // 32 buckets per wave, 128 keys per step: 512 contiguous bytes per row and step
+    constexpr int kSlab = 4 * 32 * kBT, kKeys = 32 * kKT;
+    FM_REQUIRE(ceil_div(C, kSlab) <= 65535, FM_ERR_UNSUPPORTED, "fm_project: C too large");
+    // enough key ranges for ~4 workgroups per CU, each at least 8 steps long
+    const int64_t n_steps = ceil_div(N, kKeys);
+    const int64_t slabs = int64_t(ceil_div(C, kSlab)) * H;
+    int64_t ranges = std::max<int64_t>(1, std::min<int64_t>(ceil_div(1024, slabs), ceil_div(n_steps, 8)));
+    const int steps_per_wg = int(ceil_div(n_steps, ranges));
+    ranges = ceil_div(n_steps, steps_per_wg);
+    hipLaunchKernelGGL((project_stream_bf16_d128_kernel<kBT, kKT>),
+                       dim3(unsigned(ranges), unsigned(ceil_div(C, kSlab)), unsigned(H)), dim3(256), 0, st,
+                       (const bf16_t*)A, (const bf16_t*)K, Y, C, N, ldy, steps_per_wg);
+  } else if (dtype == FM_BF16 && d % 16 == 0) {
     FM_REQUIRE(ceil_div(C, 128) <= 65535, FM_ERR_UNSUPPORTED, "fm_project: C too large");
     size_t lds = std::max(size_t(2) * 128 * (d + 8) * sizeof(bf16_t), size_t(128) * kProjYLd * sizeof(float));
     FM_ALLOW_LDS(project_bf16_kernel, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_project: lds");

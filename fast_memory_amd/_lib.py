@@ -55,6 +55,7 @@ SIGNATURES = {
     "fm_index_append": (c_int, [P, P, c_int, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P, P]),
     "fm_segment_sum": (c_int, [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_debug_force_generic": (None, [c_int]),
+    "fm_debug_argtopz_exact_only": (None, [c_int]),
     "fm_debug_copy": (c_int, [P, P, c_int64, P]),
     "fm_debug_read": (c_int, [P, c_int64, P, P]),
     "fm_debug_set_phase_events": (None, [P, c_int]),

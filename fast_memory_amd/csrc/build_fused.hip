@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void gather_sample_kernel(const bf16_t* __rest
 }
 
 // tau[row] = a lower bound of the rank-th largest value of the sampled row that
-// at least `rank` sampled values reach (value bits only: 12+10+10).
+// at least `rank` sampled values reach (value bits only: 11+11+10).
 __global__ __launch_bounds__(kSelThreads) void row_threshold_kernel(const float* __restrict__ Ys,
                                                                     int ns, int64_t ld, int rank,
                                                                     float* __restrict__ tau,

@@ -4,41 +4,164 @@
 // Y[r,:], ordered by (value descending, index ascending); -0 == +0, NaN is the
 // largest value.
 //
-// One workgroup per row: radix select of the Zc-th largest composite (every
-// pass re-reads the row and histograms one digit in LDS; the loop stops as soon
-// as the bin that holds the cut is wanted whole), one more read collects the
-// exactly Zc survivors into LDS, bitonic sort there, indices out.
-// HBM traffic: (passes + 1) reads of the row, typically 4; LDS 8*pow2(Zc) + 16 KiB.
+// One workgroup per row.  Two ways to the same result:
+//  * sampled (long rows, Z <= 8192): 1/16 of the row is read as whole 128-byte
+//    lines spread over the row and kept in registers; the sample's value of rank
+//    mu + 4 sqrt(mu) + 3 (mu = Z n_sample / N) is a threshold that at least Z
+//    elements of the row reach in all but about one row in 30 000.  ONE read of
+//    the row then collects the elements that reach it into LDS (about 1.3-1.6 Z),
+//    and the exact cut, the sort and the output run on those.  HBM traffic: 1.06
+//    reads of the row.
+//  * exact passes (every other shape, and any row whose sample misled: fewer than
+//    Z or more than the buffer's capacity collected, e.g. rows of mostly equal
+//    values): radix select of the Zc-th largest composite, each pass re-reading
+//    the row and histogramming one digit in LDS, stopping as soon as the bin that
+//    holds the cut is wanted whole; one more read collects the exactly Zc
+//    survivors.  HBM traffic: (passes + 1) reads of the row, typically 4.
+// Then the bitonic sort in LDS, indices (and values) out.  The result does not
+// depend on which way a row took.  LDS: max(8 pow2(Zc) * 17/16, 8 cap) + 16 KiB.
 #include "select.hpp"
 
 namespace fm {
 
+bool g_argtopz_exact_only = false;  // test hook: fm_debug_argtopz_exact_only
+
+constexpr int kSampleRegs = 32;  // sampled elements per thread: samples of up to 32768 elements
+constexpr int kCollectRegs = 16; // collected candidates per thread: capacity up to 16384
+
+struct SamplePlan {
+  int n_lines;      // sampled 128-byte lines (32 floats each); 0 = exact passes only
+  int line_stride;  // in lines
+  int rank;
+  int cap;          // candidates the LDS buffer takes
+};
+
+static SamplePlan sample_plan(int N, int Zc, int P, int nt) {
+  SamplePlan p{0, 0, 0, 0};
+  if (N < 65536 || int64_t(Zc) * 8 > N || P > 8 * nt) return p;
+  const int lines = N / 32;                         // whole lines only; a ragged tail is never sampled
+  int stride = 16;
+  while (lines / stride > kSampleRegs * nt / 32) stride *= 2;
+  const int n_lines = lines / stride;
+  const double ns = 32.0 * n_lines;
+  const double mu = double(Zc) * ns / N;
+  const int rank = int(mu + 4.0 * sqrt(mu) + 3.0);
+  const double m_exp = double(rank) * N / ns, m_sd = double(N) / ns * sqrt(double(rank));
+  int cap = 2 * P;
+  while (cap < m_exp + 5.0 * m_sd && cap < kCollectRegs * nt) cap *= 2;
+  if (cap < m_exp + 5.0 * m_sd || rank * 4 > ns) return p;
+  p.n_lines = n_lines;
+  p.line_stride = stride;
+  p.rank = rank;
+  p.cap = cap;
+  return p;
+}
+
+// The sampled lines of a row, in registers.
+template <int NT>
+struct SampleRegs {
+  float v[kSampleRegs];
+  int n;
+  template <typename F>
+  __device__ __forceinline__ void operator()(F f) const {
+#pragma unroll
+    for (int r = 0; r < kSampleRegs; ++r)
+      if (r < n) f(v[r], uint32_t(threadIdx.x + r * NT));
+  }
+};
+
+// Candidates collected in LDS, dealt to the threads' registers as composites.
+struct CollectedRegs {
+  uint64_t c[kCollectRegs];
+  int n;
+  template <typename F>
+  __device__ __forceinline__ void operator()(F f) const {
+#pragma unroll
+    for (int r = 0; r < kCollectRegs; ++r)
+      if (r < n) f(key_to_float(uint32_t(c[r] >> 32)), 0xffffffffu - uint32_t(c[r]));
+  }
+};
+
 // row_map / n_rows_dev are optional: when given, workgroup b works on input row
 // b and writes output row row_map[b], and exits if b >= min(*n_rows_dev, grid).
-__global__ __launch_bounds__(kSelThreads) void argtopz_kernel(
+template <int NT>
+__global__ __launch_bounds__(NT) void argtopz_kernel(
     const float* __restrict__ Y, int N, int64_t ldy, int Zc, int P, int32_t* __restrict__ idx_out,
-    float* __restrict__ val_out, const int32_t* __restrict__ row_map, const int32_t* __restrict__ n_rows_dev) {
-  extern __shared__ uint64_t buf[];  // P composites
+    float* __restrict__ val_out, const int32_t* __restrict__ row_map, const int32_t* __restrict__ n_rows_dev,
+    SamplePlan sp) {
+  extern __shared__ uint64_t buf[];  // P composites in the sort's layout; before that, up to sp.cap candidates
   __shared__ SelectShared sh;
   if (n_rows_dev && int(blockIdx.x) >= *n_rows_dev) return;
   const int64_t out_row = row_map ? row_map[blockIdx.x] : int64_t(blockIdx.x);
-  DenseRow src{Y + int64_t(blockIdx.x) * ldy, N};
-  const uint64_t cut = radix_select_cut(src, Zc, 6, sh);
-  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + out_row * Zc, val_out ? val_out + out_row * Zc : nullptr);
+  const float* row = Y + int64_t(blockIdx.x) * ldy;
+  int32_t* out = idx_out + out_row * Zc;
+  float* vout = val_out ? val_out + out_row * Zc : nullptr;
+  DenseRowT<NT> src{row, N};
+  if (sp.n_lines > 0) {
+    const int tid = threadIdx.x;
+    SampleRegs<NT> smp;
+    const int n_s = sp.n_lines * 32;
+    smp.n = tid < n_s ? (n_s - tid + NT - 1) / NT : 0;
+#pragma unroll
+    for (int r = 0; r < kSampleRegs; ++r) {
+      const int j = tid + r * NT;  // sample element j = element (j % 32) of sampled line j / 32
+      if (r < smp.n) smp.v[r] = row[(int64_t(j >> 5) * sp.line_stride << 5) + (j & 31)];
+    }
+    const uint64_t tau = radix_select_cut<NT>(smp, sp.rank, 3, sh) & 0xffffffff00000000ull;  // value bits only
+    if (tid == 0) sh.cnt = 0;
+    __syncthreads();
+    src([&](float y, uint32_t i) {
+      const uint64_t c = composite(y, i);
+      if (c >= tau) {
+        const int pos = atomicAdd(&sh.cnt, 1);
+        if (pos < sp.cap) buf[pos] = c;
+      }
+    });
+    __syncthreads();
+    const int m = sh.cnt;
+    if (m >= Zc && m <= sp.cap) {
+      CollectedRegs cr;
+      cr.n = tid < m ? (m - tid + NT - 1) / NT : 0;
+#pragma unroll
+      for (int r = 0; r < kCollectRegs; ++r)
+        if (r < cr.n) cr.c[r] = buf[tid + r * NT];
+      const uint64_t cut = radix_select_cut<NT>(cr, Zc, 6, sh);  // (its barriers order the reads above before the writes below)
+      collect_sort_write(cr, cut, Zc, P, buf, sh, out, vout);
+      return;
+    }
+    __syncthreads();  // every thread has read sh.cnt before the exact passes reuse it
+  }
+  const uint64_t cut = radix_select_cut<NT>(src, Zc, 6, sh);
+  collect_sort_write(src, cut, Zc, P, buf, sh, out, vout);
 }
 
 int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out, float* val_out,
                    const int32_t* row_map, const int32_t* n_rows_dev, hipStream_t st) {
   const int P = next_pow2(Zc);
-  FM_ALLOW_LDS(argtopz_kernel, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
-  hipLaunchKernelGGL(argtopz_kernel, dim3(unsigned(rows)), dim3(kSelThreads),
-                     sort_lds_bytes(P), st, Y, N, ldy, Zc, P, idx_out, val_out, row_map, n_rows_dev);
+  // Two 512-thread workgroups share a CU where one of 1024 threads would have it alone: one row's
+  // sort overlaps the other's read.  The narrow form needs the sampled path (its registers then hold
+  // all a thread keeps) and lists of at most 4096.
+  SamplePlan sp = sample_plan(N, Zc, P, 512);
+  const bool narrow = sp.n_lines > 0 && !g_argtopz_exact_only;
+  if (!narrow) sp = g_argtopz_exact_only ? SamplePlan{0, 0, 0, 0} : sample_plan(N, Zc, P, kSelThreads);
+  const size_t lds = std::max(sort_lds_bytes(P), size_t(sp.cap) * sizeof(uint64_t));
+  if (narrow) {
+    FM_ALLOW_LDS(argtopz_kernel<512>, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
+    hipLaunchKernelGGL(argtopz_kernel<512>, dim3(unsigned(rows)), dim3(512), lds, st, Y, N, ldy, Zc, P, idx_out,
+                       val_out, row_map, n_rows_dev, sp);
+  } else {
+    FM_ALLOW_LDS(argtopz_kernel<kSelThreads>, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
+    hipLaunchKernelGGL(argtopz_kernel<kSelThreads>, dim3(unsigned(rows)), dim3(kSelThreads), lds, st, Y, N, ldy, Zc,
+                       P, idx_out, val_out, row_map, n_rows_dev, sp);
+  }
   return launch_status("argtopz");
 }
 
 }  // namespace fm
 
 extern "C" size_t fm_argtopz_workspace(int64_t, int, int) { return 0; }
+
+extern "C" void fm_debug_argtopz_exact_only(int on) { fm::g_argtopz_exact_only = on != 0; }
 
 extern "C" int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, int Z,
                               int32_t* idx_out, float* val_out, void* ws, size_t ws_bytes, void* stream) {

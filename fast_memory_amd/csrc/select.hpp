@@ -17,7 +17,7 @@
 namespace fm {
 
 constexpr int kSelThreads = 1024;
-constexpr int kSelMaxBins = 4096;
+constexpr int kSelMaxBins = 2048;
 
 __device__ __forceinline__ uint64_t composite(float y, uint32_t i) {
   return (uint64_t(float_key(y)) << 32) | uint64_t(0xffffffffu - i);
@@ -37,7 +37,7 @@ struct SelectShared {
 };
 
 // Finds a cut such that exactly `need0` composites of the source are >= cut,
-// looking at no more than `max_passes` digits (12,10,10 value bits, then
+// looking at no more than `max_passes` digits (11,11,10 value bits, then
 // 11,11,10 index bits).  With all 6 passes the cut is exact; with fewer it is a
 // lower bound of the need0-th largest composite (at least need0 are >= cut).
 // Every thread of the workgroup (NT threads, a power of two between 64 and 1024) must call
@@ -51,7 +51,7 @@ __device__ __forceinline__ uint64_t radix_select_cut(Source& src, int need0, int
     sh.need = need0;
     sh.hit = 0;
   }
-  const int kBits[6] = {12, 10, 10, 11, 11, 10};
+  const int kBits[6] = {11, 11, 10, 11, 11, 10};
   int top = 64;  // bits [top,64) of the cut are known and equal sh.prefix
   for (int pass = 0; pass < max_passes; ++pass) {
     const int bits = kBits[pass];
@@ -296,7 +296,8 @@ __device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, in
 
 // Dense fp32 row as a source; 128-bit loads on the aligned body, kUnroll of
 // them in flight per thread.
-struct DenseRow {
+template <int NT = kSelThreads>
+struct DenseRowT {
   const float* row;
   int N;
   static constexpr int kUnroll = 8;
@@ -308,16 +309,16 @@ struct DenseRow {
     if (tid < head) f(row[tid], uint32_t(tid));
     const int nvec = (N - head) >> 2;
     const float4* v = reinterpret_cast<const float4*>(row + head);
-    for (int i0 = tid; i0 < nvec; i0 += kSelThreads * kUnroll) {
+    for (int i0 = tid; i0 < nvec; i0 += NT * kUnroll) {
       float4 x[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
-        int i = i0 + u * kSelThreads;
+        int i = i0 + u * NT;
         if (i < nvec) x[u] = v[i];
       }
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
-        int i = i0 + u * kSelThreads;
+        int i = i0 + u * NT;
         if (i < nvec) {
           uint32_t b = uint32_t(head + 4 * i);
           f(x[u].x, b);
@@ -331,6 +332,8 @@ struct DenseRow {
     if (tail0 + tid < N) f(row[tail0 + tid], uint32_t(tail0 + tid));
   }
 };
+
+using DenseRow = DenseRowT<>;
 
 static inline int next_pow2(int x) {
   int p = 1;

@@ -358,6 +358,11 @@ def segment_sum(X: torch.Tensor, perm: torch.Tensor, seg_off: torch.Tensor, seg_
     return out
 
 
+def argtopz_exact_only(on: bool) -> None:
+    """Diagnostic switch: dense arg-top-Z by exact radix passes only (no sampled one-pass form)."""
+    _lib.load().fm_debug_argtopz_exact_only(int(on))
+
+
 def force_generic_kernels(on: bool) -> None:
     """Diagnostic switch: route attention through the generic kernels."""
     _lib.load().fm_debug_force_generic(int(on))

@@ -63,7 +63,10 @@ int fm_project(const void* A, const void* K, float* Y, int H, int C, int N, int 
  * replaces torch.topk at memory.py:273 / triton_kernel.py:278.  Output row r =
  * the min(Z,N) indices of the largest entries of Y[r,:], ordered by value
  * descending then index ascending (the first Z entries of a stable descending
- * sort; -0 == +0; NaN is the largest).  idx_out is [rows, min(Z,N)] int32;
+ * sort; -0 == +0; NaN is the largest).  Long rows with Z <= 8192 are read once
+ * (a threshold from a 1/16 sample, then one collecting pass; a row the sample
+ * misleads falls back to exact radix passes), others about four times; the
+ * result is the same.  idx_out is [rows, min(Z,N)] int32;
  * val_out (may be NULL) receives the selected values in the same order (-0 as
  * +0): the lists' values are what fm_index_append needs to extend an index. */
 size_t fm_argtopz_workspace(int64_t rows, int N, int Z);
@@ -259,6 +262,11 @@ int fm_segment_sum(const void* X, const int32_t* perm, const int32_t* seg_off, c
 /* Diagnostic: 1 routes the attention entry points through the generic kernels
  * (used by tests to compare the two implementations), 0 restores dispatch. */
 void fm_debug_force_generic(int on);
+
+/* Diagnostic: 1 makes fm_argtopz_f32 (and the chunked index build) take the exact
+ * multi-pass selection for every row instead of the sampled one-pass form (tests
+ * compare the two), 0 restores dispatch. */
+void fm_debug_argtopz_exact_only(int on);
 
 /* Diagnostic: hand the fused index build up to 5 hipEvent_t (host array that
  * must stay valid; NULL clears) which it records on its stream before phase 0

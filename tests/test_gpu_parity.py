@@ -99,6 +99,35 @@ def test_argtopz_max_z_long_row(ops):
     check_topz(ops, Y, 16384)
 
 
+def test_argtopz_sampled_one_pass_equals_exact_passes(ops):
+    """Long rows with Z <= 8192 take the sampled one-pass selection; rows the sample misleads fall back inside
+    the kernel.  Both must give the lists of the exact multi-pass selection, bit for bit."""
+    g = gen(210)
+    N = 131072 + 37                                          # ragged tail, rows not 16-byte aligned after row 0
+    Y = torch.randn(12, N, generator=g)
+    Y[1] = torch.randn(N, generator=g).round()               # heavy ties: a few dozen distinct values
+    Y[2] = 1.0                                               # all equal: the threshold keeps the whole row
+    Y[3, ::7] = float("inf")
+    Y[4, 5::3] = float("nan")
+    Y[5] = torch.where(torch.arange(N) % 16 == 0, Y[5] + 100.0, Y[5])     # the large values sit on the sampled lines' lanes
+    Y[6, :N // 2] -= 50.0                                    # all large values in the second half
+    Y[7] = torch.arange(N, dtype=torch.float32)              # ascending: the top is the tail, which is never sampled
+    Y[8] = -torch.arange(N, dtype=torch.float32)
+    Y[9, 1000:1000 + 3000] = 7.0                             # a tie block that straddles the cut
+    Yd = dev(Y)
+    for Z in (128, 1000, 4096, 8192):
+        fast, fv = ops.argtopz(Yd, Z, return_values=True)
+        ops.argtopz_exact_only(True)
+        try:
+            exact, ev = ops.argtopz(Yd, Z, return_values=True)
+        finally:
+            ops.argtopz_exact_only(False)
+        assert torch.equal(fast, exact), f"Z={Z}: rows {(fast != exact).any(dim=1).nonzero().flatten().tolist()} differ"
+        assert torch.equal(fv.view(torch.int32), ev.view(torch.int32))
+        rows = [0, 1, 5, 9]
+        assert torch.equal(fast[rows].cpu().long(), O.argtopz(Y[rows], Z))
+
+
 def test_argtopz_rejects_oversize_z(ops):
     Y = torch.zeros(1, 40000, device="cuda")
     with pytest.raises(RuntimeError):

@@ -318,7 +318,7 @@ __global__ __launch_bounds__(256) void hash_attn_mfma_kernel(
 // bucket among the G hashes with the queries that chose it, or exits if there are
 // fewer distinct buckets.  Each bucket is read once, and a row's buckets in parallel.  Rows are described by fm_rowdesc; A, K, V
 // and the bucket lists of all rows are packed back to back.
-__global__ __launch_bounds__(256) void decode_hash_attn_kernel(
+__global__ __launch_bounds__(256, 2) void decode_hash_attn_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ A_all, const bf16_t* __restrict__ K_all,
     const bf16_t* __restrict__ V_all, const int32_t* __restrict__ idx_all,
     const fm_rowdesc* __restrict__ desc, int G, float scale2, bf16_t* __restrict__ out,

@@ -347,7 +347,8 @@ def main():
                 "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms,
                 "hit_buckets": hit, "mfma_tflops": alg_flops / attn_ms / 1e9}
-    log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M query-heads/s; attention kernel "
+    log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M {'keys/s' if args.config == 'c4' else 'query-heads/s'}"
+        f"; attention kernel "
         f"{attn_ms:.2f} ms = {achieved:.0f} GB/s algorithmic ({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak); "
         f"parts {parts_ms}")
 

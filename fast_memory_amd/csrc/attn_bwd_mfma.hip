@@ -57,6 +57,19 @@ __device__ __forceinline__ uint32_t b_pack(float lo, float hi) {
   return *reinterpret_cast<uint32_t*>(&y);
 }
 
+constexpr int kStLd = 136;  // bf16 elements per staged partial row (128 + 8: 16-byte aligned, banks spread)
+
+// Sum of two rows of eight bf16, rounded to nearest even.
+__device__ __forceinline__ uint4 add_bf16x8(uint4 a, uint4 b) {
+  const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    o[e] = b_pack(__uint_as_float(aw[e] << 16) + __uint_as_float(bw[e] << 16),
+                  __uint_as_float(aw[e] & 0xffff0000u) + __uint_as_float(bw[e] & 0xffff0000u));
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 struct BwdBlock {
   uint4 k[2][4];   // K rows as MFMA operand: [key tile][contraction step], lane (g,c): key c, columns 32s+8g..
   uint4 vk[2][4];  // V rows in the same layout
@@ -85,31 +98,25 @@ __device__ __forceinline__ void bwd_load_block(BwdBlock& r, const bf16_t* __rest
   }
 }
 
-__global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
-    const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
-    const int32_t* __restrict__ q_perm, const fm_item* __restrict__ items, const int32_t* __restrict__ n_items,
-    const bf16_t* __restrict__ out, const float* __restrict__ lse, const bf16_t* __restrict__ dout,
-    bf16_t* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv, int Sq, int N, int C, float sm_scale) {
-  __shared__ __attribute__((aligned(16))) float red[4 * 8 * 4 * 64];  // dQ partials [wave][t][r][lane]
-  __shared__ int q_rows[16];
-  if (int(blockIdx.x) >= *n_items) return;
-  const fm_item it = items[blockIdx.x];
-  const int q0 = int(blockIdx.y) * 16;  // this workgroup's query tile inside the item
-  if (q0 >= it.n_q) return;
-  const int n_q = min(16, it.n_q - q0);
-  const int64_t bkt = int64_t(it.row) * C + it.bucket;
-  const int cnt = bucket_cnt[bkt];
-  if (threadIdx.x < 16) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_perm[it.q_start + q0 + threadIdx.x] : -1;
+// One 16-query tile of a bucket: q_list[0..n_q) are the tile's query rows (inside row `qbase / Sq`).
+// STAGED = false: dK and dV contributions are added atomically into the keys' rows of dKb / dVb (fp32).
+// STAGED = true:  they go to the bucket's own partial rows dkp / dvp [list position][128] in bf16, one row
+//                 per listed key, stored (first tile of the bucket) or added to what the earlier tiles
+//                 left (the workgroup owns the bucket, so no atomics); a second kernel sums every key's
+//                 partial rows over the buckets that list it.
+template <bool STAGED, bool FIRST_TILE>
+__device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ out,
+                                         const float* __restrict__ lse, const bf16_t* __restrict__ dout,
+                                         const int32_t* __restrict__ q_list, int n_q, int64_t qbase,
+                                         const bf16_t* __restrict__ Kb, const bf16_t* __restrict__ Vb,
+                                         const int32_t* __restrict__ idx, int cnt, int N, float sm_scale,
+                                         bf16_t* __restrict__ dq, float* __restrict__ dKb, float* __restrict__ dVb,
+                                         bf16_t* dkp, bf16_t* dvp, bf16_t* dump, float* red, int* q_rows,
+                                         bf16_t* stage) {
+  if (threadIdx.x < 16) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_list[threadIdx.x] : -1;
   __syncthreads();
   const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int g = l >> 4, c = l & 15;
-  const int64_t qbase = int64_t(it.row) * Sq;
-  const bf16_t* Kb = k + int64_t(it.row) * N * kBD;
-  const bf16_t* Vb = v + int64_t(it.row) * N * kBD;
-  float* dKb = dk + int64_t(it.row) * N * kBD;
-  float* dVb = dv + int64_t(it.row) * N * kBD;
-  const int32_t* idx = k_idx + bucket_off[bkt];
   const float scale2 = sm_scale * kLog2e;
 
   // ---- the tile's Q, dO rows: operand fragments in both orientations, lse and D ----
@@ -167,11 +174,13 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
   for (int t = 0; t < 8; ++t) dQ[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int nblk = (cnt + 31) / 32;
+  // Nothing in the block loop branches around a memory instruction: loads past the end of the list are
+  // clamped to its last entry and stores of the staged form are redirected to a dump row, so the
+  // compiler knows how many memory operations follow each load and the wait for a prefetched block does
+  // not drain the stores behind it (loads and stores share one completion counter).
   auto rows_of = [&](int b) -> int {
-    const int kp = b * 32 + (l & 31);
-    int r = 0;
-    if (kp < cnt) r = idx[kp];
-    return min(max(r, 0), N - 1);
+    const int kp = min(b * 32 + (l & 31), max(cnt - 1, 0));
+    return min(max(idx[kp], 0), N - 1);
   };
 
   auto compute = [&](const BwdBlock& kv, int b) {
@@ -240,43 +249,94 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
       // instruction covers, per lane group, 16 consecutive floats (a 64-byte line) of one key's row
       const bf16x4s pA = b_as_bf16x4(make_uint2(b_pack(pr[0], pr[1]), b_pack(pr[2], pr[3])));
       const bf16x4s dsA = b_as_bf16x4(make_uint2(b_pack(dsr[0], dsr[1]), b_pack(dsr[2], dsr[3])));
-      int64_t rowoff[4];
-      bool rok[4];
+      if (STAGED) {
+        // The transposed tiles (the same registers with the operands swapped): lane (g,c) holds key c and
+        // the four consecutive columns 16t + 4g .. +3.  They go through a slab of LDS private to the wave
+        // ([dV | dK][16 keys][136]) and leave as whole rows: 16 adjacent lanes store the 256 bytes of one
+        // key's partial row, an instruction 1 KB of consecutive list positions.
+        bf16_t* slab = stage + w * (2 * 16 * kStLd);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        rowoff[r] = int64_t(__shfl(kv.rk[kt], 4 * g + r)) * kBD + c;
-        rok[r] = kp0 + 16 * kt + 4 * g + r < cnt;
-      }
+        for (int t = 0; t < 8; ++t) {
+          const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+          const f32x4 tv = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(b_as_bf16x4(doT[t]), pA, z, 0, 0, 0);
+          const f32x4 tk = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(b_as_bf16x4(qT[t]), dsA, z, 0, 0, 0);
+          *reinterpret_cast<uint2*>(slab + c * kStLd + 16 * t + 4 * g) =
+              make_uint2(b_pack(tv[0], tv[1]), b_pack(tv[2], tv[3]));
+          *reinterpret_cast<uint2*>(slab + (16 + c) * kStLd + 16 * t + 4 * g) =
+              make_uint2(b_pack(tk[0], tk[1]), b_pack(tk[2], tk[3]));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront", "local");  // LDS only: the wave's writes before its reads below
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        const f32x4 tv = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pA, b_as_bf16x4(doT[t]), z, 0, 0, 0);
-        const f32x4 tk = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(dsA, b_as_bf16x4(qT[t]), z, 0, 0, 0);
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (rok[r]) {
-            unsafeAtomicAdd(dVb + rowoff[r] + 16 * t, tv[r]);
-            unsafeAtomicAdd(dKb + rowoff[r] + 16 * t, tk[r]);
+        for (int i = 0; i < 4; ++i) {
+          const int rr = 4 * i + g;  // key row of the tile; lane chunk c = 16 bytes of it
+          uint4 xv = *reinterpret_cast<const uint4*>(slab + rr * kStLd + 8 * c);
+          uint4 xk = *reinterpret_cast<const uint4*>(slab + (16 + rr) * kStLd + 8 * c);
+          const int pos = kp0 + 16 * kt + rr;
+          const bool ok = pos < cnt;
+          uint4* pv = reinterpret_cast<uint4*>((ok ? dvp + int64_t(pos) * kBD : dump + g * kBD) + 8 * c);
+          uint4* pk = reinterpret_cast<uint4*>((ok ? dkp + int64_t(pos) * kBD : dump + (4 + g) * kBD) + 8 * c);
+          if (!FIRST_TILE) {  // (compile time: a load here, even skipped, would make every store wait)
+            xv = add_bf16x8(xv, *pv);
+            xk = add_bf16x8(xk, *pk);
           }
+          *pv = xv;
+          *pk = xk;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront", "local");  // reads done before the next tile's writes
+      } else {
+        int64_t rowoff[4];
+        bool rok[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          rowoff[r] = int64_t(__shfl(kv.rk[kt], 4 * g + r)) * kBD + c;
+          rok[r] = kp0 + 16 * kt + 4 * g + r < cnt;
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+          const f32x4 tv = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pA, b_as_bf16x4(doT[t]), z, 0, 0, 0);
+          const f32x4 tk = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(dsA, b_as_bf16x4(qT[t]), z, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (rok[r]) {
+              unsafeAtomicAdd(dVb + rowoff[r] + 16 * t, tv[r]);
+              unsafeAtomicAdd(dKb + rowoff[r] + 16 * t, tk[r]);
+            }
+        }
       }
     }
   };
 
   // ---- main loop: this wave's blocks w, w+4, ..., one block in flight ----
-  BwdBlock ra, rb;
-  int b = w;
-  if (b < nblk) bwd_load_block(ra, Kb, Vb, rows_of(b), g, c);
-  while (b < nblk) {
-    const int b1 = b + 4, b2 = b + 8;
-    if (b1 < nblk) bwd_load_block(rb, Kb, Vb, rows_of(b1), g, c);
-    compute(ra, b);
-    if (b1 >= nblk) break;
-    if (b2 < nblk) bwd_load_block(ra, Kb, Vb, rows_of(b2), g, c);
-    compute(rb, b1);
-    b = b2;
+  if (STAGED) {
+    // Two workgroups share a CU (the kernel is held to 256 registers per lane): while one wave waits
+    // for its block, the waves of the other workgroup compute.  A wave keeps one block in registers
+    // and has the list rows of its next block on the way.
+    BwdBlock ra;
+    int rows_nx = rows_of(w);
+    for (int b = w; b < nblk; b += 4) {
+      const int rows = rows_nx;
+      rows_nx = rows_of(b + 4);
+      bwd_load_block(ra, Kb, Vb, rows, g, c);
+      compute(ra, b);
+    }
+  } else {
+    BwdBlock ra, rb;
+    int b = w;
+    if (b < nblk) bwd_load_block(ra, Kb, Vb, rows_of(b), g, c);
+    while (b < nblk) {
+      const int b1 = b + 4, b2 = b + 8;
+      if (b1 < nblk) bwd_load_block(rb, Kb, Vb, rows_of(b1), g, c);
+      compute(ra, b);
+      if (b1 >= nblk) break;
+      if (b2 < nblk) bwd_load_block(ra, Kb, Vb, rows_of(b2), g, c);
+      compute(rb, b1);
+      b = b2;
+    }
   }
 
   // ---- dQ: add the four waves' partial sums, write the tile's rows ----
+  if (STAGED) __syncthreads();  // red shares its LDS with the waves' staging slabs: every wave is past its blocks
 #pragma unroll
   for (int t = 0; t < 8; ++t)
 #pragma unroll
@@ -296,6 +356,70 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
         make_uint4(b_pack(o[0], o[1]), b_pack(o[2], o[3]), b_pack(o[4], o[5]), b_pack(o[6], o[7]));
 }
 
+// grid (items, FM_QTILE / 16): one workgroup per (work item, 16-query tile); dK, dV by atomic adds.
+__global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
+    const int32_t* __restrict__ q_perm, const fm_item* __restrict__ items, const int32_t* __restrict__ n_items,
+    const bf16_t* __restrict__ out, const float* __restrict__ lse, const bf16_t* __restrict__ dout,
+    bf16_t* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv, int Sq, int N, int C, float sm_scale) {
+  __shared__ __attribute__((aligned(16))) float red[4 * 8 * 4 * 64];  // dQ partials [wave][t][r][lane]
+  __shared__ int q_rows[16];
+  if (int(blockIdx.x) >= *n_items) return;
+  const fm_item it = items[blockIdx.x];
+  const int q0 = int(blockIdx.y) * 16;  // this workgroup's query tile inside the item
+  if (q0 >= it.n_q) return;
+  const int64_t bkt = int64_t(it.row) * C + it.bucket;
+  bwd_tile<false, true>(q, out, lse, dout, q_perm + it.q_start + q0, min(16, it.n_q - q0), int64_t(it.row) * Sq,
+                  k + int64_t(it.row) * N * kBD, v + int64_t(it.row) * N * kBD, k_idx + bucket_off[bkt],
+                  bucket_cnt[bkt], N, sm_scale, dq, dk + int64_t(it.row) * N * kBD, dv + int64_t(it.row) * N * kBD,
+                  nullptr, nullptr, nullptr, red, q_rows, nullptr);
+}
+
+// grid (C, rows): one workgroup per (row, bucket) takes the bucket's query tiles one after the other;
+// dK, dV partial rows of the bucket go to dkp / dvp at (flat list position - pos0); dump: 8 rows of
+// 128 bf16 that take the stores of a block's positions past the end of a list.
+__global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
+    const int32_t* __restrict__ q_perm, const int32_t* __restrict__ bin_off, const int32_t* __restrict__ bin_count,
+    const bf16_t* __restrict__ out, const float* __restrict__ lse, const bf16_t* __restrict__ dout,
+    bf16_t* __restrict__ dq, bf16_t* dkp, bf16_t* dvp, bf16_t* dump, int64_t pos0, int row0, int Sq, int N, int C,
+    float sm_scale) {
+  // the waves' staging slabs ([wave][dV | dK][16][kStLd] bf16) during a tile's blocks, then the dQ partial
+  // sums ([wave][t][r][lane] fp32) at its end
+  __shared__ __attribute__((aligned(16))) unsigned char lds_buf[4 * 2 * 16 * kStLd * sizeof(bf16_t)];
+  static_assert(sizeof(lds_buf) >= 4 * 8 * 4 * 64 * sizeof(float), "dQ partials fit the staging slabs");
+  __shared__ int q_rows[16];
+  float* red = reinterpret_cast<float*>(lds_buf);
+  bf16_t* stage = reinterpret_cast<bf16_t*>(lds_buf);
+  const int row = row0 + blockIdx.y;
+  const int64_t bkt = int64_t(row) * C + blockIdx.x;
+  const int nq = bin_count[bkt];
+  const int64_t off = bucket_off[bkt];
+  if (nq <= 0) {  // nobody hashed here: the bucket contributes zero rows
+    const int64_t n16 = int64_t(bucket_cnt[bkt]) * (kBD * sizeof(bf16_t) / 16);
+    uint4* zk = reinterpret_cast<uint4*>(dkp + (off - pos0) * kBD);
+    uint4* zv = reinterpret_cast<uint4*>(dvp + (off - pos0) * kBD);
+    for (int64_t i = threadIdx.x; i < n16; i += 256) zk[i] = zv[i] = make_uint4(0, 0, 0, 0);
+    return;
+  }
+  const int32_t* ql = q_perm + bin_off[bkt];
+  const bf16_t* Kb = k + int64_t(row) * N * kBD;
+  const bf16_t* Vb = v + int64_t(row) * N * kBD;
+  const int cnt = bucket_cnt[bkt];
+  bf16_t* dkb = dkp + (off - pos0) * kBD;
+  bf16_t* dvb = dvp + (off - pos0) * kBD;
+  // the first tile stores the bucket's partial rows, the others add to them
+  bwd_tile<true, true>(q, out, lse, dout, ql, min(16, nq), int64_t(row) * Sq, Kb, Vb, k_idx + off, cnt, N, sm_scale,
+                       dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage);
+  for (int q0 = 16; q0 < nq; q0 += 16) {
+    __syncthreads();  // red and q_rows are reused
+    bwd_tile<true, false>(q, out, lse, dout, ql + q0, min(16, nq - q0), int64_t(row) * Sq, Kb, Vb, k_idx + off, cnt, N,
+                          sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage);
+  }
+}
+
 bool hash_attn_bwd_mfma_supported(int d, int dtype) { return d == kBD && dtype == FM_BF16; }
 
 int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
@@ -307,6 +431,18 @@ int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_
                      (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, (const bf16_t*)out, lse,
                      (const bf16_t*)dout, (bf16_t*)dq, dk, dv, Sq, N, C, sm_scale);
   return launch_status("fm_hash_attn_bwd(mfma)");
+}
+
+int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                                  const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                                  const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
+                                  const void* dout, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0, int row0,
+                                  int rows, int Sq, int N, int C, float sm_scale, hipStream_t st) {
+  hipLaunchKernelGGL(hash_attn_bwd_staged_kernel, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,
+                     (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
+                     bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, (bf16_t*)dq, (bf16_t*)dkp,
+                     (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale);
+  return launch_status("fm_hash_attn_bwd_staged(partials)");
 }
 
 }  // namespace fm

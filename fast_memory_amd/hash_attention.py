@@ -87,7 +87,8 @@ def attention_hash(q, k, v, centroids, bucket_size, sm_scale, window=None):
 
 def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                                    out: torch.Tensor, lse: torch.Tensor, k_hashes: torch.Tensor,
-                                   k_hash_counts: torch.Tensor, q_hashes: torch.Tensor, sm_scale: float
+                                   k_hash_counts: torch.Tensor, q_hashes: torch.Tensor, sm_scale: float,
+                                   staged: Optional[bool] = None, inverse_index=None
                                    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of :func:`attention_hash_varlen` w.r.t. ``q``, ``k`` and ``v``.
 
@@ -96,6 +97,12 @@ def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torc
     ``lse`` are the forward's results (fp32 natural-log LSE) or the ones merged with further keys, in
     which case the gradients are the gathered keys' share.
 
+    :param staged: ``True`` takes the path without atomics (bf16, d=128: per-bucket partial rows, then a
+        sum per key; needs the inverse of the lists), ``False`` the atomic adds; ``None`` picks the staged
+        path when there are at least as many queries per row as buckets, i.e. when most buckets receive
+        queries.
+    :param inverse_index: ``ops.inverse_index(...)`` of these lists, if the caller keeps one (it depends on
+        the lists only); built here otherwise.
     :return: ``(dq [batch, q_seq_len, d_head], dk, dv [batch, kv_seq_len, d_head])``; ``dq`` in q's dtype,
         ``dk`` / ``dv`` in fp32 (sums over every bucket a key belongs to).
     """
@@ -107,6 +114,15 @@ def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torc
     hashes = _as_i32(q_hashes).contiguous()
     off = ops.bucket_offsets(counts)
     groups = ops.group_queries(hashes, n_buckets)
-    return ops.hash_attn_bwd(q, k, v, _as_i32(k_hashes).contiguous(), off, counts, groups, out.contiguous(),
+    lists = _as_i32(k_hashes).contiguous()
+    can_stage = q.dtype == torch.bfloat16 and d_head == 128 and lists.numel() > 0
+    if staged is None:
+        staged = can_stage and q_seq_len >= n_buckets and not ops.generic_kernels_forced()
+    if staged:
+        assert can_stage, "the staged backward takes bf16 with d_head = 128"
+        inv = inverse_index if inverse_index is not None else ops.inverse_index(lists, off, counts, k.shape[1])
+        return ops.hash_attn_bwd_staged(q, k, v, lists, off, counts, groups, inv, out.contiguous(),
+                                        lse.float().contiguous(), d_out.contiguous(), sm_scale)
+    return ops.hash_attn_bwd(q, k, v, lists, off, counts, groups, out.contiguous(),
                              lse.float().contiguous(), d_out.contiguous(), sm_scale)
 

@@ -4,6 +4,8 @@ from __future__ import annotations
 
 from typing import NamedTuple, Optional, Tuple
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -251,6 +253,66 @@ def hash_attn_bwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, o
     return dq, dk, dv
 
 
+class InverseIndex(NamedTuple):
+    """For every key the flat list positions that name it (see ``fm_inverse_index``); depends on the bucket
+    lists only, so it can be kept with them."""
+    key_off: torch.Tensor      # [H*N + 1] int32
+    inv_pos: torch.Tensor      # [T] int32
+    row_pos: Tuple[int, ...]   # H + 1 host integers: flat list position where each row's lists begin
+
+
+def inverse_index(k_idx: torch.Tensor, bucket_off: torch.Tensor, bucket_cnt: torch.Tensor, N: int) -> InverseIndex:
+    """Inverse of the flat bucket lists ``k_idx`` (row-major (row, bucket) order, ``bucket_off`` / ``bucket_cnt``
+    [H,C]) over keys 0..N-1 of every row.  Synchronises once (the rows' list boundaries are read back)."""
+    _dev(k_idx, bucket_off, bucket_cnt)
+    H, C = bucket_cnt.shape
+    T = int(k_idx.numel())
+    assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and bucket_off.dtype == torch.int64
+    lib = _lib.load()
+    dev = k_idx.device
+    key_off = torch.empty(H * N + 1, dtype=torch.int32, device=dev)
+    inv_pos = torch.empty(T, dtype=torch.int32, device=dev)
+    ws = _ws(lib.fm_inverse_index_workspace(T, H, N), k_idx)
+    check(lib.fm_inverse_index(_p(k_idx), _p(bucket_off), _p(bucket_cnt), H, C, int(N), T, _p(key_off), _p(inv_pos),
+                               _p(ws), ws.numel(), _stream(k_idx)))
+    row_pos = tuple(bucket_off[:, 0].cpu().tolist()) + (T,)
+    assert int(bucket_off[-1, -1]) + int(bucket_cnt[-1, -1]) == T, "k_idx must hold exactly the listed entries"
+    return InverseIndex(key_off, inv_pos, row_pos)
+
+
+def hash_attn_bwd_staged(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, inv: InverseIndex, out, lse,
+                         dout, sm_scale: float, dk: Optional[torch.Tensor] = None,
+                         dv: Optional[torch.Tensor] = None, workspace_bytes: int = 24 << 30):
+    """:func:`hash_attn_bwd` without atomics (bf16, d = 128): per-bucket partial rows in a workspace, then a
+    sum per key over the list positions that name it (``inv`` from :func:`inverse_index`).  Same results to
+    rounding (the partial rows are bf16), in a fixed summation order."""
+    _dev(q, k, v, k_idx, bucket_off, bucket_cnt, out, lse, dout)
+    H, Sq, d = q.shape
+    _, N, _ = k.shape
+    C = bucket_cnt.shape[-1]
+    assert k.shape == v.shape and out.shape == q.shape and dout.shape == q.shape and lse.shape == (H, Sq)
+    assert q.dtype == k.dtype == v.dtype == out.dtype == dout.dtype == torch.bfloat16 and d == 128
+    assert len(inv.row_pos) == H + 1 and inv.key_off.numel() == H * N + 1
+    dq = torch.zeros_like(q)                                  # queries of an empty bucket keep 0
+    if dk is None:
+        dk = torch.zeros((H, N, d), dtype=torch.float32, device=q.device)
+    if dv is None:
+        dv = torch.zeros((H, N, d), dtype=torch.float32, device=q.device)
+    assert dk.dtype == dv.dtype == torch.float32 and dk.shape == dv.shape == (H, N, d)
+    lib = _lib.load()
+    longest = max(inv.row_pos[h + 1] - inv.row_pos[h] for h in range(H))
+    total = inv.row_pos[H] - inv.row_pos[0]
+    need_all = lib.fm_hash_attn_bwd_staged_workspace(total)
+    ws = _ws(min(need_all, max(int(workspace_bytes), lib.fm_hash_attn_bwd_staged_workspace(longest))), q)
+    row_pos = (ctypes.c_int64 * (H + 1))(*inv.row_pos)
+    check(lib.fm_hash_attn_bwd_staged(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
+                                      _p(groups.q_perm), _p(groups.bin_off), _p(groups.bin_count), _p(out), _p(lse),
+                                      _p(dout), _p(inv.key_off), _p(inv.inv_pos), _p(dq), _p(dk),
+                                      _p(dv), H, Sq, N, d, C, ctypes.cast(row_pos, ctypes.c_void_p), float(sm_scale),
+                                      _dt(q), _p(ws), ws.numel(), _stream(q)))
+    return dq, dk, dv
+
+
 def attention_hash_varlen_i32(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: float):
     """The reference operator in one C call (triton_kernel.py:51-119) on int32 index tensors."""
     _dev(q, k, v, k_idx, bucket_cnt, q_hash)
@@ -363,6 +425,15 @@ def argtopz_exact_only(on: bool) -> None:
     _lib.load().fm_debug_argtopz_exact_only(int(on))
 
 
+_generic_forced = False
+
+
 def force_generic_kernels(on: bool) -> None:
     """Diagnostic switch: route attention through the generic kernels."""
+    global _generic_forced
+    _generic_forced = bool(on)
     _lib.load().fm_debug_force_generic(int(on))
+
+
+def generic_kernels_forced() -> bool:
+    return _generic_forced

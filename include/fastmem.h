@@ -170,6 +170,41 @@ int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t*
                      const float* lse, const void* dout, void* dq, float* dk, float* dv, int H, int Sq, int N,
                      int d, int C, float sm_scale, int dtype, void* stream);
 
+/* ---- f1, dense query sets: backward without atomics ---------------------------
+ * Same gradients as fm_hash_attn_bwd (bf16, d = 128 only).  A key's dk and dv rows
+ * collect contributions from every bucket that lists it; here each (row, bucket)
+ * workgroup writes the bucket's own partial rows (bf16, one per listed key, in the
+ * workspace) and a second kernel sums, per key, the partial rows of the list
+ * positions that name it -- full-line stores and loads in place of fp32 atomic
+ * read-modify-writes, and a fixed summation order (results do not depend on
+ * scheduling).  Pays when most buckets receive queries: a bucket without queries
+ * still costs its rows (written as zeros and read back).
+ *
+ * fm_inverse_index: the inverse of the lists, which depends on the lists only and
+ * can be kept with them.  T = number of list entries (the sum of bucket_cnt, the
+ * length of k_idx; row-major (row, bucket) order as everywhere).
+ *   key_off [H*N + 1] int32   entries of key (h, n): sorted positions
+ *                              key_off[h*N + n] .. key_off[h*N + n + 1]
+ *   inv_pos [T] int32          flat list positions, ordered by (row, key, position)
+ * fm_hash_attn_bwd_staged: q_perm, bin_off, bin_count from fm_group_queries;
+ * row_pos_host [H+1] (HOST memory) = flat list position where each row's lists
+ * begin (row_pos_host[H] = T); rows are processed in groups whose partial rows
+ * (512 bytes per list entry) fit the workspace, which must hold at least the
+ * longest row (fm_hash_attn_bwd_staged_workspace(entries of that row)).
+ * dq is written, dk and dv (fp32) are accumulated into, as in fm_hash_attn_bwd. */
+size_t fm_inverse_index_workspace(int64_t T, int H, int N);
+int fm_inverse_index(const int32_t* k_idx, const int64_t* bucket_off, const int32_t* bucket_cnt, int H,
+                     int C, int N, int64_t T, int32_t* key_off, int32_t* inv_pos, void* ws, size_t ws_bytes,
+                     void* stream);
+size_t fm_hash_attn_bwd_staged_workspace(int64_t max_row_entries);
+int fm_hash_attn_bwd_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                            const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                            const int32_t* bin_off, const int32_t* bin_count, const void* out,
+                            const float* lse, const void* dout, const int32_t* key_off,
+                            const int32_t* inv_pos, void* dq, float* dk,
+                            float* dv, int H, int Sq, int N, int d, int C, const int64_t* row_pos_host,
+                            float sm_scale, int dtype, void* ws, size_t ws_bytes, void* stream);
+
 /* ---- the reference operator in one call -------------------------------------
  * attention_hash_varlen(q,k,v,k_hashes,k_hash_counts,q_hashes,sm_scale)
  * (triton_kernel.py:51-119): bucket offsets + grouping + attention. */

@@ -32,10 +32,18 @@ def update_out_and_lse(out: Optional[torch.Tensor], lse: Optional[torch.Tensor],
 
 
 # --------------------------------------------------------------------------
+_init_cache = {}
+
+
 def init_centroids(n_buckets: int, d: int, device, dtype) -> torch.Tensor:
-    """The reference's initial centroids (memory.py:489-493)."""
-    rng = np.random.RandomState(42)
-    return torch.tensor(rng.randn(n_buckets, d), device=device, dtype=dtype, requires_grad=False)
+    """The reference's initial centroids (memory.py:489-493).  The seeded host draw and its upload cost a few
+    milliseconds, more than a K-means fit of 2 M keys: the tensor is kept per (shape, device, dtype) and a
+    copy is handed out."""
+    key = (int(n_buckets), int(d), str(torch.device(device)), dtype)
+    if key not in _init_cache:
+        rng = np.random.RandomState(42)
+        _init_cache[key] = torch.tensor(rng.randn(n_buckets, d), device=device, dtype=dtype, requires_grad=False)
+    return _init_cache[key].clone()
 
 
 @torch.no_grad()

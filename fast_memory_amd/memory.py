@@ -225,6 +225,7 @@ class Memory:
 
     def _set_lists(self, bucket_idx: torch.Tensor, bucket_val: Optional[torch.Tensor]):
         self.bucket_idx, self.bucket_val = bucket_idx, bucket_val
+        self._inverse = None
         H, C, L = bucket_idx.shape
         dev = bucket_idx.device
         self.bucket_cnt = torch.full((H, C), L, dtype=torch.int32, device=dev)
@@ -259,6 +260,7 @@ class Memory:
             res = ops.build_index(self.A, self.keys, self.Z, workspace_bytes, return_values=True)
         if res[0] is not self.bucket_idx:
             self._set_lists(*res)
+        self._inverse = None          # the lists changed (possibly in place)
         return self
 
     def save(self, path: str) -> None:
@@ -294,6 +296,34 @@ class Memory:
         groups = ops.group_queries(q_hash, self.n_buckets)
         return ops.hash_attn_fwd(q, self.keys, self.values, self.bucket_idx.reshape(-1), self.bucket_off,
                                  self.bucket_cnt, groups, sm_scale)
+
+    def inverse_index(self) -> "ops.InverseIndex":
+        """For every key the list positions that name it (kept until the lists change); the backward without
+        atomics sums a key's gradient contributions over them."""
+        if getattr(self, "_inverse", None) is None:
+            self._inverse = ops.inverse_index(self.bucket_idx.reshape(-1), self.bucket_off, self.bucket_cnt,
+                                              self.keys.shape[1])
+        return self._inverse
+
+    def attend_backward(self, d_out: torch.Tensor, q: torch.Tensor, out: torch.Tensor, lse: torch.Tensor,
+                        sm_scale: float, q_hash: Optional[torch.Tensor] = None, staged: Optional[bool] = None):
+        """Gradients of :meth:`attend` (memory.py:166-206 on the gathered pairs): ``(dq [H,Sq,d], dk, dv
+        [H,N,d] fp32)`` for ``d_out [H,Sq,d]``; ``out`` / ``lse`` are the forward's results or the ones merged
+        with the local attention (the gradients are then the memory's share).  ``staged`` as in
+        ``attention_hash_varlen_backward``; the staged form reuses :meth:`inverse_index`."""
+        q = q.contiguous()
+        if q_hash is None:
+            q_hash = self.hash(q)
+        groups = ops.group_queries(q_hash, self.n_buckets)
+        lists = self.bucket_idx.reshape(-1)
+        can_stage = q.dtype == torch.bfloat16 and q.shape[2] == 128
+        if staged is None:
+            staged = can_stage and q.shape[1] >= self.n_buckets and not ops.generic_kernels_forced()
+        args = (out.to(q.dtype).contiguous(), lse.float().contiguous(), d_out.to(q.dtype).contiguous(), sm_scale)
+        if staged:
+            return ops.hash_attn_bwd_staged(q, self.keys, self.values, lists, self.bucket_off, self.bucket_cnt,
+                                            groups, self.inverse_index(), *args)
+        return ops.hash_attn_bwd(q, self.keys, self.values, lists, self.bucket_off, self.bucket_cnt, groups, *args)
 
     def attend_with_local(self, q: torch.Tensor, k_local: torch.Tensor, v_local: torch.Tensor,
                           sm_scale: float, n_groups: int, causal: bool = True):

@@ -590,6 +590,41 @@ def test_backward_staged_equals_atomic_and_oracle(ops, ws_bytes):
     assert dk4 is dk0 and torch.allclose(dk4, dk1 + 1.0, atol=1e-6)
 
 
+def test_memory_attend_backward_against_autograd(ops):
+    """Memory.attend_backward (staged form, inverse index kept by the memory) against torch autograd of a dense
+    softmax over each query's bucket, and the kept index is rebuilt after an append."""
+    from fast_memory_amd import Memory
+    g = gen(1650)
+    H, N, C, Z, S, d = 2, 600, 5, 128, 40, 128
+    K = (torch.randn(H, N, d, generator=g) * 0.5).to(torch.bfloat16)
+    V = (torch.randn(H, N, d, generator=g) * 0.5).to(torch.bfloat16)
+    A = torch.randn(H, C, d, generator=g).to(torch.bfloat16)
+    q = (torch.randn(H, S, d, generator=g) * 0.5).to(torch.bfloat16)
+    dout = (torch.randn(H, S, d, generator=g) * 0.5).to(torch.bfloat16)
+    mem = Memory.build(*dev(K, V, A), Z, keep_values=True)
+    qd = dev(q)
+    qh = mem.hash(qd)
+    out, lse = mem.attend(qd, d ** -0.5, q_hash=qh)
+    dq, dk, dv = mem.attend_backward(dev(dout), qd, out, lse, d ** -0.5, q_hash=qh)
+    inv0 = mem.inverse_index()
+    assert mem.inverse_index() is inv0                                   # kept
+    # autograd reference in fp64 on the same lists
+    lists, qhc = mem.bucket_idx.cpu().long(), qh.cpu().long()
+    Kr, Vr, qr = K.double().requires_grad_(), V.double().requires_grad_(), q.double().requires_grad_()
+    outs = []
+    for h in range(H):
+        idx = lists[h][qhc[h]]                                            # [S, Z]
+        s = torch.einsum("sd,szd->sz", qr[h], Kr[h][idx]) * d ** -0.5
+        outs.append(torch.einsum("sz,szd->sd", torch.softmax(s, -1), Vr[h][idx]))
+    torch.stack(outs).backward(dout.double())
+    _assert_grad_close(dq, qr.grad, torch.bfloat16, "dq")
+    _assert_grad_close(dk, Kr.grad, torch.bfloat16, "dk")
+    _assert_grad_close(dv, Vr.grad, torch.bfloat16, "dv")
+    mem.append(dev(K[:, :50].contiguous()), dev(V[:, :50].contiguous()))
+    inv1 = mem.inverse_index()
+    assert inv1 is not inv0 and inv1.key_off.numel() == H * (N + 50) + 1  # rebuilt for the longer memory
+
+
 def test_ring_attention_masked_backward_with_merged_result(ops):
     # memory part of a merged attention: out / lse passed to the backward are those of the softmax over
     # bucket keys and local keys together; checked against autograd through a dense fp64 evaluation

@@ -116,13 +116,19 @@ def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torc
     groups = ops.group_queries(hashes, n_buckets)
     lists = _as_i32(k_hashes).contiguous()
     can_stage = q.dtype == torch.bfloat16 and d_head == 128 and lists.numel() > 0
-    if staged is None:
+    auto = staged is None
+    if auto:
         staged = can_stage and q_seq_len >= n_buckets and not ops.generic_kernels_forced()
     if staged:
         assert can_stage, "the staged backward takes bf16 with d_head = 128"
-        inv = inverse_index if inverse_index is not None else ops.inverse_index(lists, off, counts, k.shape[1])
-        return ops.hash_attn_bwd_staged(q, k, v, lists, off, counts, groups, inv, out.contiguous(),
-                                        lse.float().contiguous(), d_out.contiguous(), sm_scale)
+        try:
+            inv = inverse_index if inverse_index is not None else ops.inverse_index(lists, off, counts, k.shape[1])
+            return ops.hash_attn_bwd_staged(q, k, v, lists, off, counts, groups, inv, out.contiguous(),
+                                            lse.float().contiguous(), d_out.contiguous(), sm_scale)
+        except torch.cuda.OutOfMemoryError:
+            if not auto:
+                raise                      # asked for explicitly: report that its workspace does not fit
+            torch.cuda.empty_cache()       # chosen here: the atomic form needs no workspace
     return ops.hash_attn_bwd(q, k, v, lists, off, counts, groups, out.contiguous(),
                              lse.float().contiguous(), d_out.contiguous(), sm_scale)
 

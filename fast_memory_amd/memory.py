@@ -317,12 +317,18 @@ class Memory:
         groups = ops.group_queries(q_hash, self.n_buckets)
         lists = self.bucket_idx.reshape(-1)
         can_stage = q.dtype == torch.bfloat16 and q.shape[2] == 128
-        if staged is None:
+        auto = staged is None
+        if auto:
             staged = can_stage and q.shape[1] >= self.n_buckets and not ops.generic_kernels_forced()
         args = (out.to(q.dtype).contiguous(), lse.float().contiguous(), d_out.to(q.dtype).contiguous(), sm_scale)
         if staged:
-            return ops.hash_attn_bwd_staged(q, self.keys, self.values, lists, self.bucket_off, self.bucket_cnt,
-                                            groups, self.inverse_index(), *args)
+            try:
+                return ops.hash_attn_bwd_staged(q, self.keys, self.values, lists, self.bucket_off, self.bucket_cnt,
+                                                groups, self.inverse_index(), *args)
+            except torch.cuda.OutOfMemoryError:
+                if not auto:
+                    raise                  # asked for explicitly: report that its workspace does not fit
+                torch.cuda.empty_cache()   # chosen here: the atomic form needs no workspace
         return ops.hash_attn_bwd(q, self.keys, self.values, lists, self.bucket_off, self.bucket_cnt, groups, *args)
 
     def attend_with_local(self, q: torch.Tensor, k_local: torch.Tensor, v_local: torch.Tensor,

@@ -1,6 +1,7 @@
 // Index build on one device (memory.py:260-278 without the collectives):
 // projection rows are produced into the caller's workspace in passes of as
-// many (head, bucket) rows as fit and handed to the selection kernel.
+// many (head, bucket) rows as fit (whole heads when several fit) and handed to
+// the selection kernel.
 #include "common.hpp"
 
 extern "C" size_t fm_build_index_workspace(int H, int C, int N, int d, int Z,
@@ -27,8 +28,20 @@ extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, fl
   const int Zc = Z < N ? Z : N;
   const size_t esz = dtype == FM_BF16 ? 2 : 4;
   float* Y = static_cast<float*>(ws);
-  // passes never straddle heads: each is a bucket range [c0, c0+nc) of one head
-  for (int h = 0; h < H; ++h) {
+  // a pass takes as many whole heads as fit, or a bucket range [c0, c0+nc) of one head
+  for (int h = 0; h < H;) {
+    if (fit >= C) {
+      const int hb = int(std::min<int64_t>(fit / C, H - h));
+      const char* Ah = static_cast<const char*>(A) + int64_t(h) * C * d * esz;
+      const char* Kh = static_cast<const char*>(K) + int64_t(h) * N * d * esz;
+      int rc = fm_project(Ah, Kh, Y, hb, C, N, d, ldy, dtype, stream);
+      if (rc) return rc;
+      rc = fm_argtopz_f32(Y, int64_t(hb) * C, N, ldy, Z, idx_out + int64_t(h) * C * Zc,
+                          val_out ? val_out + int64_t(h) * C * Zc : nullptr, nullptr, 0, stream);
+      if (rc) return rc;
+      h += hb;
+      continue;
+    }
     for (int c0 = 0; c0 < C;) {
       int nc = int(std::min<int64_t>(fit, C - c0));
       const char* Ah = static_cast<const char*>(A) + (int64_t(h) * C + c0) * d * esz;
@@ -40,6 +53,7 @@ extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, fl
       if (rc) return rc;
       c0 += nc;
     }
+    ++h;
   }
   return FM_OK;
 }

@@ -101,7 +101,7 @@ def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int =
         if unresolved == 0:
             return done()
     last_build_info.update(path="unfused")
-    full = lib.fm_build_index_workspace(H, C, N, d, int(Z), C)
+    full = lib.fm_build_index_workspace(H, C, N, d, int(Z), H * C)     # every row at once if the budget allows
     one = lib.fm_build_index_workspace(H, C, N, d, int(Z), 1)
     ws = _ws(max(one, min(full, int(workspace_bytes))), A)
     check(lib.fm_build_index(_p(A), _p(K), _p(out), _p(vals), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(),

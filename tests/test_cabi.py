@@ -42,6 +42,15 @@ def test_argument_errors_are_status_codes():
     assert lib.fm_qhash(None, None, None, None, 1, 1, 1, 8, 7, None) == 1        # bad dtype
     assert lib.fm_lse_merge(None, None, None, None, 5, 8, 0, None) == 1          # null pointers
     assert lib.fm_group_queries(None, 1, 1, 1, None, None, None, None, None, 0, None, 0, None) == 1
+    # the entry points beyond the reference's operator validate the same way, before any device call
+    assert lib.fm_index_append(None, None, 1, 1, None, None, None, None, 1, 1, 1, 1, 1, None, 0, None, None) == 1
+    assert b"fm_index_append" in lib.fm_last_error()
+    assert lib.fm_inverse_index(None, None, None, 1, 1, 1, 1, None, None, None, 0, None) == 1
+    assert lib.fm_hash_attn_bwd(None, None, None, None, None, None, None, None, None, 1, None, None, None, None,
+                                None, None, 1, 1, 1, 8, 1, 1.0, 0, None) != 0
+    assert lib.fm_hash_attn_bwd_staged(*([None] * 17), 1, 1, 1, 64, 1, None, 1.0, 1, None, 0, None) != 0   # d = 64
+    assert b"fm_hash_attn_bwd_staged" in lib.fm_last_error()
+    assert lib.fm_segment_sum(None, None, None, None, None, 1, 1, 1, 8, 0, None) != 0
     with pytest.raises(ValueError):
         _lib.check(1)
 
@@ -52,6 +61,10 @@ def test_workspace_queries():
     assert lib.fm_build_index_workspace(8, 2048, 1048576, 128, 16384, 1) == 1048576 * 4
     assert lib.fm_attention_hash_varlen_workspace(2, 16, 100) > 0
     assert lib.fm_group_queries_workspace(1, 8, 24) >= 8 * 4
+    assert lib.fm_index_append_workspace(2, 3, 5) >= 2 * 3 * 8 * 4           # rows padded to 16 bytes
+    assert lib.fm_hash_attn_bwd_staged_workspace(1000) >= 1000 * 512         # two bf16 rows of 128 per list entry
+    assert lib.fm_inverse_index_workspace(1000, 1, 100) >= 3 * 1000 * 4
+    assert lib.fm_inverse_index_workspace(0, 1, 100) == 0
 
 
 def test_ops_refuse_cpu_tensors():

@@ -287,9 +287,11 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
   };
   // Emission: every lane pops up to two mask bits per column half (lowest register first), reads
   // those values back from its LDS dump (all four reads in flight together) and appends
-  // (value bits, key code) to its segment.  The key code is  first key of the half-tile + 16*(l/32)
-  // + register; fused_key_of_code() turns it into the key index.  A lane without bits reads a
-  // harmless word below its column and stores nothing.
+  // (value bits, key code) pairs to its segment, both pairs of a column half with one 16-byte store:
+  // when only one bit was popped, the second pair lands beyond the cursor and the next append
+  // overwrites it (the overflow guard keeps 16 slots free).  The key code is  first key of the
+  // half-tile + 16*(l/32) + register; fused_key_of_code() turns it into the key index.  A lane
+  // without bits reads a harmless word below its column and stores nothing.
   auto emit = [&](auto check_n, uint32_t code0) {
     bool has[4];
     int r[4];
@@ -297,6 +299,9 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
       uint32_t& m = msk[p >> 1];
+      if constexpr (decltype(check_n)::value) {  // the ragged last tile: drop the bits of rows past N first
+        while (m != 0 && fused_key_of_code(code0 + uint32_t(__builtin_ffs(int(m)) - 1)) >= uint32_t(N)) m &= m - 1u;
+      }
       has[p] = m != 0;
       r[p] = __builtin_ffs(int(m)) - 1;
       m &= m - 1u;
@@ -306,14 +311,13 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     // keep the four reads together ahead of the predicated stores (one LDS round trip, not four)
     asm volatile("" : "+v"(y[0]), "+v"(y[1]), "+v"(y[2]), "+v"(y[3]));
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const int ni = p >> 1;
-      const uint32_t code = code0 + uint32_t(r[p]);
-      bool ok = has[p];
-      if constexpr (decltype(check_n)::value) ok = ok && fused_key_of_code(code) < uint32_t(N);
-      if (ok) {
-        *reinterpret_cast<uint2*>(cbase + off[ni]) = make_uint2(__float_as_uint(y[p]), code);
-        off[ni] += 8u;
+    for (int ni = 0; ni < 2; ++ni) {
+      if (has[2 * ni]) {
+        typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+        const u32x4_t rec = {__float_as_uint(y[2 * ni]), code0 + uint32_t(r[2 * ni]), __float_as_uint(y[2 * ni + 1]),
+                             code0 + uint32_t(r[2 * ni + 1])};
+        *reinterpret_cast<u32x4_t*>(cbase + off[ni]) = rec;
+        off[ni] += has[2 * ni + 1] ? 16u : 8u;
       }
     }
   };

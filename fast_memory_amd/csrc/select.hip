@@ -5,7 +5,7 @@
 // largest value.
 //
 // One workgroup per row.  Two ways to the same result:
-//  * sampled (long rows, Z <= 8192): 1/16 of the row is read as whole 128-byte
+//  * sampled (long rows): 1/16 of the row is read as whole 128-byte
 //    lines spread over the row and kept in registers; the sample's value of rank
 //    mu + 4 sqrt(mu) + 3 (mu = Z n_sample / N) is a threshold that at least Z
 //    elements of the row reach in all but about one row in 30 000.  ONE read of
@@ -28,6 +28,7 @@ bool g_argtopz_exact_only = false;  // test hook: fm_debug_argtopz_exact_only
 
 constexpr int kSampleRegs = 32;  // sampled elements per thread: samples of up to 32768 elements
 constexpr int kCollectRegs = 16; // collected candidates per thread: capacity up to 16384
+constexpr int kCollectRegsWide = 24;  // ... of the form for lists longer than 8192: up to 24576
 
 struct SamplePlan {
   int n_lines;      // sampled 128-byte lines (32 floats each); 0 = exact passes only
@@ -36,9 +37,10 @@ struct SamplePlan {
   int cap;          // candidates the LDS buffer takes
 };
 
-static SamplePlan sample_plan(int N, int Zc, int P, int nt) {
+// `wide`: the form that buffers candidate indices only (lists longer than 8 * nt).
+static SamplePlan sample_plan(int N, int Zc, int P, int nt, bool wide = false) {
   SamplePlan p{0, 0, 0, 0};
-  if (N < 65536 || int64_t(Zc) * 8 > N || P > 8 * nt) return p;
+  if (N < 65536 || int64_t(Zc) * 8 > N || (P > 8 * nt) != wide) return p;
   const int lines = N / 32;                         // whole lines only; a ragged tail is never sampled
   int stride = 16;
   while (lines / stride > kSampleRegs * nt / 32) stride *= 2;
@@ -47,8 +49,13 @@ static SamplePlan sample_plan(int N, int Zc, int P, int nt) {
   const double mu = double(Zc) * ns / N;
   const int rank = int(mu + 4.0 * sqrt(mu) + 3.0);
   const double m_exp = double(rank) * N / ns, m_sd = double(N) / ns * sqrt(double(rank));
-  int cap = 2 * P;
-  while (cap < m_exp + 5.0 * m_sd && cap < kCollectRegs * nt) cap *= 2;
+  int cap;
+  if (wide) {
+    cap = kCollectRegsWide * nt;                    // what the registers take; 4 bytes each in LDS
+  } else {
+    cap = 2 * P;
+    while (cap < m_exp + 5.0 * m_sd && cap < kCollectRegs * nt) cap *= 2;
+  }
   if (cap < m_exp + 5.0 * m_sd || rank * 4 > ns) return p;
   p.n_lines = n_lines;
   p.line_stride = stride;
@@ -71,20 +78,21 @@ struct SampleRegs {
 };
 
 // Candidates collected in LDS, dealt to the threads' registers as composites.
+template <int CR>
 struct CollectedRegs {
-  uint64_t c[kCollectRegs];
+  uint64_t c[CR];
   int n;
   template <typename F>
   __device__ __forceinline__ void operator()(F f) const {
 #pragma unroll
-    for (int r = 0; r < kCollectRegs; ++r)
+    for (int r = 0; r < CR; ++r)
       if (r < n) f(key_to_float(uint32_t(c[r] >> 32)), 0xffffffffu - uint32_t(c[r]));
   }
 };
 
 // row_map / n_rows_dev are optional: when given, workgroup b works on input row
 // b and writes output row row_map[b], and exits if b >= min(*n_rows_dev, grid).
-template <int NT>
+template <int NT, bool WIDE = false>
 __global__ __launch_bounds__(NT) void argtopz_kernel(
     const float* __restrict__ Y, int N, int64_t ldy, int Zc, int P, int32_t* __restrict__ idx_out,
     float* __restrict__ val_out, const int32_t* __restrict__ row_map, const int32_t* __restrict__ n_rows_dev,
@@ -114,17 +122,30 @@ __global__ __launch_bounds__(NT) void argtopz_kernel(
       const uint64_t c = composite(y, i);
       if (c >= tau) {
         const int pos = atomicAdd(&sh.cnt, 1);
-        if (pos < sp.cap) buf[pos] = c;
+        if (pos < sp.cap) {
+          if constexpr (WIDE)
+            reinterpret_cast<uint32_t*>(buf)[pos] = i;
+          else
+            buf[pos] = c;
+        }
       }
     });
     __syncthreads();
     const int m = sh.cnt;
     if (m >= Zc && m <= sp.cap) {
-      CollectedRegs cr;
+      constexpr int CR = WIDE ? kCollectRegsWide : kCollectRegs;
+      CollectedRegs<CR> cr;
       cr.n = tid < m ? (m - tid + NT - 1) / NT : 0;
 #pragma unroll
-      for (int r = 0; r < kCollectRegs; ++r)
-        if (r < cr.n) cr.c[r] = buf[tid + r * NT];
+      for (int r = 0; r < CR; ++r)
+        if (r < cr.n) {
+          if constexpr (WIDE) {
+            const uint32_t i = reinterpret_cast<const uint32_t*>(buf)[tid + r * NT];
+            cr.c[r] = composite(row[i], i);
+          } else {
+            cr.c[r] = buf[tid + r * NT];
+          }
+        }
       const uint64_t cut = radix_select_cut<NT>(cr, Zc, 6, sh);  // (its barriers order the reads above before the writes below)
       collect_sort_write(cr, cut, Zc, P, buf, sh, out, vout);
       return;
@@ -143,12 +164,23 @@ int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int
   // all a thread keeps) and lists of at most 4096.
   SamplePlan sp = sample_plan(N, Zc, P, 512);
   const bool narrow = sp.n_lines > 0 && !g_argtopz_exact_only;
-  if (!narrow) sp = g_argtopz_exact_only ? SamplePlan{0, 0, 0, 0} : sample_plan(N, Zc, P, kSelThreads);
-  const size_t lds = std::max(sort_lds_bytes(P), size_t(sp.cap) * sizeof(uint64_t));
+  bool wide = false;
+  if (!narrow) {
+    sp = g_argtopz_exact_only ? SamplePlan{0, 0, 0, 0} : sample_plan(N, Zc, P, kSelThreads);
+    if (sp.n_lines == 0 && !g_argtopz_exact_only) {
+      sp = sample_plan(N, Zc, P, kSelThreads, true);
+      wide = sp.n_lines > 0;
+    }
+  }
+  const size_t lds = std::max(sort_lds_bytes(P), size_t(sp.cap) * (wide ? sizeof(uint32_t) : sizeof(uint64_t)));
   if (narrow) {
     FM_ALLOW_LDS(argtopz_kernel<512>, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
     hipLaunchKernelGGL(argtopz_kernel<512>, dim3(unsigned(rows)), dim3(512), lds, st, Y, N, ldy, Zc, P, idx_out,
                        val_out, row_map, n_rows_dev, sp);
+  } else if (wide) {
+    FM_ALLOW_LDS((argtopz_kernel<kSelThreads, true>), sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
+    hipLaunchKernelGGL((argtopz_kernel<kSelThreads, true>), dim3(unsigned(rows)), dim3(kSelThreads), lds, st, Y, N,
+                       ldy, Zc, P, idx_out, val_out, row_map, n_rows_dev, sp);
   } else {
     FM_ALLOW_LDS(argtopz_kernel<kSelThreads>, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
     hipLaunchKernelGGL(argtopz_kernel<kSelThreads>, dim3(unsigned(rows)), dim3(kSelThreads), lds, st, Y, N, ldy, Zc,

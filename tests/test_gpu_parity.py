@@ -100,8 +100,9 @@ def test_argtopz_max_z_long_row(ops):
 
 
 def test_argtopz_sampled_one_pass_equals_exact_passes(ops):
-    """Long rows with Z <= 8192 take the sampled one-pass selection; rows the sample misleads fall back inside
-    the kernel.  Both must give the lists of the exact multi-pass selection, bit for bit."""
+    """Long rows take the sampled one-pass selection (lists longer than 8192 in its index-buffer form); rows
+    the sample misleads fall back inside the kernel.  Both must give the lists of the exact multi-pass
+    selection, bit for bit."""
     g = gen(210)
     N = 131072 + 37                                          # ragged tail, rows not 16-byte aligned after row 0
     Y = torch.randn(12, N, generator=g)
@@ -115,7 +116,7 @@ def test_argtopz_sampled_one_pass_equals_exact_passes(ops):
     Y[8] = -torch.arange(N, dtype=torch.float32)
     Y[9, 1000:1000 + 3000] = 7.0                             # a tie block that straddles the cut
     Yd = dev(Y)
-    for Z in (128, 1000, 4096, 8192):
+    for Z in (128, 1000, 4096, 8192, 12000, 16384):
         fast, fv = ops.argtopz(Yd, Z, return_values=True)
         ops.argtopz_exact_only(True)
         try:

@@ -128,6 +128,9 @@ def test_config5_one_million_keys_full_size(ops):
     mem = Memory.build(wl.keys, wl.values, A, Z, keep_values=True)
     check_lists_whole(mem.bucket_idx, mem.bucket_val, N)
     check_lists_sampled(ops, A, wl.keys, mem.bucket_idx, mem.bucket_val, Z, rows_per_head=2)
+    # the chunked build (projection to memory + the dense selection in its long-list form) on some rows of one head
+    part = ops.build_index(A[5:6, 700:796].contiguous(), wl.keys[5:6].contiguous(), Z, fused=False)
+    assert torch.equal(part, mem.bucket_idx[5:6, 700:796])
     q = wl.queries
     scale = d ** -0.5
     # hash: the chosen bucket holds the first maximum of the scores (sampled: the score matrix is 2 GB per head)

@@ -778,6 +778,21 @@ def test_fused_build_bit_identical_to_unfused(ops):
     assert torch.equal(fused.cpu().long(), O.argtopz(Y, Z))
 
 
+@pytest.mark.parametrize("H,C,N,Z", [(1, 513, 65536 + 31, 64),        # one bucket past a 512-bucket slab, ragged key tile
+                                     (3, 1024, 98304, 4096),           # three splits' worth of whole tiles
+                                     (2, 600, 131072 + 1, 2000),       # Z not a power of two, one key past a tile
+                                     (1, 64, 65536, 8192)])            # the longest list N/8 allows here
+def test_fused_build_shapes(ops, H, C, N, Z):
+    g = gen(910 + C)
+    K = _clustered_keys(g, H, N, 128)
+    A = torch.randn(H, C, 128, generator=g).to(torch.bfloat16)
+    Ad, Kd = dev(A, K)
+    fused, fv = ops.build_index(Ad, Kd, Z, fused=True, return_values=True)
+    assert ops.last_build_info["path"] == "fused" and ops.last_build_info["rows_unresolved"] == 0
+    unfused, uv = ops.build_index(Ad, Kd, Z, fused=False, return_values=True)
+    assert torch.equal(fused, unfused) and torch.equal(fv.view(torch.int32), uv.view(torch.int32))
+
+
 def test_fused_build_repairs_rows_whose_sampled_threshold_missed(ops):
     g = gen(901)
     H, C, N, d, Z = 1, 40, 131072, 128, 1024               # sample stride 4: keys 0,4,8,... are sampled

@@ -104,7 +104,13 @@ __device__ __forceinline__ void bwd_load_block(BwdBlock& r, const bf16_t* __rest
 //                 per listed key, stored (first tile of the bucket) or added to what the earlier tiles
 //                 left (the workgroup owns the bucket, so no atomics); a second kernel sums every key's
 //                 partial rows over the buckets that list it.
-template <bool STAGED, bool FIRST_TILE>
+//
+// PAIR (staged form only): q_list holds two tiles, 16 < n_q <= 32.  Waves 0,1 take the first and waves
+// 2,3 the second; waves w and w^2 walk the same key blocks (parity w&1) in step, and what the two tiles
+// add to a block's partial rows is summed through the waves' LDS slabs before it is stored, so the
+// bucket's K and V rows are gathered and its partial rows written once for both tiles.  The sums are
+// those of two single-tile passes (bf16(first) + bf16(second), rounded once more).
+template <bool STAGED, bool FIRST_TILE, bool PAIR = false>
 __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ out,
                                          const float* __restrict__ lse, const bf16_t* __restrict__ dout,
                                          const int32_t* __restrict__ q_list, int n_q, int64_t qbase,
@@ -113,11 +119,18 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
                                          bf16_t* __restrict__ dq, float* __restrict__ dKb, float* __restrict__ dVb,
                                          bf16_t* dkp, bf16_t* dvp, bf16_t* dump, float* red, int* q_rows,
                                          bf16_t* stage) {
-  if (threadIdx.x < 16) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_list[threadIdx.x] : -1;
+  if (threadIdx.x < (PAIR ? 32 : 16)) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_list[threadIdx.x] : -1;
   __syncthreads();
   const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int g = l >> 4, c = l & 15;
   const float scale2 = sm_scale * kLog2e;
+  const int tw = PAIR ? (w >> 1) : 0;  // this wave's tile of the pair
+  q_rows += 16 * tw;
+  auto lds_barrier = [] {  // workgroup barrier that orders LDS only (global stores stay in flight)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  };
 
   // ---- the tile's Q, dO rows: operand fragments in both orientations, lse and D ----
   const int myq = q_rows[c];  // query of lane column c (-1: none)
@@ -265,6 +278,26 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
           *reinterpret_cast<uint2*>(slab + (16 + c) * kStLd + 16 * t + 4 * g) =
               make_uint2(b_pack(tk[0], tk[1]), b_pack(tk[2], tk[3]));
         }
+        if (PAIR) {
+          // both tiles' slabs of this key tile are complete; waves of the first tile store the dV rows,
+          // waves of the second the dK rows, each the sum of the two slabs
+          lds_barrier();
+          const bf16_t* slab_a = stage + (w & 1) * (2 * 16 * kStLd) + tw * (16 * kStLd);        // first tile's wave
+          const bf16_t* slab_b = stage + ((w & 1) + 2) * (2 * 16 * kStLd) + tw * (16 * kStLd);  // second tile's wave
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int rr = 4 * i + g;
+            uint4 x = add_bf16x8(*reinterpret_cast<const uint4*>(slab_a + rr * kStLd + 8 * c),
+                                 *reinterpret_cast<const uint4*>(slab_b + rr * kStLd + 8 * c));
+            const int pos = kp0 + 16 * kt + rr;
+            const bool ok = pos < cnt;
+            bf16_t* base = tw == 0 ? dvp : dkp;
+            uint4* px = reinterpret_cast<uint4*>((ok ? base + int64_t(pos) * kBD : dump + (4 * tw + g) * kBD) + 8 * c);
+            if (!FIRST_TILE) x = add_bf16x8(x, *px);
+            *px = x;
+          }
+          lds_barrier();  // slabs read before the next key tile's writes
+        } else {
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront", "local");  // LDS only: the wave's writes before its reads below
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -283,6 +316,7 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
           *pk = xk;
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront", "local");  // reads done before the next tile's writes
+        }
       } else {
         int64_t rowoff[4];
         bool rok[4];
@@ -313,12 +347,24 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
     // for its block, the waves of the other workgroup compute.  A wave keeps one block in registers
     // and has the list rows of its next block on the way.
     BwdBlock ra;
-    int rows_nx = rows_of(w);
-    for (int b = w; b < nblk; b += 4) {
-      const int rows = rows_nx;
-      rows_nx = rows_of(b + 4);
-      bwd_load_block(ra, Kb, Vb, rows, g, c);
-      compute(ra, b);
+    if (PAIR) {
+      // every wave makes the same number of trips (the barriers inside): a block past the end is
+      // clamped, contributes zeros and stores to the dump rows
+      int rows_nx = rows_of(w & 1);
+      for (int b = w & 1; b < ((nblk + 1) & ~1); b += 2) {
+        const int rows = rows_nx;
+        rows_nx = rows_of(b + 2);
+        bwd_load_block(ra, Kb, Vb, rows, g, c);
+        compute(ra, b);
+      }
+    } else {
+      int rows_nx = rows_of(w);
+      for (int b = w; b < nblk; b += 4) {
+        const int rows = rows_nx;
+        rows_nx = rows_of(b + 4);
+        bwd_load_block(ra, Kb, Vb, rows, g, c);
+        compute(ra, b);
+      }
     }
   } else {
     BwdBlock ra, rb;
@@ -342,6 +388,21 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[((w * 8 + t) * 4 + r) * 64 + l] = dQ[t][r];
   __syncthreads();
+  if (PAIR) {
+    // the two waves of a tile add their sums; wave parity p finalises accumulator rows 2p and 2p+1
+#pragma unroll
+    for (int rr = 0; rr < 2; ++rr) {
+      const int r = 2 * (w & 1) + rr;
+      float o[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t)
+        o[t] = red[(((2 * tw) * 8 + t) * 4 + r) * 64 + l] + red[(((2 * tw + 1) * 8 + t) * 4 + r) * 64 + l];
+      if (myq >= 0)
+        *reinterpret_cast<uint4*>(dq + (qbase + myq) * kBD + 32 * g + 8 * r) =
+            make_uint4(b_pack(o[0], o[1]), b_pack(o[2], o[3]), b_pack(o[4], o[5]), b_pack(o[6], o[7]));
+    }
+    return;
+  }
   // wave w finalises accumulator row r = w: columns 32g + 8w + (0..7) of query c
   float o[8];
 #pragma unroll
@@ -390,7 +451,7 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
   // sums ([wave][t][r][lane] fp32) at its end
   __shared__ __attribute__((aligned(16))) unsigned char lds_buf[4 * 2 * 16 * kStLd * sizeof(bf16_t)];
   static_assert(sizeof(lds_buf) >= 4 * 8 * 4 * 64 * sizeof(float), "dQ partials fit the staging slabs");
-  __shared__ int q_rows[16];
+  __shared__ int q_rows[32];
   float* red = reinterpret_cast<float*>(lds_buf);
   bf16_t* stage = reinterpret_cast<bf16_t*>(lds_buf);
   const int row = row0 + blockIdx.y;
@@ -410,13 +471,26 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
   const int cnt = bucket_cnt[bkt];
   bf16_t* dkb = dkp + (off - pos0) * kBD;
   bf16_t* dvb = dvp + (off - pos0) * kBD;
-  // the first tile stores the bucket's partial rows, the others add to them
-  bwd_tile<true, true>(q, out, lse, dout, ql, min(16, nq), int64_t(row) * Sq, Kb, Vb, k_idx + off, cnt, N, sm_scale,
-                       dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage);
-  for (int q0 = 16; q0 < nq; q0 += 16) {
-    __syncthreads();  // red and q_rows are reused
-    bwd_tile<true, false>(q, out, lse, dout, ql + q0, min(16, nq - q0), int64_t(row) * Sq, Kb, Vb, k_idx + off, cnt, N,
-                          sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage);
+  // the first pass stores the bucket's partial rows, the others add to them; a pass takes two tiles
+  // when more than 16 queries are left
+  for (int q0 = 0; q0 < nq; q0 += 32) {
+    if (q0) __syncthreads();  // red and q_rows are reused
+    const int left = nq - q0;
+#define FM_BWD_PASS(FIRST, PAIRED)                                                                                   \
+  bwd_tile<true, FIRST, PAIRED>(q, out, lse, dout, ql + q0, min(PAIRED ? 32 : 16, left), int64_t(row) * Sq, Kb, Vb,  \
+                                k_idx + off, cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage)
+    if (left > 16) {
+      if (q0 == 0)
+        FM_BWD_PASS(true, true);
+      else
+        FM_BWD_PASS(false, true);
+    } else {
+      if (q0 == 0)
+        FM_BWD_PASS(true, false);
+      else
+        FM_BWD_PASS(false, false);
+    }
+#undef FM_BWD_PASS
   }
 }
 

@@ -105,12 +105,13 @@ __device__ __forceinline__ void bwd_load_block(BwdBlock& r, const bf16_t* __rest
 //                 left (the workgroup owns the bucket, so no atomics); a second kernel sums every key's
 //                 partial rows over the buckets that list it.
 //
-// PAIR (staged form only): q_list holds two tiles, 16 < n_q <= 32.  Waves 0,1 take the first and waves
-// 2,3 the second; waves w and w^2 walk the same key blocks (parity w&1) in step, and what the two tiles
-// add to a block's partial rows is summed through the waves' LDS slabs before it is stored, so the
-// bucket's K and V rows are gathered and its partial rows written once for both tiles.  The sums are
-// those of two single-tile passes (bf16(first) + bf16(second), rounded once more).
-template <bool STAGED, bool FIRST_TILE, bool PAIR = false>
+// TILES = 2 or 4 (staged form only): q_list holds up to TILES tiles, n_q <= 16 * TILES.  With two, waves
+// 0,1 take the first and waves 2,3 the second, and waves w and w^2 walk the same key blocks (parity w&1)
+// in step; with four, every wave has a tile of its own and all walk every block.  What the tiles add to
+// a block's partial rows is summed through the waves' LDS slabs before it is stored, so the bucket's K
+// and V rows are gathered and its partial rows written once for all the tiles of the pass.  The sums are
+// those of single-tile passes in tile order (bf16 rows added and rounded one by one).
+template <bool STAGED, bool FIRST_TILE, int TILES = 1>
 __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ out,
                                          const float* __restrict__ lse, const bf16_t* __restrict__ dout,
                                          const int32_t* __restrict__ q_list, int n_q, int64_t qbase,
@@ -119,12 +120,13 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
                                          bf16_t* __restrict__ dq, float* __restrict__ dKb, float* __restrict__ dVb,
                                          bf16_t* dkp, bf16_t* dvp, bf16_t* dump, float* red, int* q_rows,
                                          bf16_t* stage) {
-  if (threadIdx.x < (PAIR ? 32 : 16)) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_list[threadIdx.x] : -1;
+  if (threadIdx.x < 16 * TILES) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_list[threadIdx.x] : -1;
   __syncthreads();
   const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int g = l >> 4, c = l & 15;
   const float scale2 = sm_scale * kLog2e;
-  const int tw = PAIR ? (w >> 1) : 0;  // this wave's tile of the pair
+  constexpr bool PAIR = TILES == 2, QUAD = TILES == 4;
+  const int tw = PAIR ? (w >> 1) : QUAD ? w : 0;  // this wave's tile of the pass
   q_rows += 16 * tw;
   auto lds_barrier = [] {  // workgroup barrier that orders LDS only (global stores stay in flight)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
@@ -278,7 +280,27 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
           *reinterpret_cast<uint2*>(slab + (16 + c) * kStLd + 16 * t + 4 * g) =
               make_uint2(b_pack(tk[0], tk[1]), b_pack(tk[2], tk[3]));
         }
-        if (PAIR) {
+        if (QUAD) {
+          // the four tiles' slabs of this key tile are complete; wave 0 stores dV rows 0-7, wave 1 dV rows
+          // 8-15, waves 2 and 3 the dK rows likewise, each the sum of the four slabs in tile order
+          lds_barrier();
+          const int mat = w >> 1;  // 0: dV, 1: dK
+#pragma unroll
+          for (int ii = 0; ii < 2; ++ii) {
+            const int rr = 4 * (2 * (w & 1) + ii) + g;
+            const bf16_t* src = stage + mat * (16 * kStLd) + rr * kStLd + 8 * c;
+            uint4 x = *reinterpret_cast<const uint4*>(src);
+#pragma unroll
+            for (int j = 1; j < 4; ++j) x = add_bf16x8(x, *reinterpret_cast<const uint4*>(src + j * (2 * 16 * kStLd)));
+            const int pos = kp0 + 16 * kt + rr;
+            const bool ok = pos < cnt;
+            bf16_t* base = mat == 0 ? dvp : dkp;
+            uint4* px = reinterpret_cast<uint4*>((ok ? base + int64_t(pos) * kBD : dump + (4 * mat + g) * kBD) + 8 * c);
+            if (!FIRST_TILE) x = add_bf16x8(x, *px);
+            *px = x;
+          }
+          lds_barrier();  // slabs read before the next key tile's writes
+        } else if (PAIR) {
           // both tiles' slabs of this key tile are complete; waves of the first tile store the dV rows,
           // waves of the second the dK rows, each the sum of the two slabs
           lds_barrier();
@@ -347,7 +369,15 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
     // for its block, the waves of the other workgroup compute.  A wave keeps one block in registers
     // and has the list rows of its next block on the way.
     BwdBlock ra;
-    if (PAIR) {
+    if (QUAD) {
+      int rows_nx = rows_of(0);
+      for (int b = 0; b < nblk; ++b) {
+        const int rows = rows_nx;
+        rows_nx = rows_of(b + 1);
+        bwd_load_block(ra, Kb, Vb, rows, g, c);
+        compute(ra, b);
+      }
+    } else if (PAIR) {
       // every wave makes the same number of trips (the barriers inside): a block past the end is
       // clamped, contributes zeros and stores to the dump rows
       int rows_nx = rows_of(w & 1);
@@ -388,6 +418,19 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[((w * 8 + t) * 4 + r) * 64 + l] = dQ[t][r];
   __syncthreads();
+  if (QUAD) {
+    // a wave holds all of its tile's sums
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float o[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) o[t] = red[((w * 8 + t) * 4 + r) * 64 + l];
+      if (myq >= 0)
+        *reinterpret_cast<uint4*>(dq + (qbase + myq) * kBD + 32 * g + 8 * r) =
+            make_uint4(b_pack(o[0], o[1]), b_pack(o[2], o[3]), b_pack(o[4], o[5]), b_pack(o[6], o[7]));
+    }
+    return;
+  }
   if (PAIR) {
     // the two waves of a tile add their sums; wave parity p finalises accumulator rows 2p and 2p+1
 #pragma unroll
@@ -440,6 +483,9 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
 // grid (C, rows): one workgroup per (row, bucket) takes the bucket's query tiles one after the other;
 // dK, dV partial rows of the bucket go to dkp / dvp at (flat list position - pos0); dump: 8 rows of
 // 128 bf16 that take the stores of a block's positions past the end of a list.
+// MAXT: the most tiles a pass takes (2 or 4).  The four-tile form costs registers in every path of the
+// kernel that holds it, so it is only launched where buckets receive more than 24 queries on average.
+template <int MAXT>
 __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
@@ -451,7 +497,7 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
   // sums ([wave][t][r][lane] fp32) at its end
   __shared__ __attribute__((aligned(16))) unsigned char lds_buf[4 * 2 * 16 * kStLd * sizeof(bf16_t)];
   static_assert(sizeof(lds_buf) >= 4 * 8 * 4 * 64 * sizeof(float), "dQ partials fit the staging slabs");
-  __shared__ int q_rows[32];
+  __shared__ int q_rows[16 * MAXT];
   float* red = reinterpret_cast<float*>(lds_buf);
   bf16_t* stage = reinterpret_cast<bf16_t*>(lds_buf);
   const int row = row0 + blockIdx.y;
@@ -471,24 +517,28 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
   const int cnt = bucket_cnt[bkt];
   bf16_t* dkb = dkp + (off - pos0) * kBD;
   bf16_t* dvb = dvp + (off - pos0) * kBD;
-  // the first pass stores the bucket's partial rows, the others add to them; a pass takes two tiles
-  // when more than 16 queries are left
-  for (int q0 = 0; q0 < nq; q0 += 32) {
+  // the first pass stores the bucket's partial rows, the others add to them; a pass takes up to MAXT tiles
+  for (int q0 = 0; q0 < nq; q0 += 16 * MAXT) {
     if (q0) __syncthreads();  // red and q_rows are reused
     const int left = nq - q0;
-#define FM_BWD_PASS(FIRST, PAIRED)                                                                                   \
-  bwd_tile<true, FIRST, PAIRED>(q, out, lse, dout, ql + q0, min(PAIRED ? 32 : 16, left), int64_t(row) * Sq, Kb, Vb,  \
-                                k_idx + off, cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage)
-    if (left > 16) {
+#define FM_BWD_PASS(FIRST, NT)                                                                                        \
+  bwd_tile<true, FIRST, NT>(q, out, lse, dout, ql + q0, min(16 * NT, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,  \
+                            cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage)
+    if (MAXT == 4 && left > 32) {
       if (q0 == 0)
-        FM_BWD_PASS(true, true);
+        FM_BWD_PASS(true, MAXT);  // (MAXT, not 4: the two-tile kernel does not instantiate this form)
       else
-        FM_BWD_PASS(false, true);
+        FM_BWD_PASS(false, MAXT);
+    } else if (left > 16) {
+      if (q0 == 0)
+        FM_BWD_PASS(true, 2);
+      else
+        FM_BWD_PASS(false, 2);
     } else {
       if (q0 == 0)
-        FM_BWD_PASS(true, false);
+        FM_BWD_PASS(true, 1);
       else
-        FM_BWD_PASS(false, false);
+        FM_BWD_PASS(false, 1);
     }
 #undef FM_BWD_PASS
   }
@@ -512,10 +562,16 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
                                   const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
                                   const void* dout, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0, int row0,
                                   int rows, int Sq, int N, int C, float sm_scale, hipStream_t st) {
-  hipLaunchKernelGGL(hash_attn_bwd_staged_kernel, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,
-                     (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
-                     bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, (bf16_t*)dq, (bf16_t*)dkp,
-                     (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale);
+#define FM_BWD_STAGED(MAXT)                                                                                        \
+  hipLaunchKernelGGL(hash_attn_bwd_staged_kernel<MAXT>, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,       \
+                     (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,  \
+                     bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, (bf16_t*)dq, (bf16_t*)dkp,  \
+                     (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale)
+  if (int64_t(Sq) > 24 * int64_t(C))  // more than 24 queries per bucket on average
+    FM_BWD_STAGED(4);
+  else
+    FM_BWD_STAGED(2);
+#undef FM_BWD_STAGED
   return launch_status("fm_hash_attn_bwd_staged(partials)");
 }
 

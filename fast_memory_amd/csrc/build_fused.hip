@@ -143,14 +143,15 @@ __global__ __launch_bounds__(256) void gather_sample_kernel(const bf16_t* __rest
 
 // tau[row] = a lower bound of the rank-th largest value of the sampled row that
 // at least `rank` sampled values reach (value bits only: 11+11+10).
-__global__ __launch_bounds__(kSelThreads) void row_threshold_kernel(const float* __restrict__ Ys,
+constexpr int kTauThreads = 256;  // a sampled row is short: narrow workgroups, several rows per CU in flight
+__global__ __launch_bounds__(kTauThreads) void row_threshold_kernel(const float* __restrict__ Ys,
                                                                     int ns, int64_t ld, int rank,
                                                                     float* __restrict__ tau,
                                                                     int32_t* __restrict__ n_fail) {
   __shared__ SelectShared sh;
   if (blockIdx.x == 0 && threadIdx.x < 4) n_fail[threadIdx.x] = 0;
-  DenseRow src{Ys + int64_t(blockIdx.x) * ld, ns};
-  const uint64_t cut = radix_select_cut(src, rank, 3, sh);
+  DenseRowT<kTauThreads> src{Ys + int64_t(blockIdx.x) * ld, ns};
+  const uint64_t cut = radix_select_cut<kTauThreads>(src, rank, 3, sh);
   if (threadIdx.x == 0) tau[blockIdx.x] = key_to_float(uint32_t(cut >> 32));
 }
 
@@ -562,7 +563,7 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
                      dim3(256), 0, st, (const bf16_t*)K, Ks, N, p.ns, p.stride);
   int rc = fm_project(A, Ks, Ys, H, C, p.ns, d, p.ld_s, dtype, stream);
   if (rc) return rc;
-  hipLaunchKernelGGL(row_threshold_kernel, dim3(unsigned(rows)), dim3(kSelThreads), 0, st, Ys, p.ns,
+  hipLaunchKernelGGL(row_threshold_kernel, dim3(unsigned(rows)), dim3(kTauThreads), 0, st, Ys, p.ns,
                      p.ld_s, p.rank, tau, n_fail);
   // phase 1
   mark_phase(1, st);

@@ -470,7 +470,8 @@ __global__ __launch_bounds__(NT) void cand_select_kernel(
 
 // ---- phase 3 ---------------------------------------------------------------
 // Y of the listed (head, bucket) rows, one output column per workgroup row-slot.
-// grid (ceil(N/128), kMaxRepair); 4 waves x 32 keys.
+// grid (up to 128, kMaxRepair): a workgroup walks 128-key tiles (4 waves x 32 keys); with nothing to
+// repair the launch is 8192 workgroups that read one word and leave.
 __global__ __launch_bounds__(256) void project_listed_rows_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const int32_t* __restrict__ fail_rows,
     const int32_t* __restrict__ n_fail, float* __restrict__ Yf, int C, int N, int64_t ldy) {
@@ -479,27 +480,38 @@ __global__ __launch_bounds__(256) void project_listed_rows_kernel(
   const int row = fail_rows[slot];
   const int h = row / C;
   const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int key = blockIdx.x * 128 + w * 32 + (l & 31);
-  const uint4* pk = reinterpret_cast<const uint4*>(K + (int64_t(h) * N + min(key, N - 1)) * kFD + (l >> 5) * 8);
   const uint4* pa = reinterpret_cast<const uint4*>(A + int64_t(row) * kFD + (l >> 5) * 8);
-  f32x16 acc;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  bf16x8 bfr[8];
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
     union {
       uint4 u;
       bf16x8 b;
-    } a, b;
-    a.u = key < N ? pk[2 * ks] : make_uint4(0, 0, 0, 0);
+    } b;
     b.u = (l & 31) == 0 ? pa[2 * ks] : make_uint4(0, 0, 0, 0);  // only column 0 carries the row
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b, b.b, acc, 0, 0, 0);
+    bfr[ks] = b.b;
   }
-  if ((l & 31) == 0) {
+  for (int tile = blockIdx.x; tile * 128 < N; tile += gridDim.x) {
+    const int key = tile * 128 + w * 32 + (l & 31);
+    const uint4* pk = reinterpret_cast<const uint4*>(K + (int64_t(h) * N + min(key, N - 1)) * kFD + (l >> 5) * 8);
+    f32x16 acc;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int n = blockIdx.x * 128 + w * 32 + acc_row_32(r, l);
-      if (n < N) Yf[int64_t(slot) * ldy + n] = acc[r];
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      union {
+        uint4 u;
+        bf16x8 b;
+      } a;
+      a.u = key < N ? pk[2 * ks] : make_uint4(0, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b, bfr[ks], acc, 0, 0, 0);
+    }
+    if ((l & 31) == 0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int n = tile * 128 + w * 32 + acc_row_32(r, l);
+        if (n < N) Yf[int64_t(slot) * ldy + n] = acc[r];
+      }
     }
   }
 }
@@ -588,7 +600,7 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
 #undef FM_CAND_SELECT
   // phase 3
   mark_phase(3, st);
-  hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(ceil_div(N, 128)), kMaxRepair), dim3(256), 0,
+  hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(std::min<int64_t>(ceil_div(N, 128), 128)), kMaxRepair), dim3(256), 0,
                      st, (const bf16_t*)A, (const bf16_t*)K, fail_rows, n_fail, Yf, C, N, p.ldy);
   rc = launch_argtopz(Yf, kMaxRepair, N, p.ldy, Zc, idx_out, val_out, fail_rows, n_fail, st);
   if (rc) return rc;

@@ -330,8 +330,9 @@ __global__ __launch_bounds__(256, 2) void decode_hash_attn_kernel(
   __shared__ int q_rows[FM_QTILE];
   const int row = blockIdx.x, slot = blockIdx.y;
   const fm_rowdesc ds = desc[row];
+  const int qrow = ds.q_row1 ? ds.q_row1 - 1 : row;  // where the row's queries and results live
   const int tid = threadIdx.x, l = tid & 63, w = tid >> 6;
-  const bf16_t* qb = q + int64_t(row) * G * kD;
+  const bf16_t* qb = q + int64_t(qrow) * G * kD;
   // ---- hash on MFMA: 32 buckets x (G queries padded to 32) per v_mfma_f32_32x32x16_bf16 chain,
   //      buckets on the A operand and ascending contraction steps: the sums of the other hash
   //      kernels.  Wave w takes bucket chunks w, w+4, ...; lane (column l%32, half l/32) sees the
@@ -398,7 +399,7 @@ __global__ __launch_bounds__(256, 2) void decode_hash_attn_kernel(
       }
     }
     s_hash[tid] = bi;
-    if (slot == 0) hash_out[int64_t(row) * G + tid] = bi;
+    if (slot == 0) hash_out[int64_t(qrow) * G + tid] = bi;
   }
   __syncthreads();
   // ---- this workgroup's bucket: the slot-th distinct one among the G hashes ----
@@ -422,7 +423,7 @@ __global__ __launch_bounds__(256, 2) void decode_hash_attn_kernel(
   __syncthreads();
   const int n_q = q_rows[FM_QTILE - 1];
   attend_item<1>(qb, q_rows, n_q, Kb, Vb, idx_all + ds.idx_off + int64_t(bkt) * ds.bucket_size, ds.bucket_size,
-                 ds.n_keys, scale2, out + int64_t(row) * G * kD, lse + int64_t(row) * G, red);
+                 ds.n_keys, scale2, out + int64_t(qrow) * G * kD, lse + int64_t(qrow) * G, red);
 }
 
 // Dense attention of one token per query head over L local keys (decode): one workgroup per KV

@@ -375,6 +375,10 @@ class MemoryBatch:
             for _ in range(H):
                 rows.append([a, k, i, N | (C << 32), Z])
                 a, k, i = a + C, k + N, i + C * Z
+        # descriptors go longest lists first (a workgroup's time grows with Z, and the launch then ends
+        # evenly); each names the row of q / out it belongs to (fm_rowdesc.q_row1 = row + 1)
+        order = sorted(range(len(rows)), key=lambda r: -rows[r][4])
+        rows = [rows[r][:4] + [rows[r][4] | ((r + 1) << 32)] for r in order]
         self.desc = torch.tensor(rows, dtype=torch.int64, device=dev)
         self.shapes = [(m.keys.shape[1], m.bucket_idx.shape[1], m.bucket_idx.shape[2]) for m in mems]
 

@@ -333,7 +333,7 @@ def attention_hash_varlen_i32(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: floa
 def decode_hash_attn(q, A_all, K_all, V_all, idx_all, desc, sm_scale: float, return_scores: bool = False):
     """Hash + gathered attention for a decode batch of rows with different memories.
     q [rows,G,d]; A_all [sum C,d]; K_all,V_all [sum N,d]; idx_all flat int32; desc [rows,5] int64
-    viewed as fm_rowdesc (a_off, k_off, idx_off, (n_keys | n_buckets<<32), (bucket_size))."""
+    viewed as fm_rowdesc (a_off, k_off, idx_off, (n_keys | n_buckets<<32), (bucket_size | q_row1<<32))."""
     _dev(q, A_all, K_all, V_all, idx_all, desc)
     rows, G, d = q.shape
     assert desc.dtype == torch.int64 and desc.shape == (rows, 5) and idx_all.dtype == torch.int32

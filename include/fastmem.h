@@ -227,7 +227,10 @@ typedef struct {
   int64_t a_off;        /* first row of this row's A in A_all            */
   int64_t k_off;        /* first key row in K_all / V_all                */
   int64_t idx_off;      /* first element of its bucket lists in idx_all  */
-  int32_t n_keys, n_buckets, bucket_size, reserved;
+  int32_t n_keys, n_buckets, bucket_size;
+  int32_t q_row1;       /* 0: this row's queries are row i of q/out/lse/hash_out, i = position of the
+                           descriptor; else they are row q_row1 - 1 (descriptors may then come in any
+                           order, e.g. longest lists first so that the launch ends evenly)            */
 } fm_rowdesc;
 int fm_decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
                         const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, int d,

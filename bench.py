@@ -137,6 +137,27 @@ def bench_decode_batch(args):
             alg_bytes += len(set(hc[s, hh].tolist())) * Z * (2 * d * 2 + 4) + C * d * 2
     alg_bytes += qheads * (2 * d * 2 + 4)
     achieved = alg_bytes / attn_ms / 1e6
+    # CPU baseline: whole sequences (all heads, hash + bucket attention + local attention + merge), one
+    # after the other until the time budget is used
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import cpu_path
+        threads = min(16, os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        n_done, t_total, seqs = 0, 0.0, 0
+        while seqs < n_seq and t_total < args.cpu_seconds:
+            m = mems[seqs]
+            Kc, Vc, Ac, Lc = m.keys.cpu(), m.values.cpu(), m.A.cpu(), m.bucket_idx.cpu().long()
+            qc, klc, vlc = q[seqs].cpu(), kl[seqs].cpu(), vl[seqs].cpu()
+            for hh in range(H):
+                t_total += cpu_path.time_query_path(qc[hh], Kc[hh], Vc[hh], Ac[hh], Lc[hh], sm_scale, klc[hh], vlc[hh])
+            n_done += H * G
+            seqs += 1
+        cpu = {"value": n_done / t_total, "unit": "query-heads/s", "cores": threads, "kind": "port",
+               "sample": f"sequences 0..{seqs - 1} of {n_seq} (all {H} KV heads, {G} query heads each): hash + "
+                         f"per-bucket gathered softmax attention + local attention over 512 keys + merge; "
+                         f"{t_total:.2f} s"}
+        log(f"[bench] CPU port ({threads} threads): {cpu['value']:.0f} query-heads/s on {seqs} sequences")
     line = {
         "metric": "hashed-attn query-heads/s", "value": qheads / (ms_per_step * 1e-3), "unit": "query-heads/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
@@ -148,7 +169,7 @@ def bench_decode_batch(args):
         "roofline": {"kernel": "decode_hash_attn_kernel", "bound": "hbm", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms},
-        "cpu_baseline": None,
+        "cpu_baseline": cpu,
         "index_build": {"keys_per_s": total_keys / (build_ms * 1e-3), "ms": build_ms, "keys": total_keys},
     }
     log(f"[bench] c3 step {ms_per_step:.3f} ms -> {line['value'] / 1e6:.2f} M query-heads/s; decode kernel "

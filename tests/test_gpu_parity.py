@@ -546,13 +546,15 @@ def test_backward_mfma_and_generic_agree(ops):
             f"{name}: {(a - b).abs().max().item():.3e} vs max {b.abs().max().item():.3e}"
 
 
-@pytest.mark.parametrize("ws_bytes", [24 << 30, 1 << 20])          # everything in one pass; one row per pass
-def test_backward_staged_equals_atomic_and_oracle(ops, ws_bytes):
+@pytest.mark.parametrize("ws_bytes,C", [(24 << 30, 10), (1 << 20, 10),    # everything in one pass; one row per pass
+                                        (24 << 30, 16)])                   # fewer queries per bucket: the two-tile kernel
+def test_backward_staged_equals_atomic_and_oracle(ops, ws_bytes, C):
     """The backward without atomics (per-bucket partial rows, then a sum per key over the inverted lists)
-    against the atomic path and the oracle: buckets with several query tiles, buckets nobody hashed to,
-    ragged and empty lists, keys listed by no bucket."""
+    against the atomic path and the oracle: buckets with several query tiles (passes of one, two and four
+    tiles; the launch takes the four-tile kernel above 24 queries per bucket on average), buckets nobody
+    hashed to, ragged and empty lists, keys listed by no bucket."""
     from fast_memory_amd import attention_hash_varlen
-    B, S, N, C, Z, d = 3, 260, 1500, 10, 200, 128
+    B, S, N, Z, d = 3, 260, 1500, 200, 128
     q, k, v, kh, cnt, qh = make_attn_case(1600, B, S, N, C, Z, d, torch.bfloat16, window="ref", std=0.7)
     qh[0, :120] = 2                                             # 120 queries in one bucket: 8 tiles
     qh[qh == 7] = 8                                             # bucket 7 receives no query

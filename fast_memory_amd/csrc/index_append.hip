@@ -36,15 +36,12 @@ static_assert(kAppendPer * kSelThreads == FM_MAX_Z, "a workgroup's registers hol
 // Every thread reads its share of the old list into registers before the barrier that precedes the
 // first write, so one code path serves both modes.
 template <bool INPLACE, int PER>
-__global__ __launch_bounds__(kSelThreads) void index_append_kernel(
+__device__ __forceinline__ void append_row(
+    int64_t row, uint64_t* nb, int& s_cnt, int (&s_wlast)[PER][kAppendWaves],
     const float* __restrict__ Ynew, int64_t ldm, int M, int n_old, const int32_t* idx_in, const float* val_in, int L_in,
     int32_t* idx_out, float* val_out, int L_out, int Z, int max_new, int32_t* __restrict__ status) {
-  extern __shared__ uint64_t nb[];  // sorted survivors (sort_phys layout), then ahead[max_new]
-  __shared__ int s_cnt;
-  __shared__ int s_wlast[PER][kAppendWaves];
   int* ahead = reinterpret_cast<int*>(nb + sort_lds_bytes(max_new) / sizeof(uint64_t));  // old entries ahead of survivor r
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t row = blockIdx.x;
   const float* y = Ynew + row * ldm;
   const int32_t* ii = idx_in + row * L_in;
   const float* vi = val_in + row * L_in;
@@ -136,12 +133,55 @@ __global__ __launch_bounds__(kSelThreads) void index_append_kernel(
   }
 }
 
+// one workgroup per row
+template <bool INPLACE, int PER>
+__global__ __launch_bounds__(kSelThreads) void index_append_kernel(
+    const float* __restrict__ Ynew, int64_t ldm, int M, int n_old, const int32_t* idx_in, const float* val_in, int L_in,
+    int32_t* idx_out, float* val_out, int L_out, int Z, int max_new, int32_t* __restrict__ status) {
+  extern __shared__ uint64_t nb[];  // sorted survivors (sort_phys layout), then ahead[max_new]
+  __shared__ int s_cnt;
+  __shared__ int s_wlast[PER][kAppendWaves];
+  append_row<INPLACE, PER>(blockIdx.x, nb, s_cnt, s_wlast, Ynew, ldm, M, n_old, idx_in, val_in, L_in, idx_out, val_out,
+                           L_out, Z, max_new, status);
+}
+
+// In place with few new keys, most rows stand as they are (a new key enters a list with probability
+// about Z/N): one thread per row finds the rows some new key enters ...
+__global__ __launch_bounds__(256) void append_precheck_kernel(const float* __restrict__ Ynew, int64_t ldm, int M,
+                                                              int n_old, const int32_t* __restrict__ idx_in,
+                                                              const float* __restrict__ val_in, int L, int64_t rows,
+                                                              int32_t* __restrict__ list, int32_t* __restrict__ n_list) {
+  const int64_t row = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (row >= rows) return;
+  const uint64_t bar = composite(val_in[row * L + L - 1], uint32_t(idx_in[row * L + L - 1]));
+  bool any = false;
+  for (int j = 0; j < M; ++j) any = any || composite(Ynew[row * ldm + j], uint32_t(n_old + j)) > bar;
+  if (any) list[atomicAdd(n_list, 1)] = int32_t(row);
+}
+
+// ... and a fixed number of workgroups walks that list (the order of the list does not matter: rows
+// are independent).
+template <int PER>
+__global__ __launch_bounds__(kSelThreads) void index_append_listed_kernel(
+    const int32_t* __restrict__ list, const int32_t* __restrict__ n_list, const float* __restrict__ Ynew, int64_t ldm,
+    int M, int n_old, int32_t* idx, float* val, int L, int Z, int max_new, int32_t* __restrict__ status) {
+  extern __shared__ uint64_t nb[];
+  __shared__ int s_cnt;
+  __shared__ int s_wlast[PER][kAppendWaves];
+  const int n = *n_list;
+  for (int i = blockIdx.x; i < n; i += gridDim.x) {
+    if (i != int(blockIdx.x)) __syncthreads();  // the row before is done with the shared buffers
+    append_row<true, PER>(list[i], nb, s_cnt, s_wlast, Ynew, ldm, M, n_old, idx, val, L, idx, val, L, Z, max_new, status);
+  }
+}
+
 }  // namespace fm
 
 extern "C" size_t fm_index_append_workspace(int H, int C, int M) {
   if (H < 1 || C < 1 || M < 1) return 0;
   const int64_t ldm = (int64_t(M) + 3) / 4 * 4;
-  return size_t(H) * C * ldm * sizeof(float) + 256;
+  // projections of the new keys, then the list of rows they enter and its length
+  return fm::align_up(size_t(H) * C * ldm * sizeof(float), 256) + fm::align_up(size_t(H) * C * sizeof(int32_t), 256) + 256;
 }
 
 extern "C" int fm_index_append(const void* A, const void* K_new, int n_old, int M, const int32_t* idx_in,
@@ -182,7 +222,27 @@ extern "C" int fm_index_append(const void* A, const void* K_new, int n_old, int 
                        idx_in, val_in, L_in, idx_out, val_out, L_out, Z, max_new, status_dev);                    \
   } while (0)
   const bool small = L_in <= 8 * kSelThreads;  // 8 list entries per thread instead of 16
-  if (inplace) {
+  if (inplace && M <= 64) {
+    // few new keys, lists stay where they are: only the rows a new key enters are touched
+    const int64_t rows = int64_t(H) * C;
+    char* base = static_cast<char*>(ws) + align_up(size_t(rows) * ldm * sizeof(float), 256);
+    int32_t* list = reinterpret_cast<int32_t*>(base);
+    int32_t* n_list = reinterpret_cast<int32_t*>(base + align_up(size_t(rows) * sizeof(int32_t), 256));
+    rc = launch_fill(n_list, 1, 0, st);
+    if (rc) return rc;
+    hipLaunchKernelGGL(append_precheck_kernel, dim3(unsigned(ceil_div(rows, 256))), dim3(256), 0, st, Y, ldm, M, n_old,
+                       idx_in, val_in, L_in, rows, list, n_list);
+    const dim3 lgrid(unsigned(std::min<int64_t>(rows, 1024)));
+    if (small) {
+      FM_ALLOW_LDS((index_append_listed_kernel<8>), lds_max, "fm_index_append: lds");
+      hipLaunchKernelGGL((index_append_listed_kernel<8>), lgrid, dim3(kSelThreads), lds, st, list, n_list, Y, ldm, M,
+                         n_old, idx_out, val_out, L_in, Z, max_new, status_dev);
+    } else {
+      FM_ALLOW_LDS((index_append_listed_kernel<kAppendPer>), lds_max, "fm_index_append: lds");
+      hipLaunchKernelGGL((index_append_listed_kernel<kAppendPer>), lgrid, dim3(kSelThreads), lds, st, list, n_list, Y,
+                         ldm, M, n_old, idx_out, val_out, L_in, Z, max_new, status_dev);
+    }
+  } else if (inplace) {
     if (small) FM_APPEND_LAUNCH(true, 8); else FM_APPEND_LAUNCH(true, kAppendPer);
   } else {
     if (small) FM_APPEND_LAUNCH(false, 8); else FM_APPEND_LAUNCH(false, kAppendPer);

@@ -701,12 +701,15 @@ def test_calc_ref_centroids(ops, dtype):
     (torch.bfloat16, 2, 20, 3000, 1000, 256, 128),
     (torch.bfloat16, 1, 6, 40, 30, 64, 128),              # the lists are not full yet: they grow, then fill
     (torch.bfloat16, 1, 4, 2000, 9000, 8192, 128),        # more new keys than old ones, long lists
+    (torch.bfloat16, 2, 20, 3000, 1, 256, 128),           # few keys into full lists: only the rows they enter are touched
+    (torch.bfloat16, 2, 20, 3000, 40, 256, 128),
+    (torch.float32, 1, 9, 500, 3, 64, 32),
 ])
 def test_append_equals_rebuild(ops, dtype, H, C, N0, M, Z, d, tmp_path):
     from fast_memory_amd import Memory
     g = gen(1700 + M)
     K = torch.randn(H, N0 + 2 * M, d, generator=g).to(dtype)
-    K[:, N0 + 3] = K[:, 5]                                   # a new key that ties with an old one: the old one wins
+    K[:, N0 + min(3, M - 1)] = K[:, 5]                       # a new key that ties with an old one: the old one wins
     V = torch.randn(H, N0 + 2 * M, d, generator=g).to(dtype)
     A = torch.randn(H, C, d, generator=g).to(dtype)
     Kd, Vd, Ad = dev(K, V, A)

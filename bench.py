@@ -252,7 +252,7 @@ def main():
         log(f"[bench] index append: {append}")
 
     # component kernels of the unfused build on one chunk of rows
-    rows = min(C, max(1, min(512, ws_bytes // (N * 4))))
+    rows = min(C, max(1, min(2048, ws_bytes // (N * 4))))
     Asub = A[:1, :rows].contiguous()
     proj_ms, Y = timed(lambda: ops.project(Asub, wl.keys[:1]), reps=3, warm=1)
     sel_ms, _ = timed(lambda: ops.argtopz(Y, Z), reps=3, warm=1)

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the indexed-memory hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c5|c2|c1|c4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c5|c2|c1|c3|c4|tkperf]
 
 One "step" is one pass of the query path over the whole synthetic batch, inputs
 already resident in HBM: query hash -> grouping -> bucket-gathered attention ->
@@ -10,6 +10,9 @@ already resident in HBM: query hash -> grouping -> bucket-gathered attention ->
 (projection + arg-top-Z) and the K-means that produces A are timed beside it
 and reported in the same JSON line, as are the roofline figures of the
 dominant kernel and a CPU baseline on a bounded sample of the same workload.
+``--config tkperf`` is the shape of the reference's own performance harness
+(triton_kernel.py:507-528), whose step is the whole composite ``attention_hash``:
+index build + query hash + attention per call.
 Prints exactly one JSON line on stdout; progress goes to stderr.
 """
 from __future__ import annotations
@@ -70,6 +73,29 @@ def fused_phase_times(run):
         lib.fm_debug_set_phase_events(None, 0)
     names = ["thresholds_ms", "mfma_filter_ms", "select_ms", "repair_ms"]
     return {n: evs[i].elapsed_time(evs[i + 1]) for i, n in enumerate(names)}
+
+
+def calibrate_copy(dev):
+    """Launches copy_probe_kernel over 1 GiB: the kernel of known size that profiler HBM counters are
+    scaled against."""
+    from fast_memory_amd import _lib
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        _lib.check(_lib.load().fm_debug_copy(dst.data_ptr(), src.data_ptr(), src.numel(),
+                                             torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+
+
+def hbm_traffic(kernel, workload):
+    """HBM bytes per launch measured offline with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) and kept as
+    text under profiles/; None when no figure is recorded."""
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    if os.path.exists(tpath):
+        for ln in open(tpath):
+            if ln.strip().startswith(f"{kernel}/{workload}") and "=" in ln:
+                return float(ln.split("=")[1])
+    return None
 
 
 def bench_decode_batch(args):
@@ -177,12 +203,122 @@ def bench_decode_batch(args):
     print(json.dumps(line), flush=True)
 
 
+def bench_reference_harness(args):
+    """The reference's own performance harness (triton_kernel.py:404-412, 475-489, 507-528): 8 rows x 4
+    groups x 32768 queries, 65536 keys, d = 128, 1024 buckets of 3072 keys, q / k / v / centroids ~ N(0,1);
+    one step = attention_hash(q, k, v, centroids, bucket_size, sm_scale), i.e. index build + query hash +
+    grouping + attention, and the figure it prints is the dense-equivalent 4*B*G*S*N*d flops per second.
+    The reference runs it in fp16; bf16 here (same width; the MFMA kernels take bf16)."""
+    from fast_memory_amd import attention_hash, ops
+    B, G, S, N, d, C, Z = 8, 4, 32768, 65536, 128, 1024, 3072
+    Sq = G * S
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    g = torch.Generator(device="cpu").manual_seed(1006)
+    mk = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    k, v, centroids = mk(B, N, d), mk(B, N, d), mk(B, C, d)
+    q = torch.cat([mk(1, Sq, d) for _ in range(B)])
+    sm_scale = d ** -0.5
+    ws_bytes = int(args.workspace_gib * (1 << 30))
+
+    # the parts, each on its own
+    build_ms, lists = timed(lambda: ops.build_index(centroids, k, Z, ws_bytes), reps=3, warm=1)
+    hash_ms, qh = timed(lambda: ops.qhash(centroids, q), reps=3, warm=1)
+    group_ms, groups = timed(lambda: ops.group_queries(qh, C), reps=3, warm=1)
+    off = ops.bucket_offsets(torch.full((B, C), Z, dtype=torch.int32, device=dev))
+    cnt = torch.full((B, C), Z, dtype=torch.int32, device=dev)
+    attn_ms, (mo, ml) = timed(lambda: ops.hash_attn_fwd(q, k, v, lists.reshape(-1), off, cnt, groups, sm_scale),
+                              reps=5, warm=2)
+
+    step = lambda: attention_hash(q, k, v, centroids, Z, sm_scale)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out, lse = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    qheads = B * Sq
+    value = qheads / (ms_per_step * 1e-3)
+    dense_equiv_tflops = 4.0 * B * Sq * N * d / ms_per_step / 1e9          # what the reference prints
+    hit = int((groups.bin_count > 0).sum().item())
+    alg_bytes = hit * Z * (2 * d * 2 + 4) + qheads * (2 * d * 2 + 4)
+    alg_flops = 4.0 * d * Z * qheads
+    achieved = alg_bytes / attn_ms / 1e6
+    roofline = {"kernel": "hash_attn_staged_kernel", "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": hbm_traffic("hash_attn_staged_kernel", "tkperf"),
+                "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms, "hit_buckets": hit,
+                "mfma_tflops": alg_flops / attn_ms / 1e9,
+                "mfma_frac": alg_flops / attn_ms / 1e9 / BF16_MFMA_PEAK_TFLOPS,
+                "note": "128 queries per bucket on average: 127 flop per algorithmic byte; the kernel is bound by "
+                        "its LDS and VALU work per MFMA, not by HBM"}
+    log(f"[bench] tkperf step {ms_per_step:.2f} ms = {dense_equiv_tflops:.0f} dense-equivalent TFLOP/s; build "
+        f"{build_ms:.2f}, hash {hash_ms:.2f}, group {group_ms:.2f}, attention {attn_ms:.2f} ms "
+        f"({achieved:.0f} GB/s algorithmic, {roofline['mfma_tflops']:.0f} TFLOP/s)")
+
+    if args.calibrate_copy:
+        calibrate_copy(dev)
+
+    cpu = None
+    parity = None
+    if not args.no_cpu_baseline:
+        from oracle import cpu_path
+        threads = min(16, os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        K0, V0, A0 = k[0].cpu(), v[0].cpu(), centroids[0].cpu()
+        r = 32
+        tb0 = time.perf_counter()
+        cpu_lists = cpu_path.build_rows(A0[:r], K0, Z)
+        t_build = time.perf_counter() - tb0
+        Yg = ops.project(centroids[:1, :r].contiguous(), k[:1])[0].cpu()
+        ref_lists = torch.sort(Yg + 0.0, dim=-1, descending=True, stable=True)[1][:, :Z]
+        lists0 = lists[0].cpu().long()
+        # the query path of rows 0.. until the time budget is used (the cost is per bucket gathered)
+        n_total, t_total, rows_used = 0, 0.0, 0
+        while rows_used < B and t_total < args.cpu_seconds:
+            b = rows_used
+            t_total += cpu_path.time_query_path(q[b].cpu(), k[b].cpu(), v[b].cpu(), centroids[b].cpu(),
+                                                lists[b].cpu().long(), sm_scale)
+            n_total += Sq
+            rows_used += 1
+        t_row = t_total / rows_used + C * t_build / r                     # one row: its build + its queries
+        cpu = {"value": Sq / t_row, "unit": "query-heads/s", "cores": threads, "kind": "port",
+               "sample": f"rows 0..{rows_used - 1} of {B}: hash + per-bucket gathered softmax attention of all {Sq} "
+                         f"queries of each ({t_total:.2f} s), plus the index build of {r} of {C} bucket rows of row 0 "
+                         f"({t_build:.2f} s) extrapolated to the {C}"}
+        sel = torch.linspace(0, Sq - 1, 4096).long()
+        co, cl, ch = cpu_path.hashed_attention(q[0].cpu()[sel], K0, V0, A0, lists0, sm_scale)
+        same = qh[0].cpu().long()[sel] == ch
+        parity = {"hash_agree_frac": same.float().mean().item(),
+                  "out_max_abs_err": (out[0].float().cpu()[sel][same] - co[same]).abs().max().item(),
+                  "lse_max_abs_err": (lse[0].float().cpu()[sel][same] - cl[same]).abs().max().item(),
+                  "bucket_rows_bit_exact_vs_cpu_stable_sort_of_gpu_Y": bool(torch.equal(ref_lists, lists0[:r]))}
+        log(f"[bench] cpu baseline: {cpu['value']:.1f} query-heads/s on {threads} threads; parity {parity}")
+
+    line = {
+        "metric": "hashed-attn query-heads/s", "value": value, "unit": "query-heads/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"tkperf: the reference's performance harness, {B} rows x {G} groups x {S} queries, "
+                               f"N={N} keys, d={d}, C={C}, Z={Z}, q/k/v/centroids ~ N(0,1)",
+                   "step": "attention_hash: index build + query hash + grouping + gather attention"},
+        "roofline": roofline, "cpu_baseline": cpu,
+        "dense_equivalent_tflops": dense_equiv_tflops,
+        "step_parts_ms": {"index_build": build_ms, "qhash": hash_ms, "group": group_ms, "attention": attn_ms},
+        "index_build": {"keys_per_s": B * N / (build_ms * 1e-3), "ms": build_ms, "keys": B * N,
+                        "path": dict(ops.last_build_info)},
+        "parity_spot_check": parity,
+    }
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="c5", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--config", default="c5", choices=["c1", "c2", "c3", "c4", "c5", "tkperf"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-backward", action="store_true", help="skip timing the backward of the gathered attention")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -202,6 +338,8 @@ def main():
     _lib.load()
     if args.config == "c3":
         return bench_decode_batch(args)
+    if args.config == "tkperf":
+        return bench_reference_harness(args)
     cfg = synth.CONFIGS[args.config]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -376,14 +514,12 @@ def main():
     alg_bytes = hit * Z * (2 * d * e + 4) + qheads * (2 * d * e + 4)
     alg_flops = 4.0 * d * Z * qheads
     achieved = alg_bytes / attn_ms / 1e6
-    traffic = None
-    # measured offline with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) and kept as text under profiles/
-    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
-    if os.path.exists(tpath):
-        for ln in open(tpath):
-            if ln.strip().startswith(f"hash_attn_mfma_kernel/{cfg.name}") and "=" in ln:
-                traffic = float(ln.split("=")[1])
-    roofline = {"kernel": "hash_attn_mfma_kernel" if (d == 128 and e == 2) else "hash_attn_generic_kernel",
+    # the library's dispatch: generic kernel unless bf16 d = 128; of the two MFMA kernels, the one that
+    # stages rows in LDS from 48 queries per bucket on average
+    attn_kernel = ("hash_attn_generic_kernel" if not (d == 128 and e == 2) else
+                   "hash_attn_staged_kernel" if Sq >= 48 * C else "hash_attn_mfma_kernel")
+    traffic = hbm_traffic(attn_kernel, cfg.name)
+    roofline = {"kernel": attn_kernel,
                 "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms,
@@ -407,13 +543,7 @@ def main():
         f"{100 * achieved / read_ceiling:.1f}% of it")
 
     if args.calibrate_copy:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            _lib.check(_lib.load().fm_debug_copy(dst.data_ptr(), src.data_ptr(), src.numel(),
-                                                 torch.cuda.current_stream().cuda_stream))
-        torch.cuda.synchronize()
-        del src, dst
+        calibrate_copy(dev)
 
     # ---- CPU baseline on a bounded sample (head 0), also used as a parity spot check ----
     cpu = None
@@ -469,11 +599,7 @@ def main():
         log(f"[bench] cpu baseline: {cpu['value']:.1f} query-heads/s on {threads} threads; parity {parity}")
 
     if args.config == "c4" and fused_phases:
-        filter_traffic = None
-        if os.path.exists(tpath):
-            for ln in open(tpath):
-                if ln.strip().startswith(f"fused_filter_kernel/{cfg.name}") and "=" in ln:
-                    filter_traffic = float(ln.split("=")[1])
+        filter_traffic = hbm_traffic("fused_filter_kernel", cfg.name)
         roofline = {"kernel": "fused_filter_kernel", "bound": "mfma", "achieved": fused_phases["filter_tflops"],
                     "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": fused_phases["filter_mfma_frac"],
                     "traffic": filter_traffic, "algorithmic_flops_per_launch": 2.0 * H * C * N * d,

@@ -24,7 +24,9 @@ int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const 
                      const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, float sm_scale,
                      void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st);
 
-// 0 = automatic, 1 = force the generic kernels (used by tests to compare paths)
+// 0 = automatic, 1 = force the generic kernels (used by tests to compare paths); for the grouped
+// forward on MFMA, 2 = always the form that stages a bucket's rows in LDS, 3 = always the form that
+// gathers them into registers
 int g_force_generic = 0;
 }  // namespace fm
 
@@ -45,7 +47,7 @@ extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, con
   FM_REQUIRE(max_items >= 1 && max_items <= 0x7fffffffLL, FM_ERR_ARG,
              "fm_hash_attn_fwd: max_items=%lld", (long long)max_items);
   hipStream_t st = as_stream(stream);
-  if (!g_force_generic && hash_attn_mfma_supported(d, dtype))
+  if (g_force_generic != 1 && hash_attn_mfma_supported(d, dtype))
     return hash_attn_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items,
                           out, lse, Sq, N, d, C, sm_scale, st);
   return hash_attn_generic(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
@@ -123,7 +125,7 @@ extern "C" int fm_local_attn_fwd(const void* q, const void* k, const void* v, vo
   FM_REQUIRE(q && k && v && out && lse, FM_ERR_ARG, "fm_local_attn_fwd: null pointer");
   FM_REQUIRE(int64_t(H) * G <= 65535, FM_ERR_UNSUPPORTED, "fm_local_attn_fwd: H*G > 65535");
   hipStream_t st = as_stream(stream);
-  if (!g_force_generic && local_attn_mfma_supported(d, dtype))
+  if (g_force_generic != 1 && local_attn_mfma_supported(d, dtype))
     return local_attn_mfma(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, st);
   return local_attn_generic(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, dtype, st);
 }

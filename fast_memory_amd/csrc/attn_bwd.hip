@@ -121,7 +121,7 @@ extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, con
   FM_REQUIRE(max_items >= 1 && max_items <= 0x7fffffffLL, FM_ERR_ARG, "fm_hash_attn_bwd: max_items=%lld",
              (long long)max_items);
   hipStream_t st = as_stream(stream);
-  if (!g_force_generic && hash_attn_bwd_mfma_supported(d, dtype))
+  if (g_force_generic != 1 && hash_attn_bwd_mfma_supported(d, dtype))
     return hash_attn_bwd_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse,
                               dout, dq, dk, dv, Sq, N, C, sm_scale, st);
   if (dtype == FM_F32)

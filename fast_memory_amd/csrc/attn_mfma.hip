@@ -464,11 +464,22 @@ int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const 
 }
 bool local_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_BF16; }
 
+int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                          const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                          const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
+                          float* lse, int Sq, int N, int C, float sm_scale, hipStream_t st);
+extern int g_force_generic;
+
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
                    const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
                    float* lse, int Sq, int N, int d, int C, float sm_scale, hipStream_t st) {
   (void)d;
+  // Many queries per bucket on average (most work items full): the arithmetic outweighs the gather
+  // and the kernel that shares a bucket's rows through LDS among waves of 16 queries is the faster one.
+  if (g_force_generic == 2 || (g_force_generic == 0 && Sq >= 48 * int64_t(C)))
+    return hash_attn_mfma_staged(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out,
+                                 lse, Sq, N, C, sm_scale, st);
   FM_ALLOW_LDS(hash_attn_mfma_kernel, kRedFloats * sizeof(float), "fm_hash_attn_fwd: lds");
   hipLaunchKernelGGL(hash_attn_mfma_kernel, dim3(unsigned(max_items)), dim3(256),
                      kRedFloats * sizeof(float), st, (const bf16_t*)q, (const bf16_t*)k,

@@ -437,3 +437,13 @@ def force_generic_kernels(on: bool) -> None:
 
 def generic_kernels_forced() -> bool:
     return _generic_forced
+
+
+def grouped_forward_kernel(which: Optional[str]) -> None:
+    """Diagnostic switch for the bf16, d = 128 grouped attention forward: ``"staged"`` always takes the
+    kernel that shares a bucket's rows among its waves through LDS (the choice for many queries per
+    bucket), ``"gather"`` always the one that gathers them into registers, ``None`` restores the
+    dispatch (staged when there are at least 48 queries per bucket on average)."""
+    global _generic_forced
+    _generic_forced = False
+    _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3}[which])

@@ -252,6 +252,35 @@ def test_attention_dense_buckets(dtype, d):
     assert_attn_close(out, lse, ro, rl, dtype, f"dense d={d}")
 
 
+@pytest.mark.parametrize("which", ["staged", "gather"])
+@pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large"])
+def test_attention_grouped_forward_kernels(ops, which, case):
+    # the two bf16 d=128 forward kernels (rows shared through LDS / gathered into registers), each forced,
+    # against the oracle: ragged lists with a last tile of 1..63 keys and empty buckets; buckets with
+    # 1, 15, 16, 17, 63, 64, 65 and 200 queries (several work items, partly filled waves); the
+    # reference's large test shape, where ~20% of the buckets are empty
+    if case == "ragged":
+        q, k, v, kh, cnt, qh = make_attn_case(31, 2, 900, 5000, 24, 333, 128, torch.bfloat16, std=0.7)
+    elif case == "full-items":
+        q, k, v, kh, cnt, qh = make_attn_case(32, 2, 700, 4096, 40, 300, 128, torch.bfloat16, window="all", std=1.0)
+        sizes = [1, 15, 16, 17, 63, 64, 65, 200]
+        pos = 0
+        for b, n in enumerate(sizes):
+            qh[0, pos:pos + n] = b
+            pos += n
+        qh[0, pos:] = torch.randint(len(sizes), 40, (700 - pos,), generator=gen(33))
+    else:
+        q, k, v, kh, cnt, qh = make_attn_case(20, 1, 4 * 2040, 1023 * 60, 512, 1024, 128, torch.bfloat16)
+        assert (cnt == 0).any()
+    ops.grouped_forward_kernel(which)
+    try:
+        out, lse = run_varlen(q, k, v, kh, cnt, qh, 128 ** -0.5)
+    finally:
+        ops.grouped_forward_kernel(None)
+    ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 128 ** -0.5)
+    assert_attn_close(out, lse, ro, rl, torch.bfloat16, f"{which} {case}")
+
+
 def test_attention_special_cases():
     # C=1, Z=N: plain softmax attention; Z=1: out = V[idx]
     g = gen(22)

@@ -25,8 +25,8 @@ int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const 
                      void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st);
 
 // 0 = automatic, 1 = force the generic kernels (used by tests to compare paths); for the grouped
-// forward on MFMA, 2 = always the form that stages a bucket's rows in LDS, 3 = always the form that
-// gathers them into registers
+// forward on MFMA, 2 = always the form that stages a bucket's rows in LDS (4: two work items per
+// workgroup), 3 = always the form that gathers them into registers
 int g_force_generic = 0;
 }  // namespace fm
 

@@ -467,7 +467,7 @@ bool local_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM
 int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
                           const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                          float* lse, int Sq, int N, int C, float sm_scale, hipStream_t st);
+                          float* lse, int Sq, int N, int C, float sm_scale, bool pairs, hipStream_t st);
 extern int g_force_generic;
 
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
@@ -477,9 +477,13 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
   (void)d;
   // Many queries per bucket on average (most work items full): the arithmetic outweighs the gather
   // and the kernel that shares a bucket's rows through LDS among waves of 16 queries is the faster one.
-  if (g_force_generic == 2 || (g_force_generic == 0 && Sq >= 48 * int64_t(C)))
+  // (it addresses rows by 32-bit byte offsets: N * 256 B must stay below 4 GiB)
+  if (N <= (1 << 24) && (g_force_generic == 2 || g_force_generic == 4 || (g_force_generic == 0 && Sq >= 48 * int64_t(C)))) {
+    // from 64 queries per bucket on average, a workgroup takes two work items at once
+    const bool pairs = g_force_generic == 4 || (g_force_generic == 0 && Sq >= 64 * int64_t(C));
     return hash_attn_mfma_staged(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out,
-                                 lse, Sq, N, C, sm_scale, st);
+                                 lse, Sq, N, C, sm_scale, pairs, st);
+  }
   FM_ALLOW_LDS(hash_attn_mfma_kernel, kRedFloats * sizeof(float), "fm_hash_attn_fwd: lds");
   hipLaunchKernelGGL(hash_attn_mfma_kernel, dim3(unsigned(max_items)), dim3(256),
                      kRedFloats * sizeof(float), st, (const bf16_t*)q, (const bf16_t*)k,

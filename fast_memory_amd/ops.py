@@ -441,9 +441,10 @@ def generic_kernels_forced() -> bool:
 
 def grouped_forward_kernel(which: Optional[str]) -> None:
     """Diagnostic switch for the bf16, d = 128 grouped attention forward: ``"staged"`` always takes the
-    kernel that shares a bucket's rows among its waves through LDS (the choice for many queries per
-    bucket), ``"gather"`` always the one that gathers them into registers, ``None`` restores the
-    dispatch (staged when there are at least 48 queries per bucket on average)."""
+    kernel that shares a bucket's rows among its waves through LDS, one work item per workgroup (the
+    choice from 48 queries per bucket on average), ``"staged-pairs"`` the same kernel with two work items
+    per workgroup (from 64), ``"gather"`` always the kernel that gathers the rows into registers,
+    ``None`` restores the dispatch."""
     global _generic_forced
     _generic_forced = False
-    _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3}[which])
+    _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4}[which])

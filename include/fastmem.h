@@ -300,8 +300,9 @@ int fm_segment_sum(const void* X, const int32_t* perm, const int32_t* seg_off, c
 /* Diagnostic: 1 routes the attention entry points through the generic kernels
  * (used by tests to compare the two implementations), 0 restores dispatch.  For
  * fm_hash_attn_fwd on bf16, d = 128 only: 2 = always the kernel that stages a
- * bucket's rows in LDS (dispatch picks it at Sq >= 48 C), 3 = always the kernel
- * that gathers them into registers. */
+ * bucket's rows in LDS, one work item per workgroup (dispatch picks it at
+ * Sq >= 48 C), 4 = the same with two work items per workgroup (Sq >= 64 C),
+ * 3 = always the kernel that gathers the rows into registers. */
 void fm_debug_force_generic(int on);
 
 /* Diagnostic: 1 makes fm_argtopz_f32 (and the chunked index build) take the exact

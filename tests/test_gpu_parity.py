@@ -252,10 +252,11 @@ def test_attention_dense_buckets(dtype, d):
     assert_attn_close(out, lse, ro, rl, dtype, f"dense d={d}")
 
 
-@pytest.mark.parametrize("which", ["staged", "gather"])
+@pytest.mark.parametrize("which", ["staged", "staged-pairs", "gather"])
 @pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large"])
 def test_attention_grouped_forward_kernels(ops, which, case):
-    # the two bf16 d=128 forward kernels (rows shared through LDS / gathered into registers), each forced,
+    # the bf16 d=128 forward kernels (rows shared through LDS, one or two work items per workgroup / rows
+    # gathered into registers), each forced,
     # against the oracle: ragged lists with a last tile of 1..63 keys and empty buckets; buckets with
     # 1, 15, 16, 17, 63, 64, 65 and 200 queries (several work items, partly filled waves); the
     # reference's large test shape, where ~20% of the buckets are empty

@@ -246,8 +246,9 @@ def bench_reference_harness(args):
     alg_bytes = hit * Z * (2 * d * 2 + 4) + qheads * (2 * d * 2 + 4)
     alg_flops = 4.0 * d * Z * qheads
     achieved = alg_bytes / attn_ms / 1e6
-    roofline = {"kernel": "hash_attn_staged_kernel", "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": hbm_traffic("hash_attn_staged_kernel", "tkperf"),
+    attn_kernel = ops.hash_attn_fwd_kernel_name(B, Sq, N, d, C, torch.bfloat16)
+    roofline = {"kernel": attn_kernel, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": hbm_traffic(attn_kernel, "tkperf"),
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms, "hit_buckets": hit,
                 "mfma_tflops": alg_flops / attn_ms / 1e9,
                 "mfma_frac": alg_flops / attn_ms / 1e9 / BF16_MFMA_PEAK_TFLOPS,
@@ -514,10 +515,7 @@ def main():
     alg_bytes = hit * Z * (2 * d * e + 4) + qheads * (2 * d * e + 4)
     alg_flops = 4.0 * d * Z * qheads
     achieved = alg_bytes / attn_ms / 1e6
-    # the library's dispatch: generic kernel unless bf16 d = 128; of the two MFMA kernels, the one that
-    # stages rows in LDS from 48 queries per bucket on average
-    attn_kernel = ("hash_attn_generic_kernel" if not (d == 128 and e == 2) else
-                   "hash_attn_staged_kernel" if Sq >= 48 * C else "hash_attn_mfma_kernel")
+    attn_kernel = ops.hash_attn_fwd_kernel_name(H, Sq, N, d, C, cfg.dtype)     # what the library's dispatch took
     traffic = hbm_traffic(attn_kernel, cfg.name)
     roofline = {"kernel": attn_kernel,
                 "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -15,7 +15,8 @@ bool hash_attn_mfma_supported(int d, int dtype);
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
                    const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                   float* lse, int Sq, int N, int d, int C, float sm_scale, hipStream_t st);
+                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, hipStream_t st);
+int hash_attn_mfma_choice(int H, int Sq, int N, int C);
 bool local_attn_mfma_supported(int d, int dtype);
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
                     int S, int L, int d, float sm_scale, int causal, hipStream_t st);
@@ -31,6 +32,16 @@ int g_force_generic = 0;
 }  // namespace fm
 
 extern "C" void fm_debug_force_generic(int on) { fm::g_force_generic = on; }
+
+extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype) {
+  using namespace fm;
+  if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype)) return "hash_attn_generic_kernel";
+  switch (hash_attn_mfma_choice(H, Sq, N, C)) {
+    case 1: return "hash_attn_staged_kernel<1>";
+    case 2: return "hash_attn_staged_kernel<2>";
+    default: return "hash_attn_mfma_kernel";
+  }
+}
 
 extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
                                 const int64_t* bucket_off, const int32_t* bucket_cnt,
@@ -49,7 +60,7 @@ extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, con
   hipStream_t st = as_stream(stream);
   if (g_force_generic != 1 && hash_attn_mfma_supported(d, dtype))
     return hash_attn_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items,
-                          out, lse, Sq, N, d, C, sm_scale, st);
+                          out, lse, H, Sq, N, d, C, sm_scale, st);
   return hash_attn_generic(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
                            max_items, out, lse, Sq, N, d, C, sm_scale, dtype, st);
 }

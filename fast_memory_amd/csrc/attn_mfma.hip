@@ -470,20 +470,32 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
                           float* lse, int Sq, int N, int C, float sm_scale, bool pairs, hipStream_t st);
 extern int g_force_generic;
 
+// Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
+// staged in LDS, one work item per workgroup, 2 = staged, two items per workgroup.  Measured rule: the
+// staged kernel is at least as fast wherever the launch has work items enough to fill the chip (at
+// least 512, taking min(Sq, C) per row as their number) or buckets receive 24 queries or more on
+// average; with few and small items the four waves of the gather kernel, which share one bucket's
+// keys, finish an item sooner.  Two items per workgroup from 64 queries per bucket on average.
+// (The staged kernel addresses rows by 32-bit byte offsets: N * 256 B must stay below 4 GiB.)
+int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
+  if (g_force_generic == 3 || N > (1 << 24)) return 0;
+  if (g_force_generic == 2) return 1;
+  if (g_force_generic == 4) return 2;
+  const bool many_items = int64_t(H) * (Sq < C ? Sq : C) >= 512;
+  const bool dense = Sq >= 24 * int64_t(C);
+  if (!many_items && !dense) return 0;
+  return (Sq >= 64 * int64_t(C) && many_items) ? 2 : 1;
+}
+
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
                    const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                   float* lse, int Sq, int N, int d, int C, float sm_scale, hipStream_t st) {
+                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, hipStream_t st) {
   (void)d;
-  // Many queries per bucket on average (most work items full): the arithmetic outweighs the gather
-  // and the kernel that shares a bucket's rows through LDS among waves of 16 queries is the faster one.
-  // (it addresses rows by 32-bit byte offsets: N * 256 B must stay below 4 GiB)
-  if (N <= (1 << 24) && (g_force_generic == 2 || g_force_generic == 4 || (g_force_generic == 0 && Sq >= 48 * int64_t(C)))) {
-    // from 64 queries per bucket on average, a workgroup takes two work items at once
-    const bool pairs = g_force_generic == 4 || (g_force_generic == 0 && Sq >= 64 * int64_t(C));
+  const int choice = hash_attn_mfma_choice(H, Sq, N, C);
+  if (choice)
     return hash_attn_mfma_staged(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out,
-                                 lse, Sq, N, C, sm_scale, pairs, st);
-  }
+                                 lse, Sq, N, C, sm_scale, choice == 2, st);
   FM_ALLOW_LDS(hash_attn_mfma_kernel, kRedFloats * sizeof(float), "fm_hash_attn_fwd: lds");
   hipLaunchKernelGGL(hash_attn_mfma_kernel, dim3(unsigned(max_items)), dim3(256),
                      kRedFloats * sizeof(float), st, (const bf16_t*)q, (const bf16_t*)k,

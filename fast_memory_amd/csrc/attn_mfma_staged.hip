@@ -1,8 +1,9 @@
-// bf16 bucket-gathered attention forward for head dimension 128 (gfx950), the form for
-// launches whose work items are mostly full (many queries per bucket, e.g. the shape of the
-// reference's own performance harness, triton_kernel.py:507-528: 128 queries per bucket).
-// There the arithmetic, not the gather, is the larger part, and the register-gather kernel
-// (attn_mfma.hip) runs one wave per SIMD with every MFMA, softmax and load of a wave in series.
+// bf16 bucket-gathered attention forward for head dimension 128 (gfx950) with a bucket's rows
+// staged in LDS (triton_kernel.py:137-272).  The kernel of every launch that has work items enough
+// to fill the chip or buckets with many queries (the register-gather kernel of attn_mfma.hip keeps
+// the launches with few, small items): from the HBM-bound shapes (16 queries per bucket over a
+// million keys) to the shape of the reference's own performance harness (triton_kernel.py:507-528,
+// 128 queries per bucket), where the arithmetic is the larger part.
 //
 // Work decomposition.  One workgroup (4 waves) per work item (up to 64 queries of one bucket), or
 // per two consecutive items of a bucket; wave w carries 16 (or 32) of the queries over ALL keys of

@@ -439,12 +439,18 @@ def generic_kernels_forced() -> bool:
     return _generic_forced
 
 
+def hash_attn_fwd_kernel_name(H: int, Sq: int, N: int, d: int, C: int, dtype: torch.dtype) -> str:
+    """Name of the kernel :func:`hash_attn_fwd` launches for these extents."""
+    code = 1 if dtype == torch.bfloat16 else 0
+    return _lib.load().fm_hash_attn_fwd_kernel(H, Sq, N, d, C, code).decode()
+
+
 def grouped_forward_kernel(which: Optional[str]) -> None:
     """Diagnostic switch for the bf16, d = 128 grouped attention forward: ``"staged"`` always takes the
-    kernel that shares a bucket's rows among its waves through LDS, one work item per workgroup (the
-    choice from 48 queries per bucket on average), ``"staged-pairs"`` the same kernel with two work items
-    per workgroup (from 64), ``"gather"`` always the kernel that gathers the rows into registers,
-    ``None`` restores the dispatch."""
+    kernel that shares a bucket's rows among its waves through LDS, one work item per workgroup,
+    ``"staged-pairs"`` the same kernel with two work items per workgroup, ``"gather"`` always the kernel
+    that gathers the rows into registers, ``None`` restores the dispatch (staged unless the launch has few
+    and small work items; pairs from 64 queries per bucket on average)."""
     global _generic_forced
     _generic_forced = False
     _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4}[which])

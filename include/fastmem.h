@@ -300,10 +300,18 @@ int fm_segment_sum(const void* X, const int32_t* perm, const int32_t* seg_off, c
 /* Diagnostic: 1 routes the attention entry points through the generic kernels
  * (used by tests to compare the two implementations), 0 restores dispatch.  For
  * fm_hash_attn_fwd on bf16, d = 128 only: 2 = always the kernel that stages a
- * bucket's rows in LDS, one work item per workgroup (dispatch picks it at
- * Sq >= 48 C), 4 = the same with two work items per workgroup (Sq >= 64 C),
- * 3 = always the kernel that gathers the rows into registers. */
+ * bucket's rows in LDS, one work item per workgroup, 4 = the same with two work
+ * items per workgroup, 3 = always the kernel that gathers the rows into
+ * registers (dispatch: staged when H min(Sq, C) >= 512 or Sq >= 24 C, two items
+ * from Sq >= 64 C; gather otherwise). */
 void fm_debug_force_generic(int on);
+
+/* Diagnostic: name of the kernel fm_hash_attn_fwd launches for these extents
+ * (a static string): "hash_attn_generic_kernel", "hash_attn_mfma_kernel" (rows
+ * gathered into registers), "hash_attn_staged_kernel<1>" or "...<2>" (rows staged
+ * in LDS, one or two work items per workgroup).  bench.py names its roofline
+ * kernel with it. */
+const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype);
 
 /* Diagnostic: 1 makes fm_argtopz_f32 (and the chunked index build) take the exact
  * multi-pass selection for every row instead of the sampled one-pass form (tests

@@ -147,6 +147,8 @@ extern "C" int fm_decode_hash_attn(const void* q, const void* A_all, const void*
                                    int32_t* hash_out, float* scores_out, int dtype, void* stream) {
   using namespace fm;
   FM_REQUIRE(rows >= 0 && G >= 1 && G <= 16, FM_ERR_ARG, "fm_decode_hash_attn: rows=%d G=%d", rows, G);
+  FM_REQUIRE(int64_t(rows) * G <= 0x7fffffffLL, FM_ERR_UNSUPPORTED, "fm_decode_hash_attn: rows * G = %lld workgroups",
+             (long long)(int64_t(rows) * G));
   FM_REQUIRE(dtype == FM_BF16 && d == 128, FM_ERR_UNSUPPORTED,
              "fm_decode_hash_attn: built for bf16, d=128 (got dtype=%d d=%d)", dtype, d);
   if (rows == 0) return FM_OK;

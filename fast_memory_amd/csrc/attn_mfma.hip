@@ -328,7 +328,9 @@ __global__ __launch_bounds__(256, 2) void decode_hash_attn_kernel(
   __shared__ int s_besti[4][16];
   __shared__ int s_hash[16];
   __shared__ int q_rows[FM_QTILE];
-  const int row = blockIdx.x, slot = blockIdx.y;
+  // the G workgroups of a row are neighbours in launch order: with descriptors given longest lists
+  // first, the longest buckets of the whole batch start first
+  const int row = blockIdx.x / unsigned(G), slot = blockIdx.x % unsigned(G);
   const fm_rowdesc ds = desc[row];
   const int qrow = ds.q_row1 ? ds.q_row1 - 1 : row;  // where the row's queries and results live
   const int tid = threadIdx.x, l = tid & 63, w = tid >> 6;
@@ -456,7 +458,7 @@ bool hash_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_
 int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
                      const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, float sm_scale,
                      void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st) {
-  hipLaunchKernelGGL(decode_hash_attn_kernel, dim3(unsigned(rows), unsigned(G)), dim3(256), red_floats(1) * sizeof(float),
+  hipLaunchKernelGGL(decode_hash_attn_kernel, dim3(unsigned(rows) * unsigned(G)), dim3(256), red_floats(1) * sizeof(float),
                      st, (const bf16_t*)q, (const bf16_t*)A_all, (const bf16_t*)K_all,
                      (const bf16_t*)V_all, idx_all, desc, G, sm_scale * kLog2e, (bf16_t*)out, lse, hash_out,
                      scores_out);

@@ -282,6 +282,34 @@ def test_attention_grouped_forward_kernels(ops, which, case):
     assert_attn_close(out, lse, ro, rl, torch.bfloat16, f"{which} {case}")
 
 
+@pytest.mark.parametrize("which", ["staged", "staged-pairs", "gather", "generic"])
+def test_attention_out_of_range_list_entries_are_clamped(ops, which):
+    # the contract of every entry point: key indices outside [0, N) are clamped, never dereferenced
+    # (negative -> key 0, >= N -> key N-1); lists here hold such entries in every bucket, and lists
+    # shorter than one 64-key tile
+    N = 3000
+    q, k, v, kh, cnt, qh = make_attn_case(35, 2, 300, N, 12, 150, 128, torch.bfloat16, window="all", std=0.7)
+    kh = kh.reshape(2, 12, 150).clone()
+    kh[:, :, 3] = -7
+    kh[:, :, 77] = N + 1000
+    kh[:, :, 149] = 2 ** 31 - 1
+    cnt = cnt.clone()
+    cnt[0, 5] = 40                                               # a single ragged tile
+    cnt[1, 2] = 1
+    flat = torch.cat([kh[b, c, : int(cnt[b, c])] for b in range(2) for c in range(12)])
+    if which == "generic":
+        ops.force_generic_kernels(True)
+    else:
+        ops.grouped_forward_kernel(which)
+    try:
+        out, lse = run_varlen(q, k, v, flat, cnt, qh, 128 ** -0.5)
+    finally:
+        ops.force_generic_kernels(False)
+        ops.grouped_forward_kernel(None)
+    ro, rl = O.hashed_attention_gather(q, k, v, flat.clamp(0, N - 1), cnt, qh, 128 ** -0.5)
+    assert_attn_close(out, lse, ro, rl, torch.bfloat16, f"{which} clamped indices")
+
+
 def test_attention_special_cases():
     # C=1, Z=N: plain softmax attention; Z=1: out = V[idx]
     g = gen(22)

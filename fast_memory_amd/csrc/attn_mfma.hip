@@ -318,6 +318,10 @@ __global__ __launch_bounds__(256) void hash_attn_mfma_kernel(
 // bucket among the G hashes with the queries that chose it, or exits if there are
 // fewer distinct buckets.  Each bucket is read once, and a row's buckets in parallel.  Rows are described by fm_rowdesc; A, K, V
 // and the bucket lists of all rows are packed back to back.
+// MODE 0: hash and attend in one launch; 1: hash only (one workgroup per row, writes hash_out); 2:
+// attend only, on the hashes a MODE 1 launch left in hash_out.  Two launches take the hash off the
+// path of the G workgroups of a row, which otherwise each repeat it before their first key load.
+template <int MODE>
 __global__ __launch_bounds__(256, 2) void decode_hash_attn_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ A_all, const bf16_t* __restrict__ K_all,
     const bf16_t* __restrict__ V_all, const int32_t* __restrict__ idx_all,
@@ -330,80 +334,87 @@ __global__ __launch_bounds__(256, 2) void decode_hash_attn_kernel(
   __shared__ int q_rows[FM_QTILE];
   // the G workgroups of a row are neighbours in launch order: with descriptors given longest lists
   // first, the longest buckets of the whole batch start first
-  const int row = blockIdx.x / unsigned(G), slot = blockIdx.x % unsigned(G);
+  const int row = MODE == 1 ? int(blockIdx.x) : int(blockIdx.x / unsigned(G));
+  const int slot = MODE == 1 ? 0 : int(blockIdx.x % unsigned(G));
   const fm_rowdesc ds = desc[row];
   const int qrow = ds.q_row1 ? ds.q_row1 - 1 : row;  // where the row's queries and results live
   const int tid = threadIdx.x, l = tid & 63, w = tid >> 6;
   const bf16_t* qb = q + int64_t(qrow) * G * kD;
-  // ---- hash on MFMA: 32 buckets x (G queries padded to 32) per v_mfma_f32_32x32x16_bf16 chain,
-  //      buckets on the A operand and ascending contraction steps: the sums of the other hash
-  //      kernels.  Wave w takes bucket chunks w, w+4, ...; lane (column l%32, half l/32) sees the
-  //      scores of its query for 16 buckets of a chunk in ascending order.
-  typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
-  const int C = ds.n_buckets;
-  const int col = l & 31, hb = l >> 5;
-  bf16x8 bq[8];
-  {
-    const uint4* pq = reinterpret_cast<const uint4*>(qb + int64_t(col < G ? col : 0) * kD + hb * 8);
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) bq[ks] = as_bf16x8(col < G ? pq[2 * ks] : make_uint4(0, 0, 0, 0));
-  }
-  float best = -INFINITY;
-  int besti = 0x7fffffff;
-  for (int c0 = 32 * w; c0 < C; c0 += 128) {
-    const int cr = min(c0 + col, C - 1);
-    const uint4* pa = reinterpret_cast<const uint4*>(A_all + (ds.a_off + cr) * kD + hb * 8);
-    uint4 au[8];
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) au[ks] = pa[2 * ks];
-    f32x16 acc;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(au[ks]), bq[ks], acc, 0, 0, 0);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int c = c0 + 8 * (r >> 2) + 4 * hb + (r & 3);
-      if (c < C && col < G) {
-        if (scores_out && slot == 0) scores_out[(ds.a_off + c) * G + col] = acc[r];
-        if (besti == 0x7fffffff || acc[r] > best) {  // buckets ascend per lane
-          best = acc[r];
-          besti = c;
+  if constexpr (MODE != 2) {
+    // ---- hash on MFMA: 32 buckets x (G queries padded to 32) per v_mfma_f32_32x32x16_bf16 chain,
+    //      buckets on the A operand and ascending contraction steps: the sums of the other hash
+    //      kernels.  Wave w takes bucket chunks w, w+4, ...; lane (column l%32, half l/32) sees the
+    //      scores of its query for 16 buckets of a chunk in ascending order.
+    typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+    const int C = ds.n_buckets;
+    const int col = l & 31, hb = l >> 5;
+    bf16x8 bq[8];
+    {
+      const uint4* pq = reinterpret_cast<const uint4*>(qb + int64_t(col < G ? col : 0) * kD + hb * 8);
+  #pragma unroll
+      for (int ks = 0; ks < 8; ++ks) bq[ks] = as_bf16x8(col < G ? pq[2 * ks] : make_uint4(0, 0, 0, 0));
+    }
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int c0 = 32 * w; c0 < C; c0 += 128) {
+      const int cr = min(c0 + col, C - 1);
+      const uint4* pa = reinterpret_cast<const uint4*>(A_all + (ds.a_off + cr) * kD + hb * 8);
+      uint4 au[8];
+  #pragma unroll
+      for (int ks = 0; ks < 8; ++ks) au[ks] = pa[2 * ks];
+      f32x16 acc;
+  #pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  #pragma unroll
+      for (int ks = 0; ks < 8; ++ks)
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(au[ks]), bq[ks], acc, 0, 0, 0);
+  #pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c = c0 + 8 * (r >> 2) + 4 * hb + (r & 3);
+        if (c < C && col < G) {
+          if (scores_out && slot == 0) scores_out[(ds.a_off + c) * G + col] = acc[r];
+          if (besti == 0x7fffffff || acc[r] > best) {  // buckets ascend per lane
+            best = acc[r];
+            besti = c;
+          }
         }
       }
     }
-  }
-  // the two lane halves of a column, then the four waves: larger score wins, equal scores keep the
-  // lower bucket
-  {
-    const float ob = __shfl_xor(best, 32);
-    const int oi = __shfl_xor(besti, 32);
-    if (oi != 0x7fffffff && (besti == 0x7fffffff || ob > best || (ob == best && oi < besti))) {
-      best = ob;
-      besti = oi;
-    }
-    if (l < G) {
-      s_best[w][l] = best;
-      s_besti[w][l] = besti;
-    }
-  }
-  __syncthreads();
-  if (tid < G) {
-    float b = s_best[0][tid];
-    int bi = s_besti[0][tid];
-    for (int ww = 1; ww < 4; ++ww) {
-      const float ob = s_best[ww][tid];
-      const int oi = s_besti[ww][tid];
-      if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > b || (ob == b && oi < bi))) {
-        b = ob;
-        bi = oi;
+    // the two lane halves of a column, then the four waves: larger score wins, equal scores keep the
+    // lower bucket
+    {
+      const float ob = __shfl_xor(best, 32);
+      const int oi = __shfl_xor(besti, 32);
+      if (oi != 0x7fffffff && (besti == 0x7fffffff || ob > best || (ob == best && oi < besti))) {
+        best = ob;
+        besti = oi;
+      }
+      if (l < G) {
+        s_best[w][l] = best;
+        s_besti[w][l] = besti;
       }
     }
-    s_hash[tid] = bi;
-    if (slot == 0) hash_out[int64_t(qrow) * G + tid] = bi;
+    __syncthreads();
+    if (tid < G) {
+      float b = s_best[0][tid];
+      int bi = s_besti[0][tid];
+      for (int ww = 1; ww < 4; ++ww) {
+        const float ob = s_best[ww][tid];
+        const int oi = s_besti[ww][tid];
+        if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > b || (ob == b && oi < bi))) {
+          b = ob;
+          bi = oi;
+        }
+      }
+      s_hash[tid] = bi;
+      if (slot == 0) hash_out[int64_t(qrow) * G + tid] = bi;
+    }
+    __syncthreads();
+  } else {
+    if (tid < G) s_hash[tid] = hash_out[int64_t(qrow) * G + tid];
+    __syncthreads();
   }
-  __syncthreads();
+  if constexpr (MODE == 1) return;
   // ---- this workgroup's bucket: the slot-th distinct one among the G hashes ----
   const bf16_t* Kb = K_all + ds.k_off * kD;
   const bf16_t* Vb = V_all + ds.k_off * kD;
@@ -458,8 +469,13 @@ bool hash_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_
 int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
                      const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, float sm_scale,
                      void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st) {
-  hipLaunchKernelGGL(decode_hash_attn_kernel, dim3(unsigned(rows) * unsigned(G)), dim3(256), red_floats(1) * sizeof(float),
-                     st, (const bf16_t*)q, (const bf16_t*)A_all, (const bf16_t*)K_all,
+  // the hash of every row first (one short workgroup each), then G workgroups per row that start on
+  // their bucket at once
+  hipLaunchKernelGGL(decode_hash_attn_kernel<1>, dim3(unsigned(rows)), dim3(256), 0, st, (const bf16_t*)q,
+                     (const bf16_t*)A_all, (const bf16_t*)K_all, (const bf16_t*)V_all, idx_all, desc, G,
+                     sm_scale * kLog2e, (bf16_t*)out, lse, hash_out, scores_out);
+  hipLaunchKernelGGL(decode_hash_attn_kernel<2>, dim3(unsigned(rows) * unsigned(G)), dim3(256),
+                     red_floats(1) * sizeof(float), st, (const bf16_t*)q, (const bf16_t*)A_all, (const bf16_t*)K_all,
                      (const bf16_t*)V_all, idx_all, desc, G, sm_scale * kLog2e, (bf16_t*)out, lse, hash_out,
                      scores_out);
   return launch_status("fm_decode_hash_attn");

@@ -221,7 +221,8 @@ int fm_attention_hash_varlen(const void* q, const void* k, const void* v, const 
  * G query heads of that KV head, one token each).  A, K, V of all rows are
  * packed back to back ([sum C, d], [sum N, d]); the bucket lists likewise, each
  * row holding C*Z indices local to its own keys.  bf16, d = 128 only.
- *   q [rows,G,d] -> out [rows,G,d], lse [rows,G] fp32, hash_out [rows,G] int32;
+ *   q [rows,G,d] -> out [rows,G,d], lse [rows,G] fp32, hash_out [rows,G] int32
+ *   (required: a first launch hashes every row into it, a second reads it);
  *   scores_out (optional, [sum C, G] fp32): the scores the hashes were taken over. */
 typedef struct {
   int64_t a_off;        /* first row of this row's A in A_all            */

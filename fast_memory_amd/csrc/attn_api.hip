@@ -98,6 +98,47 @@ extern "C" size_t fm_attention_hash_varlen_workspace(int H, int C, int Sq) {
   return fm::varlen_layout(H, C, Sq).total;
 }
 
+namespace fm {
+// A query whose hash is outside [0, C) belongs to no bucket and to no work item, so the attention kernels
+// never write its rows: here it gets the result of an empty bucket, out = 0 and lse = -FLT_MAX.
+__global__ __launch_bounds__(256) void unhashed_rows_kernel(const int32_t* __restrict__ q_hash, int64_t nq,
+                                                            int C, int row_halves, uint16_t* __restrict__ out,
+                                                            float* __restrict__ lse) {
+  const int64_t i = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (i >= nq) return;
+  const int b = q_hash[i];
+  if (b >= 0 && b < C) return;
+  for (int w = lane_id(); w < row_halves; w += kWave) out[i * row_halves + w] = uint16_t(0);
+  if (lane_id() == 0) lse[i] = -FLT_MAX;
+}
+
+// bucket offsets + grouping + attention with every intermediate in the buffer at `base`
+static int varlen_run(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                      const int32_t* bucket_cnt, const int32_t* q_hash, void* out, float* lse, int H,
+                      int Sq, int N, int d, int C, float sm_scale, int dtype, char* base,
+                      const VarlenWs& w, void* stream) {
+  int64_t* bucket_off = reinterpret_cast<int64_t*>(base + w.off_bucket_off);
+  int32_t* q_perm = reinterpret_cast<int32_t*>(base + w.off_q_perm);
+  int32_t* bin_count = reinterpret_cast<int32_t*>(base + w.off_bin_count);
+  int32_t* bin_off = reinterpret_cast<int32_t*>(base + w.off_bin_off);
+  fm_item* items = reinterpret_cast<fm_item*>(base + w.off_items);
+  int32_t* n_items = reinterpret_cast<int32_t*>(base + w.off_n_items);
+  int rc = fm_bucket_offsets(bucket_cnt, int64_t(H) * C, bucket_off, stream);
+  if (rc) return rc;
+  rc = fm_group_queries(q_hash, H, C, Sq, q_perm, bin_count, bin_off, items, n_items, w.max_items,
+                        base + w.off_group, fm_group_queries_workspace(H, C, Sq), stream);
+  if (rc) return rc;
+  rc = fm_hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, w.max_items, out,
+                        lse, H, Sq, N, d, C, sm_scale, dtype, stream);
+  if (rc) return rc;
+  const int row_bytes = d * (dtype == FM_BF16 ? 2 : 4);
+  const int64_t nq = int64_t(H) * Sq;
+  hipLaunchKernelGGL(unhashed_rows_kernel, dim3(unsigned(ceil_div(nq, 4))), dim3(256), 0, as_stream(stream),
+                     q_hash, nq, C, row_bytes / 2, static_cast<uint16_t*>(out), lse);
+  return launch_status("fm_attention_hash_varlen");
+}
+}  // namespace fm
+
 extern "C" int fm_attention_hash_varlen(const void* q, const void* k, const void* v,
                                         const int32_t* k_idx, const int32_t* bucket_cnt,
                                         const int32_t* q_hash, void* out, float* lse, int H, int Sq,
@@ -110,20 +151,8 @@ extern "C" int fm_attention_hash_varlen(const void* q, const void* k, const void
   VarlenWs w = varlen_layout(H, C, Sq);
   FM_REQUIRE(ws_bytes >= w.total, FM_ERR_WORKSPACE, "fm_attention_hash_varlen: workspace %zu < %zu",
              ws_bytes, w.total);
-  char* base = static_cast<char*>(ws);
-  int64_t* bucket_off = reinterpret_cast<int64_t*>(base + w.off_bucket_off);
-  int32_t* q_perm = reinterpret_cast<int32_t*>(base + w.off_q_perm);
-  int32_t* bin_count = reinterpret_cast<int32_t*>(base + w.off_bin_count);
-  int32_t* bin_off = reinterpret_cast<int32_t*>(base + w.off_bin_off);
-  fm_item* items = reinterpret_cast<fm_item*>(base + w.off_items);
-  int32_t* n_items = reinterpret_cast<int32_t*>(base + w.off_n_items);
-  int rc = fm_bucket_offsets(bucket_cnt, int64_t(H) * C, bucket_off, stream);
-  if (rc) return rc;
-  rc = fm_group_queries(q_hash, H, C, Sq, q_perm, bin_count, bin_off, items, n_items, w.max_items,
-                        base + w.off_group, fm_group_queries_workspace(H, C, Sq), stream);
-  if (rc) return rc;
-  return fm_hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
-                          w.max_items, out, lse, H, Sq, N, d, C, sm_scale, dtype, stream);
+  return varlen_run(q, k, v, k_idx, bucket_cnt, q_hash, out, lse, H, Sq, N, d, C, sm_scale, dtype,
+                    static_cast<char*>(ws), w, stream);
 }
 
 extern "C" int fm_local_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,

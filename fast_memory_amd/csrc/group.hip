@@ -39,18 +39,14 @@ __global__ __launch_bounds__(1024) void excl_scan_i32_i64_kernel(const int32_t* 
 // block_hist is [H][NB][C], zeroed beforehand.
 __global__ __launch_bounds__(kGrpBlock) void group_rank_kernel(const int32_t* __restrict__ q_hash,
                                                                int C, int Sq, int NB,
-                                                               int32_t* __restrict__ block_hist,
-                                                               int32_t* __restrict__ bad) {
+                                                               int32_t* __restrict__ block_hist) {
   __shared__ int sh[kGrpBlock];
   const int h = blockIdx.y, blk = blockIdx.x, t = threadIdx.x;
   const int i = blk * kGrpBlock + t;
   int b = -1;
   if (i < Sq) {
     b = q_hash[int64_t(h) * Sq + i];
-    if (b < 0 || b >= C) {
-      atomicOr(bad, 1);
-      b = -1;
-    }
+    if (b < 0 || b >= C) b = -1;  // belongs to no bucket: in no bin, no work item, no q_perm slot
   }
   sh[t] = b;
   __syncthreads();
@@ -243,11 +239,10 @@ extern "C" int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int
   hipStream_t st = as_stream(stream);
   const int NB = int(ceil_div(Sq, kGrpBlock));
   int32_t* block_hist = static_cast<int32_t*>(ws);
-  int32_t* bad = block_hist + int64_t(H) * NB * C;  // one flag word after the table (inside the +256)
-  int rc = launch_fill(block_hist, int64_t(H) * NB * C + 1, 0, st);
+  int rc = launch_fill(block_hist, int64_t(H) * NB * C, 0, st);
   if (rc) return rc;
   hipLaunchKernelGGL(group_rank_kernel, dim3(NB, H), dim3(kGrpBlock), 0, st, q_hash, C, Sq, NB,
-                     block_hist, bad);
+                     block_hist);
   hipLaunchKernelGGL(group_colscan_kernel, dim3(unsigned(ceil_div(int64_t(H) * C, 256))), dim3(256),
                      0, st, block_hist, H, C, NB, bin_count);
   hipLaunchKernelGGL(group_items_kernel, dim3(1), dim3(1024), 0, st, bin_count, int64_t(H) * C, C,

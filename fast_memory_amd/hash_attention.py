@@ -32,8 +32,10 @@ def attention_hash_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     :param q_hashes: ``[batch_size, q_seq_len]`` bucket of every query
     :param sm_scale: softmax scale
     :param lse_dtype: ``torch.float32`` (default) returns the fp32 natural-log
-        LSE; ``None`` reproduces the reference's rounding of the LSE to q's
-        dtype (triton_kernel.py:111-117).
+        LSE; ``None`` follows the reference's rounding order
+        (triton_kernel.py:111-117): the base-2 LSE is rounded to q's dtype and
+        multiplied by ln 2 in that dtype (the base-2 value is recovered from
+        the fp32 natural-log one, i.e. to one fp32 rounding).
     :return: ``(out [batch, q_seq_len, d_head], lse [batch, q_seq_len])``;
         a query whose bucket holds no key gets ``out = 0`` and
         ``lse = finfo(lse.dtype).min``.
@@ -56,8 +58,12 @@ def attention_hash_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                                              _as_i32(k_hash_counts).contiguous(),
                                              _as_i32(q_hashes).contiguous(), sm_scale)
     if lse_dtype is None:
-        # the reference scales after rounding: lse2.to(q.dtype) * ln2, then nan_to_num
-        lse = lse.to(q.dtype)
+        # the reference's order (triton_kernel.py:111-117): the kernel's base-2 value is rounded to q's
+        # dtype first, the product with ln 2 is then formed in that dtype, then nan_to_num
+        empty = lse < -1e30
+        lse2 = (lse * 1.4426950408889634).to(q.dtype)
+        lse = lse2 * 0.6931471805599453
+        lse = lse.masked_fill(empty, torch.finfo(lse.dtype).min)
         lse = torch.nan_to_num(lse, nan=0.0, posinf=torch.finfo(lse.dtype).max,
                                neginf=torch.finfo(lse.dtype).min)
     elif lse_dtype != torch.float32:
@@ -123,8 +129,9 @@ def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torc
         assert can_stage, "the staged backward takes bf16 with d_head = 128"
         try:
             inv = inverse_index if inverse_index is not None else ops.inverse_index(lists, off, counts, k.shape[1])
-            return ops.hash_attn_bwd_staged(q, k, v, lists, off, counts, groups, inv, out.contiguous(),
-                                            lse.float().contiguous(), d_out.contiguous(), sm_scale)
+            if inv.row_pos[-1] > 0:        # no listed entry at all: nothing to stage, the other form handles it
+                return ops.hash_attn_bwd_staged(q, k, v, lists, off, counts, groups, inv, out.contiguous(),
+                                                lse.float().contiguous(), d_out.contiguous(), sm_scale)
         except torch.cuda.OutOfMemoryError:
             if not auto:
                 raise                      # asked for explicitly: report that its workspace does not fit

@@ -127,7 +127,9 @@ int fm_bucket_offsets(const int32_t* cnt, int64_t n, int64_t* off_out, void* str
  *   items     [max_items] out  work items {row, bucket, first sorted position,
  *                           number of queries <= FM_QTILE}
  *   n_items   [1]      out  number of items written
- * max_items must be >= fm_group_max_items(H, C, Sq). */
+ * max_items must be >= fm_group_max_items(H, C, Sq).  A query whose hash is outside
+ * [0, C) belongs to no bucket: it is counted in no bin, is part of no item and
+ * appears nowhere in q_perm (whose last slots then stay unwritten). */
 typedef struct { int32_t row, bucket, q_start, n_q; } fm_item;
 int64_t fm_group_max_items(int H, int C, int Sq);
 size_t fm_group_queries_workspace(int H, int C, int Sq);
@@ -142,7 +144,8 @@ int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int32_t* q_per
  *   k_idx flat int32, bucket_off [H*C] int64, bucket_cnt [H*C] int32
  *   q_perm, items, n_items            from fm_group_queries
  *   out [H,Sq,d] (dtype of q), lse [H,Sq] fp32 natural log, original order.
- * A query whose bucket is empty gets out = 0, lse = -FLT_MAX. */
+ * A query whose bucket is empty gets out = 0, lse = -FLT_MAX.  Rows of queries that
+ * are part of no item (hash outside [0, C), see fm_group_queries) are not written. */
 int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
                      const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                      const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
@@ -207,7 +210,9 @@ int fm_hash_attn_bwd_staged(const void* q, const void* k, const void* v, const i
 
 /* ---- the reference operator in one call -------------------------------------
  * attention_hash_varlen(q,k,v,k_hashes,k_hash_counts,q_hashes,sm_scale)
- * (triton_kernel.py:51-119): bucket offsets + grouping + attention. */
+ * (triton_kernel.py:51-119): bucket offsets + grouping + attention.  A query whose
+ * hash is outside [0, C) (the reference would fail on the index) is treated as
+ * hashed to an empty bucket: out = 0, lse = -FLT_MAX. */
 size_t fm_attention_hash_varlen_workspace(int H, int C, int Sq);
 int fm_attention_hash_varlen(const void* q, const void* k, const void* v, const int32_t* k_idx,
                              const int32_t* bucket_cnt, const int32_t* q_hash, void* out,

@@ -165,21 +165,29 @@ def test_config5_one_million_keys_full_size(ops):
 
 
 def test_config3_decode_batch_full_size(ops):
-    from fast_memory_amd import Memory, MemoryBatch, synth
-    cfg_d, H, G = 128, 8, 4
+    """Config 3 as the benchmark runs it: per sequence the clustered keys of config 2 (256-component vMF
+    mixture, kappa 20, lognormal norms), A from two K-means iterations on them, one query per head drawn
+    near a cluster centre -- the data on which a row's G queries fall into few buckets, often one."""
+    from fast_memory_amd import Memory, MemoryBatch, fit_projection, synth
+    base = synth.CONFIGS["c2"]
+    cfg_d, H, G = base.d, base.H, base.G
+    assert (cfg_d, H, G) == (128, 8, 4)
     lengths = synth.decode_lengths()
-    g = torch.Generator(device="cuda").manual_seed(1003)
-    mems = []
-    for N, C, Z in lengths:
-        K = torch.randn(H, N, cfg_d, generator=g, device="cuda").to(torch.bfloat16)
-        V = torch.randn(H, N, cfg_d, generator=g, device="cuda").to(torch.bfloat16)
-        A = torch.randn(H, C, cfg_d, generator=g, device="cuda")
-        A = (A / A.norm(dim=-1, keepdim=True)).to(torch.bfloat16)
-        mems.append(Memory.build(K, V, A, Z))
+    mems, qs, kls, vls = [], [], [], []
+    for s, (N, C, Z) in enumerate(lengths):
+        cfg = synth.Config(f"c3-seq{s}", base.dtype, H, G, cfg_d, N, C, Z, 1, 256, 20.0, 2, 512, 1003 + s)
+        wl = synth.make_workload(cfg, "cuda")
+        A = fit_projection(wl.keys, C, iters=2)
+        mems.append(Memory.build(wl.keys, wl.values, A, Z))
+        qs.append(wl.queries.reshape(H, G, cfg_d))
+        kls.append(wl.k_local)
+        vls.append(wl.v_local)
     batch = MemoryBatch(mems)
-    q = (torch.randn(len(lengths), H, G, cfg_d, generator=g, device="cuda") * 2).to(torch.bfloat16)
+    q = torch.stack(qs)
     scale = cfg_d ** -0.5
     out, lse, h, scores = batch.attend(q, scale, return_scores=True)
+    distinct = sum(len(set(h[s, hh].tolist())) for s in range(len(lengths)) for hh in range(H)) / (len(lengths) * H)
+    print(f"c3: {distinct:.2f} distinct buckets among the {G} queries of a row, on average", flush=True)
     a_off = 0
     for s, ((N, C, Z), mem) in enumerate(zip(lengths, mems)):
         sc = scores[a_off:a_off + H * C].reshape(H, C, G).transpose(1, 2)       # [H, G, C]
@@ -190,8 +198,8 @@ def test_config3_decode_batch_full_size(ops):
                 ro, rl = oracle_on_sample(q[s, hh], h[s, hh].long(), mem.bucket_idx[hh], mem.keys[hh],
                                           mem.values[hh], scale)
                 assert_attn_close(out[s, hh][None], lse[s, hh][None], ro, rl, torch.bfloat16, f"seq {s} head {hh}")
-    kl = torch.randn(len(lengths), H, 512, cfg_d, generator=g, device="cuda").to(torch.bfloat16)
-    vl = torch.randn(len(lengths), H, 512, cfg_d, generator=g, device="cuda").to(torch.bfloat16)
+    kl, vl = torch.stack(kls), torch.stack(vls)
+    assert kl.shape == (len(lengths), H, 512, cfg_d)
     mo, ml = batch.attend_with_local(q, kl, vl, scale)
     for s in range(0, len(lengths), 8):
         lo, ll = O.local_attention(q[s].cpu().reshape(1, H * G, 1, cfg_d), kl[s:s + 1].cpu(), vl[s:s + 1].cpu(),

@@ -340,7 +340,18 @@ def test_attention_reference_lse_rounding_switch():
     ro, rl = O.hashed_attention_blocked(q, k, v, kh, cnt, qh, 0.125, ref_lse_rounding=True)
     empty = qh[0] == 1
     assert (lse.cpu()[0][empty] == torch.finfo(torch.bfloat16).min).all()
-    assert torch.allclose(lse.cpu().float()[0][~empty], rl.float()[0][~empty], atol=0.07)
+    # same rounding order as triton_kernel.py:111: bf16(lse2) * ln2 in bf16.  The GPU's fp32 lse2 differs from
+    # the oracle's in the last bits (summation order), which moves a bf16 rounding only next to a tie: almost
+    # all values are identical and none is further than one bf16 step (2^-7 relative) away
+    got, ref = lse.cpu().float()[0][~empty], rl.float()[0][~empty]
+    assert (got == ref).float().mean().item() >= 0.95
+    assert ((got - ref).abs() <= ref.abs() * 2.0 ** -7 + 1e-6).all()
+    # and it is NOT the rounding of the already scaled fp32 value wherever the two orders differ
+    ro32, rl32 = O.hashed_attention_blocked(q, k, v, kh, cnt, qh, 0.125)
+    other = rl32[0][~empty].to(torch.bfloat16).float()
+    differ = other != ref
+    assert differ.any(), "case does not separate the two rounding orders"
+    assert (got[differ] == ref[differ]).float().mean().item() >= 0.9
 
 
 # ------------------------------------------------------------------ a10

@@ -16,6 +16,7 @@ FM_F32, FM_BF16 = 0, 1
 FM_MAX_Z = 16384
 FM_MAX_D = 256
 FM_QTILE = 64
+FM_STATIC_SCRATCH_BYTES = 32 << 20
 
 P = c_void_p
 
@@ -49,6 +50,8 @@ SIGNATURES = {
     "fm_attention_hash_varlen_workspace": (c_size_t, [c_int, c_int, c_int]),
     "fm_attention_hash_varlen": (c_int, [P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int,
                                          c_float, c_int, P, c_size_t, P]),
+    "fm_attention_hash_varlen_static": (c_int, [P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int,
+                                                c_float, c_int, P]),
     "fm_decode_hash_attn": (c_int, [P, P, P, P, P, P, c_int, c_int, c_int, c_float, P, P, P, P, c_int, P]),
     "fm_local_attn_fwd": (c_int, [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                   c_int, P]),

@@ -2,6 +2,8 @@
 // shapes they are built for and the generic kernels otherwise.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace fm {
 int hash_attn_generic(const void* q, const void* k, const void* v, const int32_t* k_idx,
                       const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
@@ -153,6 +155,64 @@ extern "C" int fm_attention_hash_varlen(const void* q, const void* k, const void
              ws_bytes, w.total);
   return varlen_run(q, k, v, k_idx, bucket_cnt, q_hash, out, lse, H, Sq, N, d, C, sm_scale, dtype,
                     static_cast<char*>(ws), w, stream);
+}
+
+// ---- the same operator for callers that cannot allocate ------------------------------------
+// The grouping tables, the permutation and the work items live in a device array of the library
+// itself, one copy per GPU.  In host code the array's name only stands for the symbol: the device
+// address comes from hipGetSymbolAddress, once per device, and only that pointer is used below.
+namespace fm {
+static __device__ __align__(256) unsigned char scratch[FM_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, 0 = not asked yet
+
+static int scratch_of_current_device(char** ptr_out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    set_error("fm_attention_hash_varlen_static: no current device (hipGetDevice gave %d)", dev);
+    return FM_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      set_error("fm_attention_hash_varlen_static: hipGetSymbolAddress on device %d: %s", dev,
+                hipGetErrorString(e));
+      return FM_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr_out = static_cast<char*>(g_scratch_ptr[dev]);
+  return FM_OK;
+}
+}  // namespace fm
+
+extern "C" int fm_attention_hash_varlen_static(const void* q, const void* k, const void* v,
+                                               const int32_t* k_idx, const int32_t* bucket_cnt,
+                                               const int32_t* q_hash, void* out, float* lse, int H,
+                                               int Sq, int N, int d, int C, float sm_scale, int dtype,
+                                               void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1, FM_ERR_ARG,
+             "fm_attention_hash_varlen_static: H=%d Sq=%d N=%d C=%d", H, Sq, N, C);
+  FM_REQUIRE(bucket_cnt && q_hash, FM_ERR_ARG, "fm_attention_hash_varlen_static: null pointer");
+  VarlenWs w = varlen_layout(H, C, Sq);
+  FM_REQUIRE(w.total <= size_t(FM_STATIC_SCRATCH_BYTES), FM_ERR_WORKSPACE,
+             "fm_attention_hash_varlen_static: H=%d C=%d Sq=%d needs %zu bytes of scratch, the static "
+             "array holds %zu; use fm_attention_hash_varlen with a workspace",
+             H, C, Sq, w.total, size_t(FM_STATIC_SCRATCH_BYTES));
+  char* base = nullptr;
+  int rc = scratch_of_current_device(&base);
+  if (rc) return rc;
+  // nothing in the array has to survive from an earlier call: the grouping clears its block table
+  // with a fill kernel and every other region is written before it is read
+  return varlen_run(q, k, v, k_idx, bucket_cnt, q_hash, out, lse, H, Sq, N, d, C, sm_scale, dtype,
+                    base, w, stream);
 }
 
 extern "C" int fm_local_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,

@@ -337,6 +337,24 @@ def attention_hash_varlen_i32(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: floa
     return out, lse
 
 
+def attention_hash_varlen_static_(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: float, out: torch.Tensor,
+                                  lse: torch.Tensor):
+    """:func:`attention_hash_varlen_i32` into caller-provided ``out`` / ``lse`` with no allocation at all:
+    the grouping scratch is the library's own static device array (``fm_attention_hash_varlen_static``;
+    extents beyond ``FM_STATIC_SCRATCH_BYTES`` raise).  Calls on one GPU share that array, so they must
+    not overlap."""
+    _dev(q, k, v, k_idx, bucket_cnt, q_hash, out, lse)
+    H, Sq, d = q.shape
+    _, N, _ = k.shape
+    C = bucket_cnt.shape[-1]
+    assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and q_hash.dtype == torch.int32
+    assert out.shape == q.shape and out.dtype == q.dtype and lse.shape == (H, Sq) and lse.dtype == torch.float32
+    check(_lib.load().fm_attention_hash_varlen_static(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_cnt), _p(q_hash),
+                                                      _p(out), _p(lse), H, Sq, N, d, C, float(sm_scale), _dt(q),
+                                                      _stream(q)))
+    return out, lse
+
+
 def decode_hash_attn(q, A_all, K_all, V_all, idx_all, desc, sm_scale: float, return_scores: bool = False):
     """Hash + gathered attention for a decode batch of rows with different memories.
     q [rows,G,d]; A_all [sum C,d]; K_all,V_all [sum N,d]; idx_all flat int32; desc [rows,5] int64

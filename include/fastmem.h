@@ -219,6 +219,26 @@ int fm_attention_hash_varlen(const void* q, const void* k, const void* v, const 
                              float* lse, int H, int Sq, int N, int d, int C, float sm_scale,
                              int dtype, void* ws, size_t ws_bytes, void* stream);
 
+/* ---- the same operator for callers that cannot allocate ------------------------
+ * No counterpart in the reference.  For callers that cannot obtain device memory
+ * for a workspace: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid allocation.  Identical to fm_attention_hash_varlen (same kernels,
+ * same results bit for bit) except that the grouping tables, the query
+ * permutation and the work items live in a device array of the library itself,
+ * FM_STATIC_SCRATCH_BYTES long, which every GPU the library runs on holds until
+ * the process ends.  The call allocates nothing and frees nothing; the first call
+ * on a device looks the array's address up (hipGetSymbolAddress).  Extents whose
+ * fm_attention_hash_varlen_workspace(H, C, Sq) exceeds FM_STATIC_SCRATCH_BYTES are
+ * refused with FM_ERR_WORKSPACE.  All calls on one GPU share that GPU's array:
+ * calls that overlap on one GPU (different streams or threads) race; successive
+ * calls on one stream do not (each clears what it needs to start at zero with a
+ * fill kernel, not a memset node). */
+#define FM_STATIC_SCRATCH_BYTES (32u << 20)
+int fm_attention_hash_varlen_static(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                                    const int32_t* bucket_cnt, const int32_t* q_hash, void* out,
+                                    float* lse, int H, int Sq, int N, int d, int C, float sm_scale,
+                                    int dtype, void* stream);
+
 /* ---- decode batch over memories of different sizes ---------------------------
  * The same path (query hash memory.py:281-283 + gathered attention
  * triton_kernel.py:137-272) for a batch of rows whose memories differ in N, C

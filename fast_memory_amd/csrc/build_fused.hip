@@ -434,6 +434,12 @@ struct CandRegs {
   }
 };
 
+static inline size_t cand_select_lds_bytes(int Zc, int P) {
+  const size_t binned = size_t(Zc + kSelMaxBin) * sizeof(uint64_t) + size_t(kSelBins) * sizeof(uint32_t);
+  const size_t sorted = sort_lds_bytes(P) + sizeof(SelectShared) + 8;
+  return std::max(binned, sorted);
+}
+
 // Exact top-Z (value desc, index asc) of every row's candidates: radix select of the cut,
 // collection of the Zc survivors into LDS, bitonic sort, indices out -- the code of the dense
 // arg-top-Z kernel, on ~1.2 Zc register-resident candidates instead of the N-element row.
@@ -442,9 +448,11 @@ __global__ __launch_bounds__(NT) void cand_select_kernel(
     const uint2* __restrict__ cand, const int32_t* __restrict__ cnt, int n_writers, int cap_w, int Zc, int P,
     int32_t* __restrict__ idx_out, float* __restrict__ val_out, int32_t* __restrict__ fail_rows,
     int32_t* __restrict__ n_fail) {
+  // dynamic LDS, two uses of the same bytes: [composites of the binned selection | its histogram], or,
+  // when that declines the row, [sort buffer of the radix select | its histograms]
   extern __shared__ uint64_t buf[];
-  __shared__ SelectShared sh;
   __shared__ CandCounts cc;
+  __shared__ BinShared bs;
   const int64_t row = blockIdx.x;
   const int T = NT / n_writers;  // threads per segment
   bool ok = load_cand_counts(cnt, row, n_writers, cap_w, Zc, cc);
@@ -464,8 +472,14 @@ __global__ __launch_bounds__(NT) void cand_select_kernel(
 #pragma unroll
   for (int r = 0; r < R; ++r)
     if (r < src.n) src.e[r] = seg[t + r * T];
+  int32_t* out = idx_out + row * Zc;
+  float* vout = val_out ? val_out + row * Zc : nullptr;
+  uint32_t* hist = reinterpret_cast<uint32_t*>(buf + (Zc + kSelMaxBin));
+  if (binned_select_write<NT>(src, Zc, buf, hist, bs, out, vout)) return;
+  __syncthreads();
+  SelectShared& sh = *reinterpret_cast<SelectShared*>(buf + sort_lds_bytes(P) / sizeof(uint64_t));
   const uint64_t cut = radix_select_cut<NT>(src, Zc, 6, sh);
-  collect_sort_write(src, cut, Zc, P, buf, sh, idx_out + row * Zc, val_out ? val_out + row * Zc : nullptr);
+  collect_sort_write(src, cut, Zc, P, buf, sh, out, vout);
 }
 
 // ---- phase 3 ---------------------------------------------------------------
@@ -587,8 +601,8 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   const int P = next_pow2(Zc);
 #define FM_CAND_SELECT(NT, R)                                                                           \
   do {                                                                                                  \
-    FM_ALLOW_LDS((cand_select_kernel<NT, R>), sort_lds_bytes(FM_MAX_Z), "fm_build_index_fused: lds");   \
-    hipLaunchKernelGGL((cand_select_kernel<NT, R>), dim3(unsigned(rows)), dim3(NT), sort_lds_bytes(P), st, cand, cnt, \
+    FM_ALLOW_LDS((cand_select_kernel<NT, R>), cand_select_lds_bytes(FM_MAX_Z, FM_MAX_Z), "fm_build_index_fused: lds");   \
+    hipLaunchKernelGGL((cand_select_kernel<NT, R>), dim3(unsigned(rows)), dim3(NT), cand_select_lds_bytes(Zc, P), st, cand, cnt, \
                        p.n_writers, p.cap_w, Zc, P, idx_out, val_out, fail_rows, n_fail);                      \
   } while (0)
   if (p.sel_threads == 256)

@@ -294,6 +294,129 @@ __device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, in
   }
 }
 
+// ---- selection by value bins: no radix passes, no sorting network --------------------------
+// For candidate sets that are a modest superset of the answer (the fused build's ~1.2 Zc candidates per
+// row).  The value keys are cut into up to kSelBins equal-width bins over [min, max] of the row (a shift,
+// so 2048..4096 bins are in use), descending; one histogram and a scan give every bin's first output
+// position and the bin that holds the Zc-th element; the candidates of the bins up to that one are
+// scattered into their bins' slots (any order), and every element's final position is its bin's start
+// plus the number of larger composites in its bin, counted by brute force: a bin holds a few elements,
+// a few dozen next to the cut where the values are densest.  Composites are unique, so the positions are a
+// permutation and the result is exactly "value descending, index ascending".
+// Returns false, with nothing written, when a bin is longer than kSelMaxBin (many equal or nearly equal
+// values): the caller then takes the radix select and the sorting network.
+constexpr int kSelBinBits = 12;
+constexpr int kSelBins = 1 << kSelBinBits;
+constexpr int kSelMaxBin = 256;
+
+struct BinShared {
+  uint32_t red_min[16], red_max[16];
+  int scan_tmp[17];
+  int cut_bin, n_keep, max_bin;
+};
+
+// buf holds Zc + kSelMaxBin composites, hist kSelBins words.
+template <int NT, typename Source>
+__device__ __forceinline__ bool binned_select_write(Source& src, int Zc, uint64_t* buf, uint32_t* hist,
+                                                    BinShared& bs, int32_t* __restrict__ out,
+                                                    float* __restrict__ val_out) {
+  static_assert(NT >= 256 && NT <= 1024 && kSelBins % NT == 0, "threads per row");
+  const int tid = threadIdx.x, w = tid >> 6;
+  constexpr int nw = NT / 64;
+  uint32_t mn = 0xffffffffu, mx = 0u;
+  src([&](float y, uint32_t) {
+    const uint32_t k = float_key(y);
+    mn = min(mn, k);
+    mx = max(mx, k);
+  });
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = min(mn, uint32_t(__shfl_xor(int(mn), o)));
+    mx = max(mx, uint32_t(__shfl_xor(int(mx), o)));
+  }
+  if (lane_id() == 0) {
+    bs.red_min[w] = mn;
+    bs.red_max[w] = mx;
+  }
+  for (int i = tid; i < kSelBins; i += NT) hist[i] = 0;
+  if (tid == 0) {
+    bs.max_bin = 0;
+    bs.cut_bin = -1;
+    bs.n_keep = 0;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < nw; ++i) {
+    mn = min(mn, bs.red_min[i]);
+    mx = max(mx, bs.red_max[i]);
+  }
+  if (mx < mn) return false;  // no candidate at all
+  const uint32_t range1 = mx - mn;
+  const int hb = range1 ? 32 - __clz(int(range1)) : 0;
+  const int shift = hb > kSelBinBits ? hb - kSelBinBits : 0;
+  const uint32_t top = range1 >> shift;  // < kSelBins
+  auto dbin = [&](uint32_t k) { return int(top - ((k - mn) >> shift)); };  // 0 = the largest values
+  src([&](float y, uint32_t) { atomicAdd(&hist[dbin(float_key(y))], 1u); });
+  __syncthreads();
+  {
+    constexpr int per = kSelBins / NT;
+    int h[per], local = 0;
+#pragma unroll
+    for (int j = 0; j < per; ++j) {
+      h[j] = int(hist[tid * per + j]);
+      local += h[j];
+    }
+    int total;
+    int running = block_excl_scan(local, bs.scan_tmp, &total);
+    int longest = 0;
+#pragma unroll
+    for (int j = 0; j < per; ++j) {
+      if (running < Zc) {
+        longest = max(longest, h[j]);
+        if (Zc <= running + h[j]) {
+          bs.cut_bin = tid * per + j;
+          bs.n_keep = running + h[j];
+        }
+      }
+      hist[tid * per + j] = uint32_t(running);
+      running += h[j];
+    }
+    if (longest > kSelMaxBin) atomicMax(&bs.max_bin, longest);
+  }
+  __syncthreads();
+  const int cut_bin = bs.cut_bin, n_keep = bs.n_keep;
+  if (cut_bin < 0 || bs.max_bin > kSelMaxBin) return false;  // fewer than Zc candidates, or a long bin
+  src([&](float y, uint32_t i) {
+    const int d = dbin(float_key(y));
+    if (d <= cut_bin) buf[atomicAdd(&hist[d], 1u)] = composite(y, i);
+  });
+  __syncthreads();
+  // hist[d] is now the end of bin d (for d <= cut_bin), i.e. the start of bin d + 1
+  for (int p = tid; p < n_keep; p += NT) {
+    const uint64_t c = buf[p];
+    const uint32_t clo = uint32_t(c), chi = uint32_t(c >> 32);
+    const int d = dbin(chi);
+    const int s0 = d ? int(hist[d - 1]) : 0, e0 = int(hist[d]);
+    int rank = s0;
+    for (int q = s0; q < e0; ++q) {
+      const uint64_t o = buf[q];
+      uint32_t t;
+      // rank += (c < o): the borrow of the 64-bit subtraction c - o, two full-rate instructions
+      asm("v_sub_co_u32 %0, vcc, %2, %4\n\t"
+          "v_subb_co_u32 %0, vcc, %3, %5, vcc\n\t"
+          "v_addc_co_u32 %1, vcc, 0, %1, vcc"
+          : "=&v"(t), "+v"(rank)
+          : "v"(clo), "v"(chi), "v"(uint32_t(o)), "v"(uint32_t(o >> 32))
+          : "vcc");
+    }
+    if (rank < Zc) {
+      out[rank] = int32_t(0xffffffffu - clo);
+      if (val_out) val_out[rank] = key_to_float(chi);
+    }
+  }
+  return true;
+}
+
 // Dense fp32 row as a source; 128-bit loads on the aligned body, kUnroll of
 // them in flight per thread.
 template <int NT = kSelThreads>

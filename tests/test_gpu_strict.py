@@ -241,3 +241,28 @@ def test_out_of_range_query_hash_is_an_empty_bucket(ops, dtype, d):
     groups = ops.group_queries(dev(qh_bad.int()), 5)
     assert torch.equal(groups.bin_count.cpu().long(),
                        torch.stack([torch.bincount(qh[b][good[b]], minlength=5) for b in range(2)]))
+
+
+# ------------------------------------------------------------------ a2 in the fused build: ties and long runs
+@pytest.mark.parametrize("copies", [3, 40, 700])
+def test_fused_build_with_duplicated_keys(ops, copies):
+    """The selection of the fused build places every candidate by counting the larger ones in its value
+    bin, and hands rows with very long runs of (nearly) equal values to the radix select and the sorting
+    network.  Keys repeated `copies` times give runs of exactly equal projections -- short runs stay in
+    the bins (ties by ascending index), 700 copies exceed what a bin takes -- and in every case the lists
+    must equal the stable descending sort of the GPU's own Y and those of the unfused build."""
+    g = gen(7700 + copies)
+    H, C, N, d, Z = 1, 24, 70000, 128, 2048
+    base = (torch.randn(H, N // copies + 1, d, generator=g) * 0.5)
+    K = base.repeat_interleave(copies, dim=1)[:, :N]
+    perm = torch.randperm(N, generator=g)
+    K = K[:, perm].contiguous().to(torch.bfloat16)                 # equal keys scattered over the index range
+    A = torch.randn(H, C, d, generator=g).to(torch.bfloat16)
+    Ad, Kd = dev(A, K)
+    fused, fv = ops.build_index(Ad, Kd, Z, fused=True, return_values=True)
+    assert ops.last_build_info["path"] == "fused" and ops.last_build_info["rows_unresolved"] == 0
+    Y = ops.project(Ad, Kd).cpu()
+    ref = torch.sort(Y + 0.0, dim=-1, descending=True, stable=True)
+    assert torch.equal(fused.cpu().long(), ref.indices[..., :Z]), "lists differ from the stable sort"
+    assert torch.equal(fv.cpu(), ref.values[..., :Z])
+    assert torch.equal(fused, ops.build_index(Ad, Kd, Z, fused=False))

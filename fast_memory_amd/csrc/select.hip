@@ -96,9 +96,12 @@ template <int NT, bool WIDE = false>
 __global__ __launch_bounds__(NT) void argtopz_kernel(
     const float* __restrict__ Y, int N, int64_t ldy, int Zc, int P, int32_t* __restrict__ idx_out,
     float* __restrict__ val_out, const int32_t* __restrict__ row_map, const int32_t* __restrict__ n_rows_dev,
-    SamplePlan sp) {
-  extern __shared__ uint64_t buf[];  // P composites in the sort's layout; before that, up to sp.cap candidates
-  __shared__ SelectShared sh;
+    SamplePlan sp, int sh_off) {
+  // dynamic LDS: [P composites in the sort's layout, or before that up to sp.cap candidates | SelectShared];
+  // the binned selection of the sampled path reuses all of it as [Zc + kSelMaxBin composites | histogram]
+  extern __shared__ uint64_t buf[];
+  __shared__ BinShared bs;
+  SelectShared& sh = *reinterpret_cast<SelectShared*>(reinterpret_cast<char*>(buf) + sh_off);
   if (n_rows_dev && int(blockIdx.x) >= *n_rows_dev) return;
   const int64_t out_row = row_map ? row_map[blockIdx.x] : int64_t(blockIdx.x);
   const float* row = Y + int64_t(blockIdx.x) * ldy;
@@ -118,15 +121,17 @@ __global__ __launch_bounds__(NT) void argtopz_kernel(
     const uint64_t tau = radix_select_cut<NT>(smp, sp.rank, 3, sh) & 0xffffffff00000000ull;  // value bits only
     if (tid == 0) sh.cnt = 0;
     __syncthreads();
+    // tau has value bits only, so "composite >= tau" is a comparison of values: one float compare per
+    // element of the row (NaN, the largest key, passes: it is not below anything)
+    const float tau_f = key_to_float(uint32_t(tau >> 32));
     src([&](float y, uint32_t i) {
-      const uint64_t c = composite(y, i);
-      if (c >= tau) {
+      if (!(y < tau_f)) {
         const int pos = atomicAdd(&sh.cnt, 1);
         if (pos < sp.cap) {
           if constexpr (WIDE)
             reinterpret_cast<uint32_t*>(buf)[pos] = i;
           else
-            buf[pos] = c;
+            buf[pos] = composite(y, i);
         }
       }
     });
@@ -146,7 +151,11 @@ __global__ __launch_bounds__(NT) void argtopz_kernel(
             cr.c[r] = buf[tid + r * NT];
           }
         }
-      const uint64_t cut = radix_select_cut<NT>(cr, Zc, 6, sh);  // (its barriers order the reads above before the writes below)
+      __syncthreads();  // every candidate is in registers before the buffer is written again
+      if (binned_select_write<NT>(cr, Zc, buf, reinterpret_cast<uint32_t*>(buf + (Zc + kSelMaxBin)), bs, out, vout))
+        return;
+      __syncthreads();
+      const uint64_t cut = radix_select_cut<NT>(cr, Zc, 6, sh);
       collect_sort_write(cr, cut, Zc, P, buf, sh, out, vout);
       return;
     }
@@ -172,19 +181,27 @@ int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int
       wide = sp.n_lines > 0;
     }
   }
-  const size_t lds = std::max(sort_lds_bytes(P), size_t(sp.cap) * (wide ? sizeof(uint32_t) : sizeof(uint64_t)));
+  // SelectShared sits behind the sort buffer / the candidate buffer; the binned selection needs its own extent
+  const size_t sh_off = align_up(std::max(sort_lds_bytes(P), size_t(sp.cap) * (wide ? sizeof(uint32_t) : sizeof(uint64_t))), 16);
+  const auto lds_for = [](size_t off, int zc, bool sampled) {
+    const size_t binned = sampled ? size_t(zc + kSelMaxBin) * sizeof(uint64_t) + size_t(kSelBins) * sizeof(uint32_t) : 0;
+    return std::max(off + sizeof(SelectShared), binned);
+  };
+  const size_t lds = lds_for(sh_off, Zc, sp.n_lines > 0);
+  const size_t lds_max = lds_for(align_up(std::max(sort_lds_bytes(FM_MAX_Z), size_t(kCollectRegsWide) * kSelThreads * 4), 16),
+                                 FM_MAX_Z, true);
   if (narrow) {
-    FM_ALLOW_LDS(argtopz_kernel<512>, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
+    FM_ALLOW_LDS(argtopz_kernel<512>, lds_max, "argtopz: lds");
     hipLaunchKernelGGL(argtopz_kernel<512>, dim3(unsigned(rows)), dim3(512), lds, st, Y, N, ldy, Zc, P, idx_out,
-                       val_out, row_map, n_rows_dev, sp);
+                       val_out, row_map, n_rows_dev, sp, int(sh_off));
   } else if (wide) {
-    FM_ALLOW_LDS((argtopz_kernel<kSelThreads, true>), sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
+    FM_ALLOW_LDS((argtopz_kernel<kSelThreads, true>), lds_max, "argtopz: lds");
     hipLaunchKernelGGL((argtopz_kernel<kSelThreads, true>), dim3(unsigned(rows)), dim3(kSelThreads), lds, st, Y, N,
-                       ldy, Zc, P, idx_out, val_out, row_map, n_rows_dev, sp);
+                       ldy, Zc, P, idx_out, val_out, row_map, n_rows_dev, sp, int(sh_off));
   } else {
-    FM_ALLOW_LDS(argtopz_kernel<kSelThreads>, sort_lds_bytes(FM_MAX_Z), "argtopz: lds");
+    FM_ALLOW_LDS(argtopz_kernel<kSelThreads>, lds_max, "argtopz: lds");
     hipLaunchKernelGGL(argtopz_kernel<kSelThreads>, dim3(unsigned(rows)), dim3(kSelThreads), lds, st, Y, N, ldy, Zc,
-                       P, idx_out, val_out, row_map, n_rows_dev, sp);
+                       P, idx_out, val_out, row_map, n_rows_dev, sp, int(sh_off));
   }
   return launch_status("argtopz");
 }

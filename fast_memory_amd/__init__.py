@@ -9,6 +9,8 @@ from .hash_attention import attention_hash, attention_hash_varlen, attention_has
 from .memory import (Memory, MemoryBatch, calc_ref_centroids, compute_centroids, fit_projection, init_centroids, kmeans_spherical, learn_emb_proj,  # noqa: F401
                      merge, ring_attention_masked_backward, ring_attention_masked_forward, update_out_and_lse)
 
-__all__ = ["attention_hash", "attention_hash_varlen", "attention_hash_varlen_backward", "Memory", "MemoryBatch", "calc_ref_centroids", "compute_centroids", "fit_projection",
+from .autograd import attention_hash_varlen_op, local_attention_backward, ring_cross_attention_approx  # noqa: F401,E402
+
+__all__ = ["attention_hash_varlen_op", "local_attention_backward", "ring_cross_attention_approx", "attention_hash", "attention_hash_varlen", "attention_hash_varlen_backward", "Memory", "MemoryBatch", "calc_ref_centroids", "compute_centroids", "fit_projection",
            "init_centroids", "kmeans_spherical", "learn_emb_proj", "merge", "ring_attention_masked_backward", "ring_attention_masked_forward",
            "update_out_and_lse"]

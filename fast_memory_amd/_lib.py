@@ -40,12 +40,12 @@ SIGNATURES = {
     "fm_group_queries": (c_int, [P, c_int, c_int, c_int, P, P, P, P, P, c_int64, P, c_size_t, P]),
     "fm_hash_attn_fwd": (c_int, [P, P, P, P, P, P, P, P, P, c_int64, P, P, c_int, c_int, c_int, c_int,
                                  c_int, c_float, c_int, P]),
-    "fm_hash_attn_bwd": (c_int, [P, P, P, P, P, P, P, P, P, c_int64, P, P, P, P, P, P, c_int, c_int, c_int, c_int,
+    "fm_hash_attn_bwd": (c_int, [P, P, P, P, P, P, P, P, P, c_int64, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int,
                                  c_int, c_float, c_int, P]),
     "fm_inverse_index_workspace": (c_size_t, [c_int64, c_int, c_int]),
     "fm_inverse_index": (c_int, [P, P, P, c_int, c_int, c_int, c_int64, P, P, P, c_size_t, P]),
     "fm_hash_attn_bwd_staged_workspace": (c_size_t, [c_int64]),
-    "fm_hash_attn_bwd_staged": (c_int, [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, c_int, c_int, c_int,
+    "fm_hash_attn_bwd_staged": (c_int, [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, c_int, c_int, c_int,
                                         c_int, c_int, P, c_float, c_int, P, c_size_t, P]),
     "fm_attention_hash_varlen_workspace": (c_size_t, [c_int, c_int, c_int]),
     "fm_attention_hash_varlen": (c_int, [P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int,

@@ -18,7 +18,7 @@ namespace fm {
 
 template <typename T>
 __device__ __forceinline__ void backward_one_query(const T* __restrict__ qrow, const T* __restrict__ orow,
-                                                   const T* __restrict__ dorow, float lse,
+                                                   const T* __restrict__ dorow, float lse, float dlse,
                                                    const T* __restrict__ Kb, const T* __restrict__ Vb,
                                                    const int32_t* __restrict__ idx, int cnt, int N, int d,
                                                    float sm_scale, T* __restrict__ dq_row,
@@ -34,7 +34,7 @@ __device__ __forceinline__ void backward_one_query(const T* __restrict__ qrow, c
     dov[r] = k < d ? Elem<T>::load(dorow + k) : 0.f;
     dpart += k < d ? dov[r] * Elem<T>::load(orow + k) : 0.f;
   }
-  const float D = wave_sum(dpart);
+  const float D = wave_sum(dpart) - dlse;  // dS = P (dP - D) + P dlse
   const float lse2 = lse * kLog2e;
   const float scale2 = sm_scale * kLog2e;
   for (int j0 = 0; j0 < cnt; j0 += kWave) {
@@ -81,8 +81,8 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const int32_t* __restrict__ k_idx,
     const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
     const int32_t* __restrict__ q_perm, const fm_item* __restrict__ items, const int32_t* __restrict__ n_items,
-    const T* __restrict__ out, const float* __restrict__ lse, const T* __restrict__ dout, T* __restrict__ dq,
-    float* __restrict__ dk, float* __restrict__ dv, int Sq, int N, int d, int C, float sm_scale) {
+    const T* __restrict__ out, const float* __restrict__ lse, const T* __restrict__ dout,
+    const float* __restrict__ dlse, T* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv, int Sq, int N, int d, int C, float sm_scale) {
   if (int(blockIdx.x) >= *n_items) return;
   const fm_item it = items[blockIdx.x];
   const int64_t b = int64_t(it.row) * C + it.bucket;
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_generic_kernel(
   for (int j = threadIdx.x >> 6; j < it.n_q; j += 4) {
     const int qi = q_perm[it.q_start + j];
     const int64_t qrow = int64_t(it.row) * Sq + qi;
-    backward_one_query<T>(q + qrow * d, out + qrow * d, dout + qrow * d, lse[qrow], k + kv, v + kv, idx, cnt, N, d,
+    backward_one_query<T>(q + qrow * d, out + qrow * d, dout + qrow * d, lse[qrow], dlse ? dlse[qrow] : 0.f, k + kv, v + kv, idx, cnt, N, d,
                           sm_scale, dq + qrow * d, dk + kv, dv + kv);
   }
 }
@@ -101,16 +101,16 @@ extern int g_force_generic;
 bool hash_attn_bwd_mfma_supported(int d, int dtype);
 int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                        const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
-                       int64_t max_items, const void* out, const float* lse, const void* dout, void* dq, float* dk,
-                       float* dv, int Sq, int N, int C, float sm_scale, hipStream_t st);
+                       int64_t max_items, const void* out, const float* lse, const void* dout, const float* dlse, void* dq,
+                       float* dk, float* dv, int Sq, int N, int C, float sm_scale, hipStream_t st);
 
 }  // namespace fm
 
 extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
                                 const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                                 const fm_item* items, const int32_t* n_items, int64_t max_items, const void* out,
-                                const float* lse, const void* dout, void* dq, float* dk, float* dv, int H, int Sq,
-                                int N, int d, int C, float sm_scale, int dtype, void* stream) {
+                                const float* lse, const void* dout, const float* dlse, void* dq, float* dk, float* dv,
+                                int H, int Sq, int N, int d, int C, float sm_scale, int dtype, void* stream) {
   using namespace fm;
   FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_hash_attn_bwd: H=%d Sq=%d N=%d C=%d d=%d", H, Sq, N, C, d);
@@ -123,15 +123,15 @@ extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, con
   hipStream_t st = as_stream(stream);
   if (g_force_generic != 1 && hash_attn_bwd_mfma_supported(d, dtype))
     return hash_attn_bwd_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse,
-                              dout, dq, dk, dv, Sq, N, C, sm_scale, st);
+                              dout, dlse, dq, dk, dv, Sq, N, C, sm_scale, st);
   if (dtype == FM_F32)
     hipLaunchKernelGGL(hash_attn_bwd_generic_kernel<float>, dim3(unsigned(max_items)), dim3(256), 0, st,
                        (const float*)q, (const float*)k, (const float*)v, k_idx, bucket_off, bucket_cnt, q_perm, items,
-                       n_items, (const float*)out, lse, (const float*)dout, (float*)dq, dk, dv, Sq, N, d, C, sm_scale);
+                       n_items, (const float*)out, lse, (const float*)dout, dlse, (float*)dq, dk, dv, Sq, N, d, C, sm_scale);
   else
     hipLaunchKernelGGL(hash_attn_bwd_generic_kernel<bf16_t>, dim3(unsigned(max_items)), dim3(256), 0, st,
                        (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
-                       items, n_items, (const bf16_t*)out, lse, (const bf16_t*)dout, (bf16_t*)dq, dk, dv, Sq, N, d, C,
+                       items, n_items, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, Sq, N, d, C,
                        sm_scale);
   return launch_status("fm_hash_attn_bwd");
 }

@@ -114,7 +114,7 @@ __device__ __forceinline__ void bwd_load_block(BwdBlock& r, const bf16_t* __rest
 template <bool STAGED, bool FIRST_TILE, int TILES = 1>
 __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ out,
                                          const float* __restrict__ lse, const bf16_t* __restrict__ dout,
-                                         const int32_t* __restrict__ q_list, int n_q, int64_t qbase,
+                                         const float* __restrict__ dlse, const int32_t* __restrict__ q_list, int n_q, int64_t qbase,
                                          const bf16_t* __restrict__ Kb, const bf16_t* __restrict__ Vb,
                                          const int32_t* __restrict__ idx, int cnt, int N, float sm_scale,
                                          bf16_t* __restrict__ dq, float* __restrict__ dKb, float* __restrict__ dVb,
@@ -160,6 +160,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
   }
   Dc += __shfl_xor(Dc, 16);
   Dc += __shfl_xor(Dc, 32);  // D of query c, in all four lane groups
+  // a gradient of the log-sum-exp enters dS = P (dP - D) as dS += P dlse: fold it into D
+  if (dlse != nullptr && myq >= 0) Dc -= dlse[qbase + myq];
   // a lane column without a query gets lse = +inf: every probability is 0
   const float lse2c = myq >= 0 ? lse[qbase + myq] * kLog2e : INFINITY;
   float Dq[4], lse2q[4];  // the same for queries 4g+r (the other orientation)
@@ -466,7 +468,7 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
     const int32_t* __restrict__ q_perm, const fm_item* __restrict__ items, const int32_t* __restrict__ n_items,
     const bf16_t* __restrict__ out, const float* __restrict__ lse, const bf16_t* __restrict__ dout,
-    bf16_t* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv, int Sq, int N, int C, float sm_scale) {
+    const float* __restrict__ dlse, bf16_t* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv, int Sq, int N, int C, float sm_scale) {
   __shared__ __attribute__((aligned(16))) float red[4 * 8 * 4 * 64];  // dQ partials [wave][t][r][lane]
   __shared__ int q_rows[16];
   if (int(blockIdx.x) >= *n_items) return;
@@ -474,7 +476,7 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
   const int q0 = int(blockIdx.y) * 16;  // this workgroup's query tile inside the item
   if (q0 >= it.n_q) return;
   const int64_t bkt = int64_t(it.row) * C + it.bucket;
-  bwd_tile<false, true>(q, out, lse, dout, q_perm + it.q_start + q0, min(16, it.n_q - q0), int64_t(it.row) * Sq,
+  bwd_tile<false, true>(q, out, lse, dout, dlse, q_perm + it.q_start + q0, min(16, it.n_q - q0), int64_t(it.row) * Sq,
                   k + int64_t(it.row) * N * kBD, v + int64_t(it.row) * N * kBD, k_idx + bucket_off[bkt],
                   bucket_cnt[bkt], N, sm_scale, dq, dk + int64_t(it.row) * N * kBD, dv + int64_t(it.row) * N * kBD,
                   nullptr, nullptr, nullptr, red, q_rows, nullptr);
@@ -491,7 +493,7 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
     const int32_t* __restrict__ q_perm, const int32_t* __restrict__ bin_off, const int32_t* __restrict__ bin_count,
     const bf16_t* __restrict__ out, const float* __restrict__ lse, const bf16_t* __restrict__ dout,
-    bf16_t* __restrict__ dq, bf16_t* dkp, bf16_t* dvp, bf16_t* dump, int64_t pos0, int row0, int Sq, int N, int C,
+    const float* __restrict__ dlse, bf16_t* __restrict__ dq, bf16_t* dkp, bf16_t* dvp, bf16_t* dump, int64_t pos0, int row0, int Sq, int N, int C,
     float sm_scale) {
   // the waves' staging slabs ([wave][dV | dK][16][kStLd] bf16) during a tile's blocks, then the dQ partial
   // sums ([wave][t][r][lane] fp32) at its end
@@ -522,7 +524,7 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
     if (q0) __syncthreads();  // red and q_rows are reused
     const int left = nq - q0;
 #define FM_BWD_PASS(FIRST, NT)                                                                                        \
-  bwd_tile<true, FIRST, NT>(q, out, lse, dout, ql + q0, min(16 * NT, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,  \
+  bwd_tile<true, FIRST, NT>(q, out, lse, dout, dlse, ql + q0, min(16 * NT, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,  \
                             cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage)
     if (MAXT == 4 && left > 32) {
       if (q0 == 0)
@@ -548,24 +550,24 @@ bool hash_attn_bwd_mfma_supported(int d, int dtype) { return d == kBD && dtype =
 
 int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                        const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
-                       int64_t max_items, const void* out, const float* lse, const void* dout, void* dq, float* dk,
-                       float* dv, int Sq, int N, int C, float sm_scale, hipStream_t st) {
+                       int64_t max_items, const void* out, const float* lse, const void* dout, const float* dlse, void* dq,
+                       float* dk, float* dv, int Sq, int N, int C, float sm_scale, hipStream_t st) {
   dim3 grid = dim3(unsigned(max_items), unsigned(FM_QTILE / 16));
   hipLaunchKernelGGL(hash_attn_bwd_mfma_kernel, grid, dim3(256), 0, st, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, (const bf16_t*)out, lse,
-                     (const bf16_t*)dout, (bf16_t*)dq, dk, dv, Sq, N, C, sm_scale);
+                     (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, Sq, N, C, sm_scale);
   return launch_status("fm_hash_attn_bwd(mfma)");
 }
 
 int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, const int32_t* k_idx,
                                   const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                                   const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
-                                  const void* dout, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0, int row0,
-                                  int rows, int Sq, int N, int C, float sm_scale, hipStream_t st) {
+                                  const void* dout, const float* dlse, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0,
+                                  int row0, int rows, int Sq, int N, int C, float sm_scale, hipStream_t st) {
 #define FM_BWD_STAGED(MAXT)                                                                                        \
   hipLaunchKernelGGL(hash_attn_bwd_staged_kernel<MAXT>, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,       \
                      (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,  \
-                     bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, (bf16_t*)dq, (bf16_t*)dkp,  \
+                     bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, (bf16_t*)dkp,  \
                      (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale)
   if (int64_t(Sq) > 24 * int64_t(C))  // more than 24 queries per bucket on average
     FM_BWD_STAGED(4);

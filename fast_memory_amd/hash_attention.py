@@ -94,7 +94,8 @@ def attention_hash(q, k, v, centroids, bucket_size, sm_scale, window=None):
 def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                                    out: torch.Tensor, lse: torch.Tensor, k_hashes: torch.Tensor,
                                    k_hash_counts: torch.Tensor, q_hashes: torch.Tensor, sm_scale: float,
-                                   staged: Optional[bool] = None, inverse_index=None
+                                   staged: Optional[bool] = None, inverse_index=None,
+                                   d_lse: Optional[torch.Tensor] = None
                                    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of :func:`attention_hash_varlen` w.r.t. ``q``, ``k`` and ``v``.
 
@@ -107,6 +108,8 @@ def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torc
         sum per key; needs the inverse of the lists), ``False`` the atomic adds; ``None`` picks the staged
         path when there are at least as many queries per row as buckets, i.e. when most buckets receive
         queries.
+    :param d_lse: gradient w.r.t. the returned (natural-log, fp32) LSE ``[batch, q_seq_len]``, for callers that
+        differentiate through a merge of partial results done outside; ``None`` = zero.
     :param inverse_index: ``ops.inverse_index(...)`` of these lists, if the caller keeps one (it depends on
         the lists only); built here otherwise.
     :return: ``(dq [batch, q_seq_len, d_head], dk, dv [batch, kv_seq_len, d_head])``; ``dq`` in q's dtype,
@@ -131,11 +134,11 @@ def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torc
             inv = inverse_index if inverse_index is not None else ops.inverse_index(lists, off, counts, k.shape[1])
             if inv.row_pos[-1] > 0:        # no listed entry at all: nothing to stage, the other form handles it
                 return ops.hash_attn_bwd_staged(q, k, v, lists, off, counts, groups, inv, out.contiguous(),
-                                                lse.float().contiguous(), d_out.contiguous(), sm_scale)
+                                                lse.float().contiguous(), d_out.contiguous(), sm_scale, dlse=d_lse)
         except torch.cuda.OutOfMemoryError:
             if not auto:
                 raise                      # asked for explicitly: report that its workspace does not fit
             torch.cuda.empty_cache()       # chosen here: the atomic form needs no workspace
     return ops.hash_attn_bwd(q, k, v, lists, off, counts, groups, out.contiguous(),
-                             lse.float().contiguous(), d_out.contiguous(), sm_scale)
+                             lse.float().contiguous(), d_out.contiguous(), sm_scale, dlse=d_lse)
 

@@ -229,11 +229,14 @@ def hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, s
 
 
 def hash_attn_bwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, out, lse, dout, sm_scale: float,
-                  dk: Optional[torch.Tensor] = None, dv: Optional[torch.Tensor] = None):
+                  dk: Optional[torch.Tensor] = None, dv: Optional[torch.Tensor] = None,
+                  dlse: Optional[torch.Tensor] = None):
     """Backward of :func:`hash_attn_fwd` (memory.py:166-206 on the gathered pairs).  ``out`` / ``lse`` are
     the forward's result or the merged one; ``dout [H,Sq,d]``.  Returns ``dq`` (dtype of q) and the fp32
-    ``dk``, ``dv [H,N,d]``; when ``dk`` / ``dv`` are given the gradients are added into them."""
+    ``dk``, ``dv [H,N,d]``; when ``dk`` / ``dv`` are given the gradients are added into them.  ``dlse [H,Sq]``
+    fp32 (optional) is the gradient w.r.t. the returned log-sum-exp."""
     _dev(q, k, v, k_idx, bucket_off, bucket_cnt, out, lse, dout)
+    dlse = _check_dlse(dlse, lse)
     H, Sq, d = q.shape
     _, N, _ = k.shape
     C = bucket_cnt.shape[-1]
@@ -248,9 +251,16 @@ def hash_attn_bwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, o
     assert dk.dtype == dv.dtype == torch.float32 and dk.shape == dv.shape == (H, N, d)
     check(_lib.load().fm_hash_attn_bwd(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
                                        _p(groups.q_perm), _p(groups.items), _p(groups.n_items), groups.max_items,
-                                       _p(out), _p(lse), _p(dout), _p(dq), _p(dk), _p(dv), H, Sq, N, d, C,
+                                       _p(out), _p(lse), _p(dout), _p(dlse), _p(dq), _p(dk), _p(dv), H, Sq, N, d, C,
                                        float(sm_scale), _dt(q), _stream(q)))
     return dq, dk, dv
+
+
+def _check_dlse(dlse: Optional[torch.Tensor], lse: torch.Tensor) -> Optional[torch.Tensor]:
+    if dlse is None:
+        return None
+    assert dlse.shape == lse.shape and dlse.is_cuda
+    return dlse.to(torch.float32).contiguous()
 
 
 class InverseIndex(NamedTuple):
@@ -289,11 +299,13 @@ def inverse_index(k_idx: torch.Tensor, bucket_off: torch.Tensor, bucket_cnt: tor
 
 def hash_attn_bwd_staged(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, inv: InverseIndex, out, lse,
                          dout, sm_scale: float, dk: Optional[torch.Tensor] = None,
-                         dv: Optional[torch.Tensor] = None, workspace_bytes: int = 24 << 30):
+                         dv: Optional[torch.Tensor] = None, workspace_bytes: int = 24 << 30,
+                         dlse: Optional[torch.Tensor] = None):
     """:func:`hash_attn_bwd` without atomics (bf16, d = 128): per-bucket partial rows in a workspace, then a
     sum per key over the list positions that name it (``inv`` from :func:`inverse_index`).  Same results to
     rounding (the partial rows are bf16), in a fixed summation order."""
     _dev(q, k, v, k_idx, bucket_off, bucket_cnt, out, lse, dout)
+    dlse = _check_dlse(dlse, lse)
     H, Sq, d = q.shape
     _, N, _ = k.shape
     C = bucket_cnt.shape[-1]
@@ -314,7 +326,7 @@ def hash_attn_bwd_staged(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGr
     row_pos = (ctypes.c_int64 * (H + 1))(*inv.row_pos)
     check(lib.fm_hash_attn_bwd_staged(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
                                       _p(groups.q_perm), _p(groups.bin_off), _p(groups.bin_count), _p(out), _p(lse),
-                                      _p(dout), _p(inv.key_off), _p(inv.inv_pos), _p(dq), _p(dk),
+                                      _p(dout), _p(dlse), _p(inv.key_off), _p(inv.inv_pos), _p(dq), _p(dk),
                                       _p(dv), H, Sq, N, d, C, ctypes.cast(row_pos, ctypes.c_void_p), float(sm_scale),
                                       _dt(q), _p(ws), ws.numel(), _stream(q)))
     return dq, dk, dv

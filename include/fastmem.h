@@ -161,6 +161,8 @@ int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t*
  *                                      with further keys (the gradients are then
  *                                      the gathered keys' share)
  *   dout [H,Sq,d]                      gradient of the loss w.r.t. out
+ *   dlse [H,Sq] fp32, may be NULL      gradient of the loss w.r.t. lse (a caller that merges
+ *                                      partial results by their lse outside has one; NULL = 0)
  *   dq [H,Sq,d] (dtype of q)           written; a query whose bucket is empty gets 0
  *   dk, dv [H,N,d] fp32                ACCUMULATED into (atomic adds): zero them
  *                                      before the first call; several calls
@@ -170,8 +172,8 @@ int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t*
 int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
                      const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                      const fm_item* items, const int32_t* n_items, int64_t max_items, const void* out,
-                     const float* lse, const void* dout, void* dq, float* dk, float* dv, int H, int Sq, int N,
-                     int d, int C, float sm_scale, int dtype, void* stream);
+                     const float* lse, const void* dout, const float* dlse, void* dq, float* dk, float* dv, int H,
+                     int Sq, int N, int d, int C, float sm_scale, int dtype, void* stream);
 
 /* ---- f1, dense query sets: backward without atomics ---------------------------
  * Same gradients as fm_hash_attn_bwd (bf16, d = 128 only).  A key's dk and dv rows
@@ -203,8 +205,8 @@ size_t fm_hash_attn_bwd_staged_workspace(int64_t max_row_entries);
 int fm_hash_attn_bwd_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
                             const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                             const int32_t* bin_off, const int32_t* bin_count, const void* out,
-                            const float* lse, const void* dout, const int32_t* key_off,
-                            const int32_t* inv_pos, void* dq, float* dk,
+                            const float* lse, const void* dout, const float* dlse,
+                            const int32_t* key_off, const int32_t* inv_pos, void* dq, float* dk,
                             float* dv, int H, int Sq, int N, int d, int C, const int64_t* row_pos_host,
                             float sm_scale, int dtype, void* ws, size_t ws_bytes, void* stream);
 

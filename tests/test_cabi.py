@@ -47,8 +47,8 @@ def test_argument_errors_are_status_codes():
     assert b"fm_index_append" in lib.fm_last_error()
     assert lib.fm_inverse_index(None, None, None, 1, 1, 1, 1, None, None, None, 0, None) == 1
     assert lib.fm_hash_attn_bwd(None, None, None, None, None, None, None, None, None, 1, None, None, None, None,
-                                None, None, 1, 1, 1, 8, 1, 1.0, 0, None) != 0
-    assert lib.fm_hash_attn_bwd_staged(*([None] * 17), 1, 1, 1, 64, 1, None, 1.0, 1, None, 0, None) != 0   # d = 64
+                                None, None, None, 1, 1, 1, 8, 1, 1.0, 0, None) != 0
+    assert lib.fm_hash_attn_bwd_staged(*([None] * 18), 1, 1, 1, 64, 1, None, 1.0, 1, None, 0, None) != 0   # d = 64
     assert b"fm_hash_attn_bwd_staged" in lib.fm_last_error()
     assert lib.fm_segment_sum(None, None, None, None, None, 1, 1, 1, 8, 0, None) != 0
     with pytest.raises(ValueError):

@@ -286,14 +286,15 @@ def bench_reference_harness(args):
     groups x 32768 queries, 65536 keys, d = 128, 1024 buckets of 3072 keys, q / k / v / centroids ~ N(0,1);
     one step = attention_hash(q, k, v, centroids, bucket_size, sm_scale), i.e. index build + query hash +
     grouping + attention, and the figure it prints is the dense-equivalent 4*B*G*S*N*d flops per second.
-    The reference runs it in fp16; bf16 here (same width; the MFMA kernels take bf16)."""
+    fp16 as in the reference (triton_kernel.py:496); ``--tk-dtype bf16`` runs the same shape in bf16."""
     from fast_memory_amd import attention_hash, ops
     B, G, S, N, d, C, Z = 8, 4, 32768, 65536, 128, 1024, 3072
     Sq = G * S
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     g = torch.Generator(device="cpu").manual_seed(1006)
-    mk = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    tk_dtype = torch.float16 if args.tk_dtype == "fp16" else torch.bfloat16
+    mk = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float32).to(tk_dtype).to(dev)
     k, v, centroids = mk(B, N, d), mk(B, N, d), mk(B, C, d)
     q = torch.cat([mk(1, Sq, d) for _ in range(B)])
     sm_scale = d ** -0.5
@@ -324,7 +325,7 @@ def bench_reference_harness(args):
     alg_bytes = hit * Z * (2 * d * 2 + 4) + qheads * (2 * d * 2 + 4)
     alg_flops = 4.0 * d * Z * qheads
     achieved = alg_bytes / attn_ms / 1e6
-    attn_kernel = ops.hash_attn_fwd_kernel_name(B, Sq, N, d, C, torch.bfloat16)
+    attn_kernel = ops.hash_attn_fwd_kernel_name(B, Sq, N, d, C, tk_dtype)
     roofline = {"kernel": attn_kernel, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": hbm_traffic(attn_kernel, "tkperf"),
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms, "hit_buckets": hit,
@@ -379,7 +380,8 @@ def bench_reference_harness(args):
     line = {
         "metric": "hashed-attn query-heads/s", "value": value, "unit": "query-heads/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16" if tk_dtype == torch.float16 else "bf16",
+        "data": "synthetic",
         "config": {"workload": f"tkperf: the reference's performance harness, {B} rows x {G} groups x {S} queries, "
                                f"N={N} keys, d={d}, C={C}, Z={Z}, q/k/v/centroids ~ N(0,1)",
                    "step": "attention_hash: index build + query hash + grouping + gather attention"},
@@ -403,6 +405,8 @@ def main():
     ap.add_argument("--no-backward", action="store_true", help="skip timing the backward of the gathered attention")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--workspace-gib", type=float, default=8.0)
+    ap.add_argument("--tk-dtype", default="fp16", choices=["fp16", "bf16"],
+                    help="element type of --config tkperf (the reference's harness runs fp16)")
     ap.add_argument("--no-control", action="store_true",
                     help="skip the no-reuse control of the attention roofline (69 GB of K and V listed once)")
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -12,7 +12,7 @@ from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfastmem.so")
 
-FM_F32, FM_BF16 = 0, 1
+FM_F32, FM_BF16, FM_F16 = 0, 1, 2
 FM_MAX_Z = 16384
 FM_MAX_D = 256
 FM_QTILE = 64

@@ -13,11 +13,11 @@ int hash_attn_generic(const void* q, const void* k, const void* v, const int32_t
 int local_attn_generic(const void* q, const void* k, const void* v, void* out, float* lse, int H,
                        int G, int S, int L, int d, float sm_scale, int causal, int dtype,
                        hipStream_t st);
-bool hash_attn_mfma_supported(int d, int dtype);
+bool hash_attn_mfma_supported(int d, int dtype, int N);
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
                    const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, hipStream_t st);
+                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype, hipStream_t st);
 int hash_attn_mfma_choice(int H, int Sq, int N, int C);
 bool local_attn_mfma_supported(int d, int dtype);
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
@@ -37,8 +37,10 @@ extern "C" void fm_debug_force_generic(int on) { fm::g_force_generic = on; }
 
 extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype) {
   using namespace fm;
-  if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype)) return "hash_attn_generic_kernel";
-  switch (hash_attn_mfma_choice(H, Sq, N, C)) {
+  if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype, N)) return "hash_attn_generic_kernel";
+  const int choice = hash_attn_mfma_choice(H, Sq, N, C);
+  if (dtype == FM_F16) return choice == 2 ? "hash_attn_staged_kernel<2, f16>" : "hash_attn_staged_kernel<1, f16>";
+  switch (choice) {
     case 1: return "hash_attn_staged_kernel<1>";
     case 2: return "hash_attn_staged_kernel<2>";
     default: return "hash_attn_mfma_kernel";
@@ -53,16 +55,16 @@ extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, con
   using namespace fm;
   FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_hash_attn_fwd: H=%d Sq=%d N=%d C=%d d=%d", H, Sq, N, C, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_hash_attn_fwd: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_hash_attn_fwd: dtype=%d", dtype);
   FM_REQUIRE(q && k && v && k_idx && bucket_off && bucket_cnt && q_perm && items && n_items && out &&
                  lse,
              FM_ERR_ARG, "fm_hash_attn_fwd: null pointer");
   FM_REQUIRE(max_items >= 1 && max_items <= 0x7fffffffLL, FM_ERR_ARG,
              "fm_hash_attn_fwd: max_items=%lld", (long long)max_items);
   hipStream_t st = as_stream(stream);
-  if (g_force_generic != 1 && hash_attn_mfma_supported(d, dtype))
+  if (g_force_generic != 1 && hash_attn_mfma_supported(d, dtype, N))
     return hash_attn_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items,
-                          out, lse, H, Sq, N, d, C, sm_scale, st);
+                          out, lse, H, Sq, N, d, C, sm_scale, dtype, st);
   return hash_attn_generic(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
                            max_items, out, lse, Sq, N, d, C, sm_scale, dtype, st);
 }
@@ -133,7 +135,7 @@ static int varlen_run(const void* q, const void* k, const void* v, const int32_t
   rc = fm_hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, w.max_items, out,
                         lse, H, Sq, N, d, C, sm_scale, dtype, stream);
   if (rc) return rc;
-  const int row_bytes = d * (dtype == FM_BF16 ? 2 : 4);
+  const int row_bytes = d * dtype_bytes(dtype);
   const int64_t nq = int64_t(H) * Sq;
   hipLaunchKernelGGL(unhashed_rows_kernel, dim3(unsigned(ceil_div(nq, 4))), dim3(256), 0, as_stream(stream),
                      q_hash, nq, C, row_bytes / 2, static_cast<uint16_t*>(out), lse);
@@ -221,7 +223,7 @@ extern "C" int fm_local_attn_fwd(const void* q, const void* k, const void* v, vo
   using namespace fm;
   FM_REQUIRE(H >= 1 && G >= 1 && S >= 1 && L >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_local_attn_fwd: H=%d G=%d S=%d L=%d d=%d", H, G, S, L, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_local_attn_fwd: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_local_attn_fwd: dtype=%d", dtype);
   FM_REQUIRE(q && k && v && out && lse, FM_ERR_ARG, "fm_local_attn_fwd: null pointer");
   FM_REQUIRE(int64_t(H) * G <= 65535, FM_ERR_UNSUPPORTED, "fm_local_attn_fwd: H*G > 65535");
   hipStream_t st = as_stream(stream);

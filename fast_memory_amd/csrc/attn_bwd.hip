@@ -114,7 +114,7 @@ extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, con
   using namespace fm;
   FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_hash_attn_bwd: H=%d Sq=%d N=%d C=%d d=%d", H, Sq, N, C, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_hash_attn_bwd: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_hash_attn_bwd: dtype=%d", dtype);
   FM_REQUIRE(q && k && v && k_idx && bucket_off && bucket_cnt && q_perm && items && n_items && out && lse && dout &&
                  dq && dk && dv,
              FM_ERR_ARG, "fm_hash_attn_bwd: null pointer");
@@ -128,10 +128,15 @@ extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, con
     hipLaunchKernelGGL(hash_attn_bwd_generic_kernel<float>, dim3(unsigned(max_items)), dim3(256), 0, st,
                        (const float*)q, (const float*)k, (const float*)v, k_idx, bucket_off, bucket_cnt, q_perm, items,
                        n_items, (const float*)out, lse, (const float*)dout, dlse, (float*)dq, dk, dv, Sq, N, d, C, sm_scale);
-  else
+  else if (dtype == FM_BF16)
     hipLaunchKernelGGL(hash_attn_bwd_generic_kernel<bf16_t>, dim3(unsigned(max_items)), dim3(256), 0, st,
                        (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
                        items, n_items, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, Sq, N, d, C,
+                       sm_scale);
+  else
+    hipLaunchKernelGGL(hash_attn_bwd_generic_kernel<f16_t>, dim3(unsigned(max_items)), dim3(256), 0, st,
+                       (const f16_t*)q, (const f16_t*)k, (const f16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
+                       items, n_items, (const f16_t*)out, lse, (const f16_t*)dout, dlse, (f16_t*)dq, dk, dv, Sq, N, d, C,
                        sm_scale);
   return launch_status("fm_hash_attn_bwd");
 }

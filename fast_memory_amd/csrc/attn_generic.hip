@@ -181,10 +181,14 @@ int hash_attn_generic(const void* q, const void* k, const void* v, const int32_t
     hipLaunchKernelGGL(hash_attn_generic_kernel<float>, dim3(unsigned(max_items), kGenQSplit), dim3(256), 0, st,
                        (const float*)q, (const float*)k, (const float*)v, k_idx, bucket_off,
                        bucket_cnt, q_perm, items, n_items, (float*)out, lse, Sq, N, d, C, scale2);
-  else
+  else if (dtype == FM_BF16)
     hipLaunchKernelGGL(hash_attn_generic_kernel<bf16_t>, dim3(unsigned(max_items), kGenQSplit), dim3(256), 0,
                        st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off,
                        bucket_cnt, q_perm, items, n_items, (bf16_t*)out, lse, Sq, N, d, C, scale2);
+  else
+    hipLaunchKernelGGL(hash_attn_generic_kernel<f16_t>, dim3(unsigned(max_items), kGenQSplit), dim3(256), 0,
+                       st, (const f16_t*)q, (const f16_t*)k, (const f16_t*)v, k_idx, bucket_off,
+                       bucket_cnt, q_perm, items, n_items, (f16_t*)out, lse, Sq, N, d, C, scale2);
   return launch_status("fm_hash_attn_fwd(generic)");
 }
 
@@ -197,9 +201,13 @@ int local_attn_generic(const void* q, const void* k, const void* v, void* out, f
     hipLaunchKernelGGL(local_attn_generic_kernel<float>, grid, dim3(256), 0, st, (const float*)q,
                        (const float*)k, (const float*)v, (float*)out, lse, G, S, L, d, scale2,
                        causal);
-  else
+  else if (dtype == FM_BF16)
     hipLaunchKernelGGL(local_attn_generic_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)q,
                        (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)out, lse, G, S, L, d, scale2,
+                       causal);
+  else
+    hipLaunchKernelGGL(local_attn_generic_kernel<f16_t>, grid, dim3(256), 0, st, (const f16_t*)q,
+                       (const f16_t*)k, (const f16_t*)v, (f16_t*)out, lse, G, S, L, d, scale2,
                        causal);
   return launch_status("fm_local_attn_fwd(generic)");
 }

@@ -464,7 +464,11 @@ int local_attn_decode(const void* q, const void* k, const void* v, void* out, fl
   return launch_status("fm_local_attn_fwd(decode)");
 }
 
-bool hash_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_BF16; }
+// bf16: every shape (the register-gather kernel below takes what the staged kernel does not); fp16 has the
+// staged kernel only, which addresses rows by 32-bit byte offsets
+bool hash_attn_mfma_supported(int d, int dtype, int N) {
+  return d == kD && (dtype == FM_BF16 || (dtype == FM_F16 && N <= (1 << 24)));
+}
 
 int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
                      const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, float sm_scale,
@@ -485,7 +489,7 @@ bool local_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM
 int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
                           const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                          float* lse, int Sq, int N, int C, float sm_scale, bool pairs, hipStream_t st);
+                          float* lse, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, hipStream_t st);
 extern int g_force_generic;
 
 // Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
@@ -508,12 +512,13 @@ int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
                    const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, hipStream_t st) {
+                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype, hipStream_t st) {
   (void)d;
-  const int choice = hash_attn_mfma_choice(H, Sq, N, C);
+  int choice = hash_attn_mfma_choice(H, Sq, N, C);
+  if (dtype == FM_F16 && choice == 0) choice = 1;
   if (choice)
     return hash_attn_mfma_staged(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out,
-                                 lse, Sq, N, C, sm_scale, choice == 2, st);
+                                 lse, Sq, N, C, sm_scale, choice == 2, dtype == FM_F16, st);
   FM_ALLOW_LDS(hash_attn_mfma_kernel, kRedFloats * sizeof(float), "fm_hash_attn_fwd: lds");
   hipLaunchKernelGGL(hash_attn_mfma_kernel, dim3(unsigned(max_items)), dim3(256),
                      kRedFloats * sizeof(float), st, (const bf16_t*)q, (const bf16_t*)k,

@@ -8,7 +8,7 @@ namespace fm {
 // CU.  2: a workgroup takes two consecutive items of a bucket (128 queries; the workgroup of the second
 // item exits), each LDS operand read feeds two MFMAs, two workgroups per CU: half the LDS reads,
 // staging and barriers per query -- the form for buckets that receive 64 queries or more on average.
-template <int NQW>
+template <int NQW, bool F16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 - NQW))) void hash_attn_staged_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off,
@@ -23,9 +23,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 
   if (NQW == 2) {
     // the items of a bucket are consecutive and their queries contiguous: this workgroup takes items
     // 2j and 2j+1 of the bucket, the one launched for item 2j+1 has nothing to do
-    int first = blockIdx.x;
-    while (first > 0 && items[first - 1].row == it.row && items[first - 1].bucket == it.bucket) --first;
-    if ((int(blockIdx.x) - first) & 1) return;
+    // (the bucket's first item by a galloping then a binary search over the item list: a bucket that holds most
+    // of a row's queries has thousands of items, and a linear walk back would be that many dependent loads)
+    const int me = blockIdx.x;
+    auto same = [&](int i) { return items[i].row == it.row && items[i].bucket == it.bucket; };
+    int lo = me, step = 1;                         // invariant: items lo..me belong to the bucket
+    while (lo - step >= 0 && same(lo - step)) {
+      lo -= step;
+      step <<= 1;
+    }
+    int bad = max(lo - step, -1);                  // -1 or an item of another bucket, bad < lo
+    while (lo - bad > 1) {
+      const int mid = (lo + bad) >> 1;
+      if (same(mid))
+        lo = mid;
+      else
+        bad = mid;
+    }
+    if ((me - lo) & 1) return;
     if (int(blockIdx.x) + 1 < n_it) {
       const fm_item nx = items[blockIdx.x + 1];
       if (nx.row == it.row && nx.bucket == it.bucket) n_q += nx.n_q;
@@ -33,7 +48,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 
   }
   const int64_t bkt = int64_t(it.row) * C + it.bucket;
   const int64_t qbase = int64_t(it.row) * Sq;
-  attend_staged<NQW>(q + qbase * kSD, q_perm + it.q_start, n_q, k + int64_t(it.row) * N * kSD,
+  attend_staged<NQW, F16>(q + qbase * kSD, q_perm + it.q_start, n_q, k + int64_t(it.row) * N * kSD,
                      v + int64_t(it.row) * N * kSD, k_idx + bucket_off[bkt], bucket_cnt[bkt], N, scale2,
                      out + qbase * kSD, lse + qbase, st_lds);
 }
@@ -41,18 +56,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 
 int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
                           const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                          float* lse, int Sq, int N, int C, float sm_scale, bool pairs, hipStream_t st) {
+                          float* lse, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, hipStream_t st) {
   constexpr size_t kTileBytes = kStagedTileBytes;
-  if (pairs) {
-    FM_ALLOW_LDS(hash_attn_staged_kernel<2>, 2 * kTileBytes, "fm_hash_attn_fwd: lds");
-    hipLaunchKernelGGL(hash_attn_staged_kernel<2>, dim3(unsigned(max_items)), dim3(256), 2 * kTileBytes, st,
-                       (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm, items,
-                       n_items, (bf16_t*)out, lse, Sq, N, C, sm_scale * kLog2e);
-  } else {
-    hipLaunchKernelGGL(hash_attn_staged_kernel<1>, dim3(unsigned(max_items)), dim3(256), kTileBytes, st,
-                       (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm, items,
-                       n_items, (bf16_t*)out, lse, Sq, N, C, sm_scale * kLog2e);
-  }
+#define FM_STAGED_LAUNCH(NQW, F16)                                                                                   \
+  do {                                                                                                               \
+    FM_ALLOW_LDS((hash_attn_staged_kernel<NQW, F16>), NQW * kTileBytes, "fm_hash_attn_fwd: lds");                     \
+    hipLaunchKernelGGL((hash_attn_staged_kernel<NQW, F16>), dim3(unsigned(max_items)), dim3(256), NQW * kTileBytes,  \
+                       st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt,      \
+                       q_perm, items, n_items, (bf16_t*)out, lse, Sq, N, C, sm_scale * kLog2e);                      \
+  } while (0)
+  if (pairs && f16)
+    FM_STAGED_LAUNCH(2, true);
+  else if (pairs)
+    FM_STAGED_LAUNCH(2, false);
+  else if (f16)
+    FM_STAGED_LAUNCH(1, true);
+  else
+    FM_STAGED_LAUNCH(1, false);
+#undef FM_STAGED_LAUNCH
   return launch_status("fm_hash_attn_fwd(mfma, staged)");
 }
 

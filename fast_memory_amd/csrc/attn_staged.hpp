@@ -1,4 +1,4 @@
-// bf16 bucket-gathered attention forward for head dimension 128 (gfx950) with a bucket's rows
+// bf16 / fp16 bucket-gathered attention forward for head dimension 128 (gfx950) with a bucket's rows
 // staged in LDS (triton_kernel.py:137-272).  The kernel of every launch that has work items enough
 // to fill the chip or buckets with many queries (the register-gather kernel of attn_mfma.hip keeps
 // the launches with few, small items): from the HBM-bound shapes (16 queries per bucket over a
@@ -21,12 +21,12 @@
 //                  that order, so neither P nor V is shuffled.  Lane (g,c) holds
 //                  O[query c][16t + 4g .. 16t + 4g + 3], t = 0..7.
 // Softmax as in the reference kernel (triton_kernel.py:248-263): base 2 with sm_scale*log2(e),
-// fp32 running max and denominator, denominator from unrounded p, p rounded to bf16 before P.V.
+// fp32 running max and denominator, denominator from unrounded p, p rounded to the input type before P.V.
 //
 // Roofline: HBM for the algorithmic bytes (cnt*(2*128*2+4) per bucket), MFMA for 4*128 flops per
 // query-key pair; at 128 queries per bucket the two are within a factor of three of each other.
 #pragma once
-#include "common.hpp"
+#include "mma16.hpp"
 
 namespace fm {
 
@@ -86,7 +86,7 @@ constexpr size_t kStagedTileBytes = size_t(kSK * kSKld + kSD * kSVld) * sizeof(b
 // point to global memory or LDS) over the cnt keys idx[0..cnt) of one bucket.  Called by all 256
 // threads of a workgroup; lds holds NQW tile buffers of kStagedTileBytes.  NQW = 16-query tiles per
 // wave: the workgroup takes up to 64 * NQW queries.
-template <int NQW>
+template <int NQW, bool F16 = false>
 __device__ __forceinline__ void attend_staged(
     const bf16_t* __restrict__ Qb, const int* __restrict__ q_rows, int n_q, const bf16_t* __restrict__ Kb,
     const bf16_t* __restrict__ Vb, const int32_t* __restrict__ idx, int cnt, int N, float scale2,
@@ -194,11 +194,10 @@ __device__ __forceinline__ void attend_staged(
     for (int st = 0; st < 4; ++st) {
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&bK[(kt * 16 + c) * kSKld + 8 * g + 32 * st]);
+        const uint4 a = *reinterpret_cast<const uint4*>(&bK[(kt * 16 + c) * kSKld + 8 * g + 32 * st]);
 #pragma unroll
         for (int qt = 0; qt < NQW; ++qt)
-          s[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              a, st_as_bf16x8(qf[qt][st]), st == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[qt][kt], 0, 0, 0);
+          s[qt][kt] = Mma<F16>::m16(a, qf[qt][st], st == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[qt][kt]);
       }
     }
     if (kp0 + kSK > cnt) {  // the bucket's last, ragged tile
@@ -249,8 +248,8 @@ __device__ __forceinline__ void attend_staged(
         }
 #pragma unroll
         for (int r = 0; r < 8; ++r) lsum[qt] += p[r];
-        pf[qt][h] = make_uint4(st_pack_bf16(p[0], p[1]), st_pack_bf16(p[2], p[3]), st_pack_bf16(p[4], p[5]),
-                               st_pack_bf16(p[6], p[7]));
+        pf[qt][h] = make_uint4(Mma<F16>::pack2(p[0], p[1]), Mma<F16>::pack2(p[2], p[3]), Mma<F16>::pack2(p[4], p[5]),
+                               Mma<F16>::pack2(p[6], p[7]));
       }
     }
     // ---- O^T += Vt.P^T (32-key half outermost, for the same reason) ----
@@ -258,10 +257,9 @@ __device__ __forceinline__ void attend_staged(
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
       for (int t8 = 0; t8 < 8; ++t8) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&bV[(16 * t8 + c) * kSVld + 8 * g + 32 * h]);
+        const uint4 a = *reinterpret_cast<const uint4*>(&bV[(16 * t8 + c) * kSVld + 8 * g + 32 * h]);
 #pragma unroll
-        for (int qt = 0; qt < NQW; ++qt)
-          O[qt][t8] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, st_as_bf16x8(pf[qt][h]), O[qt][t8], 0, 0, 0);
+        for (int qt = 0; qt < NQW; ++qt) O[qt][t8] = Mma<F16>::m16(a, pf[qt][h], O[qt][t8]);
       }
     }
   };
@@ -343,8 +341,8 @@ __device__ __forceinline__ void attend_staged(
 #pragma unroll
       for (int t8 = 0; t8 < 8; ++t8) {
         uint2 o;
-        o.x = st_pack_bf16(O[qt][t8][0] * inv, O[qt][t8][1] * inv);
-        o.y = st_pack_bf16(O[qt][t8][2] * inv, O[qt][t8][3] * inv);
+        o.x = Mma<F16>::pack2(O[qt][t8][0] * inv, O[qt][t8][1] * inv);
+        o.y = Mma<F16>::pack2(O[qt][t8][2] * inv, O[qt][t8][3] * inv);
         *reinterpret_cast<uint2*>(po + 16 * t8) = o;
       }
       if (g == 0) Lb[qrow[qt]] = empty ? -FLT_MAX : (m[qt] + __builtin_amdgcn_logf(ltot)) * kLn2;

@@ -63,7 +63,7 @@ struct FusedPlan {
 };
 
 static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& p) {
-  if (dtype != FM_BF16 || d != kFD) return false;
+  if ((dtype != FM_BF16 && dtype != FM_F16) || d != kFD) return false;
   if (N < 65536 || int64_t(Z) * 8 > N || Z > FM_MAX_Z || Z < 64) return false;
   p.slabs = int(ceil_div(C, kFSlab));
   const int64_t ntiles = ceil_div(N, kFKeys);
@@ -173,6 +173,7 @@ __global__ __launch_bounds__(kTauThreads) void row_threshold_kernel(const float*
 //     value back from its LDS dump and appends (value, key) to its segment.
 // The compute waves issue stores only, so they never stall on a memory counter;
 // the two waves that share a SIMD overlap one's MFMAs with the other's VALU work.
+template <bool F16>
 __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const float* __restrict__ tau,
     uint2* __restrict__ cand, int32_t* __restrict__ cnt, int C, int N, int n_splits, int cap_w) {
@@ -346,8 +347,8 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
           for (int r = 0; r < 16; ++r) acc[ni][r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-          acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], bfrag[0][ks], acc[0], 0, 0, 0);
-          acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], bfrag[1][ks], acc[1], 0, 0, 0);
+          acc[0] = mfma32<F16>(a[ks], bfrag[0][ks], acc[0]);
+          acc[1] = mfma32<F16>(a[ks], bfrag[1][ks], acc[1]);
         }
         if (half == 0) {
 #pragma unroll
@@ -486,6 +487,7 @@ __global__ __launch_bounds__(NT) void cand_select_kernel(
 // Y of the listed (head, bucket) rows, one output column per workgroup row-slot.
 // grid (up to 128, kMaxRepair): a workgroup walks 128-key tiles (4 waves x 32 keys); with nothing to
 // repair the launch is 8192 workgroups that read one word and leave.
+template <bool F16>
 __global__ __launch_bounds__(256) void project_listed_rows_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const int32_t* __restrict__ fail_rows,
     const int32_t* __restrict__ n_fail, float* __restrict__ Yf, int C, int N, int64_t ldy) {
@@ -518,7 +520,7 @@ __global__ __launch_bounds__(256) void project_listed_rows_kernel(
         bf16x8 b;
       } a;
       a.u = key < N ? pk[2 * ks] : make_uint4(0, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b, bfr[ks], acc, 0, 0, 0);
+      acc = mfma32<F16>(a.b, bfr[ks], acc);
     }
     if ((l & 31) == 0) {
 #pragma unroll
@@ -565,7 +567,7 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
   FM_REQUIRE(A && K && idx_out && ws && status_dev, FM_ERR_ARG, "fm_build_index_fused: null pointer");
   FusedPlan p;
   FM_REQUIRE(fused_plan(H, C, N, d, Z, dtype, p), FM_ERR_UNSUPPORTED,
-             "fm_build_index_fused: shape not eligible (needs bf16, d=128, N >= 65536, 64 <= Z <= N/8)");
+             "fm_build_index_fused: shape not eligible (needs bf16 or fp16, d=128, N >= 65536, 64 <= Z <= N/8)");
   FM_REQUIRE(ws_bytes >= p.total, FM_ERR_WORKSPACE, "fm_build_index_fused: workspace %zu < %zu", ws_bytes,
              p.total);
   FM_REQUIRE(H <= 65535 && int64_t(H) * C <= 0x7fffffffLL, FM_ERR_UNSUPPORTED,
@@ -593,9 +595,14 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
                      p.ld_s, p.rank, tau, n_fail);
   // phase 1
   mark_phase(1, st);
-  hipLaunchKernelGGL(fused_filter_kernel, dim3(unsigned(p.n_splits), unsigned(p.slabs), unsigned(H)),
-                     dim3(kFThreads), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N,
-                     p.n_splits, p.cap_w);
+  if (dtype == FM_F16)
+    hipLaunchKernelGGL(fused_filter_kernel<true>, dim3(unsigned(p.n_splits), unsigned(p.slabs), unsigned(H)),
+                       dim3(kFThreads), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N, p.n_splits,
+                       p.cap_w);
+  else
+    hipLaunchKernelGGL(fused_filter_kernel<false>, dim3(unsigned(p.n_splits), unsigned(p.slabs), unsigned(H)),
+                       dim3(kFThreads), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N, p.n_splits,
+                       p.cap_w);
   // phase 2
   mark_phase(2, st);
   const int P = next_pow2(Zc);
@@ -614,8 +621,13 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
 #undef FM_CAND_SELECT
   // phase 3
   mark_phase(3, st);
-  hipLaunchKernelGGL(project_listed_rows_kernel, dim3(unsigned(std::min<int64_t>(ceil_div(N, 128), 128)), kMaxRepair), dim3(256), 0,
-                     st, (const bf16_t*)A, (const bf16_t*)K, fail_rows, n_fail, Yf, C, N, p.ldy);
+  const dim3 rgrid = dim3(unsigned(std::min<int64_t>(ceil_div(N, 128), 128)), kMaxRepair);
+  if (dtype == FM_F16)
+    hipLaunchKernelGGL(project_listed_rows_kernel<true>, rgrid, dim3(256), 0, st, (const bf16_t*)A, (const bf16_t*)K,
+                       fail_rows, n_fail, Yf, C, N, p.ldy);
+  else
+    hipLaunchKernelGGL(project_listed_rows_kernel<false>, rgrid, dim3(256), 0, st, (const bf16_t*)A, (const bf16_t*)K,
+                       fail_rows, n_fail, Yf, C, N, p.ldy);
   rc = launch_argtopz(Yf, kMaxRepair, N, p.ldy, Zc, idx_out, val_out, fail_rows, n_fail, st);
   if (rc) return rc;
   hipLaunchKernelGGL(fused_status_kernel, dim3(1), dim3(1), 0, st, n_fail, status_dev);

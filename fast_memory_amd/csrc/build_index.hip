@@ -26,7 +26,7 @@ extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, fl
   FM_REQUIRE(fit >= 1, FM_ERR_WORKSPACE, "fm_build_index: workspace %zu holds no row of %lld floats",
              ws_bytes, (long long)ldy);
   const int Zc = Z < N ? Z : N;
-  const size_t esz = dtype == FM_BF16 ? 2 : 4;
+  const size_t esz = size_t(dtype_bytes(dtype));
   float* Y = static_cast<float*>(ws);
   // a pass takes as many whole heads as fit, or a bucket range [c0, c0+nc) of one head
   for (int h = 0; h < H;) {

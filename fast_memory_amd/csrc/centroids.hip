@@ -224,15 +224,18 @@ extern "C" int fm_segment_sum(const void* X, const int32_t* perm, const int32_t*
   using namespace fm;
   FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG, "fm_segment_sum: H=%d C=%d N=%d d=%d",
              H, C, N, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_segment_sum: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_segment_sum: dtype=%d", dtype);
   FM_REQUIRE(X && perm && seg_off && seg_cnt && sum_out, FM_ERR_ARG, "fm_segment_sum: null pointer");
   FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_segment_sum: H > 65535");
   dim3 grid = dim3(unsigned(C), unsigned(H));
   if (dtype == FM_F32)
     hipLaunchKernelGGL(segment_sum_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)X, perm,
                        seg_off, seg_cnt, sum_out, C, N, d);
-  else
+  else if (dtype == FM_BF16)
     hipLaunchKernelGGL(segment_sum_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream), (const bf16_t*)X, perm,
+                       seg_off, seg_cnt, sum_out, C, N, d);
+  else
+    hipLaunchKernelGGL(segment_sum_kernel<f16_t>, grid, dim3(256), 0, as_stream(stream), (const f16_t*)X, perm,
                        seg_off, seg_cnt, sum_out, C, N, d);
   return launch_status("fm_segment_sum");
 }
@@ -241,7 +244,7 @@ extern "C" int fm_l2_normalize(const void* X, void* Xn, int64_t rows, int d, flo
                                void* stream) {
   using namespace fm;
   FM_REQUIRE(rows >= 0 && d >= 1, FM_ERR_ARG, "fm_l2_normalize: rows=%lld d=%d", (long long)rows, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_l2_normalize: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_l2_normalize: dtype=%d", dtype);
   if (rows == 0) return FM_OK;
   FM_REQUIRE(X && Xn, FM_ERR_ARG, "fm_l2_normalize: null pointer");
   FM_REQUIRE(ceil_div(rows, 4) <= 0x7fffffffLL, FM_ERR_UNSUPPORTED, "fm_l2_normalize: too many rows");
@@ -253,9 +256,12 @@ extern "C" int fm_l2_normalize(const void* X, void* Xn, int64_t rows, int d, flo
   } else if (dtype == FM_F32)
     hipLaunchKernelGGL(l2_normalize_kernel<float>, grid, dim3(256), 0, as_stream(stream),
                        (const float*)X, (float*)Xn, rows, d, eps);
-  else
+  else if (dtype == FM_BF16)
     hipLaunchKernelGGL(l2_normalize_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream),
                        (const bf16_t*)X, (bf16_t*)Xn, rows, d, eps);
+  else
+    hipLaunchKernelGGL(l2_normalize_kernel<f16_t>, grid, dim3(256), 0, as_stream(stream),
+                       (const f16_t*)X, (f16_t*)Xn, rows, d, eps);
   return launch_status("fm_l2_normalize");
 }
 
@@ -264,16 +270,19 @@ extern "C" int fm_topk_mean(const void* Xn, const int32_t* top_idx, void* A_out,
   using namespace fm;
   FM_REQUIRE(C >= 1 && H >= 1 && G >= 1 && N >= 1 && k >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_topk_mean: C=%d H=%d G=%d N=%d k=%d d=%d", C, H, G, N, k, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_topk_mean: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_topk_mean: dtype=%d", dtype);
   FM_REQUIRE(Xn && top_idx && A_out, FM_ERR_ARG, "fm_topk_mean: null pointer");
   FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_topk_mean: H > 65535");
   dim3 grid = dim3(unsigned(C), unsigned(H));
   if (dtype == FM_F32)
     hipLaunchKernelGGL(topk_mean_kernel<float>, grid, dim3(256), 0, as_stream(stream),
                        (const float*)Xn, top_idx, (float*)A_out, H, G, N, k, d, normalize);
-  else
+  else if (dtype == FM_BF16)
     hipLaunchKernelGGL(topk_mean_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream),
                        (const bf16_t*)Xn, top_idx, (bf16_t*)A_out, H, G, N, k, d, normalize);
+  else
+    hipLaunchKernelGGL(topk_mean_kernel<f16_t>, grid, dim3(256), 0, as_stream(stream),
+                       (const f16_t*)Xn, top_idx, (f16_t*)A_out, H, G, N, k, d, normalize);
   return launch_status("fm_topk_mean");
 }
 
@@ -283,7 +292,7 @@ extern "C" int fm_segment_mean(const void* X, const int32_t* perm, const int32_t
   using namespace fm;
   FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_segment_mean: H=%d C=%d N=%d d=%d", H, C, N, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_segment_mean: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_segment_mean: dtype=%d", dtype);
   FM_REQUIRE(X && perm && seg_off && seg_cnt && prev && cent_out, FM_ERR_ARG,
              "fm_segment_mean: null pointer");
   FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_segment_mean: H > 65535");
@@ -295,9 +304,13 @@ extern "C" int fm_segment_mean(const void* X, const int32_t* perm, const int32_t
     hipLaunchKernelGGL(segment_mean_kernel<float>, grid, dim3(256), 0, as_stream(stream),
                        (const float*)X, perm, seg_off, seg_cnt, (const float*)prev,
                        (float*)cent_out, C, N, d);
-  else
+  else if (dtype == FM_BF16)
     hipLaunchKernelGGL(segment_mean_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream),
                        (const bf16_t*)X, perm, seg_off, seg_cnt, (const bf16_t*)prev,
                        (bf16_t*)cent_out, C, N, d);
+  else
+    hipLaunchKernelGGL(segment_mean_kernel<f16_t>, grid, dim3(256), 0, as_stream(stream),
+                       (const f16_t*)X, perm, seg_off, seg_cnt, (const f16_t*)prev,
+                       (f16_t*)cent_out, C, N, d);
   return launch_status("fm_segment_mean");
 }

@@ -55,6 +55,12 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {  // round to nearest ev
   return bf16_t(u >> 16);
 }
 
+struct f16_t {  // raw IEEE half bits (a type of its own: bf16_t is the plain uint16_t)
+  uint16_t b;
+};
+static inline bool dtype_ok(int dtype) { return dtype == FM_F32 || dtype == FM_BF16 || dtype == FM_F16; }
+static inline int dtype_bytes(int dtype) { return dtype == FM_F32 ? 4 : 2; }
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
   static constexpr int dtype = FM_F32;
@@ -67,6 +73,15 @@ template <> struct Elem<bf16_t> {
   __device__ static __forceinline__ float load(const bf16_t* p) { return bf16_to_f32(*p); }
   __device__ static __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
   __device__ static __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+};
+
+template <> struct Elem<f16_t> {
+  static constexpr int dtype = FM_F16;
+  __device__ static __forceinline__ float load(const f16_t* p) { return float(__builtin_bit_cast(_Float16, p->b)); }
+  __device__ static __forceinline__ void store(f16_t* p, float v) {
+    p->b = __builtin_bit_cast(uint16_t, _Float16(v));  // round to nearest even
+  }
+  __device__ static __forceinline__ float round(float v) { return float(_Float16(v)); }
 };
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }

@@ -40,7 +40,7 @@ extern "C" int fm_lse_merge(float* out, float* lse, const void* block_out, const
                             int64_t Q, int d, int dtype, void* stream) {
   using namespace fm;
   FM_REQUIRE(Q >= 0 && d >= 1, FM_ERR_ARG, "fm_lse_merge: Q=%lld d=%d", (long long)Q, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_lse_merge: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_lse_merge: dtype=%d", dtype);
   if (Q == 0) return FM_OK;
   FM_REQUIRE(out && lse && block_out && block_lse, FM_ERR_ARG, "fm_lse_merge: null pointer");
   FM_REQUIRE(ceil_div(Q, 4) <= 0x7fffffffLL, FM_ERR_UNSUPPORTED, "fm_lse_merge: Q too large");
@@ -48,8 +48,11 @@ extern "C" int fm_lse_merge(float* out, float* lse, const void* block_out, const
   if (dtype == FM_F32)
     hipLaunchKernelGGL(lse_merge_kernel<float>, grid, dim3(256), 0, as_stream(stream), out, lse,
                        (const float*)block_out, block_lse, Q, d);
-  else
+  else if (dtype == FM_BF16)
     hipLaunchKernelGGL(lse_merge_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream), out, lse,
                        (const bf16_t*)block_out, block_lse, Q, d);
+  else
+    hipLaunchKernelGGL(lse_merge_kernel<f16_t>, grid, dim3(256), 0, as_stream(stream), out, lse,
+                       (const f16_t*)block_out, block_lse, Q, d);
   return launch_status("fm_lse_merge");
 }

@@ -13,6 +13,18 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 
+// v_mfma_f32_32x32x16_bf16 or, with F16, v_mfma_f32_32x32x16_f16 on the same registers (the fragment layouts
+// are the same; a kernel instantiated with F16 reads IEEE half data through its bf16_t pointers)
+template <bool F16>
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  if constexpr (F16) {
+    typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 h8;
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+}
+
 __device__ __forceinline__ int acc_row_32(int r, int lane) {
   return 8 * (r >> 2) + ((lane >> 5) << 2) + (r & 3);
 }
@@ -34,6 +46,7 @@ __device__ __forceinline__ void stage_rows_bf16(bf16_t* dst, int ld, const bf16_
 // acc[mi][ni] = sum over k of sa[mi*32 + i][k] * sb[ni*32 + j][k], contraction
 // in ascending 16-element steps (the order every projection-type kernel
 // shares, so equal operands give bit-equal sums).  d % 16 == 0.
+template <bool F16 = false>
 __device__ __forceinline__ void mfma_tile_64x64(const bf16_t* sa, const bf16_t* sb, int ld, int d,
                                                 f32x16 (&acc)[2][2]) {
   const int l = lane_id();
@@ -56,7 +69,7 @@ __device__ __forceinline__ void mfma_tile_64x64(const bf16_t* sa, const bf16_t* 
     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
-        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+        acc[mi][ni] = mfma32<F16>(a[mi], b[ni], acc[mi][ni]);
   }
 }
 

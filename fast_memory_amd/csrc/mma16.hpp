@@ -1,0 +1,44 @@
+// The two 16-bit element types of the MFMA kernels behind one interface: operands travel as raw
+// 128-bit registers (eight elements), only the MFMA instruction and the fp32 -> 16-bit rounding
+// differ between bf16 and fp16 (fp16 is what the reference's performance harness runs,
+// triton_kernel.py:496).  Fragment layouts of the f16 and bf16 forms of an instruction are the same.
+#pragma once
+#include "common.hpp"
+
+namespace fm {
+
+template <bool F16>
+struct Mma {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 b8;
+  typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 h8;
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 b2;
+  typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 h2;
+  typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f2;
+  typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f4;
+  typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f16v;
+
+  // v_mfma_f32_16x16x32_{bf16,f16}
+  __device__ static __forceinline__ f4 m16(uint4 a, uint4 b, f4 c) {
+    if constexpr (F16)
+      return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, a), __builtin_bit_cast(b8, b), c, 0, 0, 0);
+  }
+  // v_mfma_f32_32x32x16_{bf16,f16}
+  __device__ static __forceinline__ f16v m32(uint4 a, uint4 b, f16v c) {
+    if constexpr (F16)
+      return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(b8, a), __builtin_bit_cast(b8, b), c, 0, 0, 0);
+  }
+  // two floats rounded to nearest even and packed (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32)
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+    f2 x = {lo, hi};
+    if constexpr (F16)
+      return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, h2));
+    else
+      return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, b2));
+  }
+};
+
+}  // namespace fm

@@ -16,6 +16,7 @@ namespace fm {
 // ---------------------------------------------------------------------------
 constexpr int kProjYLd = 132;  // floats per staged output row (128 + 4 pad)
 
+template <bool F16>
 __global__ __launch_bounds__(256) void project_bf16_kernel(const bf16_t* __restrict__ A,
                                                            const bf16_t* __restrict__ K,
                                                            float* __restrict__ Y, int C, int N,
@@ -36,7 +37,7 @@ __global__ __launch_bounds__(256) void project_bf16_kernel(const bf16_t* __restr
   const int w = threadIdx.x >> 6, l = lane_id();
   const int wm = w >> 1, wn = w & 1;  // wm: key half, wn: bucket half
   f32x16 acc[2][2];
-  mfma_tile_64x64(sK + (wm * 64) * lds_ld, sA + (wn * 64) * lds_ld, lds_ld, d, acc);
+  mfma_tile_64x64<F16>(sK + (wm * 64) * lds_ld, sA + (wn * 64) * lds_ld, lds_ld, d, acc);
   __syncthreads();  // operands consumed; the same LDS now takes the output tile
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi)
@@ -97,7 +98,7 @@ __device__ __forceinline__ void ps_fetch(u32x4 (&st)[NCH], const bf16_t* __restr
 }
 
 // BT bucket tiles per wave (the slab of a workgroup is 4 * 32 BT buckets), KT key tiles per step.
-template <int BT, int KT>
+template <int BT, int KT, bool F16>
 __global__ __launch_bounds__(256) void project_stream_bf16_d128_kernel(const bf16_t* __restrict__ A,
                                                                        const bf16_t* __restrict__ K,
                                                                        float* __restrict__ Y, int C, int N,
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(256) void project_stream_bf16_d128_kernel(const bf1
       for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
-          acc[bt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[bt][ks], kf[kt], acc[bt][kt], 0, 0, 0);
+          acc[bt][kt] = mfma32<F16>(af[bt][ks], kf[kt], acc[bt][kt]);
     }
     // store: wave-uniform 64-bit base per (tile, register) + one 32-bit lane offset
     const int n0 = step * kKeys;
@@ -273,6 +274,7 @@ __global__ __launch_bounds__(256) void qhash_generic_kernel(const T* __restrict_
 // and combined across the two lane halves and the two bucket-side waves at the
 // end.
 // ---------------------------------------------------------------------------
+template <bool F16>
 __global__ __launch_bounds__(256) void qhash_bf16_kernel(const bf16_t* __restrict__ A,
                                                          const bf16_t* __restrict__ q,
                                                          int32_t* __restrict__ hash_out,
@@ -298,7 +300,7 @@ __global__ __launch_bounds__(256) void qhash_bf16_kernel(const bf16_t* __restric
     stage_rows_bf16(sA, lds_ld, Ah, c0, C, d, 128);
     __syncthreads();
     f32x16 acc[2][2];
-    mfma_tile_64x64(sA + (wm * 64) * lds_ld, sB + (wn * 64) * lds_ld, lds_ld, d, acc);
+    mfma_tile_64x64<F16>(sA + (wm * 64) * lds_ld, sB + (wn * 64) * lds_ld, lds_ld, d, acc);
 #pragma unroll
     for (int ni = 0; ni < 2; ++ni) {
       int i = i0 + wn * 64 + ni * 32 + (l & 31);
@@ -394,7 +396,7 @@ __device__ __forceinline__ void argmax_pair(float (&best)[2], int (&pos)[2], con
 // argmax over the finished sub-tile (ME) of the tile before it and the LDS reads of the next
 // half step's A fragments spread between them.  sched_barrier pins the interleaving: an MFMA
 // keeps the matrix pipe busy for 32 cycles, the six VALU instructions behind it take 24.
-template <int ME, bool MFMA, bool PREFETCH, int I>
+template <bool F16, int ME, bool MFMA, bool PREFETCH, int I>
 __device__ __forceinline__ void qs_half_step(f32x16 (&accM)[2], const f32x16 (&accE)[2], const bf16x8 (&af)[8],
                                              bf16x8 (&af_next)[8], const bf16_t* next_lds,
                                              const bf16x8 (&bfrag)[2][8], float (&best)[2], int (&pos)[2]) {
@@ -405,18 +407,19 @@ __device__ __forceinline__ void qs_half_step(f32x16 (&accM)[2], const f32x16 (&a
         f32x16 z;
 #pragma unroll
         for (int r = 0; r < 16; ++r) z[r] = 0.f;
-        accM[ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks], bfrag[ni][ks], z, 0, 0, 0);
+        accM[ni] = mfma32<F16>(af[ks], bfrag[ni][ks], z);
       } else {
-        accM[ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks], bfrag[ni][ks], accM[ni], 0, 0, 0);
+        accM[ni] = mfma32<F16>(af[ks], bfrag[ni][ks], accM[ni]);
       }
     }
     if constexpr (PREFETCH && ni == 0) af_next[ks] = *reinterpret_cast<const bf16x8*>(next_lds + ks * 16);
     argmax_pair<ME, 2 * I>(best, pos, accE);
     __builtin_amdgcn_sched_barrier(0);
-    qs_half_step<ME, MFMA, PREFETCH, I + 1>(accM, accE, af, af_next, next_lds, bfrag, best, pos);
+    qs_half_step<F16, ME, MFMA, PREFETCH, I + 1>(accM, accE, af, af_next, next_lds, bfrag, best, pos);
   }
 }
 
+template <bool F16>
 __global__ __launch_bounds__(512) void qhash_stream_kernel(const bf16_t* __restrict__ A,
                                                            const bf16_t* __restrict__ q,
                                                            int32_t* __restrict__ hash_out, int C, int Sq) {
@@ -481,8 +484,8 @@ __global__ __launch_bounds__(512) void qhash_stream_kernel(const bf16_t* __restr
     f32x16 z;
 #pragma unroll
     for (int r = 0; r < 16; ++r) z[r] = 0.f;
-    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af0[ks], bfrag[0][ks], ks ? acc[0][0] : z, 0, 0, 0);
-    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af0[ks], bfrag[1][ks], ks ? acc[0][1] : z, 0, 0, 0);
+    acc[0][0] = mfma32<F16>(af0[ks], bfrag[0][ks], ks ? acc[0][0] : z);
+    acc[0][1] = mfma32<F16>(af0[ks], bfrag[1][ks], ks ? acc[0][1] : z);
     af1[ks] = *reinterpret_cast<const bf16x8*>(frag_ptr(0, 1) + ks * 16);
   }
   for (int t = 0; t < ntiles; ++t) {
@@ -491,18 +494,18 @@ __global__ __launch_bounds__(512) void qhash_stream_kernel(const bf16_t* __restr
     {
       const float b0 = best[0], b1 = best[1];
       if (more)
-        qs_half_step<0, true, true, 0>(acc[1], acc[0], af1, af0, frag_ptr((t + 1) & 1, 0), bfrag, best, pos);
+        qs_half_step<F16, 0, true, true, 0>(acc[1], acc[0], af1, af0, frag_ptr((t + 1) & 1, 0), bfrag, best, pos);
       else
-        qs_half_step<0, true, false, 0>(acc[1], acc[0], af1, af0, nullptr, bfrag, best, pos);
+        qs_half_step<F16, 0, true, false, 0>(acc[1], acc[0], af1, af0, nullptr, bfrag, best, pos);
       if (best[0] != b0) btile[0] = t;
       if (best[1] != b1) btile[1] = t;
     }
     {
       const float b0 = best[0], b1 = best[1];
       if (more)
-        qs_half_step<1, true, true, 0>(acc[0], acc[1], af0, af1, frag_ptr((t + 1) & 1, 1), bfrag, best, pos);
+        qs_half_step<F16, 1, true, true, 0>(acc[0], acc[1], af0, af1, frag_ptr((t + 1) & 1, 1), bfrag, best, pos);
       else
-        qs_half_step<1, false, false, 0>(acc[0], acc[1], af0, af1, nullptr, bfrag, best, pos);
+        qs_half_step<F16, 1, false, false, 0>(acc[0], acc[1], af0, af1, nullptr, bfrag, best, pos);
       if (best[0] != b0) btile[0] = t;
       if (best[1] != b1) btile[1] = t;
     }
@@ -533,12 +536,13 @@ extern "C" int fm_project(const void* A, const void* K, float* Y, int H, int C, 
   FM_REQUIRE(H >= 0 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_project: H=%d C=%d N=%d d=%d", H, C, N, d);
   FM_REQUIRE(ldy >= N && ldy < (int64_t(1) << 29), FM_ERR_ARG, "fm_project: ldy=%lld, N=%d", (long long)ldy, N);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_project: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_project: dtype=%d", dtype);
   if (H == 0) return FM_OK;
   FM_REQUIRE(A && K && Y, FM_ERR_ARG, "fm_project: null pointer");
   FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_project: H=%d > 65535", H);
   hipStream_t st = as_stream(stream);
-  if (dtype == FM_BF16 && d == 128) {
+  const bool h16 = dtype == FM_BF16 || dtype == FM_F16;  // 16-bit elements: MFMA kernels
+  if (h16 && d == 128) {
     constexpr int kBT = 1, kKT = 4;  // 32 buckets per wave, 128 keys per step: 512 contiguous bytes per row and step
     constexpr int kSlab = 4 * 32 * kBT, kKeys = 32 * kKT;
     FM_REQUIRE(ceil_div(C, kSlab) <= 65535, FM_ERR_UNSUPPORTED, "fm_project: C too large");
@@ -548,27 +552,40 @@ extern "C" int fm_project(const void* A, const void* K, float* Y, int H, int C, 
     int64_t ranges = std::max<int64_t>(1, std::min<int64_t>(ceil_div(1024, slabs), ceil_div(n_steps, 8)));
     const int steps_per_wg = int(ceil_div(n_steps, ranges));
     ranges = ceil_div(n_steps, steps_per_wg);
-    hipLaunchKernelGGL((project_stream_bf16_d128_kernel<kBT, kKT>),
-                       dim3(unsigned(ranges), unsigned(ceil_div(C, kSlab)), unsigned(H)), dim3(256), 0, st,
-                       (const bf16_t*)A, (const bf16_t*)K, Y, C, N, ldy, steps_per_wg);
-  } else if (dtype == FM_BF16 && d % 16 == 0) {
+    const dim3 grid = dim3(unsigned(ranges), unsigned(ceil_div(C, kSlab)), unsigned(H));
+    if (dtype == FM_F16)
+      hipLaunchKernelGGL((project_stream_bf16_d128_kernel<kBT, kKT, true>), grid, dim3(256), 0, st, (const bf16_t*)A,
+                         (const bf16_t*)K, Y, C, N, ldy, steps_per_wg);
+    else
+      hipLaunchKernelGGL((project_stream_bf16_d128_kernel<kBT, kKT, false>), grid, dim3(256), 0, st, (const bf16_t*)A,
+                         (const bf16_t*)K, Y, C, N, ldy, steps_per_wg);
+  } else if (h16 && d % 16 == 0) {
     FM_REQUIRE(ceil_div(C, 128) <= 65535, FM_ERR_UNSUPPORTED, "fm_project: C too large");
     size_t lds = std::max(size_t(2) * 128 * (d + 8) * sizeof(bf16_t), size_t(128) * kProjYLd * sizeof(float));
-    FM_ALLOW_LDS(project_bf16_kernel, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_project: lds");
+    FM_ALLOW_LDS(project_bf16_kernel<false>, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_project: lds");
+    FM_ALLOW_LDS(project_bf16_kernel<true>, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_project: lds");
     dim3 grid = dim3(unsigned(ceil_div(N, 128)), unsigned(ceil_div(C, 128)), unsigned(H));
-    hipLaunchKernelGGL(project_bf16_kernel, grid, dim3(256), lds, st, (const bf16_t*)A,
-                       (const bf16_t*)K, Y, C, N, d, ldy);
+    if (dtype == FM_F16)
+      hipLaunchKernelGGL(project_bf16_kernel<true>, grid, dim3(256), lds, st, (const bf16_t*)A, (const bf16_t*)K, Y, C,
+                         N, d, ldy);
+    else
+      hipLaunchKernelGGL(project_bf16_kernel<false>, grid, dim3(256), lds, st, (const bf16_t*)A, (const bf16_t*)K, Y, C,
+                         N, d, ldy);
   } else {
     size_t lds = size_t(64) * (d + 1) * sizeof(float);
     dim3 grid = dim3(unsigned(ceil_div(N, 64)), unsigned(H));
     FM_ALLOW_LDS(project_generic_kernel<float>, 64 * (FM_MAX_D + 1) * 4, "fm_project: lds");
     FM_ALLOW_LDS(project_generic_kernel<bf16_t>, 64 * (FM_MAX_D + 1) * 4, "fm_project: lds");
+    FM_ALLOW_LDS(project_generic_kernel<f16_t>, 64 * (FM_MAX_D + 1) * 4, "fm_project: lds");
     if (dtype == FM_F32)
       hipLaunchKernelGGL(project_generic_kernel<float>, grid, dim3(256), lds, st, (const float*)A,
                          (const float*)K, Y, C, N, d, ldy);
-    else
+    else if (dtype == FM_BF16)
       hipLaunchKernelGGL(project_generic_kernel<bf16_t>, grid, dim3(256), lds, st,
                          (const bf16_t*)A, (const bf16_t*)K, Y, C, N, d, ldy);
+    else
+      hipLaunchKernelGGL(project_generic_kernel<f16_t>, grid, dim3(256), lds, st,
+                         (const f16_t*)A, (const f16_t*)K, Y, C, N, d, ldy);
   }
   return launch_status("fm_project");
 }
@@ -578,32 +595,46 @@ extern "C" int fm_qhash(const void* A, const void* q, int32_t* hash_out, float* 
   using namespace fm;
   FM_REQUIRE(H >= 0 && C >= 1 && Sq >= 0 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_qhash: H=%d C=%d Sq=%d d=%d", H, C, Sq, d);
-  FM_REQUIRE(dtype == FM_F32 || dtype == FM_BF16, FM_ERR_ARG, "fm_qhash: dtype=%d", dtype);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_qhash: dtype=%d", dtype);
   if (H == 0 || Sq == 0) return FM_OK;
   FM_REQUIRE(A && q && hash_out, FM_ERR_ARG, "fm_qhash: null pointer");
   FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_qhash: H=%d > 65535", H);
   hipStream_t st = as_stream(stream);
-  if (dtype == FM_BF16 && d == 128 && !scores_out) {
+  const bool h16 = dtype == FM_BF16 || dtype == FM_F16;  // 16-bit elements: MFMA kernels
+  if (h16 && d == 128 && !scores_out) {
     dim3 grid = dim3(unsigned(ceil_div(Sq, 512)), unsigned(H));
-    hipLaunchKernelGGL(qhash_stream_kernel, grid, dim3(512), 0, st, (const bf16_t*)A, (const bf16_t*)q,
-                       hash_out, C, Sq);
-  } else if (dtype == FM_BF16 && d % 16 == 0) {
+    if (dtype == FM_F16)
+      hipLaunchKernelGGL(qhash_stream_kernel<true>, grid, dim3(512), 0, st, (const bf16_t*)A, (const bf16_t*)q,
+                         hash_out, C, Sq);
+    else
+      hipLaunchKernelGGL(qhash_stream_kernel<false>, grid, dim3(512), 0, st, (const bf16_t*)A, (const bf16_t*)q,
+                         hash_out, C, Sq);
+  } else if (h16 && d % 16 == 0) {
     size_t lds = size_t(2) * 128 * (d + 8) * sizeof(bf16_t);
-    FM_ALLOW_LDS(qhash_bf16_kernel, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_qhash: lds");
+    FM_ALLOW_LDS(qhash_bf16_kernel<false>, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_qhash: lds");
+    FM_ALLOW_LDS(qhash_bf16_kernel<true>, 2 * 128 * (FM_MAX_D + 8) * sizeof(bf16_t), "fm_qhash: lds");
     dim3 grid = dim3(unsigned(ceil_div(Sq, 128)), unsigned(H));
-    hipLaunchKernelGGL(qhash_bf16_kernel, grid, dim3(256), lds, st, (const bf16_t*)A,
-                       (const bf16_t*)q, hash_out, scores_out, C, Sq, d);
+    if (dtype == FM_F16)
+      hipLaunchKernelGGL(qhash_bf16_kernel<true>, grid, dim3(256), lds, st, (const bf16_t*)A, (const bf16_t*)q,
+                         hash_out, scores_out, C, Sq, d);
+    else
+      hipLaunchKernelGGL(qhash_bf16_kernel<false>, grid, dim3(256), lds, st, (const bf16_t*)A, (const bf16_t*)q,
+                         hash_out, scores_out, C, Sq, d);
   } else {
     size_t lds = size_t(64) * (d + 1) * sizeof(float);
     FM_ALLOW_LDS(qhash_generic_kernel<float>, 64 * (FM_MAX_D + 1) * 4, "fm_qhash: lds");
     FM_ALLOW_LDS(qhash_generic_kernel<bf16_t>, 64 * (FM_MAX_D + 1) * 4, "fm_qhash: lds");
+    FM_ALLOW_LDS(qhash_generic_kernel<f16_t>, 64 * (FM_MAX_D + 1) * 4, "fm_qhash: lds");
     dim3 grid = dim3(unsigned(ceil_div(Sq, 64)), unsigned(H));
     if (dtype == FM_F32)
       hipLaunchKernelGGL(qhash_generic_kernel<float>, grid, dim3(256), lds, st, (const float*)A,
                          (const float*)q, hash_out, scores_out, C, Sq, d);
-    else
+    else if (dtype == FM_BF16)
       hipLaunchKernelGGL(qhash_generic_kernel<bf16_t>, grid, dim3(256), lds, st, (const bf16_t*)A,
                          (const bf16_t*)q, hash_out, scores_out, C, Sq, d);
+    else
+      hipLaunchKernelGGL(qhash_generic_kernel<f16_t>, grid, dim3(256), lds, st, (const f16_t*)A,
+                         (const f16_t*)q, hash_out, scores_out, C, Sq, d);
   }
   return launch_status("fm_qhash");
 }

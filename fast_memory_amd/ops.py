@@ -11,12 +11,12 @@ import torch
 from . import _lib
 from ._lib import check
 
-_DT = {torch.float32: _lib.FM_F32, torch.bfloat16: _lib.FM_BF16}
+_DT = {torch.float32: _lib.FM_F32, torch.bfloat16: _lib.FM_BF16, torch.float16: _lib.FM_F16}
 
 
 def _dt(t: torch.Tensor) -> int:
     if t.dtype not in _DT:
-        raise TypeError(f"unsupported dtype {t.dtype}; libfastmem takes float32 and bfloat16")
+        raise TypeError(f"unsupported dtype {t.dtype}; libfastmem takes float32, bfloat16 and float16")
     return _DT[t.dtype]
 
 
@@ -478,8 +478,7 @@ def generic_kernels_forced() -> bool:
 
 def hash_attn_fwd_kernel_name(H: int, Sq: int, N: int, d: int, C: int, dtype: torch.dtype) -> str:
     """Name of the kernel :func:`hash_attn_fwd` launches for these extents."""
-    code = 1 if dtype == torch.bfloat16 else 0
-    return _lib.load().fm_hash_attn_fwd_kernel(H, Sq, N, d, C, code).decode()
+    return _lib.load().fm_hash_attn_fwd_kernel(H, Sq, N, d, C, _DT[dtype]).decode()
 
 
 def grouped_forward_kernel(which: Optional[str]) -> None:

@@ -11,7 +11,8 @@
  *   - every pointer is a DEVICE pointer unless the name ends in `_host`;
  *   - tensors are dense, row-major, batch-first: A [H,C,d], K/V [H,N,d],
  *     q/out [H,Sq,d] with Sq = G*S (query head hq = h*G + g, memory.py:281);
- *   - `dtype` selects the element type of q/k/v/A: FM_F32 or FM_BF16; all
+ *   - `dtype` selects the element type of q/k/v/A: FM_F32, FM_BF16 or FM_F16 (the
+ *     reference's own performance harness runs fp16, triton_kernel.py:496); all
  *     accumulation is fp32; log-sum-exp values are fp32 natural logarithms;
  *   - all index tensors are int32;
  *   - `stream` is a hipStream_t (NULL = the default stream); no entry point
@@ -40,7 +41,7 @@ typedef enum {
   FM_ERR_LAUNCH = 4       /* HIP reported an error at launch                 */
 } fm_status;
 
-typedef enum { FM_F32 = 0, FM_BF16 = 1 } fm_dtype;
+typedef enum { FM_F32 = 0, FM_BF16 = 1, FM_F16 = 2 } fm_dtype;
 
 /* Largest bucket capacity Z the selection kernels accept. */
 #define FM_MAX_Z 16384

@@ -58,6 +58,7 @@ constexpr int kCandRegsSmall = 32;  // ... with 256 or 512 threads per row
 
 struct FusedPlan {
   int ns, stride, rank, n_splits, slabs, n_writers, cap_w, sel_threads;
+  bool wide;  // phase 1 takes fused_filter_wide_kernel (slabs of 1024 buckets)
   int64_t ld_s, ldy;
   size_t off_Ks, off_Ys, off_tau, off_cand, off_cnt, off_fail, off_nfail, off_Yf, total;
 };
@@ -65,7 +66,9 @@ struct FusedPlan {
 static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& p) {
   if ((dtype != FM_BF16 && dtype != FM_F16) || d != kFD) return false;
   if (N < 65536 || int64_t(Z) * 8 > N || Z > FM_MAX_Z || Z < 64) return false;
-  p.slabs = int(ceil_div(C, kFSlab));
+  // the wide form wherever its 1024-bucket slabs are at least three quarters full
+  p.wide = C >= 768 && (C % 1024 == 0 || C % 1024 >= 768 || C >= 4096);
+  p.slabs = int(ceil_div(C, p.wide ? 1024 : kFSlab));
   const int64_t ntiles = ceil_div(N, kFKeys);
   int64_t s = ceil_div(256, int64_t(H) * p.slabs);
   s = std::max<int64_t>(1, std::min<int64_t>(32, std::min(s, ntiles)));
@@ -389,6 +392,205 @@ __global__ __launch_bounds__(kFThreads) void fused_filter_kernel(
   }
 }
 
+// ---- phase 1, wide form ------------------------------------------------------
+// The same filter for C >= 768: eight waves of 128 buckets each (a slab of 1024), no producer wave.
+//   * A key fragment read from LDS feeds four MFMAs instead of two, which halves the LDS read traffic per
+//     flop -- the LDS (fragment reads + accumulator dumps) is the busiest unit of the 64-bucket form.
+//   * The waves stage the 64-key tiles themselves: two 16-byte chunks per lane and tile, requested two
+//     tiles ahead and written to LDS one tile ahead, right after the barrier, when every vector-memory
+//     operation of the wave is at least half a tile old (loads and stores complete in issue order, so the
+//     wait for a tile's loads is also a wait for the candidate stores issued before them).
+//   * The epilogue of a tile's second half is carried over the barrier: the end of a tile period is MFMA
+//     work only, its candidate stores are issued at the start of the next period, and the two waves of a
+//     SIMD drift half a period apart, one's MFMAs facing the other's test / dump / emission.
+// Writers, key codes, segments and counts are those of the 64-bucket form: the selection does not see
+// which form ran.  256 registers per lane (128 of them the resident bucket fragments), two waves per SIMD.
+constexpr int kFWSlab = 1024;  // buckets per workgroup of the wide form (128 per wave)
+constexpr int kFWBT = 4;       // 32-bucket tiles per wave
+
+template <bool F16>
+__global__ __launch_bounds__(512) void fused_filter_wide_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const float* __restrict__ tau,
+    uint2* __restrict__ cand, int32_t* __restrict__ cnt, int C, int N, int n_splits, int cap_w) {
+  __shared__ __attribute__((aligned(16))) struct {
+    bf16_t keys[2][kFKeys * kFLd];
+    float dump[kFWaves][2 * 64 * kFDumpLd];  // [wave][tile of the pair][lane][accumulator register, padded]
+  } sm;
+  bf16_t(&sK)[2][kFKeys * kFLd] = sm.keys;
+  const int sk = blockIdx.x, slab = blockIdx.y, h = blockIdx.z;
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+  const int n_writers = 2 * n_splits;
+  const bf16_t* Kh = K + int64_t(h) * N * kFD;
+  const int ntiles = (N + kFKeys - 1) / kFKeys;
+  const int my_tiles = sk < ntiles ? (ntiles - sk + n_splits - 1) / n_splits : 0;  // tiles sk + i*n_splits
+
+  // staging: chunks tid and tid + 512 of a tile's 1024 16-byte chunks (rows tid/16 and 32 + tid/16)
+  uint4 st0, st1;
+  auto fetch = [&](int i) {
+    const int64_t key0 = (int64_t(sk) + int64_t(i) * n_splits) * kFKeys + (tid >> 4);
+    st0 = key0 < N ? reinterpret_cast<const uint4*>(Kh + key0 * kFD)[tid & 15] : make_uint4(0, 0, 0, 0);
+    st1 = key0 + 32 < N ? reinterpret_cast<const uint4*>(Kh + (key0 + 32) * kFD)[tid & 15] : make_uint4(0, 0, 0, 0);
+  };
+  auto stash = [&](int buf) {
+    *reinterpret_cast<uint4*>(&sK[buf][(tid >> 4) * kFLd + (tid & 15) * 8]) = st0;
+    *reinterpret_cast<uint4*>(&sK[buf][(32 + (tid >> 4)) * kFLd + (tid & 15) * 8]) = st1;
+  };
+
+  const int cb = slab * kFWSlab + w * (32 * kFWBT);  // this wave's first bucket
+  const bool active = cb < C;
+  const bf16_t* Ah = A + int64_t(h) * C * kFD;
+  const int64_t wg_row0 = int64_t(h) * C + int64_t(slab) * kFWSlab;
+  char* cbase = reinterpret_cast<char*>(cand + wg_row0 * n_writers * int64_t(cap_w));
+  float* dump = sm.dump[w];
+
+  bf16x8 bfrag[kFWBT][8];
+  float th[kFWBT];
+  uint32_t off[kFWBT], start[kFWBT], lim[kFWBT];
+  uint32_t ovf = 0;  // bit bt: the segment of tile bt wrapped
+#pragma unroll
+  for (int bt = 0; bt < kFWBT; ++bt) {
+    const int row = cb + bt * 32 + (l & 31);
+    const bool ok = row < C;
+    const uint4* pa = reinterpret_cast<const uint4*>(Ah + int64_t(ok ? row : 0) * kFD + (l >> 5) * 8);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      union {
+        uint4 u;
+        bf16x8 b;
+      } cvt;
+      cvt.u = ok ? pa[2 * ks] : make_uint4(0, 0, 0, 0);
+      bfrag[bt][ks] = cvt.b;
+    }
+    th[bt] = ok ? tau[int64_t(h) * C + row] : INFINITY;
+    const uint32_t rl = uint32_t(w * (32 * kFWBT) + bt * 32 + (l & 31));  // row inside the slab
+    start[bt] = ((rl * uint32_t(n_writers) + uint32_t(sk * 2 + (l >> 5))) * uint32_t(cap_w)) * 8u;
+    off[bt] = start[bt];
+    lim[bt] = start[bt] + uint32_t(cap_w - 16) * 8u;
+  }
+#pragma unroll
+  for (int bt = 0; bt < kFWBT; ++bt) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) asm volatile("" ::"v"(bfrag[bt][ks]));
+    asm volatile("" ::"v"(th[bt]));
+  }
+  const int lane_code = (l >> 5) << 4;
+  uint32_t msk[2];
+  f32x16 acc[kFWBT];
+
+  auto test_dump4 = [&](const f32x16& a, float t, int ni, int q) {
+    *reinterpret_cast<float4*>(&dump[(ni * 64 + l) * kFDumpLd + 4 * q]) =
+        make_float4(a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]);
+#pragma unroll
+    for (int j = 3; j >= 0; --j)
+      asm volatile("v_cmp_nlt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
+                   : "+v"(msk[ni])
+                   : "v"(a[4 * q + j]), "v"(t)
+                   : "vcc", "memory");
+  };
+  // one emission round over the pair of tiles bt0, bt0 + 1 (see fused_filter_kernel::emit)
+  auto emit = [&](auto check_n, auto pair, uint32_t code0) {
+    constexpr int bt0 = 2 * decltype(pair)::value;
+    bool has[4];
+    int r[4];
+    float y[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      uint32_t& m = msk[p >> 1];
+      if constexpr (decltype(check_n)::value) {
+        while (m != 0 && fused_key_of_code(code0 + uint32_t(__builtin_ffs(int(m)) - 1)) >= uint32_t(N)) m &= m - 1u;
+      }
+      has[p] = m != 0;
+      r[p] = __builtin_ffs(int(m)) - 1;
+      m &= m - 1u;
+    }
+#pragma unroll
+    for (int p = 0; p < 4; ++p) y[p] = dump[((p >> 1) * 64 + l) * kFDumpLd + r[p]];
+    asm volatile("" : "+v"(y[0]), "+v"(y[1]), "+v"(y[2]), "+v"(y[3]));
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni) {
+      if (has[2 * ni]) {
+        typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+        const u32x4_t rec = {__float_as_uint(y[2 * ni]), code0 + uint32_t(r[2 * ni]), __float_as_uint(y[2 * ni + 1]),
+                             code0 + uint32_t(r[2 * ni + 1])};
+        *reinterpret_cast<u32x4_t*>(cbase + off[bt0 + ni]) = rec;
+        off[bt0 + ni] += has[2 * ni + 1] ? 16u : 8u;
+      }
+    }
+  };
+  auto epi_pair = [&](auto pair, uint32_t code0, bool check_n) {
+    constexpr int bt0 = 2 * decltype(pair)::value;
+    msk[0] = msk[1] = 0;
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q = 3; q >= 0; --q) test_dump4(acc[bt0 + ni], th[bt0 + ni], ni, q);
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+      if (off[bt0 + ni] > lim[bt0 + ni]) {  // fewer than 16 free slots: wrap and mark the row for repair
+        off[bt0 + ni] = start[bt0 + ni];
+        ovf |= 1u << (bt0 + ni);
+      }
+    if (check_n) {
+      do {
+        emit(std::true_type{}, pair, code0);
+      } while (__ballot((msk[0] | msk[1]) != 0));
+    } else {
+      do {
+        emit(std::false_type{}, pair, code0);
+      } while (__ballot((msk[0] | msk[1]) != 0));
+    }
+  };
+  // 32 MFMAs: 32 keys (half `half` of tile i) x this wave's 128 buckets
+  auto mfma_half = [&](int i, int half) {
+    const bf16_t* pa = &sK[i & 1][(half * 32 + (l & 31)) * kFLd + (l >> 5) * 8];
+#pragma unroll
+    for (int bt = 0; bt < kFWBT; ++bt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[bt][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const bf16x8 a = *reinterpret_cast<const bf16x8*>(pa + ks * 16);
+#pragma unroll
+      for (int bt = 0; bt < kFWBT; ++bt) acc[bt] = mfma32<F16>(a, bfrag[bt][ks], acc[bt]);
+    }
+  };
+  // test, dump and emission of the accumulators of (tile i, half): the pair of tiles 0, 1, then 2, 3
+  auto epi_half = [&](int i, int half) {
+    const int kbase = (sk + i * n_splits) * kFKeys;
+    const bool check_n = kbase + kFKeys > N;
+    const uint32_t code0 = uint32_t(kbase + half * 32 + lane_code);
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // every accumulator pass retired
+    epi_pair(std::integral_constant<int, 0>{}, code0, check_n);
+    epi_pair(std::integral_constant<int, 1>{}, code0, check_n);
+  };
+
+  if (my_tiles > 0) {
+    fetch(0);
+    stash(0);
+  }
+  if (my_tiles > 1) fetch(1);
+  __syncthreads();
+  for (int i = 0; i < my_tiles; ++i) {
+    if (i + 1 < my_tiles) stash((i + 1) & 1);  // into the buffer tile i - 1 was read from
+    if (i + 2 < my_tiles) fetch(i + 2);
+    if (active) {
+      if (i > 0) epi_half(i - 1, 1);
+      mfma_half(i, 0);
+      epi_half(i, 0);
+      mfma_half(i, 1);
+    }
+    __syncthreads();
+  }
+  if (active && my_tiles > 0) epi_half(my_tiles - 1, 1);
+#pragma unroll
+  for (int bt = 0; bt < kFWBT; ++bt) {
+    const int row = cb + bt * 32 + (l & 31);
+    if (row < C)
+      cnt[(int64_t(h) * C + row) * n_writers + sk * 2 + (l >> 5)] =
+          ((ovf >> bt) & 1u) ? cap_w + 1 : int32_t((off[bt] - start[bt]) >> 3);
+  }
+}
+
 // ---- phase 2 ---------------------------------------------------------------
 // Per-writer candidate counts of a row in LDS; returns false (to all threads) if a segment
 // overflowed or the row has fewer than Zc candidates, i.e. the sampled threshold failed.
@@ -595,14 +797,21 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
                      p.ld_s, p.rank, tau, n_fail);
   // phase 1
   mark_phase(1, st);
-  if (dtype == FM_F16)
-    hipLaunchKernelGGL(fused_filter_kernel<true>, dim3(unsigned(p.n_splits), unsigned(p.slabs), unsigned(H)),
-                       dim3(kFThreads), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N, p.n_splits,
-                       p.cap_w);
-  else
-    hipLaunchKernelGGL(fused_filter_kernel<false>, dim3(unsigned(p.n_splits), unsigned(p.slabs), unsigned(H)),
-                       dim3(kFThreads), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N, p.n_splits,
-                       p.cap_w);
+  {
+    const dim3 grid = dim3(unsigned(p.n_splits), unsigned(p.slabs), unsigned(H));
+#define FM_FILTER(KERNEL, THREADS)                                                                          \
+  hipLaunchKernelGGL(KERNEL, grid, dim3(THREADS), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N, \
+                     p.n_splits, p.cap_w)
+    if (p.wide && dtype == FM_F16)
+      FM_FILTER(fused_filter_wide_kernel<true>, 512);
+    else if (p.wide)
+      FM_FILTER(fused_filter_wide_kernel<false>, 512);
+    else if (dtype == FM_F16)
+      FM_FILTER(fused_filter_kernel<true>, kFThreads);
+    else
+      FM_FILTER(fused_filter_kernel<false>, kFThreads);
+#undef FM_FILTER
+  }
   // phase 2
   mark_phase(2, st);
   const int P = next_pow2(Zc);

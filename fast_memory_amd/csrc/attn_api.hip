@@ -39,6 +39,8 @@ extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int 
   using namespace fm;
   if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype, N)) return "hash_attn_generic_kernel";
   const int choice = hash_attn_mfma_choice(H, Sq, N, C);
+  if (choice && N > (1 << 24))
+    return dtype == FM_F16 ? "hash_attn_staged_kernel<1, f16, 64-bit rows>" : "hash_attn_staged_kernel<1, 64-bit rows>";
   if (dtype == FM_F16) return choice == 2 ? "hash_attn_staged_kernel<2, f16>" : "hash_attn_staged_kernel<1, f16>";
   switch (choice) {
     case 1: return "hash_attn_staged_kernel<1>";

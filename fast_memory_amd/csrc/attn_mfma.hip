@@ -464,10 +464,9 @@ int local_attn_decode(const void* q, const void* k, const void* v, void* out, fl
   return launch_status("fm_local_attn_fwd(decode)");
 }
 
-// bf16: every shape (the register-gather kernel below takes what the staged kernel does not); fp16 has the
-// staged kernel only, which addresses rows by 32-bit byte offsets
 bool hash_attn_mfma_supported(int d, int dtype, int N) {
-  return d == kD && (dtype == FM_BF16 || (dtype == FM_F16 && N <= (1 << 24)));
+  (void)N;
+  return d == kD && (dtype == FM_BF16 || dtype == FM_F16);
 }
 
 int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
@@ -498,15 +497,15 @@ extern int g_force_generic;
 // least 512, taking min(Sq, C) per row as their number) or buckets receive 24 queries or more on
 // average; with few and small items the four waves of the gather kernel, which share one bucket's
 // keys, finish an item sooner.  Two items per workgroup from 64 queries per bucket on average.
-// (The staged kernel addresses rows by 32-bit byte offsets: N * 256 B must stay below 4 GiB.)
+// (Beyond 2^24 keys the staged kernel runs in its form with 64-bit row offsets, one item per workgroup.)
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
-  if (g_force_generic == 3 || N > (1 << 24)) return 0;
+  if (g_force_generic == 3) return 0;
   if (g_force_generic == 2) return 1;
   if (g_force_generic == 4) return 2;
   const bool many_items = int64_t(H) * (Sq < C ? Sq : C) >= 512;
   const bool dense = Sq >= 24 * int64_t(C);
   if (!many_items && !dense) return 0;
-  return (Sq >= 64 * int64_t(C) && many_items) ? 2 : 1;
+  return (Sq >= 64 * int64_t(C) && many_items && N <= (1 << 24)) ? 2 : 1;
 }
 
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,

@@ -8,7 +8,7 @@ namespace fm {
 // CU.  2: a workgroup takes two consecutive items of a bucket (128 queries; the workgroup of the second
 // item exits), each LDS operand read feeds two MFMAs, two workgroups per CU: half the LDS reads,
 // staging and barriers per query -- the form for buckets that receive 64 queries or more on average.
-template <int NQW, bool F16>
+template <int NQW, bool F16, bool BIGN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 - NQW))) void hash_attn_staged_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off,
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 
   }
   const int64_t bkt = int64_t(it.row) * C + it.bucket;
   const int64_t qbase = int64_t(it.row) * Sq;
-  attend_staged<NQW, F16>(q + qbase * kSD, q_perm + it.q_start, n_q, k + int64_t(it.row) * N * kSD,
+  attend_staged<NQW, F16, BIGN>(q + qbase * kSD, q_perm + it.q_start, n_q, k + int64_t(it.row) * N * kSD,
                      v + int64_t(it.row) * N * kSD, k_idx + bucket_off[bkt], bucket_cnt[bkt], N, scale2,
                      out + qbase * kSD, lse + qbase, st_lds);
 }
@@ -58,14 +58,20 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
                           float* lse, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, hipStream_t st) {
   constexpr size_t kTileBytes = kStagedTileBytes;
-#define FM_STAGED_LAUNCH(NQW, F16)                                                                                   \
+#define FM_STAGED_LAUNCH(NQW, F16) FM_STAGED_LAUNCH3(NQW, F16, false)
+#define FM_STAGED_LAUNCH3(NQW, F16, BIGN)                                                                                   \
   do {                                                                                                               \
-    FM_ALLOW_LDS((hash_attn_staged_kernel<NQW, F16>), NQW * kTileBytes, "fm_hash_attn_fwd: lds");                     \
-    hipLaunchKernelGGL((hash_attn_staged_kernel<NQW, F16>), dim3(unsigned(max_items)), dim3(256), NQW * kTileBytes,  \
+    FM_ALLOW_LDS((hash_attn_staged_kernel<NQW, F16, BIGN>), NQW * kTileBytes, "fm_hash_attn_fwd: lds");                     \
+    hipLaunchKernelGGL((hash_attn_staged_kernel<NQW, F16, BIGN>), dim3(unsigned(max_items)), dim3(256), NQW * kTileBytes,  \
                        st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt,      \
                        q_perm, items, n_items, (bf16_t*)out, lse, Sq, N, C, sm_scale * kLog2e);                      \
   } while (0)
-  if (pairs && f16)
+  if (N > (1 << 24)) {  // 64-bit row offsets; one work item per workgroup only
+    if (f16)
+      FM_STAGED_LAUNCH3(1, true, true);
+    else
+      FM_STAGED_LAUNCH3(1, false, true);
+  } else if (pairs && f16)
     FM_STAGED_LAUNCH(2, true);
   else if (pairs)
     FM_STAGED_LAUNCH(2, false);
@@ -74,6 +80,7 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
   else
     FM_STAGED_LAUNCH(1, false);
 #undef FM_STAGED_LAUNCH
+#undef FM_STAGED_LAUNCH3
   return launch_status("fm_hash_attn_fwd(mfma, staged)");
 }
 

@@ -86,7 +86,9 @@ constexpr size_t kStagedTileBytes = size_t(kSK * kSKld + kSD * kSVld) * sizeof(b
 // point to global memory or LDS) over the cnt keys idx[0..cnt) of one bucket.  Called by all 256
 // threads of a workgroup; lds holds NQW tile buffers of kStagedTileBytes.  NQW = 16-query tiles per
 // wave: the workgroup takes up to 64 * NQW queries.
-template <int NQW, bool F16 = false>
+// BIGN: rows are addressed by 64-bit byte offsets (memories of more than 2^24 keys; a few more address
+// instructions per tile), otherwise by 32-bit ones (N * 256 B < 4 GiB).
+template <int NQW, bool F16 = false, bool BIGN = false>
 __device__ __forceinline__ void attend_staged(
     const bf16_t* __restrict__ Qb, const int* __restrict__ q_rows, int n_q, const bf16_t* __restrict__ Kb,
     const bf16_t* __restrict__ Vb, const int32_t* __restrict__ idx, int cnt, int N, float scale2,
@@ -137,14 +139,20 @@ __device__ __forceinline__ void attend_staged(
   const int vj = l & 15, vc = 4 * w + (l >> 4);
   const int kchunk = tid & 15, krow = tid >> 4;
   // (positions past the end of the list read row 0: their scores are masked, their p is 0)
-  // (row offsets as unsigned 32-bit byte offsets from the uniform bases: N * 256 < 2^32, checked by the host)
+  // (row offsets as unsigned 32-bit byte offsets from the uniform bases unless BIGN: N * 256 < 2^32, checked by the host)
   const char* Kc = reinterpret_cast<const char*>(Kb) + 16 * kchunk;
   const char* Vc = reinterpret_cast<const char*>(Vb) + 16 * vc;
   auto k_row = [&](int rows, int p) {
-    return *reinterpret_cast<const uint4*>(Kc + (uint32_t(__shfl(rows, p)) << 8));
+    if constexpr (BIGN)
+      return *reinterpret_cast<const uint4*>(Kc + (uint64_t(uint32_t(__shfl(rows, p))) << 8));
+    else
+      return *reinterpret_cast<const uint4*>(Kc + (uint32_t(__shfl(rows, p)) << 8));
   };
   auto v_row = [&](int rows, int p) {
-    return *reinterpret_cast<const uint4*>(Vc + (uint32_t(__shfl(rows, p)) << 8));
+    if constexpr (BIGN)
+      return *reinterpret_cast<const uint4*>(Vc + (uint64_t(uint32_t(__shfl(rows, p))) << 8));
+    else
+      return *reinterpret_cast<const uint4*>(Vc + (uint32_t(__shfl(rows, p)) << 8));
   };
 #define FM_STAGED_LOAD_TILE(rows_raw)                      \
   do {                                                     \

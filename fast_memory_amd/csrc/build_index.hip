@@ -7,12 +7,12 @@
 extern "C" size_t fm_build_index_workspace(int H, int C, int N, int d, int Z,
                                            int64_t rows_per_pass) {
   (void)d;
-  (void)Z;
   if (H < 1 || C < 1 || N < 1) return 0;
   int64_t rows = rows_per_pass < 1 ? 1 : rows_per_pass;
   if (rows > int64_t(H) * C) rows = int64_t(H) * C;
   int64_t ldy = (int64_t(N) + 3) / 4 * 4;
-  return size_t(rows) * size_t(ldy) * sizeof(float);
+  // lists longer than FM_MAX_Z are sorted in memory: that scratch sits in front of the projection rows
+  return fm::align_up(fm_argtopz_workspace(int64_t(H) * C, N, Z), 256) + size_t(rows) * size_t(ldy) * sizeof(float);
 }
 
 extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, float* val_out, int H, int C,
@@ -22,6 +22,12 @@ extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, fl
              "fm_build_index: H=%d C=%d N=%d d=%d Z=%d", H, C, N, d, Z);
   FM_REQUIRE(A && K && idx_out && ws, FM_ERR_ARG, "fm_build_index: null pointer");
   const int64_t ldy = (int64_t(N) + 3) / 4 * 4;  // rows start 16-byte aligned
+  const size_t sel_ws = align_up(fm_argtopz_workspace(int64_t(H) * C, N, Z), 256);
+  FM_REQUIRE(ws_bytes > sel_ws, FM_ERR_WORKSPACE, "fm_build_index: workspace %zu does not hold the selection scratch %zu",
+             ws_bytes, sel_ws);
+  void* const sel = ws;
+  ws = static_cast<char*>(ws) + sel_ws;
+  ws_bytes -= sel_ws;
   const int64_t fit = int64_t(ws_bytes / (size_t(ldy) * sizeof(float)));
   FM_REQUIRE(fit >= 1, FM_ERR_WORKSPACE, "fm_build_index: workspace %zu holds no row of %lld floats",
              ws_bytes, (long long)ldy);
@@ -37,7 +43,7 @@ extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, fl
       int rc = fm_project(Ah, Kh, Y, hb, C, N, d, ldy, dtype, stream);
       if (rc) return rc;
       rc = fm_argtopz_f32(Y, int64_t(hb) * C, N, ldy, Z, idx_out + int64_t(h) * C * Zc,
-                          val_out ? val_out + int64_t(h) * C * Zc : nullptr, nullptr, 0, stream);
+                          val_out ? val_out + int64_t(h) * C * Zc : nullptr, sel, sel_ws, stream);
       if (rc) return rc;
       h += hb;
       continue;
@@ -49,7 +55,7 @@ extern "C" int fm_build_index(const void* A, const void* K, int32_t* idx_out, fl
       int rc = fm_project(Ah, Kh, Y, 1, nc, N, d, ldy, dtype, stream);
       if (rc) return rc;
       rc = fm_argtopz_f32(Y, nc, N, ldy, Z, idx_out + (int64_t(h) * C + c0) * Zc,
-                          val_out ? val_out + (int64_t(h) * C + c0) * Zc : nullptr, nullptr, 0, stream);
+                          val_out ? val_out + (int64_t(h) * C + c0) * Zc : nullptr, sel, sel_ws, stream);
       if (rc) return rc;
       c0 += nc;
     }

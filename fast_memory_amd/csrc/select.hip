@@ -165,6 +165,74 @@ __global__ __launch_bounds__(NT) void argtopz_kernel(
   collect_sort_write(src, cut, Zc, P, buf, sh, out, vout);
 }
 
+// ---- lists longer than FM_MAX_Z ------------------------------------------------------------------
+// The Zc survivors do not fit LDS.  Per row: the exact cut by radix passes over the row (as above), the
+// exactly Zc composites >= cut collected into a slot of the caller's workspace, padded to a power of two,
+// and a plain bitonic network over that slot in global memory (it stays in L2: 8 bytes per entry).  A
+// workgroup owns one slot and walks rows blockIdx.x, blockIdx.x + gridDim.x, ...  Slow next to the LDS
+// forms (about a millisecond per row of 65536) and without any limit on Z or on the values.
+constexpr int kBigSlots = 1024;  // workgroups, and workspace slots, of a launch
+
+__global__ __launch_bounds__(kSelThreads) void argtopz_big_kernel(const float* __restrict__ Y, int64_t rows, int N,
+                                                                  int64_t ldy, int Zc, int P,
+                                                                  int32_t* __restrict__ idx_out,
+                                                                  float* __restrict__ val_out,
+                                                                  uint64_t* __restrict__ slots) {
+  __shared__ SelectShared sh;
+  uint64_t* buf = slots + int64_t(blockIdx.x) * P;
+  const int tid = threadIdx.x;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    DenseRowT<kSelThreads> src{Y + row * ldy, N};
+    const uint64_t cut = radix_select_cut<kSelThreads>(src, Zc, 6, sh);
+    if (tid == 0) sh.cnt = 0;
+    __syncthreads();
+    src([&](float y, uint32_t i) {
+      const uint64_t c = composite(y, i);
+      if (c >= cut) {
+        const int pos = atomicAdd(&sh.cnt, 1);
+        if (pos < P) buf[pos] = c;
+      }
+    });
+    for (int i = Zc + tid; i < P; i += kSelThreads) buf[i] = 0;
+    __syncthreads();
+    for (int k = 2; k <= P; k <<= 1)
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        for (int t = tid; t < (P >> 1); t += kSelThreads) {
+          const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+          const int q = i | j;
+          const uint64_t a = buf[i], b = buf[q];
+          const bool desc = (i & k) == 0;
+          if (desc ? (a < b) : (a > b)) {
+            buf[i] = b;
+            buf[q] = a;
+          }
+        }
+        __syncthreads();
+      }
+    for (int i = tid; i < Zc; i += kSelThreads) {
+      const uint64_t c = buf[i];
+      idx_out[row * Zc + i] = int32_t(0xffffffffu - uint32_t(c));
+      if (val_out) val_out[row * Zc + i] = key_to_float(uint32_t(c >> 32));
+    }
+    __syncthreads();  // the slot and sh are reused by the next row
+  }
+}
+
+size_t argtopz_big_workspace(int64_t rows, int Zc) {
+  if (Zc <= FM_MAX_Z || rows < 1) return 0;
+  return size_t(std::min<int64_t>(rows, kBigSlots)) * size_t(next_pow2(Zc)) * sizeof(uint64_t);
+}
+
+int launch_argtopz_big(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out, float* val_out,
+                       void* ws, size_t ws_bytes, hipStream_t st) {
+  FM_REQUIRE(ws && ws_bytes >= argtopz_big_workspace(rows, Zc), FM_ERR_WORKSPACE,
+             "arg-top-Z with min(Z, N) = %d > FM_MAX_Z needs a workspace of %zu bytes (fm_argtopz_workspace), got %zu", Zc,
+             argtopz_big_workspace(rows, Zc), ws_bytes);
+  hipLaunchKernelGGL(argtopz_big_kernel, dim3(unsigned(std::min<int64_t>(rows, kBigSlots))), dim3(kSelThreads), 0, st, Y,
+                     rows, N, ldy, Zc, next_pow2(Zc), idx_out, val_out, static_cast<uint64_t*>(ws));
+  return launch_status("argtopz(big)");
+}
+
 int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out, float* val_out,
                    const int32_t* row_map, const int32_t* n_rows_dev, hipStream_t st) {
   const int P = next_pow2(Zc);
@@ -208,15 +276,16 @@ int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int
 
 }  // namespace fm
 
-extern "C" size_t fm_argtopz_workspace(int64_t, int, int) { return 0; }
+extern "C" size_t fm_argtopz_workspace(int64_t rows, int N, int Z) {
+  if (rows < 1 || N < 1 || Z < 1) return 0;
+  return fm::argtopz_big_workspace(rows, Z < N ? Z : N);
+}
 
 extern "C" void fm_debug_argtopz_exact_only(int on) { fm::g_argtopz_exact_only = on != 0; }
 
 extern "C" int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, int Z,
                               int32_t* idx_out, float* val_out, void* ws, size_t ws_bytes, void* stream) {
   using namespace fm;
-  (void)ws;
-  (void)ws_bytes;
   FM_REQUIRE(rows >= 0 && N >= 1 && Z >= 1, FM_ERR_ARG, "fm_argtopz_f32: rows=%lld N=%d Z=%d",
              (long long)rows, N, Z);
   FM_REQUIRE(ldy >= N, FM_ERR_ARG, "fm_argtopz_f32: ldy=%lld < N=%d", (long long)ldy, N);
@@ -224,7 +293,7 @@ extern "C" int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, 
   FM_REQUIRE(Y && idx_out, FM_ERR_ARG, "fm_argtopz_f32: null pointer");
   FM_REQUIRE(rows <= 0x7fffffffLL, FM_ERR_UNSUPPORTED, "fm_argtopz_f32: too many rows");
   const int Zc = Z < N ? Z : N;
-  FM_REQUIRE(Zc <= FM_MAX_Z, FM_ERR_UNSUPPORTED, "fm_argtopz_f32: min(Z,N)=%d exceeds FM_MAX_Z=%d",
-             Zc, FM_MAX_Z);
+  if (Zc > FM_MAX_Z)  // lists that do not fit LDS: sorted in the workspace
+    return launch_argtopz_big(Y, rows, N, ldy, Zc, idx_out, val_out, ws, ws_bytes, as_stream(stream));
   return launch_argtopz(Y, rows, N, ldy, Zc, idx_out, val_out, nullptr, nullptr, as_stream(stream));
 }

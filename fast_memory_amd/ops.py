@@ -63,7 +63,10 @@ def argtopz(Y: torch.Tensor, Z: int, return_values: bool = False):
     Zc = min(int(Z), N)
     out = torch.empty((*Y.shape[:-1], Zc), dtype=torch.int32, device=Y.device)
     vals = torch.empty(out.shape, dtype=torch.float32, device=Y.device) if return_values else None
-    check(_lib.load().fm_argtopz_f32(_p(Y), rows, N, N, int(Z), _p(out), _p(vals), None, 0, _stream(Y)))
+    lib = _lib.load()
+    nws = lib.fm_argtopz_workspace(rows, N, int(Z))             # non-zero only for lists longer than FM_MAX_Z
+    ws = _ws(nws, Y) if nws else None
+    check(lib.fm_argtopz_f32(_p(Y), rows, N, N, int(Z), _p(out), _p(vals), _p(ws), nws, _stream(Y)))
     return (out, vals) if return_values else out
 
 
@@ -374,6 +377,10 @@ def decode_hash_attn(q, A_all, K_all, V_all, idx_all, desc, sm_scale: float, ret
     _dev(q, A_all, K_all, V_all, idx_all, desc)
     rows, G, d = q.shape
     assert desc.dtype == torch.int64 and desc.shape == (rows, 5) and idx_all.dtype == torch.int32
+    if G > 16:      # the kernel takes up to 16 query heads per row: more go through in groups of 16
+        parts = [decode_hash_attn(q[:, g0:g0 + 16].contiguous(), A_all, K_all, V_all, idx_all, desc, sm_scale,
+                                  return_scores) for g0 in range(0, G, 16)]
+        return tuple(torch.cat([p[j] for p in parts], dim=1) for j in range(len(parts[0])))
     out = torch.empty_like(q)
     lse = torch.empty((rows, G), dtype=torch.float32, device=q.device)
     h = torch.empty((rows, G), dtype=torch.int32, device=q.device)

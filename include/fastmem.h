@@ -43,7 +43,9 @@ typedef enum {
 
 typedef enum { FM_F32 = 0, FM_BF16 = 1, FM_F16 = 2 } fm_dtype;
 
-/* Largest bucket capacity Z the selection kernels accept. */
+/* Longest list min(Z, N) the selection sorts inside LDS.  Longer lists are accepted by fm_argtopz_f32 and
+ * fm_build_index (sorted in the workspace, markedly slower); fm_build_index_fused and fm_index_append take
+ * lists up to FM_MAX_Z only. */
 #define FM_MAX_Z 16384
 /* Largest head dimension. */
 #define FM_MAX_D 256
@@ -69,7 +71,8 @@ int fm_project(const void* A, const void* K, float* Y, int H, int C, int N, int 
  * misleads falls back to exact radix passes), others about four times; the
  * result is the same.  idx_out is [rows, min(Z,N)] int32;
  * val_out (may be NULL) receives the selected values in the same order (-0 as
- * +0): the lists' values are what fm_index_append needs to extend an index. */
+ * +0): the lists' values are what fm_index_append needs to extend an index.
+ * fm_argtopz_workspace is 0 unless min(Z, N) > FM_MAX_Z. */
 size_t fm_argtopz_workspace(int64_t rows, int N, int Z);
 int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, int Z, int32_t* idx_out,
                    float* val_out, void* ws, size_t ws_bytes, void* stream);

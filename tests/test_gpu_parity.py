@@ -129,10 +129,15 @@ def test_argtopz_sampled_one_pass_equals_exact_passes(ops):
         assert torch.equal(fast[rows].cpu().long(), O.argtopz(Y[rows], Z))
 
 
-def test_argtopz_rejects_oversize_z(ops):
+def test_argtopz_beyond_fm_max_z_needs_its_workspace(ops, lib):
+    # lists longer than FM_MAX_Z are sorted in a workspace (tests/test_gpu_limits.py checks the results);
+    # without one the call is refused with a status code, before any launch
     Y = torch.zeros(1, 40000, device="cuda")
-    with pytest.raises(RuntimeError):
-        ops.argtopz(Y, 20000)
+    out = torch.empty(1, 20000, dtype=torch.int32, device="cuda")
+    assert lib.fm_argtopz_workspace(1, 40000, 20000) == 32768 * 8
+    assert lib.fm_argtopz_workspace(1, 40000, 16384) == 0
+    assert lib.fm_argtopz_f32(Y.data_ptr(), 1, 40000, 40000, 20000, out.data_ptr(), None, None, 0, None) == 3
+    assert b"workspace" in lib.fm_last_error()
 
 
 def test_build_index_matches_project_then_select(ops):

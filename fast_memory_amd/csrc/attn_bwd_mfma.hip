@@ -487,6 +487,8 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
 // 128 bf16 that take the stores of a block's positions past the end of a list.
 // MAXT: the most tiles a pass takes (2 or 4).  The four-tile form costs registers in every path of the
 // kernel that holds it, so it is only launched where buckets receive more than 24 queries on average.
+constexpr int kStagedMaxQ = 256;  // queries of a bucket that go through its bf16 partial rows
+
 template <int MAXT>
 __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
@@ -519,10 +521,14 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
   const int cnt = bucket_cnt[bkt];
   bf16_t* dkb = dkp + (off - pos0) * kBD;
   bf16_t* dvb = dvp + (off - pos0) * kBD;
-  // the first pass stores the bucket's partial rows, the others add to them; a pass takes up to MAXT tiles
-  for (int q0 = 0; q0 < nq; q0 += 16 * MAXT) {
+  // the first pass stores the bucket's partial rows, the others add to them; a pass takes up to MAXT tiles.
+  // The partial rows are bf16 and every pass after the first rounds them again, so only the first
+  // kStagedMaxQ queries of a bucket go through them; a bucket that receives more (a heavily skewed hash)
+  // adds the rest straight into dK / dV with fp32 atomic adds (hash_attn_bwd_excess_kernel).
+  const int nq_staged = min(nq, kStagedMaxQ);
+  for (int q0 = 0; q0 < nq_staged; q0 += 16 * MAXT) {
     if (q0) __syncthreads();  // red and q_rows are reused
-    const int left = nq - q0;
+    const int left = nq_staged - q0;
 #define FM_BWD_PASS(FIRST, NT)                                                                                        \
   bwd_tile<true, FIRST, NT>(q, out, lse, dout, dlse, ql + q0, min(16 * NT, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,  \
                             cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage)
@@ -546,6 +552,31 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
   }
 }
 
+// grid (C, rows): the queries of a bucket beyond the first kStagedMaxQ, 16 at a time, with atomic adds into
+// dK / dV; a workgroup whose bucket has no such query (nearly all of them) reads one word and leaves.
+__global__ __launch_bounds__(256) void hash_attn_bwd_excess_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
+    const int32_t* __restrict__ q_perm, const int32_t* __restrict__ bin_off, const int32_t* __restrict__ bin_count,
+    const bf16_t* __restrict__ out, const float* __restrict__ lse, const bf16_t* __restrict__ dout,
+    const float* __restrict__ dlse, bf16_t* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv, int row0,
+    int Sq, int N, int C, float sm_scale) {
+  __shared__ __attribute__((aligned(16))) float red[4 * 8 * 4 * 64];
+  __shared__ int q_rows[16];
+  const int row = row0 + blockIdx.y;
+  const int64_t bkt = int64_t(row) * C + blockIdx.x;
+  const int nq = bin_count[bkt];
+  if (nq <= kStagedMaxQ) return;
+  const int32_t* ql = q_perm + bin_off[bkt];
+  for (int q0 = kStagedMaxQ; q0 < nq; q0 += 16) {
+    if (q0 > kStagedMaxQ) __syncthreads();  // red and q_rows are reused
+    bwd_tile<false, true>(q, out, lse, dout, dlse, ql + q0, min(16, nq - q0), int64_t(row) * Sq,
+                          k + int64_t(row) * N * kBD, v + int64_t(row) * N * kBD, k_idx + bucket_off[bkt],
+                          bucket_cnt[bkt], N, sm_scale, dq, dk + int64_t(row) * N * kBD, dv + int64_t(row) * N * kBD,
+                          nullptr, nullptr, nullptr, red, q_rows, nullptr);
+  }
+}
+
 bool hash_attn_bwd_mfma_supported(int d, int dtype) { return d == kBD && dtype == FM_BF16; }
 
 int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
@@ -563,7 +594,8 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
                                   const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                                   const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
                                   const void* dout, const float* dlse, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0,
-                                  int row0, int rows, int Sq, int N, int C, float sm_scale, hipStream_t st) {
+                                  int row0, int rows, int Sq, int N, int C, float sm_scale, float* dk, float* dv,
+                                  hipStream_t st) {
 #define FM_BWD_STAGED(MAXT)                                                                                        \
   hipLaunchKernelGGL(hash_attn_bwd_staged_kernel<MAXT>, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,       \
                      (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,  \
@@ -574,6 +606,11 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
   else
     FM_BWD_STAGED(2);
 #undef FM_BWD_STAGED
+  if (Sq > kStagedMaxQ)  // some bucket may hold more queries than go through its partial rows
+    hipLaunchKernelGGL(hash_attn_bwd_excess_kernel, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,
+                       (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
+                       bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, row0,
+                       Sq, N, C, sm_scale);
   return launch_status("fm_hash_attn_bwd_staged(partials)");
 }
 

@@ -36,7 +36,7 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
                                   const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                                   const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
                                   const void* dout, const float* dlse, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0,
-                                  int row0, int rows, int Sq, int N, int C, float sm_scale,
+                                  int row0, int rows, int Sq, int N, int C, float sm_scale, float* dk, float* dv,
                                   hipStream_t st);  // attn_bwd_mfma.hip
 
 // ---- inverse index ------------------------------------------------------------
@@ -228,7 +228,7 @@ extern "C" int fm_hash_attn_bwd_staged(const void* q, const void* k, const void*
       bf16_t* dvp = dkp + size_t(n_pos) * 128;
       bf16_t* dump = dvp + size_t(n_pos) * 128;
       int rc = hash_attn_bwd_staged_partials(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, bin_off, bin_count, out,
-                                             lse, dout, dlse, dq, dkp, dvp, dump, pos0, h0, h1 - h0, Sq, N, C, sm_scale, st);
+                                             lse, dout, dlse, dq, dkp, dvp, dump, pos0, h0, h1 - h0, Sq, N, C, sm_scale, dk, dv, st);
       if (rc) return rc;
       const int64_t n_keys = int64_t(h1 - h0) * N;
       hipLaunchKernelGGL(bwd_reduce_kernel, dim3(unsigned(ceil_div(n_keys, int64_t(4)))), dim3(256), 0, st, dkp, dvp,

@@ -186,7 +186,8 @@ int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t*
  * workspace) and a second kernel sums, per key, the partial rows of the list
  * positions that name it -- full-line stores and loads in place of fp32 atomic
  * read-modify-writes, and a fixed summation order (results do not depend on
- * scheduling).  Pays when most buckets receive queries: a bucket without queries
+ * scheduling; only the first 256 queries of a bucket go through its partial
+ * rows, a bucket that receives more adds the rest with fp32 atomic adds).  Pays when most buckets receive queries: a bucket without queries
  * still costs its rows (written as zeros and read back).
  *
  * fm_inverse_index: the inverse of the lists, which depends on the lists only and

@@ -49,6 +49,7 @@ def build(force: bool = True, jobs: int = 8) -> str:
     srcs = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
     hdrs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
     hdrs.append(os.path.join(os.path.dirname(HERE), "include", "fastmem.h"))
+    hdrs.append(os.path.join(os.path.dirname(HERE), "include", "fastmem_debug.h"))
     newest_hdr = max(os.path.getmtime(h) for h in hdrs)
     todo = []
     for s in srcs:

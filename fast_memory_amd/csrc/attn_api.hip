@@ -30,10 +30,10 @@ int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const 
 // 0 = automatic, 1 = force the generic kernels (used by tests to compare paths); for the grouped
 // forward on MFMA, 2 = always the form that stages a bucket's rows in LDS (4: two work items per
 // workgroup), 3 = always the form that gathers them into registers
-int g_force_generic = 0;
+std::atomic<int> g_force_generic{0};
 }  // namespace fm
 
-extern "C" void fm_debug_force_generic(int on) { fm::g_force_generic = on; }
+extern "C" void fm_debug_force_generic(int on) { fm::g_force_generic.store(on, std::memory_order_relaxed); }
 
 extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype) {
   using namespace fm;

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_generic_kernel(
   }
 }
 
-extern int g_force_generic;
+extern std::atomic<int> g_force_generic;
 bool hash_attn_bwd_mfma_supported(int d, int dtype);
 int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                        const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items, const int32_t* n_items,

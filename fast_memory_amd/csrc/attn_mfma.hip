@@ -489,7 +489,7 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
                           const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
                           float* lse, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, hipStream_t st);
-extern int g_force_generic;
+extern std::atomic<int> g_force_generic;
 
 // Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
 // staged in LDS, one work item per workgroup, 2 = staged, two items per workgroup.  Measured rule: the

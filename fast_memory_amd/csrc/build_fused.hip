@@ -741,15 +741,20 @@ __global__ void fused_status_kernel(const int32_t* __restrict__ n_fail, int32_t*
 }
 
 // optional phase markers for profiling: events recorded after phases 0, 1, 2, 3
+// (process-wide and guarded by a mutex: a build that runs while another thread sets or clears the
+// markers records into the old set or the new one, never into a half-written pair)
+static std::mutex g_phase_mu;
 static hipEvent_t* g_phase_events = nullptr;
 static int g_n_phase_events = 0;
 static inline void mark_phase(int i, hipStream_t st) {
+  std::lock_guard<std::mutex> lk(g_phase_mu);
   if (g_phase_events && i < g_n_phase_events) (void)hipEventRecord(g_phase_events[i], st);
 }
 
 }  // namespace fm
 
 extern "C" void fm_debug_set_phase_events(void** events, int n) {
+  std::lock_guard<std::mutex> lk(fm::g_phase_mu);
   fm::g_phase_events = reinterpret_cast<hipEvent_t*>(events);
   fm::g_n_phase_events = events ? n : 0;
 }

@@ -3,8 +3,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <float.h>
+#include <atomic>
+#include <mutex>
 
-#include "../../include/fastmem.h"
+#include "../../include/fastmem_debug.h"
 
 namespace fm {
 

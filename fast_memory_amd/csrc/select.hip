@@ -24,7 +24,7 @@
 
 namespace fm {
 
-bool g_argtopz_exact_only = false;  // test hook: fm_debug_argtopz_exact_only
+std::atomic<bool> g_argtopz_exact_only{false};  // test hook: fm_debug_argtopz_exact_only
 
 constexpr int kSampleRegs = 32;  // sampled elements per thread: samples of up to 32768 elements
 constexpr int kCollectRegs = 16; // collected candidates per thread: capacity up to 16384

@@ -1,0 +1,57 @@
+/*
+ * fastmem_debug.h -- test and measurement hooks of libfastmem.so.
+ *
+ * None of these has a counterpart in the reference.  The switches (fm_debug_force_generic,
+ * fm_debug_argtopz_exact_only, fm_debug_set_phase_events) are PROCESS-WIDE state, read by every call on
+ * every stream: they exist so that tests can compare two implementations of one operator and so that the
+ * benchmark can time the phases of the fused build; a production caller never touches them.  The probes
+ * (fm_debug_copy, fm_debug_read) are plain kernels of known size.
+ */
+#ifndef FASTMEM_DEBUG_H
+#define FASTMEM_DEBUG_H
+
+#include "fastmem.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Diagnostic: 1 routes the attention entry points through the generic kernels
+ * (used by tests to compare the two implementations), 0 restores dispatch.  For
+ * fm_hash_attn_fwd on bf16, d = 128 only: 2 = always the kernel that stages a
+ * bucket's rows in LDS, one work item per workgroup, 4 = the same with two work
+ * items per workgroup, 3 = always the kernel that gathers the rows into
+ * registers (dispatch: staged when H min(Sq, C) >= 512 or Sq >= 24 C, two items
+ * from Sq >= 64 C; gather otherwise). */
+void fm_debug_force_generic(int on);
+
+/* Diagnostic: name of the kernel fm_hash_attn_fwd launches for these extents
+ * (a static string): "hash_attn_generic_kernel", "hash_attn_mfma_kernel" (rows
+ * gathered into registers), "hash_attn_staged_kernel<1>" or "...<2>" (rows staged
+ * in LDS, one or two work items per workgroup).  bench.py names its roofline
+ * kernel with it. */
+const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype);
+
+/* Diagnostic: 1 makes fm_argtopz_f32 (and the chunked index build) take the exact
+ * multi-pass selection for every row instead of the sampled one-pass form (tests
+ * compare the two), 0 restores dispatch. */
+void fm_debug_argtopz_exact_only(int on);
+
+/* Diagnostic: hand the fused index build up to 5 hipEvent_t (host array that
+ * must stay valid; NULL clears) which it records on its stream before phase 0
+ * (thresholds), 1 (MFMA filter), 2 (selection), 3 (repair) and at the end. */
+void fm_debug_set_phase_events(void** events, int n);
+
+/* Diagnostic: streaming copy of nbytes (multiple of 16) device to device; the
+ * known-size kernel that profiler HBM counters are calibrated against. */
+int fm_debug_copy(void* dst, const void* src, int64_t nbytes, void* stream);
+
+/* Diagnostic: read-only stream over nbytes (multiple of 32768) of device memory;
+ * nothing is written (sink: 4 bytes of device memory, left untouched).  Times the
+ * read bandwidth a kernel reaches on the device. */
+int fm_debug_read(const void* src, int64_t nbytes, void* sink, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTMEM_DEBUG_H */

@@ -13,9 +13,18 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def header_symbols():
+    syms = set()
+    for name in ("fastmem.h", "fastmem_debug.h"):
+        text = open(os.path.join(ROOT, "include", name)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        syms |= set(re.findall(r"\b(fm_[a-z0-9_]+)\s*\(", text))
+    return sorted(syms)
+
+
+def test_production_header_declares_no_debug_hook():
     text = open(os.path.join(ROOT, "include", "fastmem.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(fm_[a-z0-9_]+)\s*\(", text)))
+    assert "fm_debug_" not in text
 
 
 def test_library_exports_every_declared_symbol():

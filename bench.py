@@ -695,8 +695,9 @@ def main():
             f"passes {['%.2f' % t for t in t_all]} s; parity {parity}")
 
     if args.config == "c4" and fused_phases:
-        filter_traffic = hbm_traffic("fused_filter_kernel", cfg.name)
-        roofline = {"kernel": "fused_filter_kernel", "bound": "mfma", "achieved": fused_phases["filter_tflops"],
+        filter_kernel = ops.fused_filter_kernel_name(H, C, N, d, Z, cfg.dtype)
+        filter_traffic = hbm_traffic(filter_kernel, cfg.name)
+        roofline = {"kernel": filter_kernel, "bound": "mfma", "achieved": fused_phases["filter_tflops"],
                     "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": fused_phases["filter_mfma_frac"],
                     "traffic": filter_traffic, "algorithmic_flops_per_launch": 2.0 * H * C * N * d,
                     "avg_launch_ms": fused_phases["mfma_filter_ms"]}

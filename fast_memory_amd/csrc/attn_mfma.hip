@@ -489,23 +489,31 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
                           const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
                           float* lse, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, hipStream_t st);
+int hash_attn_mfma_ring(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
+                        const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items,
+                        const int32_t* n_items, int64_t max_items, void* out, float* lse, int Sq, int N, int C,
+                        float sm_scale, bool f16, hipStream_t st);
 extern std::atomic<int> g_force_generic;
 
 // Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
-// staged in LDS, one work item per workgroup, 2 = staged, two items per workgroup.  Measured rule: the
-// staged kernel is at least as fast wherever the launch has work items enough to fill the chip (at
-// least 512, taking min(Sq, C) per row as their number) or buckets receive 24 queries or more on
-// average; with few and small items the four waves of the gather kernel, which share one bucket's
-// keys, finish an item sooner.  Two items per workgroup from 64 queries per bucket on average.
+// staged in LDS through registers, one work item per workgroup, 2 = the same, two items per workgroup,
+// 3 = rows loaded straight into LDS, two items per workgroup (attn_ring.hpp).  Measured rule: the
+// staged kernel is at least as fast as the register-gather one wherever the launch has work items enough
+// to fill the chip (at least 512, taking min(Sq, C) per row as their number) or buckets receive 24 queries
+// or more on average; with few and small items the four waves of the gather kernel, which share one
+// bucket's keys, finish an item sooner.  From 64 queries per bucket on average, two items per workgroup,
+// with the direct loads (13 % faster than form 2 at 128 queries per bucket; form 2 stays for tests to
+// compare against).
 // (Beyond 2^24 keys the staged kernel runs in its form with 64-bit row offsets, one item per workgroup.)
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
   if (g_force_generic == 3) return 0;
   if (g_force_generic == 2) return 1;
-  if (g_force_generic == 4) return 2;
+  if (g_force_generic == 4) return N <= (1 << 24) ? 2 : 1;
+  if (g_force_generic == 5) return N <= (1 << 24) ? 3 : 1;
   const bool many_items = int64_t(H) * (Sq < C ? Sq : C) >= 512;
   const bool dense = Sq >= 24 * int64_t(C);
   if (!many_items && !dense) return 0;
-  return (Sq >= 64 * int64_t(C) && many_items && N <= (1 << 24)) ? 2 : 1;
+  return (Sq >= 64 * int64_t(C) && many_items && N <= (1 << 24)) ? 3 : 1;
 }
 
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
@@ -515,6 +523,9 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
   (void)d;
   int choice = hash_attn_mfma_choice(H, Sq, N, C);
   if (dtype == FM_F16 && choice == 0) choice = 1;
+  if (choice == 3)
+    return hash_attn_mfma_ring(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse, Sq,
+                               N, C, sm_scale, dtype == FM_F16, st);
   if (choice)
     return hash_attn_mfma_staged(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out,
                                  lse, Sq, N, C, sm_scale, choice == 2, dtype == FM_F16, st);

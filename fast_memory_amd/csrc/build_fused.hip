@@ -759,6 +759,12 @@ extern "C" void fm_debug_set_phase_events(void** events, int n) {
   fm::g_n_phase_events = events ? n : 0;
 }
 
+extern "C" const char* fm_build_index_fused_kernel(int H, int C, int N, int d, int Z, int dtype) {
+  fm::FusedPlan p;
+  if (H < 1 || C < 1 || N < 1 || !fm::fused_plan(H, C, N, d, Z, dtype, p)) return nullptr;
+  return p.wide ? "fused_filter_wide_kernel" : "fused_filter_kernel";
+}
+
 extern "C" size_t fm_build_index_fused_workspace(int H, int C, int N, int d, int Z, int dtype) {
   fm::FusedPlan p;
   if (H < 1 || C < 1 || N < 1 || !fm::fused_plan(H, C, N, d, Z, dtype, p)) return 0;

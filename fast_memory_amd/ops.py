@@ -483,17 +483,24 @@ def generic_kernels_forced() -> bool:
     return _generic_forced
 
 
+def fused_filter_kernel_name(H: int, C: int, N: int, d: int, Z: int, dtype: torch.dtype):
+    """Name of the filter kernel the fused index build launches for these extents (None: shape not taken)."""
+    name = _lib.load().fm_build_index_fused_kernel(H, C, N, d, Z, _DT[dtype])
+    return name.decode() if name else None
+
+
 def hash_attn_fwd_kernel_name(H: int, Sq: int, N: int, d: int, C: int, dtype: torch.dtype) -> str:
     """Name of the kernel :func:`hash_attn_fwd` launches for these extents."""
     return _lib.load().fm_hash_attn_fwd_kernel(H, Sq, N, d, C, _DT[dtype]).decode()
 
 
 def grouped_forward_kernel(which: Optional[str]) -> None:
-    """Diagnostic switch for the bf16, d = 128 grouped attention forward: ``"staged"`` always takes the
+    """Diagnostic switch for the bf16 / fp16, d = 128 grouped attention forward: ``"staged"`` always takes the
     kernel that shares a bucket's rows among its waves through LDS, one work item per workgroup,
-    ``"staged-pairs"`` the same kernel with two work items per workgroup, ``"gather"`` always the kernel
+    ``"staged-pairs"`` the same kernel with two work items per workgroup, ``"ring"`` the kernel whose rows
+    go from global memory straight into LDS (two items per workgroup), ``"gather"`` always the kernel
     that gathers the rows into registers, ``None`` restores the dispatch (staged unless the launch has few
-    and small work items; pairs from 64 queries per bucket on average)."""
+    and small work items; the direct loads from 64 queries per bucket on average)."""
     global _generic_forced
     _generic_forced = False
-    _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4}[which])
+    _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4, "ring": 5}[which])

@@ -32,6 +32,12 @@ void fm_debug_force_generic(int on);
  * kernel with it. */
 const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype);
 
+/* Diagnostic: name of the filter kernel fm_build_index_fused launches for these
+ * extents (a static string): "fused_filter_kernel" (four waves over a slab of 256
+ * buckets) or "fused_filter_wide_kernel" (eight waves over a slab of 1024); NULL
+ * where the fused build does not take the shape. */
+const char* fm_build_index_fused_kernel(int H, int C, int N, int d, int Z, int dtype);
+
 /* Diagnostic: 1 makes fm_argtopz_f32 (and the chunked index build) take the exact
  * multi-pass selection for every row instead of the sampled one-pass form (tests
  * compare the two), 0 restores dispatch. */

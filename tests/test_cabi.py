@@ -89,7 +89,7 @@ def test_grouped_forward_dispatch_rule():
     name = lambda *a: lib.fm_hash_attn_fwd_kernel(*a).decode()
     assert name(8, 32768, 1048576, 128, 2048, 1) == "hash_attn_staged_kernel<1>"      # 1 M keys, 16 queries / bucket
     assert name(8, 8192, 32768, 128, 256, 1) == "hash_attn_staged_kernel<1>"          # prefill chunk, 32 / bucket
-    assert name(8, 131072, 65536, 128, 1024, 1) == "hash_attn_staged_kernel<2>"       # reference harness, 128 / bucket
+    assert name(8, 131072, 65536, 128, 1024, 1) == "hash_attn_ring_kernel"       # reference harness, 128 / bucket
     assert name(1, 64, 262144, 128, 64, 1) == "hash_attn_mfma_kernel"                 # few, small work items
     assert name(1, 2048, 262144, 128, 64, 1) == "hash_attn_staged_kernel<1>"          # few buckets, many queries each
     assert name(8, 8192, 1 << 25, 128, 256, 1) == "hash_attn_staged_kernel<1, 64-bit rows>"   # beyond 32-bit byte offsets

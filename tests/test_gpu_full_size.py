@@ -212,9 +212,9 @@ def test_config3_decode_batch_full_size(ops):
 
 def test_reference_harness_shape_kernels_agree(ops):
     """The shape of the reference's performance harness (triton_kernel.py:507-528): 8 rows x 131072 queries,
-    65536 keys, 1024 buckets of 3072 keys, N(0,1) inputs.  Dispatch takes the staged kernel with two work
-    items per workgroup; the register-gather kernel, an independent implementation, must agree with it on
-    every query, and sampled queries must agree with the fp64 oracle."""
+    65536 keys, 1024 buckets of 3072 keys, N(0,1) inputs.  Dispatch takes the kernel that loads a bucket's rows
+    straight into LDS, two work items per workgroup; the register-gather kernel, an independent implementation,
+    must agree with it on every query, and sampled queries must agree with the fp64 oracle."""
     from fast_memory_amd import attention_hash
     B, Sq, N, d, C, Z = 8, 131072, 65536, 128, 1024, 3072
     g = torch.Generator().manual_seed(1006)
@@ -222,7 +222,7 @@ def test_reference_harness_shape_kernels_agree(ops):
     k, v, A = mk(B, N, d), mk(B, N, d), mk(B, C, d)
     q = torch.cat([mk(1, Sq, d) for _ in range(B)])
     scale = d ** -0.5
-    assert ops.hash_attn_fwd_kernel_name(B, Sq, N, d, C, torch.bfloat16) == "hash_attn_staged_kernel<2>"
+    assert ops.hash_attn_fwd_kernel_name(B, Sq, N, d, C, torch.bfloat16) == "hash_attn_ring_kernel"
     out, lse = attention_hash(q, k, v, A, Z, scale)
     ops.grouped_forward_kernel("gather")
     try:

@@ -257,7 +257,7 @@ def test_attention_dense_buckets(dtype, d):
     assert_attn_close(out, lse, ro, rl, dtype, f"dense d={d}")
 
 
-@pytest.mark.parametrize("which", ["staged", "staged-pairs", "gather"])
+@pytest.mark.parametrize("which", ["staged", "staged-pairs", "ring", "gather"])
 @pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large"])
 def test_attention_grouped_forward_kernels(ops, which, case):
     # the bf16 d=128 forward kernels (rows shared through LDS, one or two work items per workgroup / rows
@@ -287,7 +287,7 @@ def test_attention_grouped_forward_kernels(ops, which, case):
     assert_attn_close(out, lse, ro, rl, torch.bfloat16, f"{which} {case}")
 
 
-@pytest.mark.parametrize("which", ["staged", "staged-pairs", "gather", "generic"])
+@pytest.mark.parametrize("which", ["staged", "staged-pairs", "ring", "gather", "generic"])
 def test_attention_out_of_range_list_entries_are_clamped(ops, which):
     # the contract of every entry point: key indices outside [0, N) are clamped, never dereferenced
     # (negative -> key 0, >= N -> key N-1); lists here hold such entries in every bucket, and lists

@@ -271,7 +271,8 @@ def bench_decode_batch(args):
                                f"Z=round(4 sqrt N), 1 token per query head ({qheads} query-heads), 512 local keys",
                    "step": "batched hash + gather attention (one launch) + local attention + merge"},
         "roofline": {"kernel": "decode_hash_attn_kernel", "bound": "hbm", "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": hbm_traffic("decode_hash_attn_kernel", "c3-varlen-decode-bf16"),
                      "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms},
         "cpu_baseline": cpu,
         "index_build": {"keys_per_s": total_keys / (build_ms * 1e-3), "ms": build_ms, "keys": total_keys},

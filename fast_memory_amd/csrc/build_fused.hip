@@ -84,13 +84,16 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   const int P = next_pow2(Z);
   bool found = false;
   double m_exp = 0;
-  for (int ns_try : {16384, 32768}) {
+  for (int ns_try : {4096, 8192, 16384, 32768}) {
     p.stride = N / ns_try;
     p.ns = N / p.stride;
     const double mu = double(Z) * p.ns / N;
     p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
     if (p.rank * 4 > p.ns) continue;
     m_exp = double(p.rank) * N / p.ns;
+    // (the two small samples only where they keep at most 32 % more candidates than Z: short memories with
+    // long lists, where a 16 K sample would be a quarter of all keys and phase 0 a quarter of the projection)
+    if (ns_try < 16384 && m_exp > 1.32 * Z) continue;
     const double per_w = m_exp / p.n_writers;
     const double sd_w = sqrt(pow(double(N) / p.ns * sqrt(double(p.rank)) / p.n_writers, 2) + per_w);
     for (int nt = 256; nt <= kSelThreads && !found; nt *= 2)

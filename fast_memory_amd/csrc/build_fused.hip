@@ -641,7 +641,7 @@ struct CandRegs {
 };
 
 static inline size_t cand_select_lds_bytes(int Zc, int P) {
-  const size_t binned = size_t(Zc + kSelMaxBin) * sizeof(uint64_t) + size_t(kSelBins) * sizeof(uint32_t);
+  const size_t binned = binned_lds_bytes(Zc);
   const size_t sorted = sort_lds_bytes(P) + sizeof(SelectShared) + 8;
   return std::max(binned, sorted);
 }

@@ -252,7 +252,7 @@ int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int
   // SelectShared sits behind the sort buffer / the candidate buffer; the binned selection needs its own extent
   const size_t sh_off = align_up(std::max(sort_lds_bytes(P), size_t(sp.cap) * (wide ? sizeof(uint32_t) : sizeof(uint64_t))), 16);
   const auto lds_for = [](size_t off, int zc, bool sampled) {
-    const size_t binned = sampled ? size_t(zc + kSelMaxBin) * sizeof(uint64_t) + size_t(kSelBins) * sizeof(uint32_t) : 0;
+    const size_t binned = sampled ? binned_lds_bytes(zc) : 0;
     return std::max(off + sizeof(SelectShared), binned);
   };
   const size_t lds = lds_for(sh_off, Zc, sp.n_lines > 0);

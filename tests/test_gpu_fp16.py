@@ -67,6 +67,31 @@ def test_attention_forward_fp16(ops, B, S, N, C, Z, d):
     assert (out.float().cpu() - ro.float()).abs().max().item() < 4e-3
 
 
+def test_attention_forward_fp16_many_queries_per_bucket(ops):
+    # the kernels for buckets with many queries (two work items per workgroup; rows through staging registers,
+    # or loaded straight into LDS), each forced, in fp16: against the oracle and bit for bit against each
+    # other.  Buckets of 1, 64, 65, 128, 129 and 300 queries; ragged lists.
+    from fast_memory_amd import attention_hash_varlen
+    q, k, v, kh, cnt, qh = make_attn_case(9411, 2, 900, 4000, 10, 700, 128, F16, window="ref")
+    sizes = [1, 64, 65, 128, 129, 300]
+    pos = 0
+    for b, n in enumerate(sizes):
+        qh[0, pos:pos + n] = b
+        pos += n
+    qh[0, pos:] = 7
+    ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 128 ** -0.5)
+    outs = {}
+    for which in ("staged-pairs", "ring"):
+        ops.grouped_forward_kernel(which)
+        try:
+            out, lse = attention_hash_varlen(*dev(q, k, v, kh, cnt, qh), 128 ** -0.5)
+        finally:
+            ops.grouped_forward_kernel(None)
+        assert_attn_close(out, lse, ro, rl, F16, f"fp16 {which}")
+        outs[which] = (out, lse)
+    assert torch.equal(outs["ring"][0], outs["staged-pairs"][0]) and torch.equal(outs["ring"][1], outs["staged-pairs"][1])
+
+
 def test_composite_local_merge_and_backward_fp16(ops):
     from fast_memory_amd import Memory, attention_hash, fit_projection
     g = gen(9400)

@@ -29,7 +29,8 @@ int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const 
 
 // 0 = automatic, 1 = force the generic kernels (used by tests to compare paths); for the grouped
 // forward on MFMA, 2 = always the form that stages a bucket's rows in LDS (4: two work items per
-// workgroup), 3 = always the form that gathers them into registers
+// workgroup), 5 = always the form that loads them straight into LDS, 3 = always the form that gathers them
+// into registers
 std::atomic<int> g_force_generic{0};
 }  // namespace fm
 

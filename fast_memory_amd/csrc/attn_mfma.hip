@@ -497,13 +497,12 @@ extern std::atomic<int> g_force_generic;
 
 // Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
 // staged in LDS through registers, one work item per workgroup, 2 = the same, two items per workgroup,
-// 3 = rows loaded straight into LDS, two items per workgroup (attn_ring.hpp).  Measured rule: the
+// 3 = rows loaded straight into LDS, three items per workgroup (attn_ring.hpp).  Measured rule: the
 // staged kernel is at least as fast as the register-gather one wherever the launch has work items enough
 // to fill the chip (at least 512, taking min(Sq, C) per row as their number) or buckets receive 24 queries
 // or more on average; with few and small items the four waves of the gather kernel, which share one
-// bucket's keys, finish an item sooner.  From 64 queries per bucket on average, two items per workgroup,
-// with the direct loads (13 % faster than form 2 at 128 queries per bucket; form 2 stays for tests to
-// compare against).
+// bucket's keys, finish an item sooner.  From 64 queries per bucket on average, form 3 (17 % faster than
+// form 2 at 128 queries per bucket; form 2 stays for tests to compare against).
 // (Beyond 2^24 keys the staged kernel runs in its form with 64-bit row offsets, one item per workgroup.)
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
   if (g_force_generic == 3) return 0;

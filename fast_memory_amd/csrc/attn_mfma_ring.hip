@@ -1,6 +1,6 @@
 // Grouped launch of the bucket-gathered attention whose rows go from global memory straight into LDS
-// (attn_ring.hpp): one workgroup per two consecutive work items of a bucket (128 queries), the form for
-// buckets with many queries.
+// (attn_ring.hpp): one workgroup per three consecutive work items of a bucket (192 queries, 48 per wave),
+// the form for buckets with many queries.  A bucket of up to 192 queries is swept once.
 #include "attn_ring.hpp"
 
 namespace fm {
@@ -23,8 +23,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   int me = blockIdx.x;
   if ((me | 63) < n_it) me = (me & ~63) | ((me & 7) << 3) | ((me >> 3) & 7);
   const fm_item it = items[me];
-  // The items of a bucket are consecutive and their queries contiguous: the workgroup of item lo + 2j takes
-  // the items lo + 2j and lo + 2j + 1 of the bucket, the one launched for item lo + 2j + 1 has nothing to do.
+  // The items of a bucket are consecutive and their queries contiguous: the workgroup of item lo + 3j takes
+  // the items lo + 3j .. lo + 3j + 2 of the bucket, the ones launched for the other two have nothing to do.
   // (The bucket's first item by a galloping, then a binary search: a bucket may have thousands of items.)
   auto same = [&](int i) { return items[i].row == it.row && items[i].bucket == it.bucket; };
   int lo = me, step = 1;  // invariant: items lo..me belong to the bucket
@@ -40,14 +40,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     else
       bad = mid;
   }
-  if ((me - lo) & 1) return;
+  if ((me - lo) % 3) return;
   int n_q = it.n_q;
-  if (me + 1 < n_it && same(me + 1)) n_q += items[me + 1].n_q;
+  if (me + 1 < n_it && same(me + 1)) {
+    n_q += items[me + 1].n_q;
+    if (me + 2 < n_it && same(me + 2)) n_q += items[me + 2].n_q;
+  }
   const int64_t bkt = int64_t(it.row) * C + it.bucket;
   const int64_t qbase = int64_t(it.row) * Sq;
-  attend_ring<2, F16>(q + qbase * kSD, q_perm + it.q_start, n_q, k + int64_t(it.row) * N * kSD,
+  attend_ring<3, F16>(q + qbase * kSD, q_perm + it.q_start, n_q, k + int64_t(it.row) * N * kSD,
                       v + int64_t(it.row) * N * kSD, k_idx + bucket_off[bkt], bucket_cnt[bkt], N, scale2,
-                      out + qbase * kSD, lse + qbase, ring_lds);
+                      out + qbase * kSD, lse + qbase, ring_lds, it.bucket);
 }
 
 int hash_attn_mfma_ring(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,

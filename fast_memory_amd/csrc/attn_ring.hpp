@@ -30,9 +30,17 @@
 // t - 1, whose buffers are free), request tile t + 1 and the list entries of tile t + 2, then
 // S^T = K Q^T, the softmax and O^T += V^T P^T.
 //
-// Measured at the reference's harness shape (fp16, 128 queries per bucket, 3072 keys): 2.66 ms against
-// 3.05 ms for the staged kernel with two items per workgroup.
+// A wave takes up to three tiles of 16 queries (a workgroup 192 queries: three consecutive work items of a
+// bucket), dealt to the waves in turn so that their shares differ by one tile at most, and runs a copy of the
+// loop compiled for the number of tiles it has.  250 registers, none spilled: a spill inside the loop would be
+// reloaded by a vector-memory instruction, and the wait for it would also wait for the rows on their way.
+//
+// Measured at the reference's harness shape (fp16, 128 queries per bucket on average, half of the buckets
+// above 128, 3072 keys): 2.51 ms against 3.05 ms for the staged kernel with two items per workgroup (2.62 ms
+// with two tiles per wave, where a bucket of 129-192 queries was swept by two workgroups).
 #pragma once
+#include <type_traits>
+
 #include "attn_staged.hpp"
 
 namespace fm {
@@ -71,14 +79,14 @@ __device__ __forceinline__ const T* ring_uniform_ptr(const T* p) {
 }
 
 // The attention of n_q <= 64 NQW queries (rows q_rows[0..n_q) of Qb / Ob / Lb) over the cnt keys
-// idx[0..cnt) of one bucket; called by all 256 threads of a workgroup (wave w takes queries 16 NQW w ..),
-// lds = kRingLdsBytes of LDS.
+// idx[0..cnt) of one bucket; called by all 256 threads of a workgroup (a wave takes up to NQW <= 3 tiles of
+// 16 queries), lds = kRingLdsBytes of LDS.
 // Rows are addressed by 32-bit byte offsets: N * 256 < 2^32 (checked by the host).
 template <int NQW, bool F16>
 __device__ __forceinline__ void attend_ring(const bf16_t* __restrict__ Qb, const int* __restrict__ q_rows, int n_q,
                                             const bf16_t* Kb, const bf16_t* Vb, const int32_t* idx, int cnt, int N,
                                             float scale2, bf16_t* __restrict__ Ob, float* __restrict__ Lb,
-                                            bf16_t* lds_generic) {
+                                            bf16_t* lds_generic, int rot) {
   lds_char_t* const lds = (lds_char_t*)lds_generic;
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane(uint32_t(uintptr_t(lds)));
   const int tid = threadIdx.x, l = tid & 63;
@@ -91,19 +99,21 @@ __device__ __forceinline__ void attend_ring(const bf16_t* __restrict__ Qb, const
   auto swz = [](int r) { return ((r & 7) << 1) | ((r >> 3) & 1); };
 
   // ---- this lane's queries (column c of each of wave w's NQW tiles) ----
-  const int nqt_w = min(max((n_q - 16 * NQW * w + 15) >> 4, 0), NQW);
-  const bool wave_on = nqt_w > 0;
-  bool q_ok[NQW];
-  int64_t qrow[NQW];
+  // The 16-query tiles are dealt to the waves in turn, tile j to wave (j + rot) % 4 as its tile j / 4, so a
+  // wave's share differs from another's by one tile at most (9 tiles: 3, 2, 2, 2), and `rot` (the caller
+  // passes the bucket number) moves the wave with the extra tile, and with it the SIMD, from bucket to bucket.
+  const int wl = (w - rot) & 3;
+  const int n_qt = (n_q + 15) >> 4;
+  const int nqt_w = min(max((n_qt - wl + 3) >> 2, 0), NQW);  // tiles of this wave that hold queries
   uint4 qf[NQW][4];
 #pragma unroll
   for (int qt = 0; qt < NQW; ++qt) {
-    const int jq = 16 * (NQW * w + qt) + c;
-    q_ok[qt] = jq < n_q;
-    qrow[qt] = q_ok[qt] ? q_rows[jq] : 0;
-    const uint4* pq = reinterpret_cast<const uint4*>(Qb + qrow[qt] * kSD + 8 * g);
+    const int jq = 16 * (wl + 4 * qt) + c;
+    const bool ok = jq < n_q;
+    const int64_t qrow = ok ? q_rows[jq] : 0;
+    const uint4* pq = reinterpret_cast<const uint4*>(Qb + qrow * kSD + 8 * g);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) qf[qt][s] = q_ok[qt] ? pq[4 * s] : make_uint4(0, 0, 0, 0);
+    for (int s = 0; s < 4; ++s) qf[qt][s] = ok ? pq[4 * s] : make_uint4(0, 0, 0, 0);
   }
   f32x4 O[NQW][8];
   float m[NQW], lsum[NQW];
@@ -157,17 +167,21 @@ __device__ __forceinline__ void attend_ring(const bf16_t* __restrict__ Qb, const
   const int vbase = vrl * 256 + ((((c & 3) >> 1) ^ swz(vrl)) << 4) + (c & 1) * 8;  // ^ (t8 << 5)
   const lds_char_t* const ring = lds + kRIdsBytes;
 
-  auto scores = [&](int t, int slot, f32x4 (&s)[NQW][4]) {
+  // (T_ = std::integral_constant: the number of this wave's query tiles the call works on)
+  // (kb, vb: kbase and vbase through an empty asm statement of the caller, once per tile, so that the
+  // 12 operand addresses are formed again with an XOR each instead of living in registers through the loop)
+  auto scores = [&](auto T_, int t, int slot, int kb, f32x4 (&s)[NQW][4]) {
+    constexpr int T = decltype(T_)::value;
     const lds_char_t* const bK = ring + slot * kRSlotBytes;
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) {
         const ring_u32x4 a_ =
-            *reinterpret_cast<const __attribute__((address_space(3))) ring_u32x4*>(bK + kt * 4096 + (kbase ^ (st << 6)));
+            *reinterpret_cast<const __attribute__((address_space(3))) ring_u32x4*>(bK + kt * 4096 + (kb ^ (st << 6)));
         const uint4 a = make_uint4(a_[0], a_[1], a_[2], a_[3]);
 #pragma unroll
-        for (int qt = 0; qt < NQW; ++qt)
+        for (int qt = 0; qt < T; ++qt)
           s[qt][kt] = Mma<F16>::m16(a, qf[qt][st], st == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[qt][kt]);
       }
     }
@@ -179,14 +193,15 @@ __device__ __forceinline__ void attend_ring(const bf16_t* __restrict__ Qb, const
         for (int r = 0; r < 4; ++r)
           if (kp0 + 16 * kt + 4 * g + r >= cnt) {
 #pragma unroll
-            for (int qt = 0; qt < NQW; ++qt) s[qt][kt][r] = -INFINITY;
+            for (int qt = 0; qt < T; ++qt) s[qt][kt][r] = -INFINITY;
           }
     }
   };
   // online softmax as in attn_staged.hpp (triton_kernel.py:248-263)
-  auto softmax = [&](f32x4 (&s)[NQW][4], uint4 (&pf)[NQW][2]) {
+  auto softmax = [&](auto T_, f32x4 (&s)[NQW][4], uint4 (&pf)[NQW][2]) {
+    constexpr int T = decltype(T_)::value;
 #pragma unroll
-    for (int qt = 0; qt < NQW; ++qt) {
+    for (int qt = 0; qt < T; ++qt) {
       float mx = st_max3(s[qt][0][0], s[qt][0][1], s[qt][0][2]);
       mx = st_max3(mx, s[qt][0][3], s[qt][1][0]);
       mx = st_max3(mx, s[qt][1][1], s[qt][1][2]);
@@ -224,14 +239,15 @@ __device__ __forceinline__ void attend_ring(const bf16_t* __restrict__ Qb, const
       }
     }
   };
-  auto weighted_values = [&](int slot, const uint4 (&pf)[NQW][2]) {
+  auto weighted_values = [&](auto T_, int slot, int vb, const uint4 (&pf)[NQW][2]) {
+    constexpr int T = decltype(T_)::value;
     const lds_char_t* const bV = ring + slot * kRSlotBytes;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
       for (int t8 = 0; t8 < 8; ++t8) {
         // contraction slots 8g .. 8g+3: keys 4g .. 4g+3 of key tile 2h; slots 8g+4 .. 8g+7: the same of key tile 2h+1
-        const lds_char_t* p = bV + h * 8192 + (vbase ^ (t8 << 5));
+        const lds_char_t* p = bV + h * 8192 + (vb ^ (t8 << 5));
         const ring_short4 lo =
             __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ring_short4*)p);
         const ring_short4 hi =
@@ -243,61 +259,79 @@ __device__ __forceinline__ void attend_ring(const bf16_t* __restrict__ Qb, const
         a.s4[0] = lo;
         a.s4[1] = hi;
 #pragma unroll
-        for (int qt = 0; qt < NQW; ++qt) O[qt][t8] = Mma<F16>::m16(a.u, pf[qt][h], O[qt][t8]);
+        for (int qt = 0; qt < T; ++qt) O[qt][t8] = Mma<F16>::m16(a.u, pf[qt][h], O[qt][t8]);
       }
     }
   };
 
-  if (ntiles > 0) {
-    // ---- prologue: list entries of tile 0, then tile 0 and the list entries of tile 1 ----
-    issue_ids(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    read_rows(0);
-    if (ntiles > 1) issue_ids(1);
-    issue_tile(0);
-    // two tiles per round, so that the buffers are compile-time constants
-    for (int t0 = 0; t0 < ntiles; t0 += 2) {
+  // The work of a wave that has T of its NQW query tiles: the loop over the bucket's tiles and the
+  // write-out, compiled once for every T so that a wave runs neither MFMAs nor softmax for tiles it does
+  // not have (the waves of a workgroup meet at the barriers all the same: every copy has one per tile).
+  auto run = [&](auto T_) {
+    constexpr int T = decltype(T_)::value;
+    if (ntiles > 0) {
+      // ---- prologue: list entries of tile 0, then tile 0 and the list entries of tile 1 ----
+      issue_ids(0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      read_rows(0);
+      if (ntiles > 1) issue_ids(1);
+      issue_tile(0);
+      // two tiles per round, so that the buffers are compile-time constants
+      for (int t0 = 0; t0 < ntiles; t0 += 2) {
 #pragma unroll
-      for (int par = 0; par < 2; ++par) {
-        const int t = t0 + par;
-        if (t >= ntiles) break;
-        f32x4 s_[NQW][4];
-        uint4 pf_[NQW][2];
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        ring_barrier();  // tile t is in place (and this wave's list entries of tile t + 1); every wave has finished tile t - 1
-        if (t + 1 < ntiles) {
-          read_rows(t + 1);
-          if (t + 2 < ntiles) issue_ids(t + 2);
-          issue_tile(1 - par);
-        }
-        if (wave_on) {
-          scores(t, 2 * par, s_);
-          softmax(s_, pf_);
-          weighted_values(2 * par + 1, pf_);
+        for (int par = 0; par < 2; ++par) {
+          const int t = t0 + par;
+          if (t >= ntiles) break;
+          f32x4 s_[NQW][4];
+          uint4 pf_[NQW][2];
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          ring_barrier();  // tile t is in place (and this wave's list entries of tile t + 1); every wave has finished tile t - 1
+          if (t + 1 < ntiles) {
+            read_rows(t + 1);
+            if (t + 2 < ntiles) issue_ids(t + 2);
+            issue_tile(1 - par);
+          }
+          if (T > 0) {
+            constexpr int TT = T > 0 ? T : 1;
+            int kb = kbase, vb = vbase;
+            asm volatile("" : "+v"(kb), "+v"(vb));
+            scores(std::integral_constant<int, TT>{}, t, 2 * par, kb, s_);
+            softmax(std::integral_constant<int, TT>{}, s_, pf_);
+            weighted_values(std::integral_constant<int, TT>{}, 2 * par + 1, vb, pf_);
+          }
         }
       }
     }
-  }
-
-  // ---- finish: lane (g,c) holds dims 16t + 4g + r of query c of each tile ----
+    // ---- finish: lane (g,c) holds dims 16t + 4g + r of query c of each tile ----
 #pragma unroll
-  for (int qt = 0; qt < NQW; ++qt) {
-    float ltot = lsum[qt] + __shfl_xor(lsum[qt], 16);
-    ltot += __shfl_xor(ltot, 32);
-    const bool empty = (m[qt] == -INFINITY);
-    const float inv = empty ? 0.f : 1.f / ltot;
-    if (q_ok[qt]) {
-      bf16_t* po = Ob + qrow[qt] * kSD + 4 * g;
+    for (int qt = 0; qt < T; ++qt) {
+      float ltot = lsum[qt] + __shfl_xor(lsum[qt], 16);
+      ltot += __shfl_xor(ltot, 32);
+      const bool empty = (m[qt] == -INFINITY);
+      const float inv = empty ? 0.f : 1.f / ltot;
+      const int jq = 16 * (wl + 4 * qt) + c;  // (looked up again rather than kept in registers through the loop)
+      if (jq < n_q) {
+        const int64_t qrow = q_rows[jq];
+        bf16_t* po = Ob + qrow * kSD + 4 * g;
 #pragma unroll
-      for (int t8 = 0; t8 < 8; ++t8) {
-        uint2 o;
-        o.x = Mma<F16>::pack2(O[qt][t8][0] * inv, O[qt][t8][1] * inv);
-        o.y = Mma<F16>::pack2(O[qt][t8][2] * inv, O[qt][t8][3] * inv);
-        *reinterpret_cast<uint2*>(po + 16 * t8) = o;
+        for (int t8 = 0; t8 < 8; ++t8) {
+          uint2 o;
+          o.x = Mma<F16>::pack2(O[qt][t8][0] * inv, O[qt][t8][1] * inv);
+          o.y = Mma<F16>::pack2(O[qt][t8][2] * inv, O[qt][t8][3] * inv);
+          *reinterpret_cast<uint2*>(po + 16 * t8) = o;
+        }
+        if (g == 0) Lb[qrow] = empty ? -FLT_MAX : (m[qt] + __builtin_amdgcn_logf(ltot)) * kLn2;
       }
-      if (g == 0) Lb[qrow[qt]] = empty ? -FLT_MAX : (m[qt] + __builtin_amdgcn_logf(ltot)) * kLn2;
     }
-  }
+  };
+  if (nqt_w == NQW)
+    run(std::integral_constant<int, NQW>{});
+  else if (NQW > 1 && nqt_w == NQW - 1)
+    run(std::integral_constant<int, (NQW > 1 ? NQW - 1 : 0)>{});
+  else if (NQW > 2 && nqt_w == NQW - 2)
+    run(std::integral_constant<int, (NQW > 2 ? NQW - 2 : 0)>{});
+  else
+    run(std::integral_constant<int, 0>{});
 }
 
 }  // namespace fm

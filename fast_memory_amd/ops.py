@@ -498,7 +498,7 @@ def grouped_forward_kernel(which: Optional[str]) -> None:
     """Diagnostic switch for the bf16 / fp16, d = 128 grouped attention forward: ``"staged"`` always takes the
     kernel that shares a bucket's rows among its waves through LDS, one work item per workgroup,
     ``"staged-pairs"`` the same kernel with two work items per workgroup, ``"ring"`` the kernel whose rows
-    go from global memory straight into LDS (two items per workgroup), ``"gather"`` always the kernel
+    go from global memory straight into LDS (three items per workgroup), ``"gather"`` always the kernel
     that gathers the rows into registers, ``None`` restores the dispatch (staged unless the launch has few
     and small work items; the direct loads from 64 queries per bucket on average)."""
     global _generic_forced

@@ -18,18 +18,21 @@ extern "C" {
 
 /* Diagnostic: 1 routes the attention entry points through the generic kernels
  * (used by tests to compare the two implementations), 0 restores dispatch.  For
- * fm_hash_attn_fwd on bf16, d = 128 only: 2 = always the kernel that stages a
+ * fm_hash_attn_fwd on bf16 / fp16, d = 128 only: 2 = always the kernel that stages a
  * bucket's rows in LDS, one work item per workgroup, 4 = the same with two work
- * items per workgroup, 3 = always the kernel that gathers the rows into
- * registers (dispatch: staged when H min(Sq, C) >= 512 or Sq >= 24 C, two items
- * from Sq >= 64 C; gather otherwise). */
+ * items per workgroup, 5 = always the kernel that loads the rows straight into
+ * LDS (three items per workgroup), 3 = always the kernel that gathers the rows
+ * into registers (dispatch: staged when H min(Sq, C) >= 512 or Sq >= 24 C, the
+ * direct loads from Sq >= 64 C; gather otherwise). */
 void fm_debug_force_generic(int on);
 
 /* Diagnostic: name of the kernel fm_hash_attn_fwd launches for these extents
  * (a static string): "hash_attn_generic_kernel", "hash_attn_mfma_kernel" (rows
  * gathered into registers), "hash_attn_staged_kernel<1>" or "...<2>" (rows staged
- * in LDS, one or two work items per workgroup).  bench.py names its roofline
- * kernel with it. */
+ * in LDS through registers, one or two work items per workgroup),
+ * "hash_attn_ring_kernel" (rows loaded straight into LDS, three work items per
+ * workgroup); ", f16>" / "<f16>" marks the fp16 forms, "64-bit rows" the form for
+ * memories of more than 2^24 keys.  bench.py names its roofline kernel with it. */
 const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype);
 
 /* Diagnostic: name of the filter kernel fm_build_index_fused launches for these

@@ -68,7 +68,7 @@ def test_attention_forward_fp16(ops, B, S, N, C, Z, d):
 
 
 def test_attention_forward_fp16_many_queries_per_bucket(ops):
-    # the kernels for buckets with many queries (two work items per workgroup; rows through staging registers,
+    # the kernels for buckets with many queries (two or three work items per workgroup; rows through staging registers,
     # or loaded straight into LDS), each forced, in fp16: against the oracle and bit for bit against each
     # other.  Buckets of 1, 64, 65, 128, 129 and 300 queries; ragged lists.
     from fast_memory_amd import attention_hash_varlen

@@ -213,7 +213,7 @@ def test_config3_decode_batch_full_size(ops):
 def test_reference_harness_shape_kernels_agree(ops):
     """The shape of the reference's performance harness (triton_kernel.py:507-528): 8 rows x 131072 queries,
     65536 keys, 1024 buckets of 3072 keys, N(0,1) inputs.  Dispatch takes the kernel that loads a bucket's rows
-    straight into LDS, two work items per workgroup; the register-gather kernel, an independent implementation,
+    straight into LDS, three work items per workgroup; the register-gather kernel, an independent implementation,
     must agree with it on every query, and sampled queries must agree with the fp64 oracle."""
     from fast_memory_amd import attention_hash
     B, Sq, N, d, C, Z = 8, 131072, 65536, 128, 1024, 3072

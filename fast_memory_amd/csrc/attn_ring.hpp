@@ -4,7 +4,7 @@
 // as attn_staged.hpp; what differs is how a bucket's rows reach LDS.
 //
 // In attn_staged.hpp a tile's rows wait in registers between their load and their place in LDS (32
-// registers a thread), V is transposed on the way with VALU work, and two barriers frame every tile.
+// registers a thread) and V is transposed on the way with VALU work.
 // Here the rows go from global memory straight into LDS (global_load_lds_dwordx4: lane i of a wave's
 // load writes 16 bytes at M0 + 16 i):
 //   * LDS holds two tiles of 64 keys (K and V, 64 rows x 256 B each): the one being read and the next,

@@ -497,12 +497,16 @@ extern std::atomic<int> g_force_generic;
 
 // Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
 // staged in LDS through registers, one work item per workgroup, 2 = the same, two items per workgroup,
-// 3 = rows loaded straight into LDS, three items per workgroup (attn_ring.hpp).  Measured rule: the
-// staged kernel is at least as fast as the register-gather one wherever the launch has work items enough
-// to fill the chip (at least 512, taking min(Sq, C) per row as their number) or buckets receive 24 queries
-// or more on average; with few and small items the four waves of the gather kernel, which share one
-// bucket's keys, finish an item sooner.  From 64 queries per bucket on average, form 3 (17 % faster than
-// form 2 at 128 queries per bucket; form 2 stays for tests to compare against).
+// 3 = rows loaded straight into LDS, three items per workgroup (attn_ring.hpp).  Measured rule: a kernel
+// that shares a bucket's rows through LDS is at least as fast as the register-gather one wherever the launch
+// has work items enough to fill the chip (at least 512, taking min(Sq, C) per row as their number) or buckets
+// receive 24 queries or more on average; with few and small items the four waves of the gather kernel, which
+// share one bucket's keys, finish an item sooner.  From 24 queries per bucket on average form 3, below that
+// form 1.  (On keys that stay in the last-level cache form 3 is ahead at every density measured: 65536 keys,
+// 1024 buckets of 3072, 16 / 32 / 64 / 128 queries per bucket: 1.51 / 1.57 / 1.69 / 2.51 ms against 1.54 /
+// 1.67 / 2.30 / 3.05 ms; on a million keys with 16 queries per bucket, where the rows come from HBM and what
+// counts is the bytes in flight, form 1 with its three workgroups per CU is 1 % ahead.  Form 2 stays for
+// tests to compare against.)
 // (Beyond 2^24 keys the staged kernel runs in its form with 64-bit row offsets, one item per workgroup.)
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
   if (g_force_generic == 3) return 0;
@@ -512,7 +516,7 @@ int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
   const bool many_items = int64_t(H) * (Sq < C ? Sq : C) >= 512;
   const bool dense = Sq >= 24 * int64_t(C);
   if (!many_items && !dense) return 0;
-  return (Sq >= 64 * int64_t(C) && many_items && N <= (1 << 24)) ? 3 : 1;
+  return (dense && N <= (1 << 24)) ? 3 : 1;
 }
 
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,

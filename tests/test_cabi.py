@@ -88,11 +88,12 @@ def test_grouped_forward_dispatch_rule():
     lib = _lib.load()
     name = lambda *a: lib.fm_hash_attn_fwd_kernel(*a).decode()
     assert name(8, 32768, 1048576, 128, 2048, 1) == "hash_attn_staged_kernel<1>"      # 1 M keys, 16 queries / bucket
-    assert name(8, 8192, 32768, 128, 256, 1) == "hash_attn_staged_kernel<1>"          # prefill chunk, 32 / bucket
+    assert name(8, 8192, 32768, 128, 256, 1) == "hash_attn_ring_kernel"               # prefill chunk, 32 / bucket
     assert name(8, 131072, 65536, 128, 1024, 1) == "hash_attn_ring_kernel"       # reference harness, 128 / bucket
     assert name(1, 64, 262144, 128, 64, 1) == "hash_attn_mfma_kernel"                 # few, small work items
-    assert name(1, 2048, 262144, 128, 64, 1) == "hash_attn_staged_kernel<1>"          # few buckets, many queries each
+    assert name(1, 2048, 262144, 128, 64, 1) == "hash_attn_ring_kernel"               # few buckets, many queries each
     assert name(8, 8192, 1 << 25, 128, 256, 1) == "hash_attn_staged_kernel<1, 64-bit rows>"   # beyond 32-bit byte offsets
-    assert name(8, 8192, 32768, 128, 256, 2) == "hash_attn_staged_kernel<1, f16>"     # fp16 (FM_F16 = 2)
+    assert name(8, 8192, 32768, 128, 256, 2) == "hash_attn_ring_kernel<f16>"          # fp16 (FM_F16 = 2)
+    assert name(8, 4096, 32768, 128, 256, 2) == "hash_attn_staged_kernel<1, f16>"     # fp16, 16 / bucket
     assert name(1, 64, 1 << 25, 128, 64, 1) == "hash_attn_mfma_kernel"                # few small items, any N
     assert name(1, 512, 4096, 64, 64, 0) == "hash_attn_generic_kernel"                # fp32 / d != 128

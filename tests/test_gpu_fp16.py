@@ -50,15 +50,16 @@ def test_fused_build_fp16_bit_identical(ops):
     assert torch.equal(fused.cpu().long(), O.argtopz(ops.project(Ad, Kd).cpu(), Z))
 
 
-@pytest.mark.parametrize("B,S,N,C,Z,d", [(2, 300, 3000, 9, 500, 128),       # staged MFMA kernel, one item per workgroup
-                                         (1, 2000, 2000, 8, 333, 128),      # 250 queries per bucket: two items per workgroup
+@pytest.mark.parametrize("B,S,N,C,Z,d", [(2, 300, 3000, 9, 500, 128),       # 33 queries per bucket: rows loaded straight into LDS
+                                         (2, 600, 3000, 64, 200, 128),      # 9 per bucket, 128 items: staged, one item per workgroup
+                                         (1, 2000, 2000, 8, 333, 128),      # 250 queries per bucket
                                          (2, 70, 300, 6, 40, 64)])          # generic kernel
 def test_attention_forward_fp16(ops, B, S, N, C, Z, d):
     from fast_memory_amd import attention_hash_varlen
     q, k, v, kh, cnt, qh = make_attn_case(9300 + S, B, S, N, C, Z, d, F16, window="ref")
     if d == 128:
         name = ops.hash_attn_fwd_kernel_name(B, S, N, d, C, F16)
-        assert name.startswith("hash_attn_staged_kernel") and "f16" in name, name
+        assert name.startswith(("hash_attn_staged_kernel", "hash_attn_ring_kernel")) and "f16" in name, name
     out, lse = attention_hash_varlen(*dev(q, k, v, kh, cnt, qh), d ** -0.5)
     assert out.dtype == F16
     ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, d ** -0.5)

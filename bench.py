@@ -332,8 +332,9 @@ def bench_reference_harness(args):
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms, "hit_buckets": hit,
                 "mfma_tflops": alg_flops / attn_ms / 1e9,
                 "mfma_frac": alg_flops / attn_ms / 1e9 / BF16_MFMA_PEAK_TFLOPS,
-                "note": "128 queries per bucket on average: 127 flop per algorithmic byte; the kernel is bound by "
-                        "its LDS and VALU work per MFMA, not by HBM"}
+                "note": "128 queries per bucket on average: 127 flop per algorithmic byte; the rows come from the "
+                        "last-level cache, not from HBM; the kernel is bound by the MFMA and softmax work of a SIMD, "
+                        "which issue one after the other, and by the wait for the next tile's rows"}
     log(f"[bench] tkperf step {ms_per_step:.2f} ms = {dense_equiv_tflops:.0f} dense-equivalent TFLOP/s; build "
         f"{build_ms:.2f}, hash {hash_ms:.2f}, group {group_ms:.2f}, attention {attn_ms:.2f} ms "
         f"({achieved:.0f} GB/s algorithmic, {roofline['mfma_tflops']:.0f} TFLOP/s)")

@@ -258,13 +258,13 @@ def test_attention_dense_buckets(dtype, d):
 
 
 @pytest.mark.parametrize("which", ["staged", "staged-pairs", "ring", "gather"])
-@pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large"])
+@pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large", "heavy-bucket"])
 def test_attention_grouped_forward_kernels(ops, which, case):
     # the bf16 d=128 forward kernels (rows shared through LDS, one or two work items per workgroup / rows
     # gathered into registers), each forced,
     # against the oracle: ragged lists with a last tile of 1..63 keys and empty buckets; buckets with
     # 1, 15, 16, 17, 63, 64, 65 and 200 queries (several work items, partly filled waves); the
-    # reference's large test shape, where ~20% of the buckets are empty
+    # reference's large test shape, where ~20% of the buckets are empty; one bucket with 3000 queries
     if case == "ragged":
         q, k, v, kh, cnt, qh = make_attn_case(31, 2, 900, 5000, 24, 333, 128, torch.bfloat16, std=0.7)
     elif case == "full-items":
@@ -275,6 +275,14 @@ def test_attention_grouped_forward_kernels(ops, which, case):
             qh[0, pos:pos + n] = b
             pos += n
         qh[0, pos:] = torch.randint(len(sizes), 40, (700 - pos,), generator=gen(33))
+    elif case == "heavy-bucket":
+        # most of a row's queries in one bucket (dozens of work items of the same bucket), a bucket of exactly
+        # 192 and one of 193 queries (the most a workgroup of the direct-load kernel takes, and one more)
+        q, k, v, kh, cnt, qh = make_attn_case(34, 2, 3600, 3000, 12, 260, 128, torch.bfloat16, std=0.8)
+        qh[0, :3000] = 5
+        qh[0, 3000:3192] = 7
+        qh[0, 3192:3385] = 2
+        qh[0, 3385:] = torch.randint(8, 12, (3600 - 3385,), generator=gen(35))
     else:
         q, k, v, kh, cnt, qh = make_attn_case(20, 1, 4 * 2040, 1023 * 60, 512, 1024, 128, torch.bfloat16)
         assert (cnt == 0).any()

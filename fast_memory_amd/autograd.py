@@ -138,17 +138,20 @@ _notbad_attention_hash_varlen.register_autograd(_notbad_backward, setup_context=
 _prefix_lists = {}
 
 
-def _causal_prefix_lists(H: int, S: int, L: int, causal: bool, device):
-    """Bucket lists that express the dense local attention as a gathered one: token t of every query head is
-    "hashed" to bucket t, whose list is the keys it may see, 0 .. t + (L - S) (all L keys without the causal
-    mask, one bucket).  Kept per shape."""
-    key = (H, S, L, bool(causal), str(device))
+_PREFIX_CHUNK_ENTRIES = 1 << 24   # list entries per KV head and call of the gathered backward (64 MiB of int32)
+
+
+def _causal_prefix_lists(H: int, t0: int, t1: int, S: int, L: int, causal: bool, device):
+    """Bucket lists that express the dense local attention of tokens t0 .. t1-1 as a gathered one: token t of
+    every query head is "hashed" to bucket t - t0, whose list is the keys it may see, 0 .. t + (L - S) (all L
+    keys without the causal mask, one bucket).  The last one built is kept."""
+    key = (H, t0, t1, S, L, bool(causal), str(device))
     if key not in _prefix_lists:
         if causal:
-            lim = (torch.arange(S, device=device) + (L - S + 1)).clamp(min=0, max=L)          # keys seen by token t
+            lim = (torch.arange(t0, t1, device=device) + (L - S + 1)).clamp(min=0, max=L)    # keys seen by token t
             j = torch.arange(L, device=device)
-            flat1 = j.expand(S, L)[j[None, :] < lim[:, None]].to(torch.int32)                # row-major (t, key)
-            cnt = lim.to(torch.int32).unsqueeze(0).expand(H, S).contiguous()
+            flat1 = j.expand(t1 - t0, L)[j[None, :] < lim[:, None]].to(torch.int32)          # row-major (t, key)
+            cnt = lim.to(torch.int32).unsqueeze(0).expand(H, t1 - t0).contiguous()
         else:
             flat1 = torch.arange(L, device=device, dtype=torch.int32)
             cnt = torch.full((H, 1), L, dtype=torch.int32, device=device)
@@ -165,18 +168,30 @@ def local_attention_backward(d_out, q, k, v, out, lse, sm_scale: float, causal: 
     ``(dq [H*G,S,d], dk, dv [H,L,d] fp32)``.
 
     The causal prefix of every token is a list of keys, so this is the backward of the gathered attention
-    with one bucket per token (shared by the G query heads of a KV head): no kernel of its own."""
+    with one bucket per token (shared by the G query heads of a KV head): no kernel of its own.  The lists
+    hold S (L - S/2) entries per KV head, so the tokens are taken in chunks that keep a call's lists below
+    2^24 entries per head (one call up to S = L = 4096); dk and dv add up over the calls."""
     HG, S, d = q.shape
     H, L, _ = k.shape
     G = HG // H
-    flat, cnt = _causal_prefix_lists(H, S, L, causal, q.device)
-    t = torch.arange(S, device=q.device, dtype=torch.int32) if causal else torch.zeros(S, dtype=torch.int32,
-                                                                                      device=q.device)
-    qh = t.repeat(H * G).reshape(H, G * S)                                                    # query g*S + t -> t
-    dq, dk, dv = attention_hash_varlen_backward(
-        d_out.reshape(H, G * S, d).contiguous(), q.reshape(H, G * S, d).contiguous(), k.contiguous(), v.contiguous(),
-        out.reshape(H, G * S, d).to(q.dtype).contiguous(), lse.reshape(H, G * S).float().contiguous(), flat, cnt, qh,
-        sm_scale, staged=False)
+    dev = q.device
+    q4, do4 = q.reshape(H, G, S, d), d_out.reshape(H, G, S, d)
+    o4, l4 = out.reshape(H, G, S, d), lse.reshape(H, G, S)
+    k, v = k.contiguous(), v.contiguous()
+    T = S if not causal else max(64, min(S, _PREFIX_CHUNK_ENTRIES // max(L, 1)))
+    dq = torch.empty((H, G, S, d), dtype=q.dtype, device=dev)
+    dk = dv = None
+    for t0 in range(0, S, T):
+        t1 = min(S, t0 + T)
+        n = t1 - t0
+        flat, cnt = _causal_prefix_lists(H, t0, t1, S, L, causal, dev)
+        t = torch.arange(n, device=dev, dtype=torch.int32) if causal else torch.zeros(n, dtype=torch.int32, device=dev)
+        qh = t.repeat(H * G).reshape(H, G * n)                                                # query g*n + t -> t
+        sl = lambda x: x[:, :, t0:t1].reshape(H, G * n, *x.shape[3:]).contiguous()
+        dq_c, dk_c, dv_c = attention_hash_varlen_backward(
+            sl(do4), sl(q4), k, v, sl(o4).to(q.dtype), sl(l4).float(), flat, cnt, qh, sm_scale, staged=False)
+        dq[:, :, t0:t1] = dq_c.reshape(H, G, n, d)
+        dk, dv = (dk_c, dv_c) if dk is None else (dk + dk_c, dv + dv_c)
     return dq.reshape(HG, S, d), dk, dv
 
 

@@ -140,10 +140,13 @@ def test_module_forward_backward_against_joint_softmax():
         assert err <= 2e-4, f"{name}: max err {err:.3e}"
 
 
-def test_local_attention_backward_bf16():
-    from fast_memory_amd import local_attention_backward, ops as _ops
+@pytest.mark.parametrize("S,L,chunk_entries", [(40, 56, None), (200, 200, 64 * 200)])   # one call; token chunks of 64
+def test_local_attention_backward_bf16(S, L, chunk_entries, monkeypatch):
+    from fast_memory_amd import autograd as fm_autograd, local_attention_backward, ops as _ops
+    if chunk_entries:
+        monkeypatch.setattr(fm_autograd, "_PREFIX_CHUNK_ENTRIES", chunk_entries)
     g = gen(8400)
-    H, G, S, L, d = 2, 4, 40, 56, 128
+    H, G, d = 2, 4, 128
     q = (torch.randn(H * G, S, d, generator=g) * 0.6).to(torch.bfloat16)
     k = (torch.randn(H, L, d, generator=g) * 0.6).to(torch.bfloat16)
     v = (torch.randn(H, L, d, generator=g) * 0.6).to(torch.bfloat16)

@@ -91,12 +91,13 @@ def cpu_timed(fn, reps=3):
     return ts[len(ts) // 2], ts
 
 
-def no_reuse_control(dev, reps=3):
+def no_reuse_control(dev, reps=3, list_order="key"):
     """fm_hash_attn_fwd on lists that name every key and value row exactly once: H = 8 rows of N = 2^24 keys,
     C = 1024 buckets of Z = 16384 keys = a seeded permutation of the keys, 16 queries per bucket (c5's
     average).  K and V are 69 GB, far beyond the 256 MB last-level cache, and no row is listed twice, so
     every gathered byte comes from HBM: the rate the gather kernel reaches here is an HBM rate, which the
-    c5 figure (every key listed in ~32 buckets) is not."""
+    c5 figure (every key listed in ~32 buckets) is not.  Timed with the lists in the order the step reads
+    them (``list_order``) and, beside it, in the other one."""
     from fast_memory_amd import ops
     H, C, Z, d, per_bucket = 8, 1024, 16384, 128, 16
     N, Sq = C * Z, per_bucket * C
@@ -109,17 +110,25 @@ def no_reuse_control(dev, reps=3):
     cnt = torch.full((H, C), Z, dtype=torch.int32, device=dev)
     off = ops.bucket_offsets(cnt)
     groups = ops.group_queries(qh, C)
-    run = lambda: ops.hash_attn_fwd(q, k, v, lists.reshape(-1), off, cnt, groups, d ** -0.5)
-    ms = min(timed(run, reps=1, warm=1 if i == 0 else 0)[0] for i in range(reps))
-    out, lse = run()
-    assert bool(torch.isfinite(lse).all())
     alg = H * C * Z * (2 * d * 2 + 4) + H * Sq * (2 * d * 2 + 4)
     res = {"kernel": ops.hash_attn_fwd_kernel_name(H, Sq, N, d, C, torch.bfloat16),
            "workload": f"H={H}, N=2^24 keys/head (K+V {2 * H * N * d * 2 / 1e9:.1f} GB), C={C}, Z={Z}: lists = a "
                        f"seeded permutation, every row listed once; {per_bucket} queries per bucket",
-           "algorithmic_bytes_per_launch": alg, "launch_ms": ms, "gbs": alg / ms / 1e6,
-           "hbm_frac": alg / ms / 1e6 / HBM_PEAK_GBS}
-    del k, v, lists, q, out, lse
+           "algorithmic_bytes_per_launch": alg}
+    flat = lists.reshape(-1)
+    for order in ("value", "key"):          # as the permutation fell (what score order amounts to), then sorted
+        if order == "key":
+            flat = ops.lists_key_order(flat, off.reshape(-1), cnt.reshape(-1), N)
+        run = lambda: ops.hash_attn_fwd(q, k, v, flat, off, cnt, groups, d ** -0.5)
+        ms = min(timed(run, reps=1, warm=1 if i == 0 else 0)[0] for i in range(reps))
+        out, lse = run()
+        assert bool(torch.isfinite(lse).all())
+        if order == list_order:
+            res.update({"list_order": order, "launch_ms": ms, "gbs": alg / ms / 1e6,
+                        "hbm_frac": alg / ms / 1e6 / HBM_PEAK_GBS})
+        else:
+            res["other_list_order"] = {"list_order": order, "launch_ms": ms, "gbs": alg / ms / 1e6}
+    del k, v, lists, flat, q, out, lse
     torch.cuda.empty_cache()
     return res
 
@@ -409,6 +418,9 @@ def main():
     ap.add_argument("--workspace-gib", type=float, default=8.0)
     ap.add_argument("--tk-dtype", default="fp16", choices=["fp16", "bf16"],
                     help="element type of --config tkperf (the reference's harness runs fp16)")
+    ap.add_argument("--list-order", default="key", choices=["key", "value"],
+                    help="order of a bucket's list as the gathered attention reads it: ascending key index (the "
+                         "copy Memory keeps for its attention) or descending score as torch.topk leaves it")
     ap.add_argument("--no-control", action="store_true",
                     help="skip the no-reuse control of the attention roofline (69 GB of K and V listed once)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -499,6 +511,11 @@ def main():
         f"{build_parts['argtopz']['hbm_gbs']:.0f} GB/s (algorithmic)")
 
     q = wl.queries
+    # the lists as the attention reads them: Memory's copy in ascending key order (made once per index)
+    ko_ms, _ = timed(lambda: ops.lists_key_order(mem.bucket_idx.reshape(-1), mem.bucket_off.reshape(-1),
+                                                 mem.bucket_cnt.reshape(-1), N), reps=2, warm=1)
+    attn_lists = mem.attention_lists(Sq) if args.list_order == "key" else mem.bucket_idx.reshape(-1)
+    log(f"[bench] lists in key order: {ko_ms:.2f} ms (once per index); the step reads them in {args.list_order} order")
     has_local = wl.k_local is not None
     attn_events = []
     part_events = {"qhash": [], "group": [], "local": [], "merge": []}
@@ -513,7 +530,7 @@ def main():
         g1.record()
         a0, a1 = ev_pair()
         a0.record()
-        mo, ml = ops.hash_attn_fwd(q, mem.keys, mem.values, mem.bucket_idx.reshape(-1), mem.bucket_off,
+        mo, ml = ops.hash_attn_fwd(q, mem.keys, mem.values, attn_lists, mem.bucket_off,
                                    mem.bucket_cnt, groups, sm_scale)
         a1.record()
         if has_local:
@@ -563,7 +580,7 @@ def main():
         dout = torch.randn_like(mo)
         dkb = torch.zeros(mem.keys.shape, dtype=torch.float32, device=dev)
         dvb = torch.zeros_like(dkb)
-        run_bwd = lambda: ops.hash_attn_bwd(q, mem.keys, mem.values, mem.bucket_idx.reshape(-1), mem.bucket_off,
+        run_bwd = lambda: ops.hash_attn_bwd(q, mem.keys, mem.values, attn_lists, mem.bucket_off,
                                             mem.bucket_cnt, groups, mo, ml, dout, sm_scale, dkb, dvb)
         bwd_ms, _ = timed(run_bwd, reps=2, warm=1)
         n_tiles = int(((groups.bin_count + 15) // 16).sum().item())       # 16-query tiles, each sweeps its bucket
@@ -576,7 +593,7 @@ def main():
             f"({backward['atomic']['atomic_gbs']:.0f} GB/s of atomic adds)")
         if d == 128 and e == 2:
             # without atomics: per-bucket partial rows + a sum per key over the inverted lists
-            lists = mem.bucket_idx.reshape(-1)
+            lists = attn_lists
             inv_ms, inv = timed(lambda: ops.inverse_index(lists, mem.bucket_off, mem.bucket_cnt, N), reps=1, warm=1)
             run_st = lambda: ops.hash_attn_bwd_staged(q, mem.keys, mem.values, lists, mem.bucket_off, mem.bucket_cnt,
                                                       groups, inv, mo, ml, dout, sm_scale, dkb, dvb)
@@ -608,7 +625,7 @@ def main():
                 "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms,
-                "hit_buckets": hit, "mfma_tflops": alg_flops / attn_ms / 1e9}
+                "hit_buckets": hit, "mfma_tflops": alg_flops / attn_ms / 1e9, "list_order": args.list_order}
     log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M {'keys/s' if args.config == 'c4' else 'query-heads/s'}"
         f"; attention kernel "
         f"{attn_ms:.2f} ms = {achieved:.0f} GB/s algorithmic ({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak); "
@@ -627,8 +644,19 @@ def main():
     log(f"[bench] streaming-read probe: {read_ceiling:.0f} GB/s; attention kernel at "
         f"{100 * achieved / read_ceiling:.1f}% of it")
 
+    if not args.no_control:
+        # the same launch over the lists in the other order (descending score, as torch.topk leaves them, is a
+        # random key order), for scale
+        other_lists = mem.bucket_idx.reshape(-1) if args.list_order == "key" else mem.attention_lists(Sq)
+        other_ms = min(timed(lambda: ops.hash_attn_fwd(q, mem.keys, mem.values, other_lists, mem.bucket_off,
+                                                       mem.bucket_cnt, groups, sm_scale), reps=2, warm=1)[0]
+                       for _ in range(2))
+        roofline["other_list_order"] = {"list_order": "value" if args.list_order == "key" else "key",
+                                        "launch_ms": other_ms, "gbs": alg_bytes / other_ms / 1e6}
+        log(f"[bench] the same launch over lists in {roofline['other_list_order']['list_order']} order: "
+            f"{other_ms:.2f} ms")
     if not args.no_control and args.config == "c5":
-        ctl = no_reuse_control(dev)
+        ctl = no_reuse_control(dev, list_order=args.list_order)
         roofline["no_reuse_control"] = ctl
         log(f"[bench] no-reuse control ({ctl['kernel']}): {ctl['launch_ms']:.2f} ms = {ctl['gbs']:.0f} GB/s "
             f"({100 * ctl['hbm_frac']:.1f}% of HBM peak) with every K/V row read once from HBM")
@@ -718,7 +746,8 @@ def main():
         "cpu_baseline": cpu,
         "index_build": {"keys_per_s": keys_per_s, "ms": build_ms, "keys": H * N, "path": build_path,
                         "fused_phases_ms": fused_phases, "unfused_parts": build_parts,
-                        "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters, "append": append},
+                        "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters, "append": append,
+                        "lists_key_order_ms": ko_ms},
         "query_path": query_path,
         "step_parts_ms": {"attention": attn_ms, **parts_ms},
         "backward": backward,

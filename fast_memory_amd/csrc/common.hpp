@@ -113,6 +113,18 @@ __device__ __forceinline__ int wave_incl_scan(int v) {
   }
   return v;
 }
+// The same scan on the data-parallel-primitive path of the VALU (no LDS-pipe permutes): shifts within the
+// 16-lane rows, then the last lane of row 0 / 2 into row 1 / 3 and lane 31 into the upper half.  Lanes
+// without a source add 0.  All 64 lanes must be active.
+__device__ __forceinline__ int wave_incl_scan_dpp(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
 __device__ __forceinline__ long long wave_incl_scan_ll(long long v) {
   int l = lane_id();
 #pragma unroll

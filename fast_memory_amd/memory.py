@@ -215,17 +215,25 @@ class Memory:
     capacity.  ``attend`` returns the attention over the hashed bucket and its
     log-sum-exp so the caller can merge it with attention over other keys
     (``merge`` / ``update_out_and_lse``).
+
+    ``bucket_idx [H,C,L]`` are the lists as ``torch.topk`` orders them (memory.py:273, descending score).
+    With ``key_order`` (the default) the attention and its backward read a copy in ascending key order,
+    made the first time a call brings at least one query per bucket and kept until the lists change: the
+    result of the gathered softmax does not depend on the order of a list, the speed of the row gathers
+    does (:func:`ops.lists_key_order`).
     """
 
     def __init__(self, keys: torch.Tensor, values: torch.Tensor, A: torch.Tensor, bucket_idx: torch.Tensor,
-                 bucket_val: Optional[torch.Tensor] = None, Z: Optional[int] = None):
+                 bucket_val: Optional[torch.Tensor] = None, Z: Optional[int] = None, key_order: bool = True):
         self.keys, self.values, self.A = keys, values, A
         self.Z = int(Z) if Z is not None else bucket_idx.shape[2]       # capacity; lists are shorter while N < Z
+        self.key_order = bool(key_order)
         self._set_lists(bucket_idx, bucket_val)
 
     def _set_lists(self, bucket_idx: torch.Tensor, bucket_val: Optional[torch.Tensor]):
-        self.bucket_idx, self.bucket_val = bucket_idx, bucket_val
+        self.bucket_idx, self.bucket_val = bucket_idx.contiguous(), bucket_val
         self._inverse = None
+        self._attn_idx = None
         H, C, L = bucket_idx.shape
         dev = bucket_idx.device
         self.bucket_cnt = torch.full((H, C), L, dtype=torch.int32, device=dev)
@@ -233,15 +241,15 @@ class Memory:
 
     @classmethod
     def build(cls, keys: torch.Tensor, values: torch.Tensor, A: torch.Tensor, Z: int,
-              workspace_bytes: int = 8 << 30, keep_values: bool = False) -> "Memory":
+              workspace_bytes: int = 8 << 30, keep_values: bool = False, key_order: bool = True) -> "Memory":
         """``keep_values`` also stores the projections of the listed keys (4 bytes per list entry), which
-        :meth:`append` needs."""
+        :meth:`append` needs; ``key_order`` as in the class description."""
         keys, values, A = keys.contiguous(), values.contiguous(), A.contiguous()
         assert keys.shape == values.shape and A.shape[0] == keys.shape[0] and A.shape[2] == keys.shape[2]
         if keep_values:
             idx, val = ops.build_index(A, keys, Z, workspace_bytes, return_values=True)
-            return cls(keys, values, A, idx, val, Z)
-        return cls(keys, values, A, ops.build_index(A, keys, Z, workspace_bytes), None, Z)
+            return cls(keys, values, A, idx, val, Z, key_order)
+        return cls(keys, values, A, ops.build_index(A, keys, Z, workspace_bytes), None, Z, key_order)
 
     def append(self, new_keys: torch.Tensor, new_values: torch.Tensor, workspace_bytes: int = 8 << 30) -> "Memory":
         """Add keys/values ``[H,M,d]`` at the end of the memory and bring the bucket lists to what a rebuild
@@ -261,6 +269,7 @@ class Memory:
         if res[0] is not self.bucket_idx:
             self._set_lists(*res)
         self._inverse = None          # the lists changed (possibly in place)
+        self._attn_idx = None
         return self
 
     def save(self, path: str) -> None:
@@ -288,20 +297,30 @@ class Memory:
         """q ``[H,Sq,d]`` -> bucket ids ``[H,Sq]`` int32."""
         return ops.qhash(self.A, q.contiguous())
 
+    def attention_lists(self, n_queries: int = 0) -> torch.Tensor:
+        """The flat lists the attention reads: the copy in ascending key order once it exists; a call with at
+        least one query per bucket (``n_queries >= C``) makes it, fewer queries do not repay the reordering
+        and read ``bucket_idx`` as it is."""
+        if self._attn_idx is None and self.key_order and n_queries >= self.n_buckets:
+            self._attn_idx = ops.lists_key_order(self.bucket_idx.reshape(-1), self.bucket_off.reshape(-1),
+                                                 self.bucket_cnt.reshape(-1), self.keys.shape[1])
+            self._inverse = None      # positions in the lists changed
+        return self._attn_idx if self._attn_idx is not None else self.bucket_idx.reshape(-1)
+
     def attend(self, q: torch.Tensor, sm_scale: float, q_hash: Optional[torch.Tensor] = None):
         """q ``[H,Sq,d]`` (Sq = G*S, query head h*G+g) -> ``(out [H,Sq,d], lse [H,Sq] fp32)``."""
         q = q.contiguous()
         if q_hash is None:
             q_hash = self.hash(q)
         groups = ops.group_queries(q_hash, self.n_buckets)
-        return ops.hash_attn_fwd(q, self.keys, self.values, self.bucket_idx.reshape(-1), self.bucket_off,
+        return ops.hash_attn_fwd(q, self.keys, self.values, self.attention_lists(q.shape[1]), self.bucket_off,
                                  self.bucket_cnt, groups, sm_scale)
 
     def inverse_index(self) -> "ops.InverseIndex":
-        """For every key the list positions that name it (kept until the lists change); the backward without
-        atomics sums a key's gradient contributions over them."""
+        """For every key the positions of :meth:`attention_lists` that name it (kept until those change); the
+        backward without atomics sums a key's gradient contributions over them."""
         if getattr(self, "_inverse", None) is None:
-            self._inverse = ops.inverse_index(self.bucket_idx.reshape(-1), self.bucket_off, self.bucket_cnt,
+            self._inverse = ops.inverse_index(self.attention_lists(), self.bucket_off, self.bucket_cnt,
                                               self.keys.shape[1])
         return self._inverse
 
@@ -315,7 +334,7 @@ class Memory:
         if q_hash is None:
             q_hash = self.hash(q)
         groups = ops.group_queries(q_hash, self.n_buckets)
-        lists = self.bucket_idx.reshape(-1)
+        lists = self.attention_lists(q.shape[1])
         can_stage = q.dtype == torch.bfloat16 and q.shape[2] == 128
         auto = staged is None
         if auto:

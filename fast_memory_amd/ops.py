@@ -231,6 +231,23 @@ def hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, s
     return out, lse
 
 
+def lists_key_order(k_idx, bucket_off, bucket_cnt, N: int, return_unsorted: bool = False):
+    """The flat lists ``k_idx`` with every bucket's entries in ascending key order (same ``bucket_off`` /
+    ``bucket_cnt``): the order in which :func:`hash_attn_fwd` and the backward read K and V fastest when many
+    queries are served (their results do not depend on the order beyond fp32 rounding; the kernel of
+    triton_kernel.py:230-272 takes the lists as stored).  A list that repeats a key or names one outside
+    ``[0, N)`` is copied unchanged; with ``return_unsorted`` also the device counter ``[1]`` of such lists."""
+    _dev(k_idx, bucket_off, bucket_cnt)
+    assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and bucket_off.dtype == torch.int64
+    assert k_idx.is_contiguous() and bucket_off.is_contiguous() and bucket_cnt.is_contiguous()
+    assert bucket_off.numel() == bucket_cnt.numel()
+    out = torch.empty_like(k_idx)
+    n_uns = torch.empty(1, dtype=torch.int32, device=k_idx.device) if return_unsorted else None
+    check(_lib.load().fm_lists_key_order(_p(k_idx), _p(bucket_off), _p(bucket_cnt), bucket_cnt.numel(), int(N),
+                                         _p(out), _p(n_uns) if n_uns is not None else None, _stream(k_idx)))
+    return (out, n_uns) if return_unsorted else out
+
+
 def hash_attn_bwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, out, lse, dout, sm_scale: float,
                   dk: Optional[torch.Tensor] = None, dv: Optional[torch.Tensor] = None,
                   dlse: Optional[torch.Tensor] = None):

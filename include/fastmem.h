@@ -157,6 +157,21 @@ int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t*
                      float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype,
                      void* stream);
 
+/* ---- lists in ascending key order, for the gathered attention ------------------
+ * The kernel of triton_kernel.py:230-272 walks a bucket's list in stored order, and
+ * softmax(q.K^T).V over a list does not depend on that order (only the rounding of
+ * the fp32 sums does).  torch.topk (memory.py:273) leaves the lists in descending
+ * score order, which is a random key order; in ascending key order a 64-key tile
+ * reads neighbouring pages of K and V, which makes fm_hash_attn_fwd and the
+ * backward 10-20 % faster where many queries are served per build (nothing to gain
+ * for a single query per row).  Same flat layout in and out (bucket_off,
+ * bucket_cnt as for fm_hash_attn_fwd, n_lists of them; k_idx_out != k_idx); any
+ * list length.  A list that names a key twice or a key outside [0, N) is copied
+ * unchanged; n_unsorted [1] (device, may be NULL) receives the number of such
+ * lists.  The value-ordered lists stay the ones fm_index_append extends. */
+int fm_lists_key_order(const int32_t* k_idx, const int64_t* bucket_off, const int32_t* bucket_cnt,
+                       int64_t n_lists, int N, int32_t* k_idx_out, int32_t* n_unsorted, void* stream);
+
 /* ---- f1: backward of the bucket-gathered attention --------------------------
  * replaces ring_attention_masked_backward (memory.py:166-206), which forms the
  * dense [S, N] probability matrix; here only a query's bucket is visited.

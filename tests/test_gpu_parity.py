@@ -214,6 +214,91 @@ def test_bucket_offsets_and_window_filter(ops):
     assert torch.equal(flat[: rflat.numel()].cpu().long(), rflat)
 
 
+def _ragged_distinct_lists(g, n_lists, N, max_len):
+    """Flat ragged lists of distinct keys (each a random subset of [0, N)), offsets, counts."""
+    cnt = torch.randint(0, max_len + 1, (n_lists,), generator=g).int()
+    cnt[0], cnt[-1] = 0, max_len                       # an empty list and a longest one
+    if n_lists > 2:
+        cnt[1] = 1
+    lists = [torch.randperm(N, generator=g)[: int(c)].int() for c in cnt]
+    off = torch.zeros(n_lists, dtype=torch.int64)
+    off[1:] = torch.cumsum(cnt.long(), 0)[:-1]
+    return lists, off, cnt
+
+
+@pytest.mark.parametrize("n_lists,N,max_len", [(40, 1000, 700),            # one pass, 256 threads
+                                               (9, 262144, 5000),          # the largest single pass of the narrow form
+                                               (6, 262145, 70000),         # 512 threads, lists longer than FM_MAX_Z
+                                               (4, 600000, 20000),         # 1024 threads, one pass
+                                               (5, 3 * (1 << 20) + 77, 3000),   # four passes, ragged last range
+                                               (3, 33, 33)])               # every key listed, one bitmap word and a bit
+def test_lists_key_order(ops, n_lists, N, max_len):
+    g = gen(420 + n_lists)
+    max_len = min(max_len, N)
+    lists, off, cnt = _ragged_distinct_lists(g, n_lists, N, max_len)
+    flat = torch.cat(lists)
+    got, n_uns = ops.lists_key_order(dev(flat), dev(off), dev(cnt), N, return_unsorted=True)
+    ref = torch.cat([torch.sort(l).values for l in lists])
+    assert int(n_uns.item()) == 0
+    assert torch.equal(got.cpu(), ref)
+
+
+def test_lists_key_order_copies_lists_it_cannot_sort(ops):
+    """A list that names a key twice counts it twice in the softmax, and one with an entry outside [0, N) is
+    whatever the caller meant: both come back unchanged (and counted), the other lists sorted."""
+    g = gen(431)
+    N = 5000
+    lists, off, cnt = _ragged_distinct_lists(g, 12, N, 900)
+    lists[3] = torch.cat([lists[3][:10], lists[3][:10], torch.randperm(N, generator=g)[:50].int()])   # repeats
+    lists[7] = torch.cat([torch.tensor([N], dtype=torch.int32), torch.randperm(N, generator=g)[:20].int()])
+    lists[9] = torch.cat([torch.randperm(N, generator=g)[:20].int(), torch.tensor([-1], dtype=torch.int32)])
+    cnt = torch.tensor([l.numel() for l in lists], dtype=torch.int32)
+    off = torch.zeros(12, dtype=torch.int64)
+    off[1:] = torch.cumsum(cnt.long(), 0)[:-1]
+    flat = torch.cat(lists)
+    got, n_uns = ops.lists_key_order(dev(flat), dev(off), dev(cnt), N, return_unsorted=True)
+    ref = torch.cat([l if i in (3, 7, 9) else torch.sort(l).values for i, l in enumerate(lists)])
+    assert int(n_uns.item()) == 3
+    assert torch.equal(got.cpu(), ref)
+
+
+def test_memory_attends_over_key_ordered_lists(ops):
+    """Memory.attend reads a key-ordered copy of the lists once a call brings a query per bucket: the same
+    sets, bucket_idx untouched, the result that of the oracle on the lists as torch.topk orders them; a
+    memory built with key_order=False reads bucket_idx itself and agrees to rounding."""
+    from fast_memory_amd import Memory
+    g = gen(432)
+    H, C, N, d, Z, S = 2, 16, 6000, 128, 512, 300
+    K = (torch.randn(H, N, d, generator=g) * 0.5).to(torch.bfloat16)
+    V = (torch.randn(H, N, d, generator=g) * 0.5).to(torch.bfloat16)
+    A = torch.randn(H, C, d, generator=g).to(torch.bfloat16)
+    q = (torch.randn(H, S, d, generator=g) * 0.5).to(torch.bfloat16)
+    mem = Memory.build(*dev(K, V, A), Z, keep_values=True)
+    plain = Memory.build(*dev(K, V, A), Z, key_order=False)
+    idx0 = mem.bucket_idx.clone()
+    few = mem.attend(dev(q[:, :8]), d ** -0.5)            # fewer queries than buckets: no copy is made
+    assert mem._attn_idx is None
+    out, lse = mem.attend(dev(q), d ** -0.5)
+    assert mem._attn_idx is not None and torch.equal(mem.bucket_idx, idx0)
+    ko = mem._attn_idx.reshape(H, C, Z).cpu()
+    assert torch.equal(ko, torch.sort(idx0.cpu(), dim=-1).values)
+    qh = mem.hash(dev(q)).cpu().long()
+    ro, rl = O.hashed_attention_gather(q, K, V, idx0.cpu().long().reshape(-1), torch.full((H, C), Z), qh, d ** -0.5)
+    assert_attn_close(out, lse, ro, rl, torch.bfloat16, "key-ordered lists")
+    po, pl = plain.attend(dev(q), d ** -0.5)
+    assert plain._attn_idx is None
+    assert_attn_close(po, pl, ro, rl, torch.bfloat16, "value-ordered lists")
+    assert (out.float() - po.float()).abs().max().item() < 4e-3 and (lse - pl).abs().max().item() < 1e-4
+    o8, l8 = mem.attend(dev(q[:, :8]), d ** -0.5)         # the copy exists now and serves small calls too
+    assert torch.allclose(o8.float(), few[0].float(), atol=4e-3) and torch.allclose(l8, few[1], atol=1e-4)
+    # appending changes the lists: the copy is dropped and made again from the new ones
+    mem.append(*dev((torch.randn(H, 40, d, generator=g) * 0.5).to(torch.bfloat16),
+                    (torch.randn(H, 40, d, generator=g) * 0.5).to(torch.bfloat16)))
+    assert mem._attn_idx is None
+    mem.attend(dev(q), d ** -0.5)
+    assert torch.equal(mem._attn_idx.reshape(H, C, Z).cpu(), torch.sort(mem.bucket_idx.cpu(), dim=-1).values)
+
+
 # ------------------------------------------------------------------ a6-a8
 def run_varlen(q, k, v, kh, cnt, qh, scale):
     from fast_memory_amd import attention_hash_varlen

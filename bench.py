@@ -620,11 +620,13 @@ def main():
     alg_flops = 4.0 * d * Z * qheads
     achieved = alg_bytes / attn_ms / 1e6
     attn_kernel = ops.hash_attn_fwd_kernel_name(H, Sq, N, d, C, cfg.dtype)     # what the library's dispatch took
-    traffic = hbm_traffic(attn_kernel, cfg.name)
+    launches = ops.hash_attn_fwd_launches(H, Sq, N, d, C, cfg.dtype)           # one per row on large memories
+    traffic = hbm_traffic(attn_kernel, cfg.name)                               # per launch, as the profiler counts
     roofline = {"kernel": attn_kernel,
                 "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms,
+                "algorithmic_bytes_per_launch": alg_bytes / launches, "avg_launch_ms": attn_ms / launches,
+                "launches_per_step": launches, "algorithmic_bytes_per_step": alg_bytes, "launches_ms_per_step": attn_ms,
                 "hit_buckets": hit, "mfma_tflops": alg_flops / attn_ms / 1e9, "list_order": args.list_order}
     log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M {'keys/s' if args.config == 'c4' else 'query-heads/s'}"
         f"; attention kernel "

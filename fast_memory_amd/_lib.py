@@ -65,6 +65,7 @@ SIGNATURES = {
     "fm_segment_sum": (c_int, [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_debug_force_generic": (None, [c_int]),
     "fm_hash_attn_fwd_kernel": (ctypes.c_char_p, [c_int] * 6),
+    "fm_hash_attn_fwd_launches": (c_int, [c_int] * 6),
     "fm_build_index_fused_kernel": (ctypes.c_char_p, [c_int] * 6),
     "fm_debug_argtopz_exact_only": (None, [c_int]),
     "fm_debug_copy": (c_int, [P, P, c_int64, P]),

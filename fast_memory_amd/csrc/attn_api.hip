@@ -19,6 +19,7 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
                    float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype, hipStream_t st);
 int hash_attn_mfma_choice(int H, int Sq, int N, int C);
+bool hash_attn_mfma_per_row(int choice, int H, int Sq, int N, int C);
 bool local_attn_mfma_supported(int d, int dtype);
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
                     int S, int L, int d, float sm_scale, int causal, hipStream_t st);
@@ -51,6 +52,14 @@ extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int 
     case 3: return "hash_attn_ring_kernel";
     default: return "hash_attn_mfma_kernel";
   }
+}
+
+extern "C" int fm_hash_attn_fwd_launches(int H, int Sq, int N, int d, int C, int dtype) {
+  using namespace fm;
+  if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype, N)) return 1;
+  int choice = hash_attn_mfma_choice(H, Sq, N, C);
+  if (dtype == FM_F16 && choice == 0) choice = 1;
+  return hash_attn_mfma_per_row(choice, H, Sq, N, C) ? H : 1;
 }
 
 extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,

@@ -488,7 +488,8 @@ bool local_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM
 int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
                           const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                          float* lse, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, hipStream_t st);
+                          float* lse, int H, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, bool per_row,
+                          hipStream_t st);
 int hash_attn_mfma_ring(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                         const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items,
                         const int32_t* n_items, int64_t max_items, void* out, float* lse, int Sq, int N, int C,
@@ -510,13 +511,21 @@ extern std::atomic<int> g_force_generic;
 // (Beyond 2^24 keys the staged kernel runs in its form with 64-bit row offsets, one item per workgroup.)
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
   if (g_force_generic == 3) return 0;
-  if (g_force_generic == 2) return 1;
+  if (g_force_generic == 2 || g_force_generic == 6) return 1;
   if (g_force_generic == 4) return N <= (1 << 24) ? 2 : 1;
   if (g_force_generic == 5) return N <= (1 << 24) ? 3 : 1;
   const bool many_items = int64_t(H) * (Sq < C ? Sq : C) >= 512;
   const bool dense = Sq >= 24 * int64_t(C);
   if (!many_items && !dense) return 0;
   return (dense && N <= (1 << 24)) ? 3 : 1;
+}
+
+// The staged kernel, one item per workgroup, goes out in one launch per row once a row's K and V outgrow
+// the last-level cache (256 MB) and the row fills the device at least twice over (768 workgroups at a time).
+bool hash_attn_mfma_per_row(int choice, int H, int Sq, int N, int C) {
+  if (choice != 1 || g_force_generic == 2) return false;
+  if (g_force_generic == 6) return true;
+  return H > 1 && int64_t(N) * kD * 4 >= (int64_t(256) << 20) && (C < Sq ? C : Sq) >= 1536;
 }
 
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
@@ -529,9 +538,11 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
   if (choice == 3)
     return hash_attn_mfma_ring(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse, Sq,
                                N, C, sm_scale, dtype == FM_F16, st);
-  if (choice)
+  if (choice) {
+    const bool per_row = hash_attn_mfma_per_row(choice, H, Sq, N, C);
     return hash_attn_mfma_staged(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out,
-                                 lse, Sq, N, C, sm_scale, choice == 2, dtype == FM_F16, st);
+                                 lse, H, Sq, N, C, sm_scale, choice == 2, dtype == FM_F16, per_row, st);
+  }
   FM_ALLOW_LDS(hash_attn_mfma_kernel, kRedFloats * sizeof(float), "fm_hash_attn_fwd: lds");
   hipLaunchKernelGGL(hash_attn_mfma_kernel, dim3(unsigned(max_items)), dim3(256),
                      kRedFloats * sizeof(float), st, (const bf16_t*)q, (const bf16_t*)k,

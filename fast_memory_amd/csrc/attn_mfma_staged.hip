@@ -14,11 +14,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off,
     const int32_t* __restrict__ bucket_cnt, const int32_t* __restrict__ q_perm,
     const fm_item* __restrict__ items, const int32_t* __restrict__ n_items,
-    bf16_t* __restrict__ out, float* __restrict__ lse, int Sq, int N, int C, float scale2) {
+    bf16_t* __restrict__ out, float* __restrict__ lse, int Sq, int N, int C, float scale2, int only_row) {
   extern __shared__ __attribute__((aligned(16))) bf16_t st_lds[];
   const int n_it = *n_items;
-  if (int(blockIdx.x) >= n_it) return;
-  const fm_item it = items[blockIdx.x];
+  int item_id = blockIdx.x;
+  if (NQW == 1 && only_row >= 0) {
+    // a launch per row: workgroup j takes the row's j-th item.  The row's first item by a search every wave
+    // runs for itself, 64 probes a round (the items are in row order).
+    const int lane = threadIdx.x & 63;
+    int lo = 0, hi = n_it;  // the first item of a row >= only_row lies in [lo, hi]
+    while (hi > lo) {
+      const int step = (hi - lo + 63) >> 6;
+      const int probe = lo + lane * step;
+      const bool ge = probe >= hi || items[probe].row >= only_row;
+      const unsigned long long m = __ballot(ge);
+      const int f = m ? __ffsll(m) - 1 : 64;  // the first lane whose probe is at or past the row
+      hi = min(hi, lo + f * step);
+      lo = f == 0 ? hi : lo + (f - 1) * step + 1;
+    }
+    item_id += lo;
+    if (item_id >= n_it || items[item_id].row != only_row) return;
+  }
+  if (item_id >= n_it) return;
+  const fm_item it = items[item_id];
   int n_q = it.n_q;
   if (NQW == 2) {
     // the items of a bucket are consecutive and their queries contiguous: this workgroup takes items
@@ -53,18 +71,50 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 
                      out + qbase * kSD, lse + qbase, st_lds);
 }
 
+#define FM_STAGED_ROW_LAUNCH(F16, BIGN)                                                                              \
+  do {                                                                                                              \
+    FM_ALLOW_LDS((hash_attn_staged_kernel<1, F16, BIGN>), kStagedTileBytes, "fm_hash_attn_fwd: lds");               \
+    hipLaunchKernelGGL((hash_attn_staged_kernel<1, F16, BIGN>), dim3(unsigned(row_items)), dim3(256),               \
+                       kStagedTileBytes, st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx,           \
+                       bucket_off, bucket_cnt, q_perm, items, n_items, (bf16_t*)out, lse, Sq, N, C,                 \
+                       sm_scale * kLog2e, row);                                                                     \
+  } while (0)
+
 int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
                           const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                          float* lse, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, hipStream_t st) {
+                          float* lse, int H, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, bool per_row,
+                          hipStream_t st) {
   constexpr size_t kTileBytes = kStagedTileBytes;
+  if (per_row && !pairs) {
+    // One launch per row, in row order.  The workgroups of a launch start together and sweep the row's K
+    // and V at about the same pace (lists in ascending key order), so a key row that several buckets list
+    // is fetched from HBM once and found in the last-level cache, or the L2, by the others; in a single
+    // launch over all rows the starts spread over the whole sweep after a few rounds of workgroups and two
+    // rows' sweeps overlap at every row boundary.  Measured on 8 rows of 2^20 keys, 2048 buckets of 16384:
+    // 14.0 ms against 15.9 ms.
+    const int64_t row_items = std::min<int64_t>(max_items, int64_t(C < Sq ? C : Sq) + Sq / FM_QTILE + 1);
+    for (int row = 0; row < H; ++row) {
+      if (N > (1 << 24)) {
+        if (f16)
+          FM_STAGED_ROW_LAUNCH(true, true);
+        else
+          FM_STAGED_ROW_LAUNCH(false, true);
+      } else if (f16) {
+        FM_STAGED_ROW_LAUNCH(true, false);
+      } else {
+        FM_STAGED_ROW_LAUNCH(false, false);
+      }
+    }
+    return launch_status("fm_hash_attn_fwd(mfma, staged, per row)");
+  }
 #define FM_STAGED_LAUNCH(NQW, F16) FM_STAGED_LAUNCH3(NQW, F16, false)
 #define FM_STAGED_LAUNCH3(NQW, F16, BIGN)                                                                                   \
   do {                                                                                                               \
     FM_ALLOW_LDS((hash_attn_staged_kernel<NQW, F16, BIGN>), NQW * kTileBytes, "fm_hash_attn_fwd: lds");                     \
     hipLaunchKernelGGL((hash_attn_staged_kernel<NQW, F16, BIGN>), dim3(unsigned(max_items)), dim3(256), NQW * kTileBytes,  \
                        st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt,      \
-                       q_perm, items, n_items, (bf16_t*)out, lse, Sq, N, C, sm_scale * kLog2e);                      \
+                       q_perm, items, n_items, (bf16_t*)out, lse, Sq, N, C, sm_scale * kLog2e, -1);                  \
   } while (0)
   if (N > (1 << 24)) {  // 64-bit row offsets; one work item per workgroup only
     if (f16)
@@ -80,6 +130,7 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
   else
     FM_STAGED_LAUNCH(1, false);
 #undef FM_STAGED_LAUNCH
+#undef FM_STAGED_ROW_LAUNCH
 #undef FM_STAGED_LAUNCH3
   return launch_status("fm_hash_attn_fwd(mfma, staged)");
 }

@@ -511,13 +511,21 @@ def hash_attn_fwd_kernel_name(H: int, Sq: int, N: int, d: int, C: int, dtype: to
     return _lib.load().fm_hash_attn_fwd_kernel(H, Sq, N, d, C, _DT[dtype]).decode()
 
 
+def hash_attn_fwd_launches(H: int, Sq: int, N: int, d: int, C: int, dtype: torch.dtype) -> int:
+    """Number of launches of that kernel one :func:`hash_attn_fwd` call makes (one per row where a row's K
+    and V outgrow the last-level cache)."""
+    return int(_lib.load().fm_hash_attn_fwd_launches(H, Sq, N, d, C, _DT[dtype]))
+
+
 def grouped_forward_kernel(which: Optional[str]) -> None:
     """Diagnostic switch for the bf16 / fp16, d = 128 grouped attention forward: ``"staged"`` always takes the
-    kernel that shares a bucket's rows among its waves through LDS, one work item per workgroup,
-    ``"staged-pairs"`` the same kernel with two work items per workgroup, ``"ring"`` the kernel whose rows
-    go from global memory straight into LDS (three items per workgroup), ``"gather"`` always the kernel
-    that gathers the rows into registers, ``None`` restores the dispatch (staged unless the launch has few
-    and small work items; the direct loads from 64 queries per bucket on average)."""
+    kernel that shares a bucket's rows among its waves through LDS, one work item per workgroup, in a single
+    launch, ``"staged-per-row"`` the same in one launch per row, ``"staged-pairs"`` the same kernel with two
+    work items per workgroup, ``"ring"`` the kernel whose rows go from global memory straight into LDS (three
+    items per workgroup), ``"gather"`` always the kernel that gathers the rows into registers, ``None``
+    restores the dispatch (staged unless the launch has few and small work items, per row when a row's K
+    and V outgrow the last-level cache; the direct loads from 64 queries per bucket on average)."""
     global _generic_forced
     _generic_forced = False
-    _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4, "ring": 5}[which])
+    _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4, "ring": 5,
+                                         "staged-per-row": 6}[which])

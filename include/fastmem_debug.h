@@ -19,7 +19,9 @@ extern "C" {
 /* Diagnostic: 1 routes the attention entry points through the generic kernels
  * (used by tests to compare the two implementations), 0 restores dispatch.  For
  * fm_hash_attn_fwd on bf16 / fp16, d = 128 only: 2 = always the kernel that stages a
- * bucket's rows in LDS, one work item per workgroup, 4 = the same with two work
+ * bucket's rows in LDS, one work item per workgroup, in a single launch, 6 = the
+ * same in one launch per row (dispatch: when a row's K and V are 256 MB or more and
+ * the row has 1536 buckets and queries or more), 4 = the staged kernel with two work
  * items per workgroup, 5 = always the kernel that loads the rows straight into
  * LDS (three items per workgroup), 3 = always the kernel that gathers the rows
  * into registers (dispatch: staged when H min(Sq, C) >= 512 or Sq >= 24 C, the
@@ -34,6 +36,12 @@ void fm_debug_force_generic(int on);
  * workgroup); ", f16>" / "<f16>" marks the fp16 forms, "64-bit rows" the form for
  * memories of more than 2^24 keys.  bench.py names its roofline kernel with it. */
 const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype);
+
+/* Diagnostic: number of launches of that kernel one fm_hash_attn_fwd call makes for
+ * these extents: 1, or H where the staged kernel goes out once per row (a row's K
+ * and V of 256 MB or more, 1536 or more buckets and queries per row).  bench.py
+ * divides its event time and the algorithmic bytes by it. */
+int fm_hash_attn_fwd_launches(int H, int Sq, int N, int d, int C, int dtype);
 
 /* Diagnostic: name of the filter kernel fm_build_index_fused launches for these
  * extents (a static string): "fused_filter_kernel" (four waves over a slab of 256

@@ -97,3 +97,13 @@ def test_grouped_forward_dispatch_rule():
     assert name(8, 4096, 32768, 128, 256, 2) == "hash_attn_staged_kernel<1, f16>"     # fp16, 16 / bucket
     assert name(1, 64, 1 << 25, 128, 64, 1) == "hash_attn_mfma_kernel"                # few small items, any N
     assert name(1, 512, 4096, 64, 64, 0) == "hash_attn_generic_kernel"                # fp32 / d != 128
+    # launches per call: one per row where a row's K and V (256 MB and more) outgrow the last-level cache and
+    # the row fills the device twice over; one otherwise
+    launches = lib.fm_hash_attn_fwd_launches
+    assert launches(8, 32768, 1048576, 128, 2048, 1) == 8
+    assert launches(8, 32768, 1048576, 128, 2048, 2) == 8
+    assert launches(1, 32768, 1048576, 128, 2048, 1) == 1                             # a single row
+    assert launches(8, 16384, 262144, 128, 1024, 1) == 1                              # 128 MB per row
+    assert launches(8, 16384, 1 << 24, 128, 1024, 1) == 1                             # too few buckets per row
+    assert launches(8, 131072, 1048576, 128, 2048, 1) == 1                            # 64 queries / bucket: other kernel
+    assert launches(8, 32768, 1048576, 64, 2048, 0) == 1                              # generic kernels

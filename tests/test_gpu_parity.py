@@ -342,7 +342,7 @@ def test_attention_dense_buckets(dtype, d):
     assert_attn_close(out, lse, ro, rl, dtype, f"dense d={d}")
 
 
-@pytest.mark.parametrize("which", ["staged", "staged-pairs", "ring", "gather"])
+@pytest.mark.parametrize("which", ["staged", "staged-per-row", "staged-pairs", "ring", "gather"])
 @pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large", "heavy-bucket"])
 def test_attention_grouped_forward_kernels(ops, which, case):
     # the bf16 d=128 forward kernels (rows shared through LDS, one or two work items per workgroup / rows
@@ -378,6 +378,50 @@ def test_attention_grouped_forward_kernels(ops, which, case):
         ops.grouped_forward_kernel(None)
     ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 128 ** -0.5)
     assert_attn_close(out, lse, ro, rl, torch.bfloat16, f"{which} {case}")
+    if which == "staged-per-row":
+        # a launch per row runs the same work items: bit-identical to the single launch (rows without any
+        # item, a row whose items end the list, a first item found in the middle of the item list)
+        ops.grouped_forward_kernel("staged")
+        try:
+            o1, l1 = run_varlen(q, k, v, kh, cnt, qh, 128 ** -0.5)
+        finally:
+            ops.grouped_forward_kernel(None)
+        assert torch.equal(out, o1) and torch.equal(lse, l1)
+
+
+def test_attention_a_launch_per_row_finds_every_rows_items(ops):
+    """Eleven rows with very different numbers of work items, among them rows whose queries all carry a hash
+    outside [0, C) (no item at all; their output rows are never written): the per-row launches write exactly
+    what the single launch writes."""
+    H, S, N, C, Z, d = 11, 520, 700, 37, 90, 128
+    q, k, v, kh, cnt, qh = make_attn_case(36, H, S, N, C, Z, d, torch.bfloat16, std=0.8)
+    qh[3] = -1
+    qh[10] = C + 5
+    qh[0] = 4                                   # one bucket, nine items
+    qh[5, :40] = torch.arange(40) % C           # the rest of row 5 in no bucket
+    qh[5, 40:] = -1
+    res = []
+    for which in ("staged", "staged-per-row"):
+        ops.grouped_forward_kernel(which)
+        try:
+            qd, kd, vd, khd, cntd, qhd = dev(q, k, v, kh, cnt, qh)
+            groups = ops.group_queries(qhd.int(), C)
+            off = ops.bucket_offsets(cntd.int())
+            out = torch.full(q.shape, 7.0, dtype=torch.bfloat16, device="cuda")
+            lse = torch.full((H, S), 7.0, dtype=torch.float32, device="cuda")
+            from fast_memory_amd import _lib
+            _lib.check(_lib.load().fm_hash_attn_fwd(
+                qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), khd.int().reshape(-1).contiguous().data_ptr(), off.data_ptr(),
+                cntd.int().contiguous().data_ptr(), groups.q_perm.data_ptr(), groups.items.data_ptr(),
+                groups.n_items.data_ptr(), groups.max_items, out.data_ptr(), lse.data_ptr(), H, S, N, d, C,
+                float(d ** -0.5), 1, torch.cuda.current_stream().cuda_stream))
+            sync()
+            res.append((out.clone(), lse.clone()))
+        finally:
+            ops.grouped_forward_kernel(None)
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    assert bool((res[1][1][3] == 7.0).all()) and bool((res[1][1][10] == 7.0).all())      # untouched rows
+    assert bool((res[1][1][0] != 7.0).all())
 
 
 @pytest.mark.parametrize("which", ["staged", "staged-pairs", "ring", "gather", "generic"])

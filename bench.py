@@ -91,13 +91,14 @@ def cpu_timed(fn, reps=3):
     return ts[len(ts) // 2], ts
 
 
-def no_reuse_control(dev, reps=3, list_order="key"):
+def no_reuse_control(dev, reps=3, list_order="key", force=None):
     """fm_hash_attn_fwd on lists that name every key and value row exactly once: H = 8 rows of N = 2^24 keys,
     C = 1024 buckets of Z = 16384 keys = a seeded permutation of the keys, 16 queries per bucket (c5's
     average).  K and V are 69 GB, far beyond the 256 MB last-level cache, and no row is listed twice, so
     every gathered byte comes from HBM: the rate the gather kernel reaches here is an HBM rate, which the
     c5 figure (every key listed in ~32 buckets) is not.  Timed with the lists in the order the step reads
-    them (``list_order``) and, beside it, in the other one."""
+    them (``list_order``) and, beside it, in the other one.  ``force`` (a name :func:`ops.grouped_forward_kernel`
+    takes) overrides the library's dispatch, which takes the kernel and the launch per row of c5 here too."""
     from fast_memory_amd import ops
     H, C, Z, d, per_bucket = 8, 1024, 16384, 128, 16
     N, Sq = C * Z, per_bucket * C
@@ -111,7 +112,9 @@ def no_reuse_control(dev, reps=3, list_order="key"):
     off = ops.bucket_offsets(cnt)
     groups = ops.group_queries(qh, C)
     alg = H * C * Z * (2 * d * 2 + 4) + H * Sq * (2 * d * 2 + 4)
+    ops.grouped_forward_kernel(force)
     res = {"kernel": ops.hash_attn_fwd_kernel_name(H, Sq, N, d, C, torch.bfloat16),
+           "launches": ops.hash_attn_fwd_launches(H, Sq, N, d, C, torch.bfloat16),
            "workload": f"H={H}, N=2^24 keys/head (K+V {2 * H * N * d * 2 / 1e9:.1f} GB), C={C}, Z={Z}: lists = a "
                        f"seeded permutation, every row listed once; {per_bucket} queries per bucket",
            "algorithmic_bytes_per_launch": alg}
@@ -128,6 +131,7 @@ def no_reuse_control(dev, reps=3, list_order="key"):
                         "hbm_frac": alg / ms / 1e6 / HBM_PEAK_GBS})
         else:
             res["other_list_order"] = {"list_order": order, "launch_ms": ms, "gbs": alg / ms / 1e6}
+    ops.grouped_forward_kernel(None)
     del k, v, lists, flat, q, out, lse
     torch.cuda.empty_cache()
     return res

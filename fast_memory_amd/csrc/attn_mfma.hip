@@ -493,7 +493,7 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
 int hash_attn_mfma_ring(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                         const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items,
                         const int32_t* n_items, int64_t max_items, void* out, float* lse, int Sq, int N, int C,
-                        float sm_scale, bool f16, hipStream_t st);
+                        float sm_scale, bool f16, int H, bool per_row, hipStream_t st);
 extern std::atomic<int> g_force_generic;
 
 // Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
@@ -502,30 +502,46 @@ extern std::atomic<int> g_force_generic;
 // that shares a bucket's rows through LDS is at least as fast as the register-gather one wherever the launch
 // has work items enough to fill the chip (at least 512, taking min(Sq, C) per row as their number) or buckets
 // receive 24 queries or more on average; with few and small items the four waves of the gather kernel, which
-// share one bucket's keys, finish an item sooner.  From 24 queries per bucket on average form 3, below that
-// form 1.  (On keys that stay in the last-level cache form 3 is ahead at every density measured: 65536 keys,
-// 1024 buckets of 3072, 16 / 32 / 64 / 128 queries per bucket: 1.51 / 1.57 / 1.69 / 2.51 ms against 1.54 /
-// 1.67 / 2.30 / 3.05 ms; on a million keys with 16 queries per bucket, where the rows come from HBM and what
-// counts is the bytes in flight, form 1 with its three workgroups per CU is 1 % ahead.  Form 2 stays for
-// tests to compare against.)
-// (Beyond 2^24 keys the staged kernel runs in its form with 64-bit row offsets, one item per workgroup.)
+// share one bucket's keys, finish an item sooner.  Of the LDS kernels form 3 wherever its 32-bit row offsets
+// reach (2^24 keys), form 1 in its form with 64-bit row offsets beyond.  Form 3 against form 1: on keys
+// that stay in the last-level cache (65536 keys, 1024 buckets of 3072, 16 / 32 / 64 / 128 queries per bucket)
+// 1.51 / 1.57 / 1.69 / 2.51 ms against 1.54 / 1.67 / 2.30 / 3.05 ms; on large memories with few queries per
+// bucket the two are level while the lists are in score order (a million keys, 16 queries per bucket: 17.9
+// against 17.8 ms) and form 3 is ahead once they are in key order (figures below).  Forms 1 and 2 stay for
+// the long memories and for tests to compare against.
+//
+// A launch per row, in row order, when K and V of all rows together are at least twice the last-level cache
+// (512 MB) and a row fills the device twice over (the direct-load kernel runs 512 workgroups at a time, the
+// staged one 768): with the lists in ascending key order the workgroups of a launch sweep the row's K and V
+// at about the same pace, and a key row that several buckets list is fetched from HBM once and found in the
+// last-level cache, or the L2, by the others; in a single launch over all rows the starts spread over the
+// whole sweep after a few rounds of workgroups and two rows' sweeps overlap at every row boundary.  Measured
+// (lists in key order; staged / direct loads in one launch, then per row): 8 rows of 2^20 keys, 2048 buckets
+// of 16384, 16 queries per bucket 15.9 / 14.6 / 14.0 / 12.3 ms; 8 rows of 2^18 keys, 1024 buckets of 4096, 8
+// queries per bucket 1.76 / 1.42 / 1.86 / 1.22 ms; 8 rows of 2^15 keys (134 MB in all), 256 buckets of 1024
+// 0.134 / 0.112 / 0.241 / 0.191 ms.
+static bool row_launches_pay(int choice, int H, int Sq, int N, int C) {
+  return H > 1 && int64_t(H) * N * kD * 4 >= (int64_t(512) << 20) && (C < Sq ? C : Sq) >= (choice == 3 ? 1024 : 1536);
+}
+
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
-  if (g_force_generic == 3) return 0;
-  if (g_force_generic == 2 || g_force_generic == 6) return 1;
-  if (g_force_generic == 4) return N <= (1 << 24) ? 2 : 1;
-  if (g_force_generic == 5) return N <= (1 << 24) ? 3 : 1;
+  const int force = g_force_generic;
+  if (force == 3) return 0;
+  if (force == 2 || force == 6) return 1;
+  if (force == 4) return N <= (1 << 24) ? 2 : 1;
+  if (force == 5 || force == 7) return N <= (1 << 24) ? 3 : 1;
   const bool many_items = int64_t(H) * (Sq < C ? Sq : C) >= 512;
   const bool dense = Sq >= 24 * int64_t(C);
   if (!many_items && !dense) return 0;
-  return (dense && N <= (1 << 24)) ? 3 : 1;
+  return N <= (1 << 24) ? 3 : 1;
 }
 
-// The staged kernel, one item per workgroup, goes out in one launch per row once a row's K and V outgrow
-// the last-level cache (256 MB) and the row fills the device at least twice over (768 workgroups at a time).
+// One launch per row (forms 1 and 3 only).
 bool hash_attn_mfma_per_row(int choice, int H, int Sq, int N, int C) {
-  if (choice != 1 || g_force_generic == 2) return false;
-  if (g_force_generic == 6) return true;
-  return H > 1 && int64_t(N) * kD * 4 >= (int64_t(256) << 20) && (C < Sq ? C : Sq) >= 1536;
+  const int force = g_force_generic;
+  if ((choice != 1 && choice != 3) || force == 2 || force == 5) return false;
+  if (force == 6 || force == 7) return true;
+  return row_launches_pay(choice, H, Sq, N, C);
 }
 
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
@@ -535,11 +551,11 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
   (void)d;
   int choice = hash_attn_mfma_choice(H, Sq, N, C);
   if (dtype == FM_F16 && choice == 0) choice = 1;
+  const bool per_row = hash_attn_mfma_per_row(choice, H, Sq, N, C);
   if (choice == 3)
     return hash_attn_mfma_ring(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse, Sq,
-                               N, C, sm_scale, dtype == FM_F16, st);
+                               N, C, sm_scale, dtype == FM_F16, H, per_row, st);
   if (choice) {
-    const bool per_row = hash_attn_mfma_per_row(choice, H, Sq, N, C);
     return hash_attn_mfma_staged(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out,
                                  lse, H, Sq, N, C, sm_scale, choice == 2, dtype == FM_F16, per_row, st);
   }

@@ -19,19 +19,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 - NQW, 4 
   const int n_it = *n_items;
   int item_id = blockIdx.x;
   if (NQW == 1 && only_row >= 0) {
-    // a launch per row: workgroup j takes the row's j-th item.  The row's first item by a search every wave
-    // runs for itself, 64 probes a round (the items are in row order).
-    const int lane = threadIdx.x & 63;
-    int lo = 0, hi = n_it;  // the first item of a row >= only_row lies in [lo, hi]
-    while (hi > lo) {
-      const int step = (hi - lo + 63) >> 6;
-      const int probe = lo + lane * step;
-      const bool ge = probe >= hi || items[probe].row >= only_row;
-      const unsigned long long m = __ballot(ge);
-      const int f = m ? __ffsll(m) - 1 : 64;  // the first lane whose probe is at or past the row
-      hi = min(hi, lo + f * step);
-      lo = f == 0 ? hi : lo + (f - 1) * step + 1;
-    }
+    // a launch per row: workgroup j takes the row's j-th item
+    const int lo = first_item_of_row(items, n_it, only_row);
     item_id += lo;
     if (item_id >= n_it || items[item_id].row != only_row) return;
   }

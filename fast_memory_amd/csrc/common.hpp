@@ -172,6 +172,24 @@ __device__ __forceinline__ long long block_excl_scan_ll(long long v, long long* 
   return res;
 }
 
+// Index of the first work item of a row >= `row` (n_it if there is none); the items are in row order.  A
+// search every wave runs for itself with all 64 lanes active, 64 probes a round: three rounds of
+// dependent loads for 2^18 items.
+__device__ __forceinline__ int first_item_of_row(const fm_item* __restrict__ items, int n_it, int row) {
+  const int lane = lane_id();
+  int lo = 0, hi = n_it;  // the answer lies in [lo, hi]
+  while (hi > lo) {
+    const int step = (hi - lo + 63) >> 6;
+    const int probe = lo + lane * step;
+    const bool ge = probe >= hi || items[probe].row >= row;
+    const unsigned long long m = __ballot(ge);
+    const int f = m ? __ffsll(m) - 1 : 64;  // the first lane whose probe is at or past the row
+    hi = min(hi, lo + f * step);
+    lo = f == 0 ? hi : lo + (f - 1) * step + 1;
+  }
+  return lo;
+}
+
 // Order-preserving map float -> uint32 (larger float <=> larger key);
 // -0 is folded onto +0 and every NaN becomes the largest key.
 __device__ __forceinline__ uint32_t float_key(float x) {

@@ -20,12 +20,13 @@ extern "C" {
  * (used by tests to compare the two implementations), 0 restores dispatch.  For
  * fm_hash_attn_fwd on bf16 / fp16, d = 128 only: 2 = always the kernel that stages a
  * bucket's rows in LDS, one work item per workgroup, in a single launch, 6 = the
- * same in one launch per row (dispatch: when a row's K and V are 256 MB or more and
- * the row has 1536 buckets and queries or more), 4 = the staged kernel with two work
- * items per workgroup, 5 = always the kernel that loads the rows straight into
- * LDS (three items per workgroup), 3 = always the kernel that gathers the rows
- * into registers (dispatch: staged when H min(Sq, C) >= 512 or Sq >= 24 C, the
- * direct loads from Sq >= 64 C; gather otherwise). */
+ * same in one launch per row; 4 = the staged kernel with two work items per
+ * workgroup; 5 = always the kernel that loads the rows straight into LDS (three
+ * items per workgroup), in a single launch, 7 = the same in one launch per row;
+ * 3 = always the kernel that gathers the rows into registers.  Dispatch: gather
+ * when H min(Sq, C) < 512 and Sq < 24 C; else the direct loads up to 2^24 keys and
+ * the staged kernel beyond; one launch per row when K and V of all rows are 512 MB
+ * or more and a row has 1024 (staged kernel: 1536) or more buckets and queries. */
 void fm_debug_force_generic(int on);
 
 /* Diagnostic: name of the kernel fm_hash_attn_fwd launches for these extents
@@ -38,8 +39,7 @@ void fm_debug_force_generic(int on);
 const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype);
 
 /* Diagnostic: number of launches of that kernel one fm_hash_attn_fwd call makes for
- * these extents: 1, or H where the staged kernel goes out once per row (a row's K
- * and V of 256 MB or more, 1536 or more buckets and queries per row).  bench.py
+ * these extents: 1, or H where the kernel goes out once per row (see above).  bench.py
  * divides its event time and the algorithmic bytes by it. */
 int fm_hash_attn_fwd_launches(int H, int Sq, int N, int d, int C, int dtype);
 

@@ -87,23 +87,30 @@ def test_grouped_forward_dispatch_rule():
     # host-only: which kernel fm_hash_attn_fwd would launch (H, Sq, N, d, C, dtype)
     lib = _lib.load()
     name = lambda *a: lib.fm_hash_attn_fwd_kernel(*a).decode()
-    assert name(8, 32768, 1048576, 128, 2048, 1) == "hash_attn_staged_kernel<1>"      # 1 M keys, 16 queries / bucket
+    assert name(8, 32768, 1048576, 128, 2048, 1) == "hash_attn_ring_kernel"           # 1 M keys, 16 queries / bucket
+    assert name(8, 16384, 262144, 128, 1024, 1) == "hash_attn_ring_kernel"            # 256 K keys, 16 queries / bucket
+    assert name(8, 32768, (1 << 24) + 64, 128, 2048, 1) == "hash_attn_staged_kernel<1, 64-bit rows>"
     assert name(8, 8192, 32768, 128, 256, 1) == "hash_attn_ring_kernel"               # prefill chunk, 32 / bucket
     assert name(8, 131072, 65536, 128, 1024, 1) == "hash_attn_ring_kernel"       # reference harness, 128 / bucket
     assert name(1, 64, 262144, 128, 64, 1) == "hash_attn_mfma_kernel"                 # few, small work items
     assert name(1, 2048, 262144, 128, 64, 1) == "hash_attn_ring_kernel"               # few buckets, many queries each
     assert name(8, 8192, 1 << 25, 128, 256, 1) == "hash_attn_staged_kernel<1, 64-bit rows>"   # beyond 32-bit byte offsets
     assert name(8, 8192, 32768, 128, 256, 2) == "hash_attn_ring_kernel<f16>"          # fp16 (FM_F16 = 2)
-    assert name(8, 4096, 32768, 128, 256, 2) == "hash_attn_staged_kernel<1, f16>"     # fp16, 16 / bucket
+    assert name(8, 4096, 32768, 128, 256, 2) == "hash_attn_ring_kernel<f16>"          # fp16, 16 / bucket
     assert name(1, 64, 1 << 25, 128, 64, 1) == "hash_attn_mfma_kernel"                # few small items, any N
     assert name(1, 512, 4096, 64, 64, 0) == "hash_attn_generic_kernel"                # fp32 / d != 128
-    # launches per call: one per row where a row's K and V (256 MB and more) outgrow the last-level cache and
-    # the row fills the device twice over; one otherwise
+    # launches per call: one per row where K and V of all rows are 512 MB or more and a row fills the device
+    # twice over; one otherwise
     launches = lib.fm_hash_attn_fwd_launches
     assert launches(8, 32768, 1048576, 128, 2048, 1) == 8
     assert launches(8, 32768, 1048576, 128, 2048, 2) == 8
     assert launches(1, 32768, 1048576, 128, 2048, 1) == 1                             # a single row
-    assert launches(8, 16384, 262144, 128, 1024, 1) == 1                              # 128 MB per row
-    assert launches(8, 16384, 1 << 24, 128, 1024, 1) == 1                             # too few buckets per row
-    assert launches(8, 131072, 1048576, 128, 2048, 1) == 1                            # 64 queries / bucket: other kernel
+    assert launches(8, 16384, 262144, 128, 1024, 1) == 8                              # 1 GB in all
+    assert launches(8, 16384, 262144, 128, 512, 1) == 1                               # too few buckets per row
+    assert launches(8, 16384, (1 << 24) + 64, 128, 1024, 1) == 1                      # ... for the staged kernel
+    assert launches(8, 8192, 32768, 128, 256, 1) == 1                                 # 134 MB in all
+    assert launches(8, 131072, 1048576, 128, 2048, 1) == 8                            # 64 queries / bucket
+    assert launches(8, 32768, (1 << 24) + 64, 128, 2048, 1) == 8                      # staged kernel, 64-bit rows
+    assert launches(8, 131072, 65536, 128, 1024, 2) == 1                              # reference harness
     assert launches(8, 32768, 1048576, 64, 2048, 0) == 1                              # generic kernels
+    assert launches(1, 64, 1048576, 128, 64, 1) == 1                                  # few small items: gather kernel

@@ -342,7 +342,7 @@ def test_attention_dense_buckets(dtype, d):
     assert_attn_close(out, lse, ro, rl, dtype, f"dense d={d}")
 
 
-@pytest.mark.parametrize("which", ["staged", "staged-per-row", "staged-pairs", "ring", "gather"])
+@pytest.mark.parametrize("which", ["staged", "staged-per-row", "staged-pairs", "ring", "ring-per-row", "gather"])
 @pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large", "heavy-bucket"])
 def test_attention_grouped_forward_kernels(ops, which, case):
     # the bf16 d=128 forward kernels (rows shared through LDS, one or two work items per workgroup / rows
@@ -378,10 +378,10 @@ def test_attention_grouped_forward_kernels(ops, which, case):
         ops.grouped_forward_kernel(None)
     ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 128 ** -0.5)
     assert_attn_close(out, lse, ro, rl, torch.bfloat16, f"{which} {case}")
-    if which == "staged-per-row":
+    if which.endswith("-per-row"):
         # a launch per row runs the same work items: bit-identical to the single launch (rows without any
         # item, a row whose items end the list, a first item found in the middle of the item list)
-        ops.grouped_forward_kernel("staged")
+        ops.grouped_forward_kernel(which[:-len("-per-row")])
         try:
             o1, l1 = run_varlen(q, k, v, kh, cnt, qh, 128 ** -0.5)
         finally:
@@ -401,7 +401,7 @@ def test_attention_a_launch_per_row_finds_every_rows_items(ops):
     qh[5, :40] = torch.arange(40) % C           # the rest of row 5 in no bucket
     qh[5, 40:] = -1
     res = []
-    for which in ("staged", "staged-per-row"):
+    for which in ("staged", "staged-per-row", "ring", "ring-per-row"):
         ops.grouped_forward_kernel(which)
         try:
             qd, kd, vd, khd, cntd, qhd = dev(q, k, v, kh, cnt, qh)
@@ -420,8 +420,10 @@ def test_attention_a_launch_per_row_finds_every_rows_items(ops):
         finally:
             ops.grouped_forward_kernel(None)
     assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
-    assert bool((res[1][1][3] == 7.0).all()) and bool((res[1][1][10] == 7.0).all())      # untouched rows
-    assert bool((res[1][1][0] != 7.0).all())
+    assert torch.equal(res[2][0], res[3][0]) and torch.equal(res[2][1], res[3][1])
+    for _, lse_r in res:
+        assert bool((lse_r[3] == 7.0).all()) and bool((lse_r[10] == 7.0).all())           # untouched rows
+        assert bool((lse_r[0] != 7.0).all())
 
 
 @pytest.mark.parametrize("which", ["staged", "staged-pairs", "ring", "gather", "generic"])

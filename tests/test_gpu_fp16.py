@@ -82,7 +82,7 @@ def test_attention_forward_fp16_many_queries_per_bucket(ops):
     qh[0, pos:] = 7
     ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 128 ** -0.5)
     outs = {}
-    for which in ("staged-pairs", "ring"):
+    for which in ("staged-pairs", "ring", "ring-per-row", "staged-per-row"):
         ops.grouped_forward_kernel(which)
         try:
             out, lse = attention_hash_varlen(*dev(q, k, v, kh, cnt, qh), 128 ** -0.5)
@@ -91,6 +91,8 @@ def test_attention_forward_fp16_many_queries_per_bucket(ops):
         assert_attn_close(out, lse, ro, rl, F16, f"fp16 {which}")
         outs[which] = (out, lse)
     assert torch.equal(outs["ring"][0], outs["staged-pairs"][0]) and torch.equal(outs["ring"][1], outs["staged-pairs"][1])
+    for which in ("ring-per-row", "staged-per-row"):          # a launch per row: the same items, the same bits
+        assert torch.equal(outs[which][0], outs["ring"][0]) and torch.equal(outs[which][1], outs["ring"][1])
 
 
 def test_composite_local_merge_and_backward_fp16(ops):

@@ -76,6 +76,12 @@ def test_attention_over_more_than_2_24_keys(ops, dtype):
     ro, rl = O.hashed_attention_gather(q.cpu(), Ks[None], Vs[None], torch.arange(C * Z), cnt.cpu().long(),
                                        qh.cpu().long(), d ** -0.5)
     assert_attn_close(out, lse, ro, rl, dtype, "N > 2^24")
+    ops.grouped_forward_kernel("staged-per-row")        # the same kernel as a launch per row (here: of the one row)
+    try:
+        op, lp = ops.attention_hash_varlen_i32(q, k, v, flat, cnt, qh, d ** -0.5)
+    finally:
+        ops.grouped_forward_kernel(None)
+    assert torch.equal(op, out) and torch.equal(lp, lse)
     if dtype == torch.bfloat16:
         ops.grouped_forward_kernel("gather")
         try:

@@ -9,8 +9,8 @@
 // decode).
 //
 // Per list, a counting sort over a bitmap of the key range in LDS: set the bit of every listed key, then
-// walk the bitmap in order.  A wave owns 2048 consecutive words per pass and takes them 64 at a time, a
-// lane a word: the wave's scan of the lanes' bit counts gives every lane its output position, and the keys
+// walk the bitmap in order.  A wave owns an equal share of a pass's words (2048 of a full range) and takes
+// them 64 at a time, a lane a word: the wave's scan of the lanes' bit counts gives every lane its output position, and the keys
 // of 64 neighbouring words land in one or two lines per store.  Ranges of NT * 1024 keys per pass, as many
 // passes as N needs; cost per list ~ N / 32 word visits + its length, independent of the order it arrives
 // in, and no limit on the length of a list (the list itself never sits in LDS).  A list that names a key
@@ -29,7 +29,6 @@ __global__ __launch_bounds__(NT) void lists_key_order_kernel(const int32_t* __re
   extern __shared__ uint32_t lo_bm[];  // 32 * NT words
   __shared__ int scan_tmp[17];
   constexpr int64_t kRange = int64_t(NT) * 1024;  // keys per pass
-  constexpr int kWaveWords = 2048;                // words of a pass a wave walks (NT / 64 waves)
   constexpr int kHeld = 16;                       // entries per thread kept in registers between passes
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = cnt[blockIdx.x];
@@ -59,15 +58,17 @@ __global__ __launch_bounds__(NT) void lists_key_order_kernel(const int32_t* __re
       for (int i = tid; i < n; i += NT) mark(src[i]);
     }
     __syncthreads();
-    const int w0 = wave * kWaveWords;
+    // the pass's words in equal shares of whole 64-word steps (2048 words a wave when the range is full)
+    const int wave_words = ((n_words + NT - 1) / NT) * 64;
+    const int w0 = wave * wave_words;
     int c = 0;
-    for (int s = w0 + lane; s < min(n_words, w0 + kWaveWords); s += 64) c += __popc(lo_bm[s]);
+    for (int s = w0 + lane; s < min(n_words, w0 + wave_words); s += 64) c += __popc(lo_bm[s]);
     c = __builtin_amdgcn_readlane(wave_incl_scan_dpp(c), 63);
     int total;
     int base = block_excl_scan(lane == 0 ? c : 0, scan_tmp, &total);
     base = written + __builtin_amdgcn_readfirstlane(base);
     if (c > 0) {
-      for (int s0 = w0; s0 < min(n_words, w0 + kWaveWords); s0 += 64) {
+      for (int s0 = w0; s0 < min(n_words, w0 + wave_words); s0 += 64) {
         const int s = s0 + lane;
         uint32_t w = s < n_words ? lo_bm[s] : 0u;
         const int pc = __popc(w);

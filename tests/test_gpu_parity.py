@@ -262,6 +262,30 @@ def test_lists_key_order_copies_lists_it_cannot_sort(ops):
     assert torch.equal(got.cpu(), ref)
 
 
+def test_attention_hash_reorders_lists_by_density(ops):
+    """The composite (triton_kernel.py:275-286) hands the attention key-ordered lists between 1 and 96 queries
+    per bucket on average: the same result as over the lists as built, and as the oracle's composite."""
+    from fast_memory_amd import attention_hash
+    from fast_memory_amd.hash_attention import sorts_lists
+    assert not sorts_lists(10, 16) and sorts_lists(16, 16) and sorts_lists(95 * 16, 16) and not sorts_lists(96 * 16, 16)
+    assert not sorts_lists(131072, 1024) and sorts_lists(32768, 2048)          # the harness shape; the 1M-key one
+    g = gen(433)
+    B, S, N, C, Z, d = 2, 700, 5000, 20, 300, 128
+    q = (torch.randn(B, S, d, generator=g) * 0.5).to(torch.bfloat16)
+    k = (torch.randn(B, N, d, generator=g) * 0.5).to(torch.bfloat16)
+    v = (torch.randn(B, N, d, generator=g) * 0.5).to(torch.bfloat16)
+    A = torch.randn(B, C, d, generator=g).to(torch.bfloat16)
+    res = {ko: attention_hash(*dev(q, k, v, A), Z, d ** -0.5, key_order=ko) for ko in (None, True, False)}
+    sync()
+    assert torch.equal(res[None][0], res[True][0]) and torch.equal(res[None][1], res[True][1])   # 35 per bucket: sorted
+    assert (res[True][0].float() - res[False][0].float()).abs().max().item() < 4e-3
+    assert (res[True][1] - res[False][1]).abs().max().item() < 1e-4
+    lists = O.argtopz(ops.project(*dev(A, k)).cpu(), Z)
+    qh = ops.qhash(*dev(A, q)).cpu().long()
+    ro, rl = O.hashed_attention_gather(q, k, v, lists.reshape(-1), torch.full((B, C), Z), qh, d ** -0.5)
+    assert_attn_close(res[None][0], res[None][1], ro, rl, torch.bfloat16, "attention_hash, key-ordered lists")
+
+
 def test_memory_attends_over_key_ordered_lists(ops):
     """Memory.attend reads a key-ordered copy of the lists once a call brings a query per bucket: the same
     sets, bucket_idx untouched, the result that of the oracle on the lists as torch.topk orders them; a

@@ -102,11 +102,13 @@ extern "C" int fm_lists_key_order(const int32_t* k_idx, const int64_t* bucket_of
   using namespace fm;
   FM_REQUIRE(n_lists >= 0 && N >= 1, FM_ERR_ARG, "fm_lists_key_order: n_lists=%lld N=%d", (long long)n_lists, N);
   FM_REQUIRE(n_lists <= 0x7fffffffLL, FM_ERR_UNSUPPORTED, "fm_lists_key_order: too many lists");
+  FM_REQUIRE(n_lists == 0 || (k_idx && bucket_off && bucket_cnt && k_idx_out), FM_ERR_ARG,
+             "fm_lists_key_order: null pointer");
+  FM_REQUIRE(n_lists == 0 || k_idx != k_idx_out, FM_ERR_ARG,
+             "fm_lists_key_order: the lists cannot be reordered in place");
   hipStream_t st = as_stream(stream);
   if (n_unsorted) hipLaunchKernelGGL(lists_zero_count_kernel, dim3(1), dim3(1), 0, st, n_unsorted);
-  if (n_lists == 0) return launch_status("fm_lists_key_order");
-  FM_REQUIRE(k_idx && bucket_off && bucket_cnt && k_idx_out, FM_ERR_ARG, "fm_lists_key_order: null pointer");
-  FM_REQUIRE(k_idx != k_idx_out, FM_ERR_ARG, "fm_lists_key_order: the lists cannot be reordered in place");
+  if (n_lists == 0) return n_unsorted ? launch_status("fm_lists_key_order") : FM_OK;
   // narrow workgroups (several per CU) while one pass of theirs covers the key range: every pass walks
   // the whole list again, so beyond that the widest form, with the fewest passes, is the fastest
   const int nt = N <= 256 * 1024 ? 256 : N <= 512 * 1024 ? 512 : 1024;

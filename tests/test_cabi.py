@@ -60,6 +60,12 @@ def test_argument_errors_are_status_codes():
     assert lib.fm_hash_attn_bwd_staged(*([None] * 18), 1, 1, 1, 64, 1, None, 1.0, 1, None, 0, None) != 0   # d = 64
     assert b"fm_hash_attn_bwd_staged" in lib.fm_last_error()
     assert lib.fm_segment_sum(None, None, None, None, None, 1, 1, 1, 8, 0, None) != 0
+    assert lib.fm_lists_key_order(None, None, None, 3, 10, None, None, None) == 1   # null pointers
+    assert b"fm_lists_key_order" in lib.fm_last_error()
+    assert lib.fm_lists_key_order(None, None, None, 3, 0, None, None, None) == 1    # N = 0
+    assert lib.fm_lists_key_order(None, None, None, 0, 10, None, None, None) == 0   # no list: nothing to do
+    assert lib.fm_lists_key_order(4096, 4096, 4096, 1, 10, 4096, None, None) == 1    # in place: refused before any launch
+    assert b"in place" in lib.fm_last_error()
     with pytest.raises(ValueError):
         _lib.check(1)
 

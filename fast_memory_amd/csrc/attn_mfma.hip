@@ -511,7 +511,7 @@ extern std::atomic<int> g_force_generic;
 // the long memories and for tests to compare against.
 //
 // A launch per row, in row order, when K and V of all rows together are at least twice the last-level cache
-// (512 MB) and a row fills the device twice over (the direct-load kernel runs 512 workgroups at a time, the
+// (512 MB), a row's are 32 MB or more, and a row fills the device twice over (the direct-load kernel runs 512 workgroups at a time, the
 // staged one 768): with the lists in ascending key order the workgroups of a launch sweep the row's K and V
 // at about the same pace, and a key row that several buckets list is fetched from HBM once and found in the
 // last-level cache, or the L2, by the others; in a single launch over all rows the starts spread over the
@@ -520,8 +520,11 @@ extern std::atomic<int> g_force_generic;
 // of 16384, 16 queries per bucket 15.9 / 14.6 / 14.0 / 12.3 ms; 8 rows of 2^18 keys, 1024 buckets of 4096, 8
 // queries per bucket 1.76 / 1.42 / 1.86 / 1.22 ms; 8 rows of 2^15 keys (134 MB in all), 256 buckets of 1024
 // 0.134 / 0.112 / 0.241 / 0.191 ms.
+// (Rows of 16 MB, 64 of them with 1024 buckets of 1024: 3.73 ms per row against 3.34 in one launch -- a launch of
+// 60 us is mostly start and tail; rows of 32 MB, 32 of them with 1024 buckets of 3072: 4.58 against 5.23.)
 static bool row_launches_pay(int choice, int H, int Sq, int N, int C) {
-  return H > 1 && int64_t(H) * N * kD * 4 >= (int64_t(512) << 20) && (C < Sq ? C : Sq) >= (choice == 3 ? 1024 : 1536);
+  return H > 1 && int64_t(H) * N * kD * 4 >= (int64_t(512) << 20) && int64_t(N) * kD * 4 >= (int64_t(32) << 20) &&
+         (C < Sq ? C : Sq) >= (choice == 3 ? 1024 : 1536);
 }
 
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {

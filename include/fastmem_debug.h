@@ -26,7 +26,8 @@ extern "C" {
  * 3 = always the kernel that gathers the rows into registers.  Dispatch: gather
  * when H min(Sq, C) < 512 and Sq < 24 C; else the direct loads up to 2^24 keys and
  * the staged kernel beyond; one launch per row when K and V of all rows are 512 MB
- * or more and a row has 1024 (staged kernel: 1536) or more buckets and queries. */
+ * or more, those of a row 32 MB or more, and a row has 1024 (staged kernel: 1536)
+ * or more buckets and queries. */
 void fm_debug_force_generic(int on);
 
 /* Diagnostic: name of the kernel fm_hash_attn_fwd launches for these extents

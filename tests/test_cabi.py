@@ -115,6 +115,8 @@ def test_grouped_forward_dispatch_rule():
     assert launches(8, 16384, 262144, 128, 512, 1) == 1                               # too few buckets per row
     assert launches(8, 16384, (1 << 24) + 64, 128, 1024, 1) == 1                      # ... for the staged kernel
     assert launches(8, 8192, 32768, 128, 256, 1) == 1                                 # 134 MB in all
+    assert launches(64, 16384, 32768, 128, 1024, 1) == 1                              # 1 GB in all, rows of 16 MB
+    assert launches(32, 16384, 65536, 128, 1024, 1) == 32                             # rows of 32 MB
     assert launches(8, 131072, 1048576, 128, 2048, 1) == 8                            # 64 queries / bucket
     assert launches(8, 32768, (1 << 24) + 64, 128, 2048, 1) == 8                      # staged kernel, 64-bit rows
     assert launches(8, 131072, 65536, 128, 1024, 2) == 1                              # reference harness

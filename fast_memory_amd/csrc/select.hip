@@ -51,7 +51,7 @@ static SamplePlan sample_plan(int N, int Zc, int P, int nt, bool wide = false) {
   const double m_exp = double(rank) * N / ns, m_sd = double(N) / ns * sqrt(double(rank));
   int cap;
   if (wide) {
-    cap = kCollectRegsWide * nt;                    // what the registers take; 4 bytes each in LDS
+    cap = kCollectRegsWide * nt;                    // what the registers take; LDS holds half of them at a time
   } else {
     cap = 2 * P;
     while (cap < m_exp + 5.0 * m_sd && cap < kCollectRegs * nt) cap *= 2;
@@ -90,6 +90,20 @@ struct CollectedRegs {
   }
 };
 
+// The same for candidates collected in two rounds (the two halves of a row): registers 0 .. CR/2 - 1 hold a
+// thread's share of the first round, the others its share of the second.
+template <int CR>
+struct CollectedHalves {
+  uint64_t c[CR];
+  int n0, n1;
+  template <typename F>
+  __device__ __forceinline__ void operator()(F f) const {
+#pragma unroll
+    for (int r = 0; r < CR; ++r)
+      if (r < CR / 2 ? r < n0 : r - CR / 2 < n1) f(key_to_float(uint32_t(c[r] >> 32)), 0xffffffffu - uint32_t(c[r]));
+  }
+};
+
 // row_map / n_rows_dev are optional: when given, workgroup b works on input row
 // b and writes output row row_map[b], and exits if b >= min(*n_rows_dev, grid).
 template <int NT, bool WIDE = false>
@@ -119,45 +133,77 @@ __global__ __launch_bounds__(NT) void argtopz_kernel(
       if (r < smp.n) smp.v[r] = row[(int64_t(j >> 5) * sp.line_stride << 5) + (j & 31)];
     }
     const uint64_t tau = radix_select_cut<NT>(smp, sp.rank, 3, sh) & 0xffffffff00000000ull;  // value bits only
-    if (tid == 0) sh.cnt = 0;
-    __syncthreads();
     // tau has value bits only, so "composite >= tau" is a comparison of values: one float compare per
     // element of the row (NaN, the largest key, passes: it is not below anything)
     const float tau_f = key_to_float(uint32_t(tau >> 32));
-    src([&](float y, uint32_t i) {
-      if (!(y < tau_f)) {
-        const int pos = atomicAdd(&sh.cnt, 1);
-        if (pos < sp.cap) {
-          if constexpr (WIDE)
-            reinterpret_cast<uint32_t*>(buf)[pos] = i;
-          else
-            buf[pos] = composite(y, i);
-        }
-      }
-    });
-    __syncthreads();
-    const int m = sh.cnt;
-    if (m >= Zc && m <= sp.cap) {
-      constexpr int CR = WIDE ? kCollectRegsWide : kCollectRegs;
-      CollectedRegs<CR> cr;
-      cr.n = tid < m ? (m - tid + NT - 1) / NT : 0;
+    if constexpr (WIDE) {
+      // Lists longer than 8 * NT: the candidates (about 1.2 Zc) do not fit LDS as composites all at once, so the
+      // row is taken in two interleaved halves; each half's candidates go to LDS as composites (sp.cap / 2
+      // slots) and from there to the threads' registers, which hold them all.  (Buffering indices only and fetching the
+      // candidates' values again afterwards moved a 128-byte line per candidate: 0.47 x the row once more.)
+      constexpr int CR = kCollectRegsWide;
+      CollectedHalves<CR> cr;
+      const int cap_h = sp.cap / 2;  // = CR / 2 * NT
+      int m_all = 0;
+      bool fits = true;
 #pragma unroll
-      for (int r = 0; r < CR; ++r)
-        if (r < cr.n) {
-          if constexpr (WIDE) {
-            const uint32_t i = reinterpret_cast<const uint32_t*>(buf)[tid + r * NT];
-            cr.c[r] = composite(row[i], i);
-          } else {
-            cr.c[r] = buf[tid + r * NT];
+      for (int h = 0; h < 2; ++h) {
+        if (tid == 0) sh.cnt = 0;
+        __syncthreads();
+        src.half(h, [&](float y, uint32_t i) {
+          if (!(y < tau_f)) {
+            const int pos = atomicAdd(&sh.cnt, 1);
+            if (pos < cap_h) buf[pos] = composite(y, i);
           }
-        }
-      __syncthreads();  // every candidate is in registers before the buffer is written again
-      if (binned_select_write<NT>(cr, Zc, buf, reinterpret_cast<uint32_t*>(buf + (Zc + kSelMaxBin)), bs, out, vout))
+        });
+        __syncthreads();
+        const int m = sh.cnt;
+        m_all += m;
+        fits = fits && m <= cap_h;
+        const int mine = tid < m ? (min(m, cap_h) - tid + NT - 1) / NT : 0;
+        if (h == 0)
+          cr.n0 = mine;
+        else
+          cr.n1 = mine;
+#pragma unroll
+        for (int r = 0; r < CR / 2; ++r)
+          if (r < mine) cr.c[h * (CR / 2) + r] = buf[tid + r * NT];
+        __syncthreads();  // every candidate of the half is in registers before the buffer is written again
+      }
+      if (fits && m_all >= Zc) {
+        if (binned_select_write<NT>(cr, Zc, buf, reinterpret_cast<uint32_t*>(buf + (Zc + kSelMaxBin)), bs, out, vout))
+          return;
+        __syncthreads();
+        const uint64_t cut = radix_select_cut<NT>(cr, Zc, 6, sh);
+        collect_sort_write(cr, cut, Zc, P, buf, sh, out, vout);
         return;
+      }
+    } else {
+      if (tid == 0) sh.cnt = 0;
       __syncthreads();
-      const uint64_t cut = radix_select_cut<NT>(cr, Zc, 6, sh);
-      collect_sort_write(cr, cut, Zc, P, buf, sh, out, vout);
-      return;
+      src([&](float y, uint32_t i) {
+        if (!(y < tau_f)) {
+          const int pos = atomicAdd(&sh.cnt, 1);
+          if (pos < sp.cap) buf[pos] = composite(y, i);
+        }
+      });
+      __syncthreads();
+      const int m = sh.cnt;
+      if (m >= Zc && m <= sp.cap) {
+        constexpr int CR = kCollectRegs;
+        CollectedRegs<CR> cr;
+        cr.n = tid < m ? (m - tid + NT - 1) / NT : 0;
+#pragma unroll
+        for (int r = 0; r < CR; ++r)
+          if (r < cr.n) cr.c[r] = buf[tid + r * NT];
+        __syncthreads();  // every candidate is in registers before the buffer is written again
+        if (binned_select_write<NT>(cr, Zc, buf, reinterpret_cast<uint32_t*>(buf + (Zc + kSelMaxBin)), bs, out, vout))
+          return;
+        __syncthreads();
+        const uint64_t cut = radix_select_cut<NT>(cr, Zc, 6, sh);
+        collect_sort_write(cr, cut, Zc, P, buf, sh, out, vout);
+        return;
+      }
     }
     __syncthreads();  // every thread has read sh.cnt before the exact passes reuse it
   }
@@ -250,13 +296,13 @@ int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int
     }
   }
   // SelectShared sits behind the sort buffer / the candidate buffer; the binned selection needs its own extent
-  const size_t sh_off = align_up(std::max(sort_lds_bytes(P), size_t(sp.cap) * (wide ? sizeof(uint32_t) : sizeof(uint64_t))), 16);
+  const size_t sh_off = align_up(std::max(sort_lds_bytes(P), (wide ? size_t(sp.cap) / 2 : size_t(sp.cap)) * sizeof(uint64_t)), 16);
   const auto lds_for = [](size_t off, int zc, bool sampled) {
     const size_t binned = sampled ? binned_lds_bytes(zc) : 0;
     return std::max(off + sizeof(SelectShared), binned);
   };
   const size_t lds = lds_for(sh_off, Zc, sp.n_lines > 0);
-  const size_t lds_max = lds_for(align_up(std::max(sort_lds_bytes(FM_MAX_Z), size_t(kCollectRegsWide) * kSelThreads * 4), 16),
+  const size_t lds_max = lds_for(align_up(std::max(sort_lds_bytes(FM_MAX_Z), size_t(kCollectRegsWide) / 2 * kSelThreads * sizeof(uint64_t)), 16),
                                  FM_MAX_Z, true);
   if (narrow) {
     FM_ALLOW_LDS(argtopz_kernel<512>, lds_max, "argtopz: lds");

@@ -484,6 +484,39 @@ struct DenseRowT {
     const int tail0 = head + 4 * nvec;
     if (tail0 + tid < N) f(row[tail0 + tid], uint32_t(tail0 + tid));
   }
+  // Half h (0 or 1) of the row: every other round of the loop above (rounds of NT * kUnroll * 4 elements,
+  // interleaved so that a trend along the row lands in both halves alike); the unaligned head and tail
+  // belong to half 0.
+  template <typename F>
+  __device__ __forceinline__ void half(int h, F f) const {
+    const int tid = threadIdx.x;
+    int head = int((4 - ((reinterpret_cast<uintptr_t>(row) >> 2) & 3)) & 3);
+    if (head > N) head = N;
+    if (h == 0 && tid < head) f(row[tid], uint32_t(tid));
+    const int nvec = (N - head) >> 2;
+    const float4* v = reinterpret_cast<const float4*>(row + head);
+    for (int i0 = tid + h * NT * kUnroll; i0 < nvec; i0 += 2 * NT * kUnroll) {
+      float4 x[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        int i = i0 + u * NT;
+        if (i < nvec) x[u] = v[i];
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        int i = i0 + u * NT;
+        if (i < nvec) {
+          uint32_t b = uint32_t(head + 4 * i);
+          f(x[u].x, b);
+          f(x[u].y, b + 1);
+          f(x[u].z, b + 2);
+          f(x[u].w, b + 3);
+        }
+      }
+    }
+    const int tail0 = head + 4 * nvec;
+    if (h == 0 && tail0 + tid < N) f(row[tail0 + tid], uint32_t(tail0 + tid));
+  }
 };
 
 using DenseRow = DenseRowT<>;

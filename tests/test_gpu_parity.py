@@ -100,8 +100,9 @@ def test_argtopz_max_z_long_row(ops):
 
 
 def test_argtopz_sampled_one_pass_equals_exact_passes(ops):
-    """Long rows take the sampled one-pass selection (lists longer than 8192 in its index-buffer form); rows
-    the sample misleads fall back inside the kernel.  Both must give the lists of the exact multi-pass
+    """Long rows take the sampled one-pass selection (lists longer than 8192 in the form that collects the
+    candidates of the two interleaved halves of a row one after the other); rows the sample misleads, or whose
+    candidates crowd into one half, fall back inside the kernel.  Both must give the lists of the exact multi-pass
     selection, bit for bit."""
     g = gen(210)
     N = 131072 + 37                                          # ragged tail, rows not 16-byte aligned after row 0

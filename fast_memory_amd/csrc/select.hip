@@ -170,14 +170,11 @@ __global__ __launch_bounds__(NT) void argtopz_kernel(
           if (r < mine) cr.c[h * (CR / 2) + r] = buf[tid + r * NT];
         __syncthreads();  // every candidate of the half is in registers before the buffer is written again
       }
-      if (fits && m_all >= Zc) {
-        if (binned_select_write<NT>(cr, Zc, buf, reinterpret_cast<uint32_t*>(buf + (Zc + kSelMaxBin)), bs, out, vout))
-          return;
-        __syncthreads();
-        const uint64_t cut = radix_select_cut<NT>(cr, Zc, 6, sh);
-        collect_sort_write(cr, cut, Zc, P, buf, sh, out, vout);
+      // (a row whose candidates the binned selection declines, e.g. thousands of equal values around the cut,
+      // goes on to the exact passes below like one the sample misled)
+      if (fits && m_all >= Zc &&
+          binned_select_write<NT>(cr, Zc, buf, reinterpret_cast<uint32_t*>(buf + (Zc + kSelMaxBin)), bs, out, vout))
         return;
-      }
     } else {
       if (tid == 0) sh.cnt = 0;
       __syncthreads();

@@ -315,7 +315,7 @@ def bench_reference_harness(args):
     ws_bytes = int(args.workspace_gib * (1 << 30))
 
     # the parts, each on its own
-    build_ms, lists = timed(lambda: ops.build_index(centroids, k, Z, ws_bytes), reps=3, warm=1)
+    build_ms, lists = timed(lambda: ops.build_index(centroids, k, Z, ws_bytes), reps=3, warm=3)
     hash_ms, qh = timed(lambda: ops.qhash(centroids, q), reps=3, warm=1)
     group_ms, groups = timed(lambda: ops.group_queries(qh, C), reps=3, warm=1)
     off = ops.bucket_offsets(torch.full((B, C), Z, dtype=torch.int32, device=dev))
@@ -467,9 +467,10 @@ def main():
         f"(keys {tuple(wl.keys.shape)} {wl.keys.dtype})")
 
     # ---- A by spherical K-means, index build (both timed, outside the step) ----
-    km_ms, A = timed(lambda: fit_projection(wl.keys, C, iters=cfg.kmeans_iters), reps=1, warm=1)
+    km_ms, A = timed(lambda: fit_projection(wl.keys, C, iters=cfg.kmeans_iters), reps=2, warm=2)
     log(f"[bench] K-means ({cfg.kmeans_iters} iterations): {km_ms:.1f} ms")
-    build_ms, mem = timed(lambda: Memory.build(wl.keys, wl.values, A, Z, workspace_bytes=ws_bytes), reps=2, warm=1)
+    # (three builds first: the first ones also pay for the allocator's first blocks of this size)
+    build_ms, mem = timed(lambda: Memory.build(wl.keys, wl.values, A, Z, workspace_bytes=ws_bytes), reps=3, warm=3)
     keys_per_s = H * N / (build_ms * 1e-3)
     log(f"[bench] index build: {build_ms:.1f} ms  ({keys_per_s / 1e6:.1f} M keys/s)")
 

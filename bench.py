@@ -170,6 +170,20 @@ def calibrate_copy(dev):
     torch.cuda.synchronize()
 
 
+def mfma_stream_probe(dev, iters=1000):
+    """bf16 MFMA rate (TFLOP/s) of a register-resident loop of nothing but MFMAs on normally distributed
+    operands: what the matrix pipes sustain on this device, for scale beside the published peak (the device
+    is power-bound there and clocks the loop lower the more the operand bits toggle)."""
+    from fast_memory_amd import _lib
+    g = torch.Generator(device="cpu").manual_seed(11)
+    operands = torch.randn(5120, generator=g).to(torch.bfloat16).to(dev)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    call = lambda: _lib.check(_lib.load().fm_debug_mfma(operands.data_ptr(), operands.numel(), iters, sink.data_ptr(),
+                                                        torch.cuda.current_stream().cuda_stream))
+    best_ms = min(timed(call, reps=1, warm=1)[0] for _ in range(5))
+    return iters * 2.0 ** 33 / best_ms / 1e9
+
+
 def hbm_traffic(kernel, workload):
     """HBM bytes per launch measured offline with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) and kept as
     text under profiles/; None when no figure is recorded."""
@@ -469,6 +483,13 @@ def main():
     # ---- A by spherical K-means, index build (both timed, outside the step) ----
     km_ms, A = timed(lambda: fit_projection(wl.keys, C, iters=cfg.kmeans_iters), reps=2, warm=2)
     log(f"[bench] K-means ({cfg.kmeans_iters} iterations): {km_ms:.1f} ms")
+    # its assignment step alone: the hash of every key against the C centroids
+    assign = None
+    if e == 2 and d == 128:
+        assign_ms, _ = timed(lambda: ops.qhash(A, wl.keys), reps=3, warm=1)
+        assign_tflops = 2.0 * H * C * N * d / assign_ms / 1e9
+        assign = {"ms": assign_ms, "tflops": assign_tflops, "mfma_frac": assign_tflops / BF16_MFMA_PEAK_TFLOPS}
+        log(f"[bench] K-means assignment (qhash of all keys): {assign}")
     # (three builds first: the first ones also pay for the allocator's first blocks of this size)
     build_ms, mem = timed(lambda: Memory.build(wl.keys, wl.values, A, Z, workspace_bytes=ws_bytes), reps=3, warm=3)
     keys_per_s = H * N / (build_ms * 1e-3)
@@ -481,6 +502,8 @@ def main():
         gemm_flops = 2.0 * H * C * N * d
         fused_phases["filter_tflops"] = gemm_flops / fused_phases["mfma_filter_ms"] / 1e9
         fused_phases["filter_mfma_frac"] = fused_phases["filter_tflops"] / BF16_MFMA_PEAK_TFLOPS
+        fused_phases["mfma_stream_probe_tflops"] = mfma_stream_probe(dev)
+        fused_phases["filter_vs_mfma_stream_probe"] = fused_phases["filter_tflops"] / fused_phases["mfma_stream_probe_tflops"]
         log(f"[bench] fused build phases (ms): {fused_phases}")
 
     # extending the index by M new keys instead of rebuilding it (same lists as a rebuild over N+M keys)
@@ -748,7 +771,9 @@ def main():
         roofline = {"kernel": filter_kernel, "bound": "mfma", "achieved": fused_phases["filter_tflops"],
                     "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": fused_phases["filter_mfma_frac"],
                     "traffic": filter_traffic, "algorithmic_flops_per_launch": 2.0 * H * C * N * d,
-                    "avg_launch_ms": fused_phases["mfma_filter_ms"]}
+                    "avg_launch_ms": fused_phases["mfma_filter_ms"],
+                    "mfma_stream_probe_tflops": fused_phases["mfma_stream_probe_tflops"],
+                    "vs_mfma_stream_probe": fused_phases["filter_vs_mfma_stream_probe"]}
     line = {
         "metric": "index-build keys/s" if args.config == "c4" else "hashed-attn query-heads/s",
         "value": value, "unit": "keys/s" if args.config == "c4" else "query-heads/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -764,7 +789,7 @@ def main():
         "cpu_baseline": cpu,
         "index_build": {"keys_per_s": keys_per_s, "ms": build_ms, "keys": H * N, "path": build_path,
                         "fused_phases_ms": fused_phases, "unfused_parts": build_parts,
-                        "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters, "append": append,
+                        "kmeans_ms": km_ms, "kmeans_iters": cfg.kmeans_iters, "kmeans_assign": assign, "append": append,
                         "lists_key_order_ms": ko_ms},
         "query_path": query_path,
         "step_parts_ms": {"attention": attn_ms, **parts_ms},

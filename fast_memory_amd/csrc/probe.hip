@@ -1,6 +1,8 @@
-// Plain streaming copy of a known size: the yardstick that HBM traffic counters
-// of the other kernels are scaled against when profiling.
+// Kernels of known size: a plain streaming copy (the yardstick that HBM traffic counters of the other
+// kernels are scaled against when profiling), a read-only stream and a register-resident MFMA stream (the
+// rates a kernel can actually reach on the device, beside the published peaks).
 #include "common.hpp"
+#include "mfma_tile.hpp"
 
 namespace fm {
 __global__ __launch_bounds__(256) void copy_probe_kernel(const uint4* __restrict__ src,
@@ -28,7 +30,60 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict
   }
   if (acc == 0x9e3779b9u && n < 0) sink[0] = acc;
 }
+
+// Register-resident stream of bf16 MFMAs: every wave loads ten operand fragments once and then issues nothing
+// but v_mfma_f32_32x32x16_bf16, four independent accumulator chains in turn (with fewer, the next instruction
+// of a chain waits for the one before it).  No memory, LDS or VALU work inside the loop: its rate is what the
+// matrix pipes sustain on this device for the operand values given -- the device is power-bound in such a loop
+// and clocks it lower the more the operand bits toggle -- i.e. the practical ceiling beside the published peak.
+constexpr int kMfmaProbeGrid = 1024;      // workgroups of 8 waves
+constexpr int kMfmaProbeOperands = 5120;  // 10 fragments x 64 lanes x 8 elements
+__global__ __launch_bounds__(512) void mfma_probe_kernel(const bf16_t* __restrict__ operands, int iters,
+                                                         float* __restrict__ sink) {
+  const int l = threadIdx.x & 63;
+  bf16x8 a[8], b[2];
+#pragma unroll
+  for (int i = 0; i < 10; ++i) {
+    union {
+      uint4 u;
+      bf16x8 v;
+    } cvt;
+    cvt.u = reinterpret_cast<const uint4*>(operands)[i * 64 + l];
+    if (i < 8)
+      a[i] = cvt.v;
+    else
+      b[i - 8] = cvt.v;
+  }
+  f32x16 acc[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[c][r] = 0.f;
+  for (int t = 0; t < iters; ++t) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[c] = mfma32<false>(a[ks], b[c & 1], acc[c]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[c][r];
+  if (s == 123456.789f && iters < 0) sink[0] = s;  // never true; keeps the loop alive
+}
 }  // namespace fm
+
+extern "C" int fm_debug_mfma(const void* operands, int64_t n_operands, int iters, void* sink, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(operands && sink && n_operands >= kMfmaProbeOperands && iters >= 0, FM_ERR_ARG,
+             "fm_debug_mfma: n_operands=%lld (at least %d bf16 values) iters=%d", (long long)n_operands,
+             kMfmaProbeOperands, iters);
+  if (iters == 0) return FM_OK;
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3(kMfmaProbeGrid), dim3(512), 0, as_stream(stream),
+                     (const bf16_t*)operands, iters, (float*)sink);
+  return launch_status("fm_debug_mfma");
+}
 
 extern "C" int fm_debug_read(const void* src, int64_t nbytes, void* sink, void* stream) {
   using namespace fm;

@@ -348,15 +348,22 @@ __global__ __launch_bounds__(256) void qhash_bf16_kernel(const bf16_t* __restric
 // ---------------------------------------------------------------------------
 // bf16 query hash, d = 128, streaming form (no scores written): a workgroup of 8
 // waves holds 512 queries as resident MFMA B fragments (64 per wave) and streams
-// the bucket rows of A through a double-buffered LDS tile of 64 rows.  One query
-// per lane column: the running maximum and its position are per-lane registers,
-// updated with three VALU instructions per accumulator register (compare, select
-// value, select the row number as an inline constant); buckets arrive in
-// ascending order, so "strictly greater" keeps the first maximum.  The loop is
-// software-pipelined in half tiles: while the MFMAs of one 32-row sub-tile run,
-// the finished sub-tile before it is scanned and the A fragments of the next are
-// read from LDS.  On this hardware VALU and MFMA time of a SIMD add up rather
-// than overlap, so the scan costs about as much as the products.  The scores are
+// the bucket rows of A through LDS tiles of 64 rows.  One query per lane column:
+// the running maximum and its position are per-lane registers, updated with three
+// VALU instructions per accumulator register (compare, select value, select the
+// row number as an inline constant); buckets arrive in ascending order, so
+// "strictly greater" keeps the first maximum.  The loop is software-pipelined in
+// tiles: the 32 MFMAs of a tile -- four independent chains, (32-row sub-tile,
+// 32-query fragment) -- alternate in the instruction stream with the scan of the
+// tile before it, which sits in a second set of accumulators, and with the LDS
+// reads of the next A fragments.  Measured on this hardware with register-resident
+// loops: with four chains the VALU work of the same wave is issued in the shadow of
+// its MFMAs (four VALU instructions per MFMA cost nothing, six cost 12 %); with two
+// chains it is not, and VALU work of the SIMD's other wave mostly adds to the MFMA
+// time.  The device is power-bound in such loops and clocks them lower the more
+// their operands toggle and the more LDS and VALU work they carry: a stream of these
+// MFMAs alone sustains 78 % of the nominal peak on operands of a few values and
+// 64 % on random ones, and with six VALU instructions per MFMA 56 %.  The scores are
 // the same MFMA sums as in qhash_bf16_kernel (same instruction, operand roles and
 // contraction order), so both kernels return identical hashes.
 // Roofline: MFMA, 2*C*d flops per query.
@@ -370,52 +377,70 @@ __device__ __forceinline__ void argmax_step(float& best, int& pos, float s) {
                : "v"(s), "n"(K)
                : "vcc");
 }
+// two steps in one statement (the compiler puts a wait state between two statements that write vcc)
+template <int K0, int K1>
+__device__ __forceinline__ void argmax_step2(float& best, int& pos, float s0, float s1) {
+  asm volatile(
+      "v_cmp_gt_f32 vcc, %2, %0\n\tv_cndmask_b32_e32 %0, %0, %2, vcc\n\tv_cndmask_b32_e64 %1, %1, %4, vcc\n\t"
+      "v_cmp_gt_f32 vcc, %3, %0\n\tv_cndmask_b32_e32 %0, %0, %3, vcc\n\tv_cndmask_b32_e64 %1, %1, %5, vcc"
+      : "+v"(best), "+v"(pos)
+      : "v"(s0), "v"(s1), "n"(K0), "n"(K1)
+      : "vcc");
+}
 
 // position of accumulator register R of the 32-row sub-tile MI inside the 64-row tile, for
 // lanes 0..31 (lanes 32..63 hold the rows 4 further down)
 constexpr int qs_row(int MI, int R) { return MI * 32 + 8 * (R >> 2) + (R & 3); }
 
-// Elements E and E+1 (of 32: query column half E/16, register E%16) of a finished sub-tile.
-// Register 0 of each half goes through plain C++ so that the compiler, which cannot see into the
-// asm, places the wait states a read of a fresh MFMA result needs; the MFMA that produced a half
-// was issued before those of anything read later.
-template <int MI, int E>
-__device__ __forceinline__ void argmax_pair(float (&best)[2], int (&pos)[2], const f32x16 (&acc)[2]) {
-  constexpr int NI = E >> 4, R = E & 15;
-  if constexpr (R == 0) {
-    const bool gt = acc[NI][0] > best[NI];
-    best[NI] = gt ? acc[NI][0] : best[NI];
-    pos[NI] = gt ? qs_row(MI, 0) : pos[NI];
-  } else {
-    argmax_step<qs_row(MI, R)>(best[NI], pos[NI], acc[NI][R]);
-  }
-  argmax_step<qs_row(MI, R + 1)>(best[NI], pos[NI], acc[NI][R + 1]);
-}
-
-// One half step of the pipeline: the 16 MFMAs of sub-tile (MM) of one tile, with the running
-// argmax over the finished sub-tile (ME) of the tile before it and the LDS reads of the next
-// half step's A fragments spread between them.  sched_barrier pins the interleaving: an MFMA
-// keeps the matrix pipe busy for 32 cycles, the six VALU instructions behind it take 24.
-template <bool F16, int ME, bool MFMA, bool PREFETCH, int I>
-__device__ __forceinline__ void qs_half_step(f32x16 (&accM)[2], const f32x16 (&accE)[2], const bf16x8 (&af)[8],
-                                             bf16x8 (&af_next)[8], const bf16_t* next_lds,
+// One tile step of the pipeline, slot I of 32: k-step I / 4, chain I % 4 = (sub-tile mi, query half ni).
+//   MFMA: X[mi][ni] += A fragment (sub-tile mi of the tile at frag_lds, k-step I / 4) x the half's queries;
+//         the two A fragments of the next k-step are read from LDS in the first slot of every k-step, the
+//         first ones of the next tile (next_lds) in that of the last.
+//   SCAN: two registers of the finished set Y.  Slots 0..15 cover sub-tile 0 (slot j: query half j % 2,
+//         registers 2 (j / 2) and the next), slots 16..31 sub-tile 1, so every query half sees its rows in
+//         ascending order.  Register 0 goes through plain C++ so that the compiler, which cannot see into
+//         the asm, places the wait states a read of a fresh MFMA result needs (the MFMA that produced an
+//         accumulator was issued before those of the accumulators read later).
+// sched_barrier pins the interleaving: an MFMA keeps the matrix pipe busy for 32 cycles, the six VALU
+// instructions behind it take 24.
+template <bool F16, bool MFMA, bool SCAN, int I>
+__device__ __forceinline__ void qs_tile_step(f32x16 (&X)[2][2], const f32x16 (&Y)[2][2], bf16x8 (&af)[2][2],
+                                             const bf16_t* frag_lds, const bf16_t* next_lds,
                                              const bf16x8 (&bfrag)[2][8], float (&best)[2], int (&pos)[2]) {
-  if constexpr (I < 16) {
-    constexpr int ks = I >> 1, ni = I & 1;
+  if constexpr (I < 32) {
+    constexpr int ks = I >> 2, mi = (I >> 1) & 1, ni = I & 1;
     if constexpr (MFMA) {
+      if constexpr ((I & 3) == 0) {
+        if constexpr (ks < 7) {
+          af[(ks + 1) & 1][0] = *reinterpret_cast<const bf16x8*>(frag_lds + (ks + 1) * 16);
+          af[(ks + 1) & 1][1] = *reinterpret_cast<const bf16x8*>(frag_lds + 32 * kQsLd + (ks + 1) * 16);
+        } else {
+          af[0][0] = *reinterpret_cast<const bf16x8*>(next_lds);
+          af[0][1] = *reinterpret_cast<const bf16x8*>(next_lds + 32 * kQsLd);
+        }
+      }
       if constexpr (ks == 0) {
         f32x16 z;
 #pragma unroll
         for (int r = 0; r < 16; ++r) z[r] = 0.f;
-        accM[ni] = mfma32<F16>(af[ks], bfrag[ni][ks], z);
+        X[mi][ni] = mfma32<F16>(af[0][mi], bfrag[ni][0], z);
       } else {
-        accM[ni] = mfma32<F16>(af[ks], bfrag[ni][ks], accM[ni]);
+        X[mi][ni] = mfma32<F16>(af[ks & 1][mi], bfrag[ni][ks], X[mi][ni]);
       }
     }
-    if constexpr (PREFETCH && ni == 0) af_next[ks] = *reinterpret_cast<const bf16x8*>(next_lds + ks * 16);
-    argmax_pair<ME, 2 * I>(best, pos, accE);
+    if constexpr (SCAN) {
+      constexpr int smi = I >> 4, sni = I & 1, r = 2 * ((I & 15) >> 1);
+      if constexpr (r == 0) {
+        const bool gt = Y[smi][sni][0] > best[sni];
+        best[sni] = gt ? Y[smi][sni][0] : best[sni];
+        pos[sni] = gt ? qs_row(smi, 0) : pos[sni];
+        argmax_step<qs_row(smi, 1)>(best[sni], pos[sni], Y[smi][sni][1]);
+      } else {
+        argmax_step2<qs_row(smi, r), qs_row(smi, r + 1)>(best[sni], pos[sni], Y[smi][sni][r], Y[smi][sni][r + 1]);
+      }
+    }
     __builtin_amdgcn_sched_barrier(0);
-    qs_half_step<F16, ME, MFMA, PREFETCH, I + 1>(accM, accE, af, af_next, next_lds, bfrag, best, pos);
+    qs_tile_step<F16, MFMA, SCAN, I + 1>(X, Y, af, frag_lds, next_lds, bfrag, best, pos);
   }
 }
 
@@ -423,7 +448,7 @@ template <bool F16>
 __global__ __launch_bounds__(512) void qhash_stream_kernel(const bf16_t* __restrict__ A,
                                                            const bf16_t* __restrict__ q,
                                                            int32_t* __restrict__ hash_out, int C, int Sq) {
-  __shared__ __attribute__((aligned(16))) bf16_t sA[2][64 * kQsLd];
+  __shared__ __attribute__((aligned(16))) bf16_t sA[3][64 * kQsLd];
   const int h = blockIdx.y;
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   const bf16_t* Ah = A + int64_t(h) * C * 128;
@@ -461,56 +486,59 @@ __global__ __launch_bounds__(512) void qhash_stream_kernel(const bf16_t* __restr
     *reinterpret_cast<uint4*>(&sA[buf][(tid >> 4) * kQsLd + (tid & 15) * 8]) = st0;
     *reinterpret_cast<uint4*>(&sA[buf][(32 + (tid >> 4)) * kQsLd + (tid & 15) * 8]) = st1;
   };
-  // LDS address of this lane's A fragment 0 of sub-tile mi of the tile in buffer buf
-  auto frag_ptr = [&](int buf, int mi) -> const bf16_t* {
-    return &sA[buf][(mi * 32 + (l & 31)) * kQsLd + (l >> 5) * 8];
-  };
+  // LDS address of this lane's A fragment 0 of sub-tile 0 of the tile in buffer buf (sub-tile 1: 32 rows on)
+  auto frag_ptr = [&](int buf) -> const bf16_t* { return &sA[buf][(l & 31) * kQsLd + (l >> 5) * 8]; };
+  // Three buffers: while tile t is multiplied, tile t + 1 is in place (its first fragments are read at the
+  // end of the step) and tile t + 2 is written; tile t + 3 is on its way from memory in registers.
   fetch(0);
   stash(0);
   if (ntiles > 1) {
     fetch(1);
     stash(1);
   }
+  if (ntiles > 2) fetch(2);
   __syncthreads();
 
-  // Pipeline over half steps: sub-tile 0 of tile t+1 is multiplied while sub-tile 1 of tile t
-  // is scanned, and the other way round; tile t+2 travels global -> registers -> LDS meanwhile.
-  f32x16 acc[2][2];
-  bf16x8 af0[8], af1[8];
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks) af0[ks] = *reinterpret_cast<const bf16x8*>(frag_ptr(0, 0) + ks * 16);
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks) {
-    f32x16 z;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) z[r] = 0.f;
-    acc[0][0] = mfma32<F16>(af0[ks], bfrag[0][ks], ks ? acc[0][0] : z);
-    acc[0][1] = mfma32<F16>(af0[ks], bfrag[1][ks], ks ? acc[0][1] : z);
-    af1[ks] = *reinterpret_cast<const bf16x8*>(frag_ptr(0, 1) + ks * 16);
-  }
-  for (int t = 0; t < ntiles; ++t) {
-    const bool more = t + 1 < ntiles;
-    if (t + 2 < ntiles) fetch(t + 2);
-    {
-      const float b0 = best[0], b1 = best[1];
-      if (more)
-        qs_half_step<F16, 0, true, true, 0>(acc[1], acc[0], af1, af0, frag_ptr((t + 1) & 1, 0), bfrag, best, pos);
-      else
-        qs_half_step<F16, 0, true, false, 0>(acc[1], acc[0], af1, af0, nullptr, bfrag, best, pos);
-      if (best[0] != b0) btile[0] = t;
-      if (best[1] != b1) btile[1] = t;
-    }
-    {
-      const float b0 = best[0], b1 = best[1];
-      if (more)
-        qs_half_step<F16, 1, true, true, 0>(acc[0], acc[1], af0, af1, frag_ptr((t + 1) & 1, 1), bfrag, best, pos);
-      else
-        qs_half_step<F16, 1, false, false, 0>(acc[0], acc[1], af0, af1, nullptr, bfrag, best, pos);
-      if (best[0] != b0) btile[0] = t;
-      if (best[1] != b1) btile[1] = t;
-    }
-    if (t + 2 < ntiles) stash(t & 1);  // the buffer of tile t: its last reads were a tile ago
+  f32x16 acc[2][2][2];  // [set][sub-tile][query half]
+  bf16x8 af[2][2];      // [k-step parity][sub-tile]
+  af[0][0] = *reinterpret_cast<const bf16x8*>(frag_ptr(0));
+  af[0][1] = *reinterpret_cast<const bf16x8*>(frag_ptr(0) + 32 * kQsLd);
+  int buf = 0;  // t % 3
+  // step t: the MFMAs of tile t into set XS, the scan of tile t - 1 in the other set
+  auto tile = [&](int t, auto XS_, auto SCAN_) {
+    constexpr int XS = decltype(XS_)::value;
+    constexpr bool SCAN = decltype(SCAN_)::value;
+    const int buf1 = buf == 2 ? 0 : buf + 1, buf2 = buf1 == 2 ? 0 : buf1 + 1;
+    if (t + 2 < ntiles) stash(buf2);  // fetched a step ago; the buffer's last reads (tile t - 1) were before the barrier
+    if (t + 3 < ntiles) fetch(t + 3);
+    const float b0 = best[0], b1 = best[1];
+    // (past the last tile the fragment reads at the end of the step fetch stale rows that nothing uses)
+    qs_tile_step<F16, true, SCAN, 0>(acc[XS], acc[1 - XS], af, frag_ptr(buf), frag_ptr(buf1), bfrag, best, pos);
+    if (best[0] != b0) btile[0] = t - 1;
+    if (best[1] != b1) btile[1] = t - 1;
+    buf = buf1;
     __syncthreads();
+  };
+  auto last_scan = [&](auto YS_) {
+    constexpr int YS = decltype(YS_)::value;
+    const float b0 = best[0], b1 = best[1];
+    qs_tile_step<F16, false, true, 0>(acc[1 - YS], acc[YS], af, nullptr, nullptr, bfrag, best, pos);
+    if (best[0] != b0) btile[0] = ntiles - 1;
+    if (best[1] != b1) btile[1] = ntiles - 1;
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  tile(0, I0{}, std::false_type{});
+  int t = 1;
+  for (; t + 1 < ntiles; t += 2) {
+    tile(t, I1{}, std::true_type{});
+    tile(t + 1, I0{}, std::true_type{});
+  }
+  if (t < ntiles) {
+    tile(t, I1{}, std::true_type{});
+    last_scan(I1{});
+  } else {
+    last_scan(I0{});
   }
 #pragma unroll
   for (int ni = 0; ni < 2; ++ni) {

@@ -5,7 +5,7 @@
  * fm_debug_argtopz_exact_only, fm_debug_set_phase_events) are PROCESS-WIDE state, read by every call on
  * every stream: they exist so that tests can compare two implementations of one operator and so that the
  * benchmark can time the phases of the fused build; a production caller never touches them.  The probes
- * (fm_debug_copy, fm_debug_read) are plain kernels of known size.
+ * (fm_debug_copy, fm_debug_read, fm_debug_mfma) are plain kernels of known size.
  */
 #ifndef FASTMEM_DEBUG_H
 #define FASTMEM_DEBUG_H
@@ -68,6 +68,12 @@ int fm_debug_copy(void* dst, const void* src, int64_t nbytes, void* stream);
  * nothing is written (sink: 4 bytes of device memory, left untouched).  Times the
  * read bandwidth a kernel reaches on the device. */
 int fm_debug_read(const void* src, int64_t nbytes, void* sink, void* stream);
+
+/* Diagnostic: a register-resident stream of v_mfma_f32_32x32x16_bf16 (no memory, LDS or VALU work in
+ * the loop) over the first 5120 bf16 values at `operands` (n_operands >= 5120): iters * 2^33 flops per call.
+ * Times the rate the matrix pipes sustain on the device for those operand values (the device clocks such a
+ * loop lower the more the operand bits toggle).  sink: 4 bytes of device memory, left untouched. */
+int fm_debug_mfma(const void* operands, int64_t n_operands, int iters, void* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -66,6 +66,8 @@ def test_argument_errors_are_status_codes():
     assert lib.fm_lists_key_order(None, None, None, 0, 10, None, None, None) == 0   # no list: nothing to do
     assert lib.fm_lists_key_order(4096, 4096, 4096, 1, 10, 4096, None, None) == 1    # in place: refused before any launch
     assert b"in place" in lib.fm_last_error()
+    assert lib.fm_debug_mfma(None, 5120, 1, None, None) == 1                          # null pointers
+    assert lib.fm_debug_mfma(4096, 100, 1, 4096, None) == 1                           # too few operands
     with pytest.raises(ValueError):
         _lib.check(1)
 

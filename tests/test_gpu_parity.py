@@ -178,6 +178,47 @@ def test_qhash(ops, dtype, H, C, S, d):
     assert torch.equal(ops.qhash(*dev(A, q)).cpu(), h)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("C", [1, 5, 33, 64, 65, 128, 129, 192, 200, 320, 2051])
+def test_qhash_streaming_kernel_tile_counts(ops, dtype, C):
+    """The streaming hash kernel (d = 128, no scores written) pipelines 64-row tiles of A through two
+    accumulator sets: one, two, three (odd) and many tiles, ragged last tiles, the maximum in the first and in
+    the last row, and equal rows in different tiles (the first must win)."""
+    g = gen(310 + C)
+    H, S = 2, 700
+    A = torch.randn(H, C, 128, generator=g).to(dtype)
+    q = torch.randn(H, S, 128, generator=g).to(dtype)
+    if C > 1:
+        A[0, C - 1] = A[0, 0]                                        # equal rows, as far apart as they get
+        A[1, C - 1] = 4 * q[1, 0]                                    # query 0 of row 1: the last bucket by far
+        if C > 70:
+            A[0, 70] = A[0, 37]                                      # equal rows in neighbouring tiles
+    h, sc = ops.qhash(*dev(A, q), return_scores=True)
+    hs = ops.qhash(*dev(A, q))                                       # the streaming kernel
+    assert torch.equal(hs.cpu().long(), O.argmax_first(sc.cpu())), "hash is not the first argmax of the scores"
+    assert torch.equal(hs, h)
+    if C > 1:
+        assert not (hs[0] == C - 1).any()
+        assert int(hs[1, 0]) == C - 1
+        if C > 70:
+            assert not (hs[0] == 70).any()
+
+
+def test_probe_kernels_run_and_write_nothing(ops):
+    """The kernels of known size that the benchmark times for scale (a read stream, an MFMA stream)."""
+    from fast_memory_amd import _lib
+    lib = _lib.load()
+    src = torch.ones(1 << 20, dtype=torch.uint8, device="cuda")
+    operands = torch.randn(5120, generator=gen(320)).to(torch.bfloat16).cuda()
+    sink = torch.zeros(2, dtype=torch.float32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.fm_debug_read(src.data_ptr(), src.numel(), sink.data_ptr(), st))
+    _lib.check(lib.fm_debug_mfma(operands.data_ptr(), operands.numel(), 3, sink.data_ptr(), st))
+    _lib.check(lib.fm_debug_mfma(operands.data_ptr(), operands.numel(), 0, sink.data_ptr(), st))
+    sync()
+    assert sink.tolist() == [0.0, 0.0]
+
+
 # ------------------------------------------------------------------ a4/a5/a16
 @pytest.mark.parametrize("H,S,C", [(1, 24, 8), (3, 1000, 17), (8, 8160, 512), (2, 300, 2048)])
 def test_group_queries(ops, H, S, C):

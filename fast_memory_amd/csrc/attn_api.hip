@@ -17,7 +17,9 @@ bool hash_attn_mfma_supported(int d, int dtype, int N);
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
                    const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype, hipStream_t st);
+                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype, void* ws, size_t ws_bytes,
+                   hipStream_t st);
+size_t hash_attn_ring_workspace(int64_t max_items);
 int hash_attn_mfma_choice(int H, int Sq, int N, int C);
 bool hash_attn_mfma_per_row(int choice, int H, int Sq, int N, int C);
 bool local_attn_mfma_supported(int d, int dtype);
@@ -62,11 +64,16 @@ extern "C" int fm_hash_attn_fwd_launches(int H, int Sq, int N, int d, int C, int
   return hash_attn_mfma_per_row(choice, H, Sq, N, C) ? H : 1;
 }
 
-extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
-                                const int64_t* bucket_off, const int32_t* bucket_cnt,
-                                const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
-                                int64_t max_items, void* out, float* lse, int H, int Sq, int N,
-                                int d, int C, float sm_scale, int dtype, void* stream) {
+extern "C" size_t fm_hash_attn_fwd_workspace(int64_t max_items) {
+  return max_items >= 1 ? fm::hash_attn_ring_workspace(max_items) : 0;
+}
+
+extern "C" int fm_hash_attn_fwd_ws(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                                   const int64_t* bucket_off, const int32_t* bucket_cnt,
+                                   const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                                   int64_t max_items, void* out, float* lse, int H, int Sq, int N,
+                                   int d, int C, float sm_scale, int dtype, void* ws, size_t ws_bytes,
+                                   void* stream) {
   using namespace fm;
   FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
              "fm_hash_attn_fwd: H=%d Sq=%d N=%d C=%d d=%d", H, Sq, N, C, d);
@@ -79,16 +86,25 @@ extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, con
   hipStream_t st = as_stream(stream);
   if (g_force_generic != 1 && hash_attn_mfma_supported(d, dtype, N))
     return hash_attn_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items,
-                          out, lse, H, Sq, N, d, C, sm_scale, dtype, st);
+                          out, lse, H, Sq, N, d, C, sm_scale, dtype, ws, ws ? ws_bytes : 0, st);
   return hash_attn_generic(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
                            max_items, out, lse, Sq, N, d, C, sm_scale, dtype, st);
+}
+
+extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                                const int64_t* bucket_off, const int32_t* bucket_cnt,
+                                const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                                int64_t max_items, void* out, float* lse, int H, int Sq, int N,
+                                int d, int C, float sm_scale, int dtype, void* stream) {
+  return fm_hash_attn_fwd_ws(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse,
+                             H, Sq, N, d, C, sm_scale, dtype, nullptr, 0, stream);
 }
 
 // workspace layout of the one-call operator
 namespace fm {
 struct VarlenWs {
   size_t off_bucket_off, off_q_perm, off_bin_count, off_bin_off, off_items, off_n_items, off_group,
-      total;
+      off_attn, total;
   int64_t max_items;
 };
 static VarlenWs varlen_layout(int H, int C, int Sq) {
@@ -107,6 +123,7 @@ static VarlenWs varlen_layout(int H, int C, int Sq) {
   w.off_items = take(size_t(w.max_items) * sizeof(fm_item));
   w.off_n_items = take(sizeof(int32_t));
   w.off_group = take(fm_group_queries_workspace(H, C, Sq));
+  w.off_attn = take(fm_hash_attn_fwd_workspace(w.max_items));
   w.total = o;
   return w;
 }
@@ -147,8 +164,9 @@ static int varlen_run(const void* q, const void* k, const void* v, const int32_t
   rc = fm_group_queries(q_hash, H, C, Sq, q_perm, bin_count, bin_off, items, n_items, w.max_items,
                         base + w.off_group, fm_group_queries_workspace(H, C, Sq), stream);
   if (rc) return rc;
-  rc = fm_hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, w.max_items, out,
-                        lse, H, Sq, N, d, C, sm_scale, dtype, stream);
+  rc = fm_hash_attn_fwd_ws(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, w.max_items, out,
+                           lse, H, Sq, N, d, C, sm_scale, dtype, base + w.off_attn,
+                           fm_hash_attn_fwd_workspace(w.max_items), stream);
   if (rc) return rc;
   const int row_bytes = d * dtype_bytes(dtype);
   const int64_t nq = int64_t(H) * Sq;

@@ -493,7 +493,7 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
 int hash_attn_mfma_ring(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                         const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items,
                         const int32_t* n_items, int64_t max_items, void* out, float* lse, int Sq, int N, int C,
-                        float sm_scale, bool f16, int H, bool per_row, hipStream_t st);
+                        float sm_scale, bool f16, int H, bool per_row, void* ws, size_t ws_bytes, hipStream_t st);
 extern std::atomic<int> g_force_generic;
 
 // Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
@@ -550,14 +550,15 @@ bool hash_attn_mfma_per_row(int choice, int H, int Sq, int N, int C) {
 int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx,
                    const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
-                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype, hipStream_t st) {
+                   float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype, void* ws, size_t ws_bytes,
+                   hipStream_t st) {
   (void)d;
   int choice = hash_attn_mfma_choice(H, Sq, N, C);
   if (dtype == FM_F16 && choice == 0) choice = 1;
   const bool per_row = hash_attn_mfma_per_row(choice, H, Sq, N, C);
   if (choice == 3)
     return hash_attn_mfma_ring(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse, Sq,
-                               N, C, sm_scale, dtype == FM_F16, H, per_row, st);
+                               N, C, sm_scale, dtype == FM_F16, H, per_row, ws, ws_bytes, st);
   if (choice) {
     return hash_attn_mfma_staged(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out,
                                  lse, H, Sq, N, C, sm_scale, choice == 2, dtype == FM_F16, per_row, st);

@@ -224,10 +224,12 @@ def hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, s
     assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and bucket_off.dtype == torch.int64
     out = torch.empty_like(q)
     lse = torch.empty((H, Sq), dtype=torch.float32, device=q.device)
-    check(_lib.load().fm_hash_attn_fwd(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
-                                       _p(groups.q_perm), _p(groups.items), _p(groups.n_items),
-                                       groups.max_items, _p(out), _p(lse), H, Sq, N, d, C,
-                                       float(sm_scale), _dt(q), _stream(q)))
+    lib = _lib.load()
+    ws = torch.empty(int(lib.fm_hash_attn_fwd_workspace(groups.max_items)), dtype=torch.uint8, device=q.device)
+    check(lib.fm_hash_attn_fwd_ws(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
+                                  _p(groups.q_perm), _p(groups.items), _p(groups.n_items),
+                                  groups.max_items, _p(out), _p(lse), H, Sq, N, d, C,
+                                  float(sm_scale), _dt(q), _p(ws), ws.numel(), _stream(q)))
     return out, lse
 
 

@@ -156,6 +156,18 @@ int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t*
                      const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
                      float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype,
                      void* stream);
+/* The same with fm_hash_attn_fwd_workspace(max_items) bytes of device memory to work in (no counterpart in
+ * the reference, whose launch grid is one program per 64 queries of a bucket, triton_kernel.py:99-106):
+ * where buckets receive more than FM_QTILE queries on average a workgroup takes three items of a bucket
+ * together, and with the workspace the groups are listed first so that every workgroup started has one --
+ * without it two of three return at once, which leaves compute units idle (1.3 x slower at 128 queries per
+ * bucket).  Same results bit for bit.  ws = NULL is fm_hash_attn_fwd. */
+size_t fm_hash_attn_fwd_workspace(int64_t max_items);
+int fm_hash_attn_fwd_ws(const void* q, const void* k, const void* v, const int32_t* k_idx,
+                        const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
+                        const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
+                        float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype,
+                        void* ws, size_t ws_bytes, void* stream);
 
 /* ---- lists in ascending key order, for the gathered attention ------------------
  * The kernel of triton_kernel.py:230-272 walks a bucket's list in stored order, and

@@ -455,6 +455,49 @@ def test_attention_grouped_forward_kernels(ops, which, case):
         assert torch.equal(out, o1) and torch.equal(lse, l1)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_with_listed_item_groups(ops, dtype):
+    """More than 64 queries per bucket on average: with its workspace the forward lists the groups of three
+    items first (fm_hash_attn_fwd_ws), without it a workgroup is started per item and two of three return.  The
+    same bits either way, over buckets of 0, 1, 2, 3, 4 and 23 items, the last item of every size, rows with and
+    without queries outside every bucket, and more than 1024 items (the listing walks them 1024 at a time)."""
+    H, S, N, C, Z, d = 3, 24000, 3000, 60, 150, 128
+    q, k, v, kh, cnt, qh = make_attn_case(37, H, S, N, C, Z, d, dtype, std=0.8)
+    sizes = [0, 1, 64, 65, 128, 129, 192, 193, 200, 256, 1450, 63]          # queries of buckets 0..11 of row 0
+    pos = 0
+    for b, n in enumerate(sizes):
+        qh[0, pos:pos + n] = b
+        pos += n
+    qh[0, pos:] = torch.randint(12, C, (S - pos,), generator=gen(38))
+    qh[1, ::7] = -1                                                          # in no bucket
+    assert ops.hash_attn_fwd_kernel_name(H, S, N, d, C, dtype).startswith("hash_attn_ring_kernel")
+    qd, kd, vd, khd, cntd, qhd = dev(q, k, v, kh, cnt, qh)
+    groups = ops.group_queries(qhd.int(), C)
+    assert int(groups.n_items.item()) > 1024
+    off = ops.bucket_offsets(cntd.int())
+    flat = khd.int().reshape(-1).contiguous()
+    from fast_memory_amd import _lib
+    lib = _lib.load()
+    res = []
+    for with_ws in (False, True):
+        out = torch.full(q.shape, 7.0, dtype=dtype, device="cuda")
+        lse = torch.full((H, S), 7.0, dtype=torch.float32, device="cuda")
+        ws = torch.empty(int(lib.fm_hash_attn_fwd_workspace(groups.max_items)) if with_ws else 0, dtype=torch.uint8,
+                         device="cuda")
+        _lib.check(lib.fm_hash_attn_fwd_ws(
+            qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), flat.data_ptr(), off.data_ptr(), cntd.int().contiguous().data_ptr(),
+            groups.q_perm.data_ptr(), groups.items.data_ptr(), groups.n_items.data_ptr(), groups.max_items,
+            out.data_ptr(), lse.data_ptr(), H, S, N, d, C, float(d ** -0.5), {torch.bfloat16: 1, torch.float16: 2}[dtype],
+            ws.data_ptr() if with_ws else None, ws.numel(), torch.cuda.current_stream().cuda_stream))
+        sync()
+        res.append((out, lse))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    assert bool((res[1][1][1, ::7] == 7.0).all())                            # rows of no bucket: untouched
+    ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh.clamp(min=0), d ** -0.5)
+    keep = qh >= 0
+    assert_attn_close(res[1][0][keep], res[1][1][keep], ro[keep], rl[keep], dtype, "listed groups")
+
+
 def test_attention_a_launch_per_row_finds_every_rows_items(ops):
     """Eleven rows with very different numbers of work items, among them rows whose queries all carry a hash
     outside [0, C) (no item at all; their output rows are never written): the per-row launches write exactly

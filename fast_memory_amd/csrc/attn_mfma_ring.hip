@@ -7,49 +7,56 @@ namespace fm {
 
 
 // heads[j] = the first item of the j-th group of up to three consecutive items of one bucket, in item order;
-// *n_heads = their number.  One workgroup walks the items 1024 at a time: an item's place in its bucket is its
-// distance from the bucket's first item (a running maximum over the indices of the items that start a bucket),
-// the groups' first items are counted and packed by a prefix sum.
-__global__ __launch_bounds__(1024) void ring_heads_kernel(const fm_item* __restrict__ items,
-                                                          const int32_t* __restrict__ n_items,
-                                                          int32_t* __restrict__ heads, int32_t* __restrict__ n_heads) {
-  __shared__ int scan_tmp[17];
-  __shared__ int wave_max[16];
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int n = *n_items;
-  int bucket_start = 0;  // index of the item that starts the bucket of the last item seen so far
-  int n_out = 0;
-  for (int c0 = 0; c0 < n; c0 += 1024) {
-    const int i = c0 + tid;
-    const bool valid = i < n;
-    fm_item it = {0, 0, 0, 0};
-    if (valid) it = items[i];
-    bool starts = valid && i == 0;
-    if (valid && i > 0) {
-      const fm_item pr = items[i - 1];
-      starts = pr.row != it.row || pr.bucket != it.bucket;
-    }
-    int s = starts ? i : -1;  // inclusive running maximum
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int t = __shfl_up(s, o);
-      if (lane >= o) s = max(s, t);
-    }
-    if (lane == 63) wave_max[w] = s;
-    __syncthreads();
-    int before = bucket_start;
-    for (int j = 0; j < w; ++j) before = max(before, wave_max[j]);
-    s = max(s, before);
-    int all = bucket_start;
-    for (int j = 0; j < 16; ++j) all = max(all, wave_max[j]);
-    const bool head = valid && (i - s) % 3 == 0;
-    int total;
-    const int pos = block_excl_scan(head ? 1 : 0, scan_tmp, &total);  // (its barriers also fence wave_max)
-    if (head) heads[n_out + pos] = i;
-    n_out += total;
-    bucket_start = all;
+// *n_heads = their number.  Two passes of one workgroup per 1024 items: the first counts the groups' first items
+// of its 1024, the second adds the counts of the workgroups before it and packs them by a prefix sum.  An item's
+// place in its bucket is its distance from the bucket's first item, found by a galloping, then a binary search
+// to the left (a bucket may have thousands of items).
+__device__ __forceinline__ bool ring_is_head(const fm_item* __restrict__ items, int i) {
+  const fm_item it = items[i];
+  auto same = [&](int j) { return items[j].row == it.row && items[j].bucket == it.bucket; };
+  int lo = i, step = 1;  // invariant: items lo..i belong to the bucket
+  while (lo - step >= 0 && same(lo - step)) {
+    lo -= step;
+    step <<= 1;
   }
-  if (tid == 0) *n_heads = n_out;
+  int bad = max(lo - step, -1);  // -1 or an item of another bucket, bad < lo
+  while (lo - bad > 1) {
+    const int mid = (lo + bad) >> 1;
+    if (same(mid))
+      lo = mid;
+    else
+      bad = mid;
+  }
+  return (i - lo) % 3 == 0;
+}
+
+__global__ __launch_bounds__(1024) void ring_heads_count_kernel(const fm_item* __restrict__ items,
+                                                                const int32_t* __restrict__ n_items,
+                                                                int32_t* __restrict__ counts) {
+  __shared__ int scan_tmp[17];
+  const int i = blockIdx.x * 1024 + threadIdx.x;
+  const bool head = i < *n_items && ring_is_head(items, i);
+  int total;
+  block_excl_scan(head ? 1 : 0, scan_tmp, &total);
+  if (threadIdx.x == 0) counts[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(1024) void ring_heads_write_kernel(const fm_item* __restrict__ items,
+                                                                const int32_t* __restrict__ n_items,
+                                                                const int32_t* __restrict__ counts,
+                                                                int32_t* __restrict__ heads,
+                                                                int32_t* __restrict__ n_heads) {
+  __shared__ int scan_tmp[17];
+  int before = 0;
+  for (int j = threadIdx.x; j < int(blockIdx.x); j += 1024) before += counts[j];
+  int base;
+  block_excl_scan(before, scan_tmp, &base);
+  const int i = blockIdx.x * 1024 + threadIdx.x;
+  const bool head = i < *n_items && ring_is_head(items, i);
+  int total;
+  const int pos = block_excl_scan(head ? 1 : 0, scan_tmp, &total);
+  if (head) heads[base + pos] = i;
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) *n_heads = base + total;
 }
 
 template <bool F16>
@@ -137,7 +144,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                       out + qbase * kSD, lse + qbase, ring_lds, it.bucket);
 }
 
-size_t hash_attn_ring_workspace(int64_t max_items) { return (size_t(max_items) + 64) * sizeof(int32_t); }
+// n_heads (64 ints reserved), heads[max_items], counts[ceil(max_items / 1024)]
+size_t hash_attn_ring_workspace(int64_t max_items) {
+  return (size_t(max_items) + 64 + size_t(ceil_div(max_items, int64_t(1024)))) * sizeof(int32_t);
+}
 
 int hash_attn_mfma_ring(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                         const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items,
@@ -155,7 +165,10 @@ int hash_attn_mfma_ring(const void* q, const void* k, const void* v, const int32
   if (!per_row && ws && ws_bytes >= hash_attn_ring_workspace(max_items) && int64_t(Sq) >= int64_t(FM_QTILE) * C) {
     n_heads = static_cast<int32_t*>(ws);
     heads = n_heads + 64;
-    hipLaunchKernelGGL(ring_heads_kernel, dim3(1), dim3(1024), 0, st, items, n_items, heads, n_heads);
+    int32_t* counts = heads + max_items;
+    const unsigned nblk = unsigned(ceil_div(max_items, int64_t(1024)));
+    hipLaunchKernelGGL(ring_heads_count_kernel, dim3(nblk), dim3(1024), 0, st, items, n_items, counts);
+    hipLaunchKernelGGL(ring_heads_write_kernel, dim3(nblk), dim3(1024), 0, st, items, n_items, counts, heads, n_heads);
   }
 #define FM_RING_LAUNCH(F16, GRID, ROW)                                                                            \
   do {                                                                                                            \

@@ -228,11 +228,13 @@ def bench_decode_batch(args):
         f"for {total_keys} keys")
     evs = []
 
-    def step(record=True):
-        a, b = ev_pair()
-        a.record()
+    def step(record=True, events=True):
+        if events:
+            a, b = ev_pair()
+            a.record()
         mo, ml, h = batch.attend(q, sm_scale)
-        b.record()
+        if events:
+            b.record()
         L = kl.shape[2]
         lo, ll = ops.local_attn_fwd(q.reshape(n_seq * H * G, 1, d), kl.reshape(n_seq * H, L, d),
                                     vl.reshape(n_seq * H, L, d), sm_scale, True)
@@ -253,6 +255,26 @@ def bench_decode_batch(args):
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     qheads = n_seq * H * G
     attn_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    # the same step recorded once into a HIP graph and replayed (the library records kernels only; torch's
+    # allocator serves the step's tensors from the graph's own pool): what a serving loop that replays pays
+    graph_replay = None
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            g_out, g_lse, g_h = step(False, events=False)
+        for _ in range(max(args.warmup, 2)):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        g_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        graph_replay = {"ms_per_step": g_ms, "value": qheads / (g_ms * 1e-3),
+                        "same_bits_as_eager": bool(torch.equal(g_out, out) and torch.equal(g_lse, lse) and torch.equal(g_h, h))}
+        log(f"[bench] c3 step replayed from a HIP graph: {g_ms:.3f} ms {graph_replay}")
+    except Exception as exc:  # a graph that cannot be captured here is reported, not fatal
+        log(f"[bench] HIP graph capture of the c3 step failed: {exc!r}")
     hc = h.cpu()
     alg_bytes = 0
     for s, (N, C, Z) in enumerate(lens):
@@ -303,6 +325,7 @@ def bench_decode_batch(args):
                      "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": attn_ms},
         "cpu_baseline": cpu,
         "index_build": {"keys_per_s": total_keys / (build_ms * 1e-3), "ms": build_ms, "keys": total_keys},
+        "graph_replay": graph_replay,
     }
     log(f"[bench] c3 step {ms_per_step:.3f} ms -> {line['value'] / 1e6:.2f} M query-heads/s; decode kernel "
         f"{attn_ms:.3f} ms = {achieved:.0f} GB/s algorithmic")

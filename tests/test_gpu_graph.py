@@ -1,0 +1,54 @@
+"""The query path under HIP graph capture: the hash of the queries and the entry point that allocates nothing
+(fm_qhash -> fm_attention_hash_varlen_static, both through the C ABI) recorded once into a graph and replayed.
+The library records kernels only (no memset or copy nodes), every replay is checked against an eager run on the
+same inputs, with eager work and synchronisations between the replays, and the inputs change between replays
+(a graph that had baked in results instead of work would show)."""
+import pytest
+import torch
+
+from fast_memory_amd import _lib, ops
+from tests.util import dev, gen, make_attn_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_hash_and_attention_replayed_from_a_graph(dtype):
+    H, S, N, C, Z, d = 4, 1500, 6000, 48, 256, 128
+    q, k, v, kh, cnt, _ = make_attn_case(41, H, S, N, C, Z, d, dtype)
+    A = torch.randn(H, C, d, generator=gen(42)).to(dtype)
+    q, k, v, A = dev(q, k, v, A)
+    kh, cnt = dev(kh.int(), cnt.int())
+    scale = d ** -0.5
+    lib = _lib.load()
+    dt = {torch.bfloat16: 1, torch.float16: 2}[dtype]
+
+    def run(qh_buf, out_buf, lse_buf):
+        st = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.fm_qhash(A.data_ptr(), q.data_ptr(), qh_buf.data_ptr(), None, H, C, S, d, dt, st))
+        _lib.check(lib.fm_attention_hash_varlen_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), kh.data_ptr(),
+                                                       cnt.data_ptr(), qh_buf.data_ptr(), out_buf.data_ptr(),
+                                                       lse_buf.data_ptr(), H, S, N, d, C, scale, dt, st))
+
+    bufs = lambda: (torch.zeros(H, S, dtype=torch.int32, device="cuda"), torch.zeros_like(q),
+                    torch.zeros(H, S, dtype=torch.float32, device="cuda"))
+    qh_e, out_e, lse_e = bufs()
+    qh_g, out_g, lse_g = bufs()
+    run(qh_e, out_e, lse_e)          # the first call on a device also looks up the static array: not under capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(qh_g, out_g, lse_g)
+    for rep in range(4):
+        if rep:                       # new queries in place: the graph reads the same buffers
+            q.copy_((torch.randn(H, S, d, generator=gen(50 + rep)) * 0.5).to(dtype))
+        graph.replay()
+        torch.cuda.synchronize()
+        run(qh_e, out_e, lse_e)       # eager, between the replays, over the same static array
+        torch.cuda.synchronize()
+        assert torch.equal(qh_g, qh_e), f"replay {rep}: hashes differ"
+        assert torch.equal(out_g.view(torch.int16), out_e.view(torch.int16)), f"replay {rep}: out differs"
+        assert torch.equal(lse_g.view(torch.int32), lse_e.view(torch.int32)), f"replay {rep}: lse differs"
+        assert float(out_g.float().abs().sum()) > 0
+    ref_out, ref_lse = ops.attention_hash_varlen_i32(q, k, v, kh, cnt, qh_e, scale)
+    assert torch.equal(out_g.view(torch.int16), ref_out.view(torch.int16)) and torch.equal(lse_g, ref_lse)

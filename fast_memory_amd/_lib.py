@@ -73,6 +73,7 @@ SIGNATURES = {
     "fm_debug_argtopz_exact_only": (None, [c_int]),
     "fm_debug_copy": (c_int, [P, P, c_int64, P]),
     "fm_debug_read": (c_int, [P, c_int64, P, P]),
+    "fm_debug_fused_filter": (None, [c_int]),
     "fm_debug_mfma": (c_int, [P, c_int64, c_int, P, P]),
     "fm_debug_set_phase_events": (None, [P, c_int]),
 }

@@ -26,19 +26,25 @@
 //
 // Results are bit-identical to fm_project + fm_argtopz_f32: both compute every Y
 // element with v_mfma_f32_32x32x16_bf16 in ascending 16-element steps with keys
-// on the A operand.
+// on the A operand (the third form of phase 1 with v_mfma_f32_16x16x32 in ascending
+// 32-element steps, which gives the same sums: the tests compare all forms).
 //
 // Roofline of phase 1: MFMA, 2*d flops per (key, bucket) pair; K is re-read once
 // per 512-bucket slab from L2.  Phases 0, 2, 3 are HBM/L2-bound and small.
+#include <atomic>
 #include <type_traits>
 
 #include "mfma_tile.hpp"
+#include "mma16.hpp"
 #include "select.hpp"
 
 namespace fm {
 
 int launch_argtopz(const float* Y, int64_t rows, int N, int64_t ldy, int Zc, int32_t* idx_out, float* val_out,
                    const int32_t* row_map, const int32_t* n_rows_dev, hipStream_t st);
+
+// 0 = the plan decides, 1 = never the form with the epilogue between the MFMAs (tests compare the two)
+std::atomic<int> g_fused_filter_form{0};
 
 constexpr int kFD = 128;          // head dimension the fused kernels are built for
 constexpr int kFWaves = 8;        // compute waves per workgroup
@@ -59,6 +65,7 @@ constexpr int kCandRegsSmall = 32;  // ... with 256 or 512 threads per row
 struct FusedPlan {
   int ns, stride, rank, n_splits, slabs, n_writers, cap_w, sel_threads;
   bool wide;  // phase 1 takes fused_filter_wide_kernel (slabs of 1024 buckets)
+  int ping;   // ... or fused_filter_ping_kernel, in its form 1, 2 or 3 (rounds and passes of the emission); 0 = not
   int64_t ld_s, ldy;
   size_t off_Ks, off_Ys, off_tau, off_cand, off_cnt, off_fail, off_nfail, off_Yf, total;
 };
@@ -74,6 +81,7 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   s = std::max<int64_t>(1, std::min<int64_t>(32, std::min(s, ntiles)));
   p.n_splits = int(s);
   p.n_writers = 2 * p.n_splits;
+  p.ping = 0;
   // Sample size and threads per row of the selection.  A smaller sample makes phase 0 cheaper and the
   // threshold noisier: a row keeps m = rank*stride +- stride*sqrt(rank) candidates, which the
   // selection must hold in registers (R per thread, T = NT / n_writers threads per writer segment,
@@ -84,29 +92,47 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   const int P = next_pow2(Z);
   bool found = false;
   double m_exp = 0;
-  for (int ns_try : {4096, 8192, 16384, 32768}) {
-    p.stride = N / ns_try;
-    p.ns = N / p.stride;
-    const double mu = double(Z) * p.ns / N;
-    p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
-    if (p.rank * 4 > p.ns) continue;
-    m_exp = double(p.rank) * N / p.ns;
-    // (the two small samples only where they keep at most 32 % more candidates than Z: short memories with
-    // long lists, where a 16 K sample would be a quarter of all keys and phase 0 a quarter of the projection)
-    if (ns_try < 16384 && m_exp > 1.32 * Z) continue;
-    const double per_w = m_exp / p.n_writers;
-    const double sd_w = sqrt(pow(double(N) / p.ns * sqrt(double(p.rank)) / p.n_writers, 2) + per_w);
-    for (int nt = 256; nt <= kSelThreads && !found; nt *= 2)
-      if (nt * 16 >= P && (nt / p.n_writers) * (nt < kSelThreads ? kCandRegsSmall : kCandRegs) >= per_w + 5.0 * sd_w) {
-        p.sel_threads = nt;
-        found = true;
-      }
-    if (found) break;
+  auto search = [&]() {
+    found = false;
+    for (int ns_try : {4096, 8192, 16384, 32768}) {
+      p.stride = N / ns_try;
+      p.ns = N / p.stride;
+      const double mu = double(Z) * p.ns / N;
+      p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
+      if (p.rank * 4 > p.ns) continue;
+      m_exp = double(p.rank) * N / p.ns;
+      // (the two small samples only where they keep at most 32 % more candidates than Z: short memories with
+      // long lists, where a 16 K sample would be a quarter of all keys and phase 0 a quarter of the projection)
+      if (ns_try < 16384 && m_exp > 1.32 * Z) continue;
+      const double per_w = m_exp / p.n_writers;
+      const double sd_w = sqrt(pow(double(N) / p.ns * sqrt(double(p.rank)) / p.n_writers, 2) + per_w);
+      for (int nt = 256; nt <= kSelThreads && !found; nt *= 2)
+        if (nt * 16 >= P && (nt / p.n_writers) * (nt < kSelThreads ? kCandRegsSmall : kCandRegs) >= per_w + 5.0 * sd_w) {
+          p.sel_threads = nt;
+          found = true;
+        }
+      if (found) break;
+    }
+    if (!found) {
+      if (p.rank * 4 > p.ns) return false;
+      p.sel_threads = kSelThreads;
+    }
+    return true;
+  };
+  // The form with the epilogue between the MFMAs where the wide form applies: a writer is a key split there.
+  // Its emission handles a lane's first NR candidates of a group (16 keys x 128 buckets) and the group's first
+  // ND * 64 in straight-line code; the forms are (NR, ND) = (4, 1), (6, 2), (7, 3), picked so that 3.5
+  // standard deviations of a group's candidates fit the passes.
+  if (p.wide && g_fused_filter_form.load(std::memory_order_relaxed) != 1) {
+    p.n_writers = p.n_splits;
+    if (search()) {
+      const double per_group = 2048.0 * m_exp / N;
+      const int nd = int(ceil((per_group + 3.5 * sqrt(per_group)) / 64.0));
+      if (nd >= 1 && nd <= 3) p.ping = nd;
+    }
+    if (!p.ping) p.n_writers = 2 * p.n_splits;
   }
-  if (!found) {
-    if (p.rank * 4 > p.ns) return false;
-    p.sel_threads = kSelThreads;
-  }
+  if (!p.ping && !search()) return false;
   p.cap_w = int(1.35 * m_exp / p.n_writers) + 64;  // > 16: the overflow guard keeps 16 slots free
   p.ld_s = (int64_t(p.ns) + 3) / 4 * 4;
   p.ldy = (int64_t(N) + 3) / 4 * 4;
@@ -594,6 +620,268 @@ __global__ __launch_bounds__(512) void fused_filter_wide_kernel(
   }
 }
 
+// ---- phase 1, form with the epilogue between the MFMAs ----------------------------------------
+// The same filter on v_mfma_f32_16x16x32 (the same sums: both instructions contract the 128 dimensions in
+// ascending order).  A wave still owns 128 buckets and takes the keys 16 at a time: a *group* is 16 keys x 128
+// buckets = eight independent accumulator chains of four k-steps, 32 MFMAs, and the accumulators of two groups fit
+// where those of one 32-key half tile were.  While the MFMAs of one group issue, the epilogue of the group
+// before it is issued between them, slot by slot (VALU work of a wave that sits between the MFMAs of four or
+// more independent chains of the same wave costs next to no time of its own on this hardware; work that
+// follows the MFMAs, as in the forms above, is only partly hidden by the SIMD's other wave).  For that the
+// epilogue is straight-line code:
+//   slots 0-7    threshold test of the group's 32 accumulator registers per lane (two VALU instructions each,
+//                the outcomes shifted into a 32-bit mask) and the dump of the registers to the wave's LDS slab;
+//   slots 8-9    a wave scan of the lanes' candidate counts: a lane's first NR candidates get places in a queue
+//                of the wave;
+//   then NR rounds in which every lane writes (lane, register) of one of its candidates to its place;
+//   then ND passes in which lane j takes the queue's j-th candidate: value from the dump, its bucket's cursor
+//   from LDS by an atomic add (a bucket belongs to one wave: no contention beyond the wave's own lanes), key
+//   code and one 8-byte store -- three stages a pass, as far apart as the step allows, each waits for LDS.
+//   Every lane stores a candidate, not only those whose bucket column it holds.
+// Candidates beyond NR per lane or ND * 64 per group (the plan picks NR and ND from the expected pass rate;
+// keys that cluster make such groups less rare than even rates would) are appended by loops after the last slot.
+// A writer is a key split, so a row has n_splits segments; records carry the same key codes as above, the
+// selection does not see which form ran.
+constexpr int kFPDumpLd = 36;   // floats per lane in the dump: 32 accumulator registers + 4 (bank spread of the 16-byte stores)
+constexpr int kFPQueue = 256;   // queue places of a group's candidates; lanes without one write behind it
+
+struct FpShared {
+  bf16_t keys[2][kFKeys * kFLd];
+  float dump[kFWaves][64 * kFPDumpLd];
+  uint32_t queue[kFWaves][kFPQueue + 64];
+  uint32_t cursor[kFWaves][128 + 64];  // a bucket's candidate count so far; lanes without a candidate add behind them
+};
+
+template <int N, typename F>
+__device__ __forceinline__ void fp_static_for(F&& f) {
+  if constexpr (N > 0) {
+    fp_static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+// key index -> the code fused_key_of_code() undoes
+__device__ __forceinline__ uint32_t fused_code_of_key(uint32_t key) {
+  return (key & ~31u) | (key & 3u) | ((key >> 1) & 12u) | ((key << 2) & 16u);
+}
+
+template <bool F16, int NR, int ND>
+__global__ __launch_bounds__(512) void fused_filter_ping_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ K, const float* __restrict__ tau,
+    uint2* __restrict__ cand, int32_t* __restrict__ cnt, int C, int N, int n_splits, int cap_w) {
+  __shared__ __attribute__((aligned(16))) FpShared sm;
+  const int sk = blockIdx.x, slab = blockIdx.y, h = blockIdx.z;
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+  const int g = l >> 4, c = l & 15;
+  const int n_writers = n_splits;
+  const bf16_t* Kh = K + int64_t(h) * N * kFD;
+  const int ntiles = (N + kFKeys - 1) / kFKeys;
+  const int my_tiles = sk < ntiles ? (ntiles - sk + n_splits - 1) / n_splits : 0;  // tiles sk + i*n_splits
+
+  // staging: chunks tid and tid + 512 of a tile's 1024 16-byte chunks (rows tid/16 and 32 + tid/16)
+  uint4 st0, st1;
+  auto fetch = [&](int i) {
+    const int64_t key0 = (int64_t(sk) + int64_t(i) * n_splits) * kFKeys + (tid >> 4);
+    st0 = key0 < N ? reinterpret_cast<const uint4*>(Kh + key0 * kFD)[tid & 15] : make_uint4(0, 0, 0, 0);
+    st1 = key0 + 32 < N ? reinterpret_cast<const uint4*>(Kh + (key0 + 32) * kFD)[tid & 15] : make_uint4(0, 0, 0, 0);
+  };
+  auto stash = [&](int buf) {
+    *reinterpret_cast<uint4*>(&sm.keys[buf][(tid >> 4) * kFLd + (tid & 15) * 8]) = st0;
+    *reinterpret_cast<uint4*>(&sm.keys[buf][(32 + (tid >> 4)) * kFLd + (tid & 15) * 8]) = st1;
+  };
+
+  const int cb = slab * kFWSlab + w * 128;  // this wave's first bucket
+  const bool active = cb < C;
+  const bf16_t* Ah = A + int64_t(h) * C * kFD;
+  const int64_t wg_row0 = int64_t(h) * C + int64_t(slab) * kFWSlab;
+  char* cbase = reinterpret_cast<char*>(cand + (wg_row0 + w * 128) * n_writers * int64_t(cap_w));
+  float* dump = sm.dump[w];
+  uint32_t* queue = sm.queue[w];
+  uint32_t* cursor = sm.cursor[w];
+  for (int t = l; t < 128 + 64; t += 64) cursor[t] = 0;
+
+  // resident bucket fragments: bucket cb + 16 bt + c, dimensions 32 ks + 8 g ..
+  uint4 bfrag[8][4];
+  float th[8];
+#pragma unroll
+  for (int bt = 0; bt < 8; ++bt) {
+    const int row = cb + bt * 16 + c;
+    const bool ok = row < C;
+    const uint4* pa = reinterpret_cast<const uint4*>(Ah + int64_t(ok ? row : 0) * kFD + g * 8);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) bfrag[bt][ks] = ok ? pa[4 * ks] : make_uint4(0, 0, 0, 0);
+    th[bt] = ok ? tau[int64_t(h) * C + row] : INFINITY;
+  }
+#pragma unroll
+  for (int bt = 0; bt < 8; ++bt) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+      asm volatile("" ::"v"(bfrag[bt][ks].x), "v"(bfrag[bt][ks].y), "v"(bfrag[bt][ks].z), "v"(bfrag[bt][ks].w));
+    asm volatile("" ::"v"(th[bt]));
+  }
+
+  f32x4 acc[2][8];  // [group parity][bucket tile]
+  uint4 af[2];      // A fragment of a k-step, [k-step parity]
+  uint32_t msk = 0, msk0 = 0;
+  int n_mine = 0, base = 0, base0 = 0, total = 0;
+  // dense passes in flight: descriptor, value, bucket, slot of lane j's candidate
+  uint32_t d_desc[ND], d_slot[ND];
+  float d_val[ND];
+  bool d_ok[ND];
+
+  // LDS address of this lane's A fragment of (buffer, half, key tile kt), k-step 0
+  auto frag_ptr = [&](int buf, int grp) -> const bf16_t* {  // grp = 2 half + kt: keys 16 grp .. of the tile
+    return &sm.keys[buf][(grp * 16 + c) * kFLd + g * 8];
+  };
+
+  // the candidate (lane L, register e) of the group whose first key is key0: checks, cursor and store
+  auto emit_one = [&](bool valid, uint32_t L, uint32_t e, float val, uint32_t key0) {
+    const uint32_t key = key0 + 4u * (L >> 4) + (e & 3u);
+    const uint32_t bl = (e >> 2) * 16u + (L & 15u);
+    valid = valid && key < uint32_t(N);
+    const uint32_t slot = atomicAdd(&cursor[valid ? bl : 128u + uint32_t(l)], 1u);
+    if (valid && slot < uint32_t(cap_w)) {
+      const uint2 rec = make_uint2(__float_as_uint(val), fused_code_of_key(key));
+      *reinterpret_cast<uint2*>(cbase + ((bl * uint32_t(n_writers) + uint32_t(sk)) * uint32_t(cap_w) + slot) * 8u) = rec;
+    }
+  };
+
+  // One group step, slot S of 32.  DO_MFMA: the MFMA (k-step S / 8, bucket tile S % 8) of the group at `fp` into
+  // acc[P]; DO_EPI: the epilogue of the group before it (acc[1 - P], first key key0_old).
+  auto group_step = [&](auto P_, auto DO_MFMA_, auto DO_EPI_, const bf16_t* fp, const bf16_t* fp_next, uint32_t key0_old) {
+    constexpr int P = decltype(P_)::value;
+    constexpr bool DO_MFMA = decltype(DO_MFMA_)::value, DO_EPI = decltype(DO_EPI_)::value;
+    fp_static_for<32>([&](auto S_) {
+      constexpr int S = decltype(S_)::value;
+      constexpr int ks = S >> 3, bt = S & 7;
+      if constexpr (DO_MFMA) {
+        if constexpr (bt == 0) {
+          if constexpr (ks < 3)
+            af[(ks + 1) & 1] = *reinterpret_cast<const uint4*>(fp + (ks + 1) * 32);
+          else if (fp_next)
+            af[0] = *reinterpret_cast<const uint4*>(fp_next);
+        }
+        acc[P][bt] = Mma<F16>::m16(af[ks & 1], bfrag[bt][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[P][bt]);
+      }
+      if constexpr (DO_EPI) {
+        constexpr int Q = 1 - P;
+        if constexpr (S < 8) {
+          // the four registers of bucket tile S: mask bit 31 - (4 bt + i)
+          if constexpr (S == 0) msk = 0;
+          asm volatile("v_cmp_nlt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc\n\t"
+                       "v_cmp_nlt_f32 vcc, %3, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc\n\t"
+                       "v_cmp_nlt_f32 vcc, %4, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc\n\t"
+                       "v_cmp_nlt_f32 vcc, %5, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
+                       : "+v"(msk)
+                       : "v"(acc[Q][S][0]), "v"(th[S]), "v"(acc[Q][S][1]), "v"(acc[Q][S][2]), "v"(acc[Q][S][3])
+                       : "vcc");
+          *reinterpret_cast<float4*>(&dump[l * kFPDumpLd + 4 * S]) =
+              make_float4(acc[Q][S][0], acc[Q][S][1], acc[Q][S][2], acc[Q][S][3]);
+        } else if constexpr (S == 8) {
+          msk0 = msk;
+          n_mine = __popc(msk);
+          base = wave_incl_scan_dpp(min(n_mine, NR));  // the queue takes a lane's first NR candidates
+        } else if constexpr (S == 9) {
+          total = __builtin_amdgcn_readlane(base, 63);
+          base -= min(n_mine, NR);
+          base0 = base;
+        } else if constexpr (S < 10 + NR) {
+          // a round: one candidate per lane to its place in the queue
+          const bool has = msk != 0u;
+          const uint32_t p = uint32_t(__builtin_ctz(msk | 0x80000000u));
+          queue[has && base < kFPQueue ? base : kFPQueue + l] = (uint32_t(l) << 5) | p;
+          base += has ? 1 : 0;
+          msk = has ? (msk & (msk - 1u)) : msk;
+        } else {
+          // dense passes: three stages a pass, staggered by one slot from pass to pass
+          constexpr int S0 = 10 + NR + 1;  // first stage of pass 0 (a slot after the last round)
+          constexpr int gap = (31 - S0 - (ND - 1)) / 2;  // as far apart as the step allows: each stage waits for LDS
+          fp_static_for<ND>([&](auto D_) {
+            constexpr int D = decltype(D_)::value;
+            if constexpr (S == S0 + D) {
+              d_ok[D] = D * 64 + l < total;
+              d_desc[D] = queue[min(D * 64 + l, kFPQueue - 1)];
+            } else if constexpr (S == S0 + D + gap) {
+              const uint32_t L = d_desc[D] >> 5, e = 31u - (d_desc[D] & 31u);
+              d_val[D] = dump[__umul24(L, kFPDumpLd) + e];
+              const uint32_t key = key0_old + 4u * (L >> 4) + (e & 3u);
+              d_ok[D] = d_ok[D] && key < uint32_t(N);
+              d_slot[D] = atomicAdd(&cursor[d_ok[D] ? (e >> 2) * 16u + (L & 15u) : 128u + uint32_t(l)], 1u);
+            } else if constexpr (S == S0 + D + 2 * gap) {
+              const uint32_t L = d_desc[D] >> 5, e = 31u - (d_desc[D] & 31u);
+              const uint32_t key = key0_old + 4u * (L >> 4) + (e & 3u);
+              const uint32_t bl = (e >> 2) * 16u + (L & 15u);
+              if (d_ok[D] && d_slot[D] < uint32_t(cap_w)) {
+                const uint2 rec = make_uint2(__float_as_uint(d_val[D]), fused_code_of_key(key));
+                *reinterpret_cast<uint2*>(cbase + (__umul24(__umul24(bl, uint32_t(n_writers)) + uint32_t(sk), uint32_t(cap_w)) + d_slot[D]) * 8u) = rec;
+              }
+            }
+          });
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if constexpr (DO_EPI) {
+      // What the rounds and passes above did not reach.  A lane's candidates beyond the NR-th are the bits the
+      // rounds left in its mask: appended here, a lane a round (keys that cluster make this less rare than even
+      // rates would: a bucket then takes most keys of a group).
+      static_assert(ND * 64 <= kFPQueue, "the passes read what the queue holds");
+      while (__ballot(msk != 0u)) {
+        const bool has = msk != 0u;
+        const uint32_t e = 31u - uint32_t(__builtin_ctz(msk | 0x80000000u));
+        emit_one(has, uint32_t(l), e, dump[l * kFPDumpLd + e], key0_old);
+        msk = has ? (msk & (msk - 1u)) : msk;
+      }
+      // ... and the candidates whose place in the queue lies beyond the passes' ND * 64 (a group with more than
+      // that many candidates in all): the lanes that hold them go through their first NR again
+      if (total > ND * 64) {
+        uint32_t m = msk0;
+        for (int k = 0; k < NR; ++k) {
+          const bool has = m != 0u;
+          const uint32_t e = 31u - uint32_t(__builtin_ctz(m | 0x80000000u));
+          emit_one(has && base0 + k >= ND * 64, uint32_t(l), e, dump[l * kFPDumpLd + e], key0_old);
+          m = has ? (m & (m - 1u)) : m;
+        }
+      }
+    }
+  };
+
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  if (my_tiles > 0) {
+    fetch(0);
+    stash(0);
+  }
+  if (my_tiles > 1) fetch(1);
+  __syncthreads();
+  uint32_t key0_prev = 0;  // first key of the group whose epilogue is pending
+  for (int i = 0; i < my_tiles; ++i) {
+    if (i + 1 < my_tiles) stash((i + 1) & 1);  // into the buffer tile i - 1 was read from
+    if (i + 2 < my_tiles) fetch(i + 2);
+    if (active) {
+      const int buf = i & 1;
+      const uint32_t kbase = uint32_t((sk + i * n_splits) * kFKeys);
+      af[0] = *reinterpret_cast<const uint4*>(frag_ptr(buf, 0));
+      if (i == 0)
+        group_step(B0{}, std::true_type{}, std::false_type{}, frag_ptr(buf, 0), frag_ptr(buf, 1), 0u);
+      else
+        group_step(B0{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 0), frag_ptr(buf, 1), key0_prev);
+      group_step(B1{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 1), frag_ptr(buf, 2), kbase);
+      group_step(B0{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 2), frag_ptr(buf, 3), kbase + 16u);
+      group_step(B1{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 3), nullptr, kbase + 32u);
+      key0_prev = kbase + 48u;
+    }
+    __syncthreads();
+  }
+  if (active && my_tiles > 0)
+    group_step(B0{}, std::false_type{}, std::true_type{}, nullptr, nullptr, key0_prev);
+  // candidate counts (beyond cap_w: the segment overflowed, the row is repaired)
+  for (int t = l; t < 128; t += 64) {
+    const int row = cb + t;
+    if (row < C) cnt[(int64_t(h) * C + row) * n_writers + sk] = int32_t(min(cursor[t], uint32_t(cap_w) + 1u));
+  }
+}
+
 // ---- phase 2 ---------------------------------------------------------------
 // Per-writer candidate counts of a row in LDS; returns false (to all threads) if a segment
 // overflowed or the row has fewer than Zc candidates, i.e. the sampled threshold failed.
@@ -756,6 +1044,8 @@ static inline void mark_phase(int i, hipStream_t st) {
 
 }  // namespace fm
 
+extern "C" void fm_debug_fused_filter(int form) { fm::g_fused_filter_form.store(form, std::memory_order_relaxed); }
+
 extern "C" void fm_debug_set_phase_events(void** events, int n) {
   std::lock_guard<std::mutex> lk(fm::g_phase_mu);
   fm::g_phase_events = reinterpret_cast<hipEvent_t*>(events);
@@ -765,7 +1055,7 @@ extern "C" void fm_debug_set_phase_events(void** events, int n) {
 extern "C" const char* fm_build_index_fused_kernel(int H, int C, int N, int d, int Z, int dtype) {
   fm::FusedPlan p;
   if (H < 1 || C < 1 || N < 1 || !fm::fused_plan(H, C, N, d, Z, dtype, p)) return nullptr;
-  return p.wide ? "fused_filter_wide_kernel" : "fused_filter_kernel";
+  return p.ping ? "fused_filter_ping_kernel" : p.wide ? "fused_filter_wide_kernel" : "fused_filter_kernel";
 }
 
 extern "C" size_t fm_build_index_fused_workspace(int H, int C, int N, int d, int Z, int dtype) {
@@ -816,7 +1106,19 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
 #define FM_FILTER(KERNEL, THREADS)                                                                          \
   hipLaunchKernelGGL(KERNEL, grid, dim3(THREADS), 0, st, (const bf16_t*)A, (const bf16_t*)K, tau, cand, cnt, C, N, \
                      p.n_splits, p.cap_w)
-    if (p.wide && dtype == FM_F16)
+    if (p.ping == 1 && dtype == FM_F16)
+      FM_FILTER((fused_filter_ping_kernel<true, 4, 1>), 512);
+    else if (p.ping == 1)
+      FM_FILTER((fused_filter_ping_kernel<false, 4, 1>), 512);
+    else if (p.ping == 2 && dtype == FM_F16)
+      FM_FILTER((fused_filter_ping_kernel<true, 6, 2>), 512);
+    else if (p.ping == 2)
+      FM_FILTER((fused_filter_ping_kernel<false, 6, 2>), 512);
+    else if (p.ping == 3 && dtype == FM_F16)
+      FM_FILTER((fused_filter_ping_kernel<true, 7, 3>), 512);
+    else if (p.ping == 3)
+      FM_FILTER((fused_filter_ping_kernel<false, 7, 3>), 512);
+    else if (p.wide && dtype == FM_F16)
       FM_FILTER(fused_filter_wide_kernel<true>, 512);
     else if (p.wide)
       FM_FILTER(fused_filter_wide_kernel<false>, 512);

@@ -2,7 +2,7 @@
  * fastmem_debug.h -- test and measurement hooks of libfastmem.so.
  *
  * None of these has a counterpart in the reference.  The switches (fm_debug_force_generic,
- * fm_debug_argtopz_exact_only, fm_debug_set_phase_events) are PROCESS-WIDE state, read by every call on
+ * fm_debug_argtopz_exact_only, fm_debug_fused_filter, fm_debug_set_phase_events) are PROCESS-WIDE state, read by every call on
  * every stream: they exist so that tests can compare two implementations of one operator and so that the
  * benchmark can time the phases of the fused build; a production caller never touches them.  The probes
  * (fm_debug_copy, fm_debug_read, fm_debug_mfma) are plain kernels of known size.
@@ -54,6 +54,11 @@ const char* fm_build_index_fused_kernel(int H, int C, int N, int d, int Z, int d
  * multi-pass selection for every row instead of the sampled one-pass form (tests
  * compare the two), 0 restores dispatch. */
 void fm_debug_argtopz_exact_only(int on);
+
+/* Diagnostic: 1 keeps the fused index build away from the filter kernel that issues its epilogue between its
+ * MFMAs (fused_filter_ping_kernel), so that it takes fused_filter_wide_kernel where it would take that one
+ * (tests compare the lists of the two); 0 restores the plan. */
+void fm_debug_fused_filter(int form);
 
 /* Diagnostic: hand the fused index build up to 5 hipEvent_t (host array that
  * must stay valid; NULL clears) which it records on its stream before phase 0

@@ -1120,6 +1120,47 @@ def test_fused_build_shapes(ops, H, C, N, Z):
     assert torch.equal(fused, unfused) and torch.equal(fv.view(torch.int32), uv.view(torch.int32))
 
 
+@pytest.mark.parametrize("dtype,H,C,N,Z,runs", [
+    (torch.bfloat16, 2, 1024, 65536 + 77, 1100, False),   # pass rate ~2 %: four rounds, one pass; a ragged key tile
+    (torch.bfloat16, 1, 900, 131072, 6000, False),        # ~6 %: seven rounds, three passes; a partial last wave
+    (torch.float16, 2, 2048, 98304, 3000, False),         # ~4 %: six rounds, two passes; two slabs
+    (torch.bfloat16, 1, 1024, 70000, 1100, True),         # the keys of a cluster side by side: a bucket takes whole
+    (torch.float16, 2, 1024, 131072, 2500, True),         # groups of 16 keys, more than the rounds and passes hold
+])
+def test_fused_build_filter_forms_agree(ops, dtype, H, C, N, Z, runs):
+    """The filter that issues its epilogue between its MFMAs (fused_filter_ping_kernel; slabs of 1024 buckets,
+    a queue of candidates per wave, fixed numbers of rounds and passes picked from the expected pass rate, loops
+    for what they do not reach) against the filter it replaces there and against the unfused build: the same
+    lists and values.  With the keys of a cluster in consecutive positions the buckets near it take most keys of
+    a group at once, which overflows the rounds and the passes."""
+    lib = _libmod().load()
+    g = gen(930 + C + Z)
+    if runs:
+        cen = torch.randn(H, 48, 128, generator=g)
+        comp = torch.sort(torch.randint(0, 48, (H, N), generator=g), dim=1).values
+        K = (torch.gather(cen, 1, comp[..., None].expand(-1, -1, 128)) + 0.3 * torch.randn(H, N, 128, generator=g)).to(dtype)
+        A = (cen[:, torch.arange(C) % 48] + 0.7 * torch.randn(H, C, 128, generator=g)).to(dtype)
+    else:
+        K = _clustered_keys(g, H, N, 128).to(dtype)
+        A = torch.randn(H, C, 128, generator=g).to(dtype)
+    Ad, Kd = dev(A, K)
+    dt = {torch.bfloat16: 1, torch.float16: 2}[dtype]
+    assert lib.fm_build_index_fused_kernel(H, C, N, 128, Z, dt) == b"fused_filter_ping_kernel"
+    new, nv = ops.build_index(Ad, Kd, Z, fused=True, return_values=True)
+    info = dict(ops.last_build_info)
+    assert info["path"] == "fused" and info["rows_unresolved"] == 0, info
+    lib.fm_debug_fused_filter(1)
+    try:
+        assert lib.fm_build_index_fused_kernel(H, C, N, 128, Z, dt) == b"fused_filter_wide_kernel"
+        old, ov = ops.build_index(Ad, Kd, Z, fused=True, return_values=True)
+        assert ops.last_build_info["path"] == "fused"
+    finally:
+        lib.fm_debug_fused_filter(0)
+    assert torch.equal(new, old) and torch.equal(nv.view(torch.int32), ov.view(torch.int32))
+    unfused, uv = ops.build_index(Ad, Kd, Z, fused=False, return_values=True)
+    assert torch.equal(new, unfused) and torch.equal(nv.view(torch.int32), uv.view(torch.int32))
+
+
 def test_fused_build_repairs_rows_whose_sampled_threshold_missed(ops):
     g = gen(901)
     H, C, N, d, Z = 1, 40, 131072, 128, 1024               # sample stride 4: keys 0,4,8,... are sampled

@@ -643,7 +643,7 @@ __global__ __launch_bounds__(512) void fused_filter_wide_kernel(
 // A writer is a key split, so a row has n_splits segments; records carry the same key codes as above, the
 // selection does not see which form ran.
 constexpr int kFPDumpLd = 36;   // floats per lane in the dump: 32 accumulator registers + 4 (bank spread of the 16-byte stores)
-constexpr int kFPQueue = 256;   // queue places of a group's candidates; lanes without one write behind it
+constexpr int kFPQueue = 448;   // queue places of a group's candidates (64 lanes x at most 7 rounds); lanes without one write behind it
 
 struct FpShared {
   bf16_t keys[2][kFKeys * kFLd];
@@ -787,11 +787,14 @@ __global__ __launch_bounds__(512) void fused_filter_ping_kernel(
           base0 = base;
         } else if constexpr (S < 10 + NR) {
           // a round: one candidate per lane to its place in the queue
+          // (a lane's places are below 64 NR; msk & (msk - 1) leaves an empty mask empty, and what a lane
+          // without a candidate writes behind the queue is read by nobody)
+          static_assert(NR * 64 <= kFPQueue, "every lane's NR places are inside the queue");
           const bool has = msk != 0u;
-          const uint32_t p = uint32_t(__builtin_ctz(msk | 0x80000000u));
-          queue[has && base < kFPQueue ? base : kFPQueue + l] = (uint32_t(l) << 5) | p;
+          const uint32_t p = uint32_t(__ffs(int(msk)) - 1);
+          queue[has ? base : kFPQueue + l] = (uint32_t(l) << 5) | (p & 31u);
           base += has ? 1 : 0;
-          msk = has ? (msk & (msk - 1u)) : msk;
+          msk &= msk - 1u;
         } else {
           // dense passes: three stages a pass, staggered by one slot from pass to pass
           constexpr int S0 = 10 + NR + 1;  // first stage of pass 0 (a slot after the last round)

@@ -83,6 +83,8 @@ extern "C" int fm_hash_attn_fwd_ws(const void* q, const void* k, const void* v, 
              FM_ERR_ARG, "fm_hash_attn_fwd: null pointer");
   FM_REQUIRE(max_items >= 1 && max_items <= 0x7fffffffLL, FM_ERR_ARG,
              "fm_hash_attn_fwd: max_items=%lld", (long long)max_items);
+  FM_REQUIRE(!ws || ws_bytes >= hash_attn_ring_workspace(max_items), FM_ERR_WORKSPACE,
+             "fm_hash_attn_fwd_ws: workspace %zu < %zu", ws_bytes, hash_attn_ring_workspace(max_items));
   hipStream_t st = as_stream(stream);
   if (g_force_generic != 1 && hash_attn_mfma_supported(d, dtype, N))
     return hash_attn_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items,

@@ -161,7 +161,8 @@ int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t*
  * where buckets receive more than FM_QTILE queries on average a workgroup takes three items of a bucket
  * together, and with the workspace the groups are listed first so that every workgroup started has one --
  * without it two of three return at once, which leaves compute units idle (1.3 x slower at 128 queries per
- * bucket).  Same results bit for bit.  ws = NULL is fm_hash_attn_fwd. */
+ * bucket).  Same results bit for bit.  ws = NULL is fm_hash_attn_fwd; a workspace smaller than that is
+ * refused (FM_ERR_WORKSPACE). */
 size_t fm_hash_attn_fwd_workspace(int64_t max_items);
 int fm_hash_attn_fwd_ws(const void* q, const void* k, const void* v, const int32_t* k_idx,
                         const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,

@@ -68,6 +68,10 @@ def test_argument_errors_are_status_codes():
     assert b"in place" in lib.fm_last_error()
     assert lib.fm_debug_mfma(None, 5120, 1, None, None) == 1                          # null pointers
     assert lib.fm_debug_mfma(4096, 100, 1, 4096, None) == 1                           # too few operands
+    assert lib.fm_hash_attn_fwd_workspace(1000) >= 1000 * 4 and lib.fm_hash_attn_fwd_workspace(0) == 0
+    p = 4096                                                                          # never dereferenced
+    assert lib.fm_hash_attn_fwd_ws(p, p, p, p, p, p, p, p, p, 1000, p, p, 1, 64, 64, 128, 4, 1.0, 1, p, 16, None) == 3
+    assert b"workspace" in lib.fm_last_error()                                        # a workspace that is too small
     with pytest.raises(ValueError):
         _lib.check(1)
 

@@ -285,6 +285,21 @@ def test_lists_key_order(ops, n_lists, N, max_len):
     assert torch.equal(got.cpu(), ref)
 
 
+def test_lists_key_order_dense_and_thin_stretches(ops):
+    """One list with a run of neighbouring keys (more keys in a stretch of the range than a wave stages at once:
+    stored lane by lane), a thin spread (staged, stored 64 at a time) and a run that ends on the last key of a
+    range whose word count is not a multiple of 4."""
+    N = 262144 + 37
+    keys = torch.cat([torch.arange(5000, 9000), torch.arange(20000, 260000, 61), torch.arange(N - 70, N)]).int()
+    flat = keys[torch.randperm(keys.numel(), generator=gen(3))].contiguous()
+    flat = torch.cat([flat, flat[:500].sort().values])        # and a second, short list
+    off = torch.tensor([0, keys.numel()], dtype=torch.int64)
+    cnt = torch.tensor([keys.numel(), 500], dtype=torch.int32)
+    got, n_uns = ops.lists_key_order(dev(flat), dev(off), dev(cnt), N, return_unsorted=True)
+    assert int(n_uns.item()) == 0
+    assert torch.equal(got.cpu(), torch.cat([keys, flat[keys.numel():]]))
+
+
 def test_lists_key_order_copies_lists_it_cannot_sort(ops):
     """A list that names a key twice counts it twice in the softmax, and one with an entry outside [0, N) is
     whatever the caller meant: both come back unchanged (and counted), the other lists sorted."""

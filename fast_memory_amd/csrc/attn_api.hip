@@ -261,6 +261,7 @@ extern "C" int fm_local_attn_fwd(const void* q, const void* k, const void* v, vo
   FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_local_attn_fwd: dtype=%d", dtype);
   FM_REQUIRE(q && k && v && out && lse, FM_ERR_ARG, "fm_local_attn_fwd: null pointer");
   FM_REQUIRE(int64_t(H) * G <= 65535, FM_ERR_UNSUPPORTED, "fm_local_attn_fwd: H*G > 65535");
+  FM_REQUIRE(S <= 65535 * 128, FM_ERR_UNSUPPORTED, "fm_local_attn_fwd: S=%d > 65535 * 128", S);
   hipStream_t st = as_stream(stream);
   if (g_force_generic != 1 && local_attn_mfma_supported(d, dtype))
     return local_attn_mfma(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, st);

@@ -19,7 +19,7 @@
 //                  with its key columns in that order, so neither P nor V is shuffled.
 // Softmax as in the gather kernel (triton_kernel.py:248-263): base 2 with
 // sm_scale*log2(e), fp32 running max and denominator, denominator from unrounded p,
-// p rounded to bf16 before P.V.
+// p rounded to bf16 before P.V; the running maximum is followed lazily (see kLazy).
 //
 // Roofline: MFMA (4*d flops per visible query-key pair); the per-element softmax
 // VALU work is of the same order as the MFMA time and does not overlap with it.
@@ -37,6 +37,7 @@ constexpr int kLQ = 128;    // queries per workgroup
 constexpr int kLK = 64;     // keys per tile
 constexpr int kLKld = 136;  // K tile row stride in LDS (elements)
 constexpr int kLVld = 72;   // Vt row stride in LDS (elements): 64 keys + 8
+constexpr float kLazy = 8.f;  // growth of a running maximum (in powers of two) that is left unfollowed
 
 __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
   f32x2 x = {lo, hi};
@@ -65,8 +66,11 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][kLD * kLVld];
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   const int col = l & 31, hb = l >> 5;
-  const int hq = blockIdx.y, hk = hq / G;
-  const int qb = int(gridDim.x) - 1 - int(blockIdx.x);  // late query blocks see most keys: start them first
+  // Late query blocks see most keys: the launch hands out the last block of every head first, then the block
+  // before it of every head, ..., so that what starts last is the shortest work and the launch ends evenly
+  // (with the blocks of a head in a row, the longest workgroup of the last head would start near the end).
+  const int hq = blockIdx.x, hk = hq / G;
+  const int qb = int(gridDim.y) - 1 - int(blockIdx.y);
   const int i0 = qb * kLQ;
   const bf16_t* Kh = k + int64_t(hk) * L * kLD;
   const bf16_t* Vh = v + int64_t(hk) * L * kLD;
@@ -81,8 +85,11 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
   const int iq = i0 + w * 32 + col;  // this lane's query
   const bool q_ok = iq < S;
   const int my_lim = q_ok ? lim_of(iq) : 0;
-  const int wave_lim_hi = lim_of(min(S - 1, i0 + w * 32 + 31));  // most keys any query of the wave sees
-  const int wave_lim_lo = (i0 + w * 32 + 31 < S) ? lim_of(i0 + w * 32) : 0;  // fewest
+  // (the same in every lane of a wave: read through one lane, so that the tests on them are scalar branches
+  // and not per-lane selects that every tile would pay for)
+  const int wq0 = i0 + __builtin_amdgcn_readfirstlane(w) * 32;
+  const int wave_lim_hi = lim_of(min(S - 1, wq0 + 31));  // most keys any query of the wave sees
+  const int wave_lim_lo = (wq0 + 31 < S) ? lim_of(wq0) : 0;  // fewest
 
   bf16x8 qf[8];
   {
@@ -90,6 +97,12 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = u4_as_bf16x8(q_ok ? pq[2 * ks] : make_uint4(0, 0, 0, 0));
   }
+  // The compiler's wait-count pass cannot see that these loads have landed by the time the loop starts (the path
+  // that skips the first tile has no wait) and would otherwise wait, in front of every tile's first MFMA, for
+  // all loads in flight: the next tile's, whose latency the double buffering is there to hide.  The empty
+  // statements read the registers (the pass waits for the loads here, once) and count as their last writers.
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
   f32x16 O[4];
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt)
@@ -99,8 +112,19 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
 
   LocalTileRegs tr;
   const int vj = l >> 2, vc = 4 * w + (l & 3);
+  const uint4* pk0 = reinterpret_cast<const uint4*>(Kh + int64_t(tid >> 4) * kLD) + (tid & 15);
+  const uint4* pv0 = reinterpret_cast<const uint4*>(Vh + int64_t(4 * vj) * kLD) + vc;
   auto load_tile = [&](int t) {
     const int kp0 = t * kLK;
+    if (kp0 + kLK <= L) {  // a whole tile: no row of it lies past the keys
+      const uint4* pk = pk0 + int64_t(kp0) * (kLD / 8);
+      const uint4* pv = pv0 + int64_t(kp0) * (kLD / 8);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) tr.k[u] = pk[16 * u * (kLD / 8)];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) tr.v[kk] = pv[kk * (kLD / 8)];
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int row = kp0 + (tid >> 4) + 16 * u;
@@ -145,17 +169,23 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
     // ---- S^T for the two 32-key blocks ----
     f32x16 s[2];
 #pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
+    for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[sb][r] = 0.f;
-      const bf16_t* pa = &sK[buf][(sb * 32 + col) * kLKld + hb * 8];
+    {
+      const bf16_t* pa = &sK[buf][col * kLKld + hb * 8];
+      // the two 32-key blocks in turn: neighbouring MFMAs do not wait for each other's sums
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks)
-        s[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(pa + ks * 16), qf[ks],
-                                                        s[sb], 0, 0, 0);
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+          s[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              *reinterpret_cast<const bf16x8*>(pa + sb * 32 * kLKld + ks * 16), qf[ks], s[sb], 0, 0, 0);
     }
-    // ---- mask (only tiles that reach past what some query of the wave sees) ----
+    // ---- mask (only tiles that reach past what some query of the wave sees; the empty statement keeps the
+    // compiler from turning the branch into per-lane selects that every tile would execute) ----
     if (kp0 + kLK > wave_lim_lo) {
+      asm volatile("");
 #pragma unroll
       for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
@@ -171,10 +201,15 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[1][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32)) * scale2;  // scale2 > 0: scaling commutes with the maximum
+    // The running maximum follows the scores only when some query's grew by more than 2^kLazy (or it sees
+    // its first key): until then the weights are taken against the older maximum and stay below 2^kLazy,
+    // which fp32 sums and the relative rounding of bf16 do not notice, and the 64 multiplications of the
+    // accumulator are spared in most tiles.  The sums, the output and the LSE are the same function of the
+    // scores either way.
     const float m_new = fmaxf(m, mx);
-    const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;  // a query that sees no key yet
-    if (__any(m_new != m)) {
-      const float alpha = __builtin_amdgcn_exp2f(m - m_sub);
+    if (__any(m_new > m + kLazy)) {
+      const float m_to = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m - m_to);
       lsum *= alpha;
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
@@ -182,6 +217,7 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
         for (int r = 0; r < 16; ++r) O[dt][r] *= alpha;
       m = m_new;
     }
+    const float m_sub = (m == -INFINITY) ? 0.f : m;  // a query that sees no key yet
     bf16x8 pf[2][2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
@@ -196,17 +232,17 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
         pf[sb][st] = u4_as_bf16x8(make_uint4(cvt_pk_bf16(p[8 * st + 0], p[8 * st + 1]), cvt_pk_bf16(p[8 * st + 2], p[8 * st + 3]),
                                              cvt_pk_bf16(p[8 * st + 4], p[8 * st + 5]), cvt_pk_bf16(p[8 * st + 6], p[8 * st + 7])));
     }
-    // ---- O^T += Vt.P^T ----
+    // ---- O^T += Vt.P^T (the four 32-row blocks of the output in turn, for the same reason) ----
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) {
-      const bf16_t* pv = &sVt[buf][(dt * 32 + col) * kLVld + hb * 8];
+    for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
-      for (int sb = 0; sb < 2; ++sb)
+      for (int st = 0; st < 2; ++st)
 #pragma unroll
-        for (int st = 0; st < 2; ++st)
+        for (int dt = 0; dt < 4; ++dt) {
+          const bf16_t* pv = &sVt[buf][(dt * 32 + col) * kLVld + hb * 8];
           O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(pv + sb * 32 + st * 16),
                                                           pf[sb][st], O[dt], 0, 0, 0);
-    }
+        }
   };
 
   if (ntiles > 0) {
@@ -242,7 +278,7 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
 
 int local_attn_dense(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G, int S,
                      int L, float sm_scale, int causal, hipStream_t st) {
-  dim3 grid = dim3(unsigned(ceil_div(S, kLQ)), unsigned(H * G));
+  dim3 grid = dim3(unsigned(H * G), unsigned(ceil_div(S, kLQ)));
   hipLaunchKernelGGL(local_attn_dense_kernel, grid, dim3(256), 0, st, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, (bf16_t*)out, lse, G, S, L, sm_scale * kLog2e, causal);
   return launch_status("fm_local_attn_fwd(dense)");

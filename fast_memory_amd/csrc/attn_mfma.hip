@@ -117,10 +117,11 @@ __device__ __forceinline__ void attend_item(
   }
 
   const int nblk = (cnt + kBlk - 1) / kBlk;
+  // (positions past the list read its last entry: the load is issued on every path, so the number of loads in
+  // flight at any point of the loop below is known to the compiler, and so are the loads of the blocks)
   auto rows_of = [&](int b) -> int {
-    const int kp = b * kBlk + (l & 31);
-    int r = 0;
-    if (kp < cnt) r = idx ? idx[kp] : kp;
+    const int kp = min(b * kBlk + (l & 31), cnt - 1);
+    const int r = idx ? idx[max(kp, 0)] : kp;
     return min(max(r, 0), N - 1);
   };
 
@@ -210,20 +211,25 @@ __device__ __forceinline__ void attend_item(
   // ---- main loop: this wave's blocks w, w+4, ..., one block in flight -------
   KVRegs ra, rb;
   int b = w;
-  // key rows are fetched two blocks ahead of the block being computed, K/V one ahead
-  if (b < nblk) load_block(ra, Kb, Vb, rows_of(b), g, c);
-  int r1 = rows_of(b + 4);
-  while (b < nblk) {
-    const int b1 = b + 4, b2 = b + 8;
-    const int r2 = rows_of(b2);
-    if (b1 < nblk) load_block(rb, Kb, Vb, r1, g, c);
-    compute(ra, b);
-    if (b1 >= nblk) break;
-    const int r3 = rows_of(b2 + 4);
-    if (b2 < nblk) load_block(ra, Kb, Vb, r2, g, c);
-    compute(rb, b1);
-    r1 = r3;
-    b = b2;
+  // Key rows are fetched two blocks ahead of the block being computed, K/V one ahead.  The loads of the block
+  // ahead go out whether or not there is one (past the end they fetch the list's last row again): with a load
+  // that some path skips, the compiler's wait in front of a block's first MFMA has to be for every load in
+  // flight, the block ahead included, and nothing is fetched ahead at all.
+  if (cnt > 0) {  // (an empty list has no entry to read)
+    load_block(ra, Kb, Vb, rows_of(b), g, c);
+    int r1 = rows_of(b + 4);
+    while (b < nblk) {
+      const int b1 = b + 4, b2 = b + 8;
+      const int r2 = rows_of(b2);
+      load_block(rb, Kb, Vb, r1, g, c);
+      compute(ra, b);
+      if (b1 >= nblk) break;
+      const int r3 = rows_of(b2 + 4);
+      load_block(ra, Kb, Vb, r2, g, c);
+      compute(rb, b1);
+      r1 = r3;
+      b = b2;
+    }
   }
 
   // ---- merge the four waves ---------------------------------------------------

@@ -139,15 +139,21 @@ extern "C" size_t fm_attention_hash_varlen_workspace(int H, int C, int Sq) {
 namespace fm {
 // A query whose hash is outside [0, C) belongs to no bucket and to no work item, so the attention kernels
 // never write its rows: here it gets the result of an empty bucket, out = 0 and lse = -FLT_MAX.
+// (a thread looks at one hash; the lanes of a wave then fill, together, the rows of those of its 64 queries that
+// have none -- usually there is nothing to fill and the launch only reads the hashes)
 __global__ __launch_bounds__(256) void unhashed_rows_kernel(const int32_t* __restrict__ q_hash, int64_t nq,
                                                             int C, int row_halves, uint16_t* __restrict__ out,
                                                             float* __restrict__ lse) {
-  const int64_t i = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
-  if (i >= nq) return;
-  const int b = q_hash[i];
-  if (b >= 0 && b < C) return;
-  for (int w = lane_id(); w < row_halves; w += kWave) out[i * row_halves + w] = uint16_t(0);
-  if (lane_id() == 0) lse[i] = -FLT_MAX;
+  const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const int b = i < nq ? q_hash[i] : 0;
+  uint64_t bad = __ballot(i < nq && (b < 0 || b >= C));
+  const int64_t i0 = i - lane_id();
+  while (bad) {
+    const int j = __ffsll((long long)bad) - 1;
+    bad &= bad - 1;
+    for (int w = lane_id(); w < row_halves; w += kWave) out[(i0 + j) * row_halves + w] = uint16_t(0);
+    if (lane_id() == 0) lse[i0 + j] = -FLT_MAX;
+  }
 }
 
 // bucket offsets + grouping + attention with every intermediate in the buffer at `base`
@@ -172,7 +178,7 @@ static int varlen_run(const void* q, const void* k, const void* v, const int32_t
   if (rc) return rc;
   const int row_bytes = d * dtype_bytes(dtype);
   const int64_t nq = int64_t(H) * Sq;
-  hipLaunchKernelGGL(unhashed_rows_kernel, dim3(unsigned(ceil_div(nq, 4))), dim3(256), 0, as_stream(stream),
+  hipLaunchKernelGGL(unhashed_rows_kernel, dim3(unsigned(ceil_div(nq, 256))), dim3(256), 0, as_stream(stream),
                      q_hash, nq, C, row_bytes / 2, static_cast<uint16_t*>(out), lse);
   return launch_status("fm_attention_hash_varlen");
 }

@@ -165,7 +165,7 @@ def test_local_attention_backward_bf16(S, L, chunk_entries, monkeypatch):
 
 
 def test_integration_snippet_runs_verbatim():
-    """The ctypes binding INTEGRATION.md shows for the reference's operator, executed as printed (in a process
+    """The ctypes binding that the integration guide prints for the reference's operator, executed as printed (in a process
     of its own: it registers the operator name this package registers too) and checked against the oracle."""
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
@@ -181,7 +181,7 @@ for dtype, d in ((torch.float32, 64), (torch.bfloat16, 128)):
     c = lambda t: t.cuda()
     out, lse = torch.ops.notbad.attention_hash_varlen(c(q), c(k), c(v), c(kh), c(cnt), c(qh), 0.17)
     ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 0.17)
-    assert_attn_close(out, lse, ro, rl, dtype, "INTEGRATION.md snippet")
+    assert_attn_close(out, lse, ro, rl, dtype, "binding snippet of the integration guide")
 print("snippet ok")
 ''' % ROOT
     r = subprocess.run([sys.executable, "-c", snippet[0] + driver], cwd=ROOT, capture_output=True, text=True,

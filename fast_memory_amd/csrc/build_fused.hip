@@ -123,11 +123,12 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   // Its emission handles a lane's first NR candidates of a group (16 keys x 128 buckets) and the group's first
   // ND * 64 in straight-line code; the forms are (NR, ND) = (4, 1), (6, 2), (7, 3), picked so that 3.5
   // standard deviations of a group's candidates fit the passes.
-  if (p.wide && g_fused_filter_form.load(std::memory_order_relaxed) != 1) {
+  const int forced = g_fused_filter_form.load(std::memory_order_relaxed);  // 1: not this form; 2, 3, 4: its ND = 1, 2, 3
+  if (p.wide && forced != 1) {
     p.n_writers = p.n_splits;
     if (search()) {
       const double per_group = 2048.0 * m_exp / N;
-      const int nd = int(ceil((per_group + 3.5 * sqrt(per_group)) / 64.0));
+      const int nd = forced >= 2 && forced <= 4 ? forced - 1 : int(ceil((per_group + 3.5 * sqrt(per_group)) / 64.0));
       if (nd >= 1 && nd <= 3) p.ping = nd;
     }
     if (!p.ping) p.n_writers = 2 * p.n_splits;

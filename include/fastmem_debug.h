@@ -57,7 +57,9 @@ void fm_debug_argtopz_exact_only(int on);
 
 /* Diagnostic: 1 keeps the fused index build away from the filter kernel that issues its epilogue between its
  * MFMAs (fused_filter_ping_kernel), so that it takes fused_filter_wide_kernel where it would take that one
- * (tests compare the lists of the two); 0 restores the plan. */
+ * (tests compare the lists of the two); 2, 3, 4 make it take that kernel, where the plan allows it, in the form
+ * whose straight-line emission covers 64, 128 or 192 candidates of a group of 16 keys x 128 buckets (the plan picks
+ * the form by the expected number; every form gives the same lists); 0 restores the plan. */
 void fm_debug_fused_filter(int form);
 
 /* Diagnostic: hand the fused index build up to 5 hipEvent_t (host array that

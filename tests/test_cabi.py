@@ -72,6 +72,10 @@ def test_argument_errors_are_status_codes():
     p = 4096                                                                          # never dereferenced
     assert lib.fm_hash_attn_fwd_ws(p, p, p, p, p, p, p, p, p, 1000, p, p, 1, 64, 64, 128, 4, 1.0, 1, p, 16, None) == 3
     assert b"workspace" in lib.fm_last_error()                                        # a workspace that is too small
+    # extents the launch shapes of the local attention cannot express are refused before any launch
+    assert lib.fm_local_attn_fwd(p, p, p, p, p, 1, 1, 65535 * 128 + 1, 16, 128, 1.0, 1, 1, None) != 0
+    assert b"fm_local_attn_fwd" in lib.fm_last_error()
+    assert lib.fm_local_attn_fwd(p, p, p, p, p, 65536, 1, 16, 16, 128, 1.0, 1, 1, None) != 0
     with pytest.raises(ValueError):
         _lib.check(1)
 

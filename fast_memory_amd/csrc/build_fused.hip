@@ -86,37 +86,53 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   // threshold noisier: a row keeps m = rank*stride +- stride*sqrt(rank) candidates, which the
   // selection must hold in registers (R per thread, T = NT / n_writers threads per writer segment,
   // whose share of m spreads by another sqrt).  The sort keeps 16 keys per thread, so P/16 threads
-  // are all it can use; fewer threads per row let several rows share a CU.  Take the smallest
-  // sample, then the fewest threads, that leave five standard deviations of room; failing that, the
-  // large sample with 1024 threads (rows that do not fit are repaired).
+  // are all it can use; fewer threads per row let several rows share a CU.  Of the samples that leave
+  // five standard deviations of room (each with the fewest threads that do), take the one with the
+  // least expected work; if none does, the large sample with 1024 threads (rows that do not fit are
+  // repaired).
   const int P = next_pow2(Z);
   bool found = false;
   double m_exp = 0;
   auto search = [&]() {
     found = false;
+    // Among the samples whose candidates the selection holds in registers, the one with the least expected work:
+    // phase 0 costs per sampled key and row, the filter's emission and the selection per candidate and row
+    // (measured on the 262 144- and the 1 M-key workloads: about 2.7 ps against 10 ps).  A short memory takes
+    // a small sample (a 16 K sample would be a quarter of its keys and phase 0 a quarter of the projection), a
+    // long one with long lists the 16 K sample that keeps fewer candidates.
+    double best = 0;
+    int best_ns = 0, best_nt = 0;
     for (int ns_try : {4096, 8192, 16384, 32768}) {
-      p.stride = N / ns_try;
-      p.ns = N / p.stride;
-      const double mu = double(Z) * p.ns / N;
-      p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
-      if (p.rank * 4 > p.ns) continue;
-      m_exp = double(p.rank) * N / p.ns;
-      // (the two small samples only where they keep at most 32 % more candidates than Z: short memories with
-      // long lists, where a 16 K sample would be a quarter of all keys and phase 0 a quarter of the projection)
-      if (ns_try < 16384 && m_exp > 1.32 * Z) continue;
-      const double per_w = m_exp / p.n_writers;
-      const double sd_w = sqrt(pow(double(N) / p.ns * sqrt(double(p.rank)) / p.n_writers, 2) + per_w);
-      for (int nt = 256; nt <= kSelThreads && !found; nt *= 2)
-        if (nt * 16 >= P && (nt / p.n_writers) * (nt < kSelThreads ? kCandRegsSmall : kCandRegs) >= per_w + 5.0 * sd_w) {
-          p.sel_threads = nt;
-          found = true;
-        }
-      if (found) break;
+      const int stride = N / ns_try;
+      if (stride < 1) continue;
+      const int ns = N / stride;
+      const double mu = double(Z) * ns / N;
+      const int rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
+      if (rank * 4 > ns) continue;
+      const double m = double(rank) * N / ns;
+      const double per_w = m / p.n_writers;
+      const double sd_w = sqrt(pow(double(N) / ns * sqrt(double(rank)) / p.n_writers, 2) + per_w);
+      int nt_ok = 0;
+      for (int nt = 256; nt <= kSelThreads && !nt_ok; nt *= 2)
+        if (nt * 16 >= P && (nt / p.n_writers) * (nt < kSelThreads ? kCandRegsSmall : kCandRegs) >= per_w + 5.0 * sd_w)
+          nt_ok = nt;
+      if (!nt_ok) continue;
+      const double cost = 2.7 * ns + 10.0 * m;
+      if (!found || cost < best) {
+        found = true;
+        best = cost;
+        best_ns = ns_try;
+        best_nt = nt_ok;
+      }
     }
-    if (!found) {
-      if (p.rank * 4 > p.ns) return false;
-      p.sel_threads = kSelThreads;
-    }
+    const int ns_take = found ? best_ns : 32768;  // none fits: the large sample, rows that do not fit are repaired
+    p.stride = std::max(1, N / ns_take);
+    p.ns = N / p.stride;
+    const double mu = double(Z) * p.ns / N;
+    p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
+    if (p.rank * 4 > p.ns) return false;
+    m_exp = double(p.rank) * N / p.ns;
+    p.sel_threads = found ? best_nt : kSelThreads;
     return true;
   };
   // The form with the epilogue between the MFMAs where the wide form applies: a writer is a key split there.

@@ -63,6 +63,7 @@ SIGNATURES = {
     "fm_l2_normalize": (c_int, [P, P, c_int64, c_int, c_float, c_int, P]),
     "fm_topk_mean": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P]),
     "fm_segment_mean": (c_int, [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
+    "fm_segment_mean_directions": (c_int, [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_float, c_int, P]),
     "fm_index_append_workspace": (c_size_t, [c_int, c_int, c_int]),
     "fm_index_append": (c_int, [P, P, c_int, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P, P]),
     "fm_segment_sum": (c_int, [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
@@ -73,6 +74,7 @@ SIGNATURES = {
     "fm_debug_argtopz_exact_only": (None, [c_int]),
     "fm_debug_copy": (c_int, [P, P, c_int64, P]),
     "fm_debug_read": (c_int, [P, c_int64, P, P]),
+    "fm_debug_gather": (c_int, [P, c_int64, c_int, P, P]),
     "fm_debug_fused_filter": (None, [c_int]),
     "fm_debug_mfma": (c_int, [P, c_int64, c_int, P, P]),
     "fm_debug_set_phase_events": (None, [P, c_int]),

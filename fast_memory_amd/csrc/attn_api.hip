@@ -26,6 +26,10 @@ bool local_attn_mfma_supported(int d, int dtype);
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
                     int S, int L, int d, float sm_scale, int causal, hipStream_t st);
 
+int launch_unlisted_rows(const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                         const int32_t* bin_off, const int32_t* bin_count, int64_t n_bins, int64_t nq,
+                         int row_bytes, void* rows, float* lse, hipStream_t st);  // group.hip
+
 int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
                      const int32_t* idx_all, const fm_rowdesc* desc, int rows, int G, float sm_scale,
                      void* out, float* lse, int32_t* hash_out, float* scores_out, hipStream_t st);
@@ -86,11 +90,17 @@ extern "C" int fm_hash_attn_fwd_ws(const void* q, const void* k, const void* v, 
   FM_REQUIRE(!ws || ws_bytes >= hash_attn_ring_workspace(max_items), FM_ERR_WORKSPACE,
              "fm_hash_attn_fwd_ws: workspace %zu < %zu", ws_bytes, hash_attn_ring_workspace(max_items));
   hipStream_t st = as_stream(stream);
+  int rc;
   if (g_force_generic != 1 && hash_attn_mfma_supported(d, dtype, N))
-    return hash_attn_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items,
-                          out, lse, H, Sq, N, d, C, sm_scale, dtype, ws, ws ? ws_bytes : 0, st);
-  return hash_attn_generic(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
+    rc = hash_attn_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items,
+                        out, lse, H, Sq, N, d, C, sm_scale, dtype, ws, ws ? ws_bytes : 0, st);
+  else
+    rc = hash_attn_generic(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items,
                            max_items, out, lse, Sq, N, d, C, sm_scale, dtype, st);
+  if (rc) return rc;
+  // queries that are part of no work item (hash outside [0, C)): the result of an empty bucket
+  return launch_unlisted_rows(q_perm, items, n_items, nullptr, nullptr, 0, int64_t(H) * Sq,
+                              d * dtype_bytes(dtype), out, lse, st);
 }
 
 extern "C" int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
@@ -137,25 +147,6 @@ extern "C" size_t fm_attention_hash_varlen_workspace(int H, int C, int Sq) {
 }
 
 namespace fm {
-// A query whose hash is outside [0, C) belongs to no bucket and to no work item, so the attention kernels
-// never write its rows: here it gets the result of an empty bucket, out = 0 and lse = -FLT_MAX.
-// (a thread looks at one hash; the lanes of a wave then fill, together, the rows of those of its 64 queries that
-// have none -- usually there is nothing to fill and the launch only reads the hashes)
-__global__ __launch_bounds__(256) void unhashed_rows_kernel(const int32_t* __restrict__ q_hash, int64_t nq,
-                                                            int C, int row_halves, uint16_t* __restrict__ out,
-                                                            float* __restrict__ lse) {
-  const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
-  const int b = i < nq ? q_hash[i] : 0;
-  uint64_t bad = __ballot(i < nq && (b < 0 || b >= C));
-  const int64_t i0 = i - lane_id();
-  while (bad) {
-    const int j = __ffsll((long long)bad) - 1;
-    bad &= bad - 1;
-    for (int w = lane_id(); w < row_halves; w += kWave) out[(i0 + j) * row_halves + w] = uint16_t(0);
-    if (lane_id() == 0) lse[i0 + j] = -FLT_MAX;
-  }
-}
-
 // bucket offsets + grouping + attention with every intermediate in the buffer at `base`
 static int varlen_run(const void* q, const void* k, const void* v, const int32_t* k_idx,
                       const int32_t* bucket_cnt, const int32_t* q_hash, void* out, float* lse, int H,
@@ -175,12 +166,21 @@ static int varlen_run(const void* q, const void* k, const void* v, const int32_t
   rc = fm_hash_attn_fwd_ws(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, w.max_items, out,
                            lse, H, Sq, N, d, C, sm_scale, dtype, base + w.off_attn,
                            fm_hash_attn_fwd_workspace(w.max_items), stream);
-  if (rc) return rc;
-  const int row_bytes = d * dtype_bytes(dtype);
-  const int64_t nq = int64_t(H) * Sq;
-  hipLaunchKernelGGL(unhashed_rows_kernel, dim3(unsigned(ceil_div(nq, 256))), dim3(256), 0, as_stream(stream),
-                     q_hash, nq, C, row_bytes / 2, static_cast<uint16_t*>(out), lse);
-  return launch_status("fm_attention_hash_varlen");
+  return rc;
+}
+
+// every argument check of the one-call operators, ahead of their first launch (a caller that records
+// the call into a graph must not be left with half a sequence)
+static int varlen_check(const char* name, const void* q, const void* k, const void* v, const int32_t* k_idx,
+                        const int32_t* bucket_cnt, const int32_t* q_hash, const void* out, const float* lse,
+                        int H, int Sq, int N, int d, int C, int dtype) {
+  FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
+             "%s: H=%d Sq=%d N=%d C=%d d=%d", name, H, Sq, N, C, d);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "%s: dtype=%d", name, dtype);
+  FM_REQUIRE(q && k && v && k_idx && bucket_cnt && q_hash && out && lse, FM_ERR_ARG, "%s: null pointer", name);
+  FM_REQUIRE(int64_t(H) * Sq <= 0x7fffffffLL && int64_t(H) * C <= 0x7fffffffLL && H <= 65535, FM_ERR_UNSUPPORTED,
+             "%s: H*Sq or H*C exceeds int32, or H > 65535", name);
+  return FM_OK;
 }
 }  // namespace fm
 
@@ -190,9 +190,9 @@ extern "C" int fm_attention_hash_varlen(const void* q, const void* k, const void
                                         int N, int d, int C, float sm_scale, int dtype, void* ws,
                                         size_t ws_bytes, void* stream) {
   using namespace fm;
-  FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1, FM_ERR_ARG,
-             "fm_attention_hash_varlen: H=%d Sq=%d N=%d C=%d", H, Sq, N, C);
-  FM_REQUIRE(ws && bucket_cnt && q_hash, FM_ERR_ARG, "fm_attention_hash_varlen: null pointer");
+  int rc = varlen_check("fm_attention_hash_varlen", q, k, v, k_idx, bucket_cnt, q_hash, out, lse, H, Sq, N, d, C, dtype);
+  if (rc) return rc;
+  FM_REQUIRE(ws, FM_ERR_ARG, "fm_attention_hash_varlen: null pointer");
   VarlenWs w = varlen_layout(H, C, Sq);
   FM_REQUIRE(ws_bytes >= w.total, FM_ERR_WORKSPACE, "fm_attention_hash_varlen: workspace %zu < %zu",
              ws_bytes, w.total);
@@ -241,16 +241,16 @@ extern "C" int fm_attention_hash_varlen_static(const void* q, const void* k, con
                                                int Sq, int N, int d, int C, float sm_scale, int dtype,
                                                void* stream) {
   using namespace fm;
-  FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1, FM_ERR_ARG,
-             "fm_attention_hash_varlen_static: H=%d Sq=%d N=%d C=%d", H, Sq, N, C);
-  FM_REQUIRE(bucket_cnt && q_hash, FM_ERR_ARG, "fm_attention_hash_varlen_static: null pointer");
+  int rc = varlen_check("fm_attention_hash_varlen_static", q, k, v, k_idx, bucket_cnt, q_hash, out, lse, H, Sq, N, d,
+                        C, dtype);
+  if (rc) return rc;
   VarlenWs w = varlen_layout(H, C, Sq);
   FM_REQUIRE(w.total <= size_t(FM_STATIC_SCRATCH_BYTES), FM_ERR_WORKSPACE,
              "fm_attention_hash_varlen_static: H=%d C=%d Sq=%d needs %zu bytes of scratch, the static "
              "array holds %zu; use fm_attention_hash_varlen with a workspace",
              H, C, Sq, w.total, size_t(FM_STATIC_SCRATCH_BYTES));
   char* base = nullptr;
-  int rc = scratch_of_current_device(&base);
+  rc = scratch_of_current_device(&base);
   if (rc) return rc;
   // nothing in the array has to survive from an earlier call: the grouping clears its block table
   // with a fill kernel and every other region is written before it is read

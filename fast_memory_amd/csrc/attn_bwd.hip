@@ -104,6 +104,10 @@ int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_
                        int64_t max_items, const void* out, const float* lse, const void* dout, const float* dlse, void* dq,
                        float* dk, float* dv, int Sq, int N, int C, float sm_scale, hipStream_t st);
 
+int launch_unlisted_rows(const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                         const int32_t* bin_off, const int32_t* bin_count, int64_t n_bins, int64_t nq,
+                         int row_bytes, void* rows, float* lse, hipStream_t st);  // group.hip
+
 }  // namespace fm
 
 extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
@@ -121,6 +125,10 @@ extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, con
   FM_REQUIRE(max_items >= 1 && max_items <= 0x7fffffffLL, FM_ERR_ARG, "fm_hash_attn_bwd: max_items=%lld",
              (long long)max_items);
   hipStream_t st = as_stream(stream);
+  // dq of the queries that are part of no work item (hash outside [0, C)): 0, as for an empty bucket
+  int rc = launch_unlisted_rows(q_perm, items, n_items, nullptr, nullptr, 0, int64_t(H) * Sq, d * dtype_bytes(dtype),
+                                dq, nullptr, st);
+  if (rc) return rc;
   if (g_force_generic != 1 && hash_attn_bwd_mfma_supported(d, dtype))
     return hash_attn_bwd_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse,
                               dout, dlse, dq, dk, dv, Sq, N, C, sm_scale, st);

@@ -32,6 +32,9 @@
 
 namespace fm {
 
+int launch_unlisted_rows(const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                         const int32_t* bin_off, const int32_t* bin_count, int64_t n_bins, int64_t nq,
+                         int row_bytes, void* rows, float* lse, hipStream_t st);  // group.hip
 int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, const int32_t* k_idx,
                                   const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                                   const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
@@ -213,6 +216,11 @@ extern "C" int fm_hash_attn_bwd_staged(const void* q, const void* k, const void*
   for (int h = 0; h < H; ++h)
     FM_REQUIRE(row_pos_host[h + 1] >= row_pos_host[h], FM_ERR_ARG, "fm_hash_attn_bwd_staged: row_pos not ascending");
   hipStream_t st = as_stream(stream);
+  {  // dq of the queries without a bucket (hash outside [0, C)): 0, as for an empty bucket
+    int rc = launch_unlisted_rows(q_perm, nullptr, nullptr, bin_off, bin_count, int64_t(H) * C, int64_t(H) * Sq,
+                                  128 * int(sizeof(bf16_t)), dq, nullptr, st);
+    if (rc) return rc;
+  }
   const size_t per_entry = 128 * sizeof(bf16_t) * 2;
   const int64_t cap = int64_t((ws_bytes - std::min<size_t>(ws_bytes, kStagedSlack)) / per_entry);
   int h0 = 0;

@@ -60,6 +60,9 @@ __device__ __forceinline__ void ring_barrier() {
   asm volatile("" ::: "memory");
 }
 
+// M0 is written inside the statements below and is not on their clobber lists: it is a reserved register of
+// the AMDGPU backend, which keeps no value live in it across an asm statement (it rewrites M0 right in front
+// of each of its own uses) and rejects it as a clobber with a warning per statement.
 // lane i of the wave: 16 bytes from base + voff(i) to LDS byte address lds_addr + 16 i
 __device__ __forceinline__ void ring_load16(uint32_t lds_addr, uint32_t voff, const void* base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(base)

@@ -976,6 +976,13 @@ __global__ __launch_bounds__(NT) void cand_select_kernel(
       int pos = atomicAdd(n_fail, 1);
       if (pos < kMaxRepair) fail_rows[pos] = int32_t(row);
     }
+    // Until the repair overwrites it the row holds keys 0 .. Zc-1: should more rows fail than the repair
+    // takes, a caller that reads the status word late (a recorded graph, a stream it does not wait for)
+    // has run its attention over valid key indices, never over uninitialised memory.
+    for (int j = threadIdx.x; j < Zc; j += NT) {
+      idx_out[row * Zc + j] = j;
+      if (val_out) val_out[row * Zc + j] = 0.f;
+    }
     return;
   }
   CandRegs<R> src;

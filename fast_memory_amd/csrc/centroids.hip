@@ -114,11 +114,13 @@ __global__ __launch_bounds__(256) void topk_mean_kernel(const T* __restrict__ Xn
 // cent[h,c,:] = normalise( mean of X[h, perm[...], :] over the cluster's members )
 // members = perm[seg_off[h,c] .. +seg_cnt[h,c]) (positions over the flattened
 // [H*N] sorted axis, values are row indices inside head h); empty -> prev.
-template <typename T>
+// NORM: the rows of X are taken as they are stored and every member contributes row / max(||row||, eps)
+// (the mean of the members' directions; nothing normalised is kept in memory).
+template <typename T, bool NORM>
 __global__ __launch_bounds__(256) void segment_mean_kernel(
     const T* __restrict__ X, const int32_t* __restrict__ perm, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_cnt, const T* __restrict__ prev, T* __restrict__ out, int C,
-    int N, int d) {
+    int N, int d, float eps) {
   __shared__ float sh[4];
   const int c = blockIdx.x, h = blockIdx.y, t = threadIdx.x;
   const int64_t hc = int64_t(h) * C + c;
@@ -128,7 +130,9 @@ __global__ __launch_bounds__(256) void segment_mean_kernel(
   float acc = 0.f;
   for (int j = 0; j < cnt; ++j) {
     int row = min(max(mem[j], 0), N - 1);
-    if (t < d) acc += Elem<T>::load(xb + int64_t(row) * d + t);
+    float x = t < d ? Elem<T>::load(xb + int64_t(row) * d + t) : 0.f;
+    if constexpr (NORM) x *= 1.f / fmaxf(sqrtf(block_sum_256(x * x, sh)), eps);
+    acc += x;
   }
   if (cnt > 0) acc /= float(cnt);
   float ss = block_sum_256(t < d ? acc * acc : 0.f, sh);
@@ -146,10 +150,12 @@ __global__ __launch_bounds__(256) void segment_mean_kernel(
 // j % 16), each lane adding its 8 dimensions of the gathered rows, four rows in flight per group;
 // the sixteen partial sums are then added in group order, so the result does not depend on
 // scheduling.  HBM-bound on the gathered rows (256 bytes per member).
+// NORM as in segment_mean_kernel: a row's squared norm is summed inside its group of 16 lanes.
+template <bool NORM>
 __global__ __launch_bounds__(256) void segment_mean_bf16_d128_kernel(
     const bf16_t* __restrict__ X, const int32_t* __restrict__ perm, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_cnt, const bf16_t* __restrict__ prev, bf16_t* __restrict__ out, int C,
-    int N) {
+    int N, float eps) {
   __shared__ float red[16][128];
   __shared__ float sh[4];
   const int c = blockIdx.x, h = blockIdx.y, t = threadIdx.x;
@@ -172,8 +178,19 @@ __global__ __launch_bounds__(256) void segment_mean_bf16_d128_kernel(
     for (int k = 0; k < U; ++k) {
       float f[8];
       cent_unpack8(u[k], f);
+      if constexpr (NORM) {
+        float ss = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += f[i];
+        for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) ss += __shfl_xor(ss, o);
+        const float inv = 1.f / fmaxf(sqrtf(ss), eps);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(f[i], inv, acc[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += f[i];
+      }
     }
   }
 #pragma unroll
@@ -286,31 +303,49 @@ extern "C" int fm_topk_mean(const void* Xn, const int32_t* top_idx, void* A_out,
   return launch_status("fm_topk_mean");
 }
 
+namespace fm {
+static int segment_mean_any(const char* name, bool norm, const void* X, const int32_t* perm, const int32_t* seg_off,
+                            const int32_t* seg_cnt, const void* prev, void* cent_out, int H, int C, int N, int d,
+                            float eps, int dtype, void* stream) {
+  FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG, "%s: H=%d C=%d N=%d d=%d", name, H, C,
+             N, d);
+  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "%s: dtype=%d", name, dtype);
+  FM_REQUIRE(X && perm && seg_off && seg_cnt && prev && cent_out, FM_ERR_ARG, "%s: null pointer", name);
+  FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "%s: H > 65535", name);
+  dim3 grid = dim3(unsigned(C), unsigned(H));
+  hipStream_t st = as_stream(stream);
+#define FM_SEGMEAN(T, NORM)                                                                                    \
+  hipLaunchKernelGGL((segment_mean_kernel<T, NORM>), grid, dim3(256), 0, st, (const T*)X, perm, seg_off, seg_cnt, \
+                     (const T*)prev, (T*)cent_out, C, N, d, eps)
+  if (dtype == FM_BF16 && d == 128) {
+    if (norm)
+      hipLaunchKernelGGL(segment_mean_bf16_d128_kernel<true>, grid, dim3(256), 0, st, (const bf16_t*)X, perm, seg_off,
+                         seg_cnt, (const bf16_t*)prev, (bf16_t*)cent_out, C, N, eps);
+    else
+      hipLaunchKernelGGL(segment_mean_bf16_d128_kernel<false>, grid, dim3(256), 0, st, (const bf16_t*)X, perm, seg_off,
+                         seg_cnt, (const bf16_t*)prev, (bf16_t*)cent_out, C, N, eps);
+  } else if (dtype == FM_F32) {
+    if (norm) FM_SEGMEAN(float, true); else FM_SEGMEAN(float, false);
+  } else if (dtype == FM_BF16) {
+    if (norm) FM_SEGMEAN(bf16_t, true); else FM_SEGMEAN(bf16_t, false);
+  } else {
+    if (norm) FM_SEGMEAN(f16_t, true); else FM_SEGMEAN(f16_t, false);
+  }
+#undef FM_SEGMEAN
+  return launch_status(name);
+}
+}  // namespace fm
+
 extern "C" int fm_segment_mean(const void* X, const int32_t* perm, const int32_t* seg_off,
                                const int32_t* seg_cnt, const void* prev, void* cent_out, int H,
                                int C, int N, int d, int dtype, void* stream) {
-  using namespace fm;
-  FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && d >= 1 && d <= FM_MAX_D, FM_ERR_ARG,
-             "fm_segment_mean: H=%d C=%d N=%d d=%d", H, C, N, d);
-  FM_REQUIRE(dtype_ok(dtype), FM_ERR_ARG, "fm_segment_mean: dtype=%d", dtype);
-  FM_REQUIRE(X && perm && seg_off && seg_cnt && prev && cent_out, FM_ERR_ARG,
-             "fm_segment_mean: null pointer");
-  FM_REQUIRE(H <= 65535, FM_ERR_UNSUPPORTED, "fm_segment_mean: H > 65535");
-  dim3 grid = dim3(unsigned(C), unsigned(H));
-  if (dtype == FM_BF16 && d == 128)
-    hipLaunchKernelGGL(segment_mean_bf16_d128_kernel, grid, dim3(256), 0, as_stream(stream), (const bf16_t*)X,
-                       perm, seg_off, seg_cnt, (const bf16_t*)prev, (bf16_t*)cent_out, C, N);
-  else if (dtype == FM_F32)
-    hipLaunchKernelGGL(segment_mean_kernel<float>, grid, dim3(256), 0, as_stream(stream),
-                       (const float*)X, perm, seg_off, seg_cnt, (const float*)prev,
-                       (float*)cent_out, C, N, d);
-  else if (dtype == FM_BF16)
-    hipLaunchKernelGGL(segment_mean_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream),
-                       (const bf16_t*)X, perm, seg_off, seg_cnt, (const bf16_t*)prev,
-                       (bf16_t*)cent_out, C, N, d);
-  else
-    hipLaunchKernelGGL(segment_mean_kernel<f16_t>, grid, dim3(256), 0, as_stream(stream),
-                       (const f16_t*)X, perm, seg_off, seg_cnt, (const f16_t*)prev,
-                       (f16_t*)cent_out, C, N, d);
-  return launch_status("fm_segment_mean");
+  return fm::segment_mean_any("fm_segment_mean", false, X, perm, seg_off, seg_cnt, prev, cent_out, H, C, N, d, 0.f,
+                              dtype, stream);
+}
+
+extern "C" int fm_segment_mean_directions(const void* X, const int32_t* perm, const int32_t* seg_off,
+                                          const int32_t* seg_cnt, const void* prev, void* cent_out, int H,
+                                          int C, int N, int d, float eps, int dtype, void* stream) {
+  return fm::segment_mean_any("fm_segment_mean_directions", true, X, perm, seg_off, seg_cnt, prev, cent_out, H, C, N,
+                              d, eps, dtype, stream);
 }

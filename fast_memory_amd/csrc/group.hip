@@ -97,8 +97,10 @@ __global__ __launch_bounds__(1024) void group_items_kernel(const int32_t* __rest
                                                            int32_t* __restrict__ bin_off,
                                                            fm_item* __restrict__ items,
                                                            int32_t* __restrict__ n_items,
-                                                           int64_t max_items) {
+                                                           int64_t max_items,
+                                                           int32_t* __restrict__ n_unlisted) {
   __shared__ int tmp[17];
+  if (threadIdx.x == 0) *n_unlisted = 0;  // the scatter pass counts the queries without a bucket from zero
   int carry_q = 0, carry_i = 0;
   for (int64_t base = 0; base < n; base += 1024) {
     int64_t g = base + threadIdx.x;
@@ -130,10 +132,15 @@ __global__ __launch_bounds__(1024) void group_items_kernel(const int32_t* __rest
 }
 
 // Pass 4: scatter.  position = bucket start + queries of the bucket in earlier
-// blocks + rank inside the block  => stable ascending order.
+// blocks + rank inside the block  => stable ascending order.  A query without a bucket (hash outside
+// [0, C)) goes behind the grouped ones: the grouped queries of all rows fill positions [0, T) of the
+// flattened axis, T = bin_off + bin_count of the last bin, and exactly H*Sq - T queries have no bucket, so
+// each takes one of the remaining slots (in no particular order) and leaves -(h*Sq + i) - 1 there, which
+// is how the attention entry points find the rows no work item writes.
 __global__ __launch_bounds__(kGrpBlock) void group_scatter_kernel(
-    const int32_t* __restrict__ q_hash, int C, int Sq, int NB,
+    const int32_t* __restrict__ q_hash, int H, int C, int Sq, int NB,
     const int32_t* __restrict__ block_hist, const int32_t* __restrict__ bin_off,
+    const int32_t* __restrict__ bin_count, int32_t* __restrict__ n_unlisted,
     int32_t* __restrict__ q_perm) {
   __shared__ int sh[kGrpBlock];
   const int h = blockIdx.y, blk = blockIdx.x, t = threadIdx.x;
@@ -145,7 +152,14 @@ __global__ __launch_bounds__(kGrpBlock) void group_scatter_kernel(
   }
   sh[t] = b;
   __syncthreads();
-  if (b < 0) return;
+  if (b < 0) {
+    if (i < Sq) {
+      const int64_t last = int64_t(H) * C - 1;
+      const int grouped = bin_off[last] + bin_count[last];
+      q_perm[grouped + atomicAdd(n_unlisted, 1)] = -int32_t(int64_t(h) * Sq + i) - 1;
+    }
+    return;
+  }
   int before = 0;
   for (int j = 0; j < t; ++j) before += (sh[j] == b);
   int pos = bin_off[int64_t(h) * C + b] + block_hist[(int64_t(h) * NB + blk) * C + b] + before;
@@ -188,6 +202,39 @@ __global__ __launch_bounds__(256) void window_compact_kernel(const int32_t* __re
     if (keep) o[base + rank] = int32_t(v - lo);
     base += __popcll(m);
   }
+}
+
+// Rows of the queries that are part of no work item (see group_scatter_kernel): `rows16` [nq, row_halves]
+// two-byte units are zeroed and `lse` (if given) set to -FLT_MAX, the result of an empty bucket.  The number
+// of grouped queries comes from the last work item, or from the last bin where there are no items at hand.
+// A wave per row; usually there is none and every wave leaves after two loads.
+__global__ __launch_bounds__(256) void unlisted_rows_kernel(
+    const int32_t* __restrict__ q_perm, const fm_item* __restrict__ items, const int32_t* __restrict__ n_items,
+    const int32_t* __restrict__ bin_off, const int32_t* __restrict__ bin_count, int64_t n_bins, int64_t nq,
+    int row_halves, uint16_t* __restrict__ rows16, float* __restrict__ lse) {
+  int64_t grouped;
+  if (items) {
+    const int n = *n_items;
+    grouped = n > 0 ? int64_t(items[n - 1].q_start) + items[n - 1].n_q : 0;
+  } else {
+    grouped = int64_t(bin_off[n_bins - 1]) + bin_count[n_bins - 1];
+  }
+  const int64_t wave = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6), n_waves = int64_t(gridDim.x) * 4;
+  for (int64_t p = grouped + wave; p < nq; p += n_waves) {
+    const int64_t g = -int64_t(q_perm[p]) - 1;
+    if (g < 0 || g >= nq) continue;  // not a slot the grouping wrote: leave everything alone
+    for (int w = lane_id(); w < row_halves; w += kWave) rows16[g * row_halves + w] = uint16_t(0);
+    if (lse && lane_id() == 0) lse[g] = -FLT_MAX;
+  }
+}
+
+int launch_unlisted_rows(const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                         const int32_t* bin_off, const int32_t* bin_count, int64_t n_bins, int64_t nq,
+                         int row_bytes, void* rows, float* lse, hipStream_t st) {
+  const unsigned blocks = unsigned(std::min<int64_t>(ceil_div(nq, 4), 256));
+  hipLaunchKernelGGL(unlisted_rows_kernel, dim3(blocks), dim3(256), 0, st, q_perm, items, n_items, bin_off,
+                     bin_count, n_bins, nq, row_bytes / 2, static_cast<uint16_t*>(rows), lse);
+  return launch_status("unlisted rows");
 }
 
 int launch_fill(int32_t* p, int64_t n, int32_t v, hipStream_t st) {
@@ -239,6 +286,9 @@ extern "C" int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int
   hipStream_t st = as_stream(stream);
   const int NB = int(ceil_div(Sq, kGrpBlock));
   int32_t* block_hist = static_cast<int32_t*>(ws);
+  // counter of the queries without a bucket: the spare 256 bytes behind the block table
+  int32_t* n_unlisted = reinterpret_cast<int32_t*>(static_cast<char*>(ws) +
+                                                   align_up(size_t(H) * size_t(NB) * size_t(C) * sizeof(int32_t), 256));
   int rc = launch_fill(block_hist, int64_t(H) * NB * C, 0, st);
   if (rc) return rc;
   hipLaunchKernelGGL(group_rank_kernel, dim3(NB, H), dim3(kGrpBlock), 0, st, q_hash, C, Sq, NB,
@@ -246,9 +296,9 @@ extern "C" int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int
   hipLaunchKernelGGL(group_colscan_kernel, dim3(unsigned(ceil_div(int64_t(H) * C, 256))), dim3(256),
                      0, st, block_hist, H, C, NB, bin_count);
   hipLaunchKernelGGL(group_items_kernel, dim3(1), dim3(1024), 0, st, bin_count, int64_t(H) * C, C,
-                     bin_off, items, n_items, max_items);
-  hipLaunchKernelGGL(group_scatter_kernel, dim3(NB, H), dim3(kGrpBlock), 0, st, q_hash, C, Sq, NB,
-                     block_hist, bin_off, q_perm);
+                     bin_off, items, n_items, max_items, n_unlisted);
+  hipLaunchKernelGGL(group_scatter_kernel, dim3(NB, H), dim3(kGrpBlock), 0, st, q_hash, H, C, Sq, NB,
+                     block_hist, bin_off, bin_count, n_unlisted, q_perm);
   return launch_status("fm_group_queries");
 }
 

@@ -31,6 +31,35 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict
   if (acc == 0x9e3779b9u && n < 0) sink[0] = acc;
 }
 
+// Gather of 256-byte rows from a region small enough to stay in the last-level cache and much larger than an
+// XCD's L2: sixteen lanes read one row with one 16-byte load each (the shape of the attention kernels' row
+// fetches), eight rows in flight per group of sixteen lanes.  The rows of a pass are a permutation of the
+// region (an odd multiplier modulo a power of two), so no row is read twice in a pass, and the groups move on by
+// 17 places from pass to pass, so the next reader of a row sits behind another L2.  Nothing is written.  From
+// the second pass on every byte comes out of the last-level cache through the fabric into an L2: the rate is
+// what that path sustains for scattered rows.
+__global__ __launch_bounds__(256) void gather_probe_kernel(const uint4* __restrict__ src, uint32_t region_rows,
+                                                           int passes, uint32_t* __restrict__ sink) {
+  constexpr int U = 8;
+  const uint32_t n_grp = gridDim.x * 16u, lane16 = threadIdx.x & 15u;
+  const uint32_t grp0 = blockIdx.x * 16u + (threadIdx.x >> 4);
+  uint32_t acc = 0;
+  for (int pass = 0; pass < passes; ++pass) {
+    const uint32_t grp = (grp0 + uint32_t(pass) * 17u) % n_grp;
+    for (uint32_t r = grp; r + (U - 1) * n_grp < region_rows; r += U * n_grp) {
+      uint4 x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t row = ((r + u * n_grp) * 0x9E3779B1u) & (region_rows - 1u);
+        x[u] = src[size_t(row) * 16u + lane16];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc ^= x[u].x ^ x[u].y ^ x[u].z ^ x[u].w;
+    }
+  }
+  if (acc == 0x9e3779b9u && passes < 0) sink[0] = acc;
+}
+
 // Register-resident stream of bf16 MFMAs: every wave loads ten operand fragments once and then issues nothing
 // but v_mfma_f32_32x32x16_bf16, four independent accumulator chains in turn (with fewer, the next instruction
 // of a chain waits for the one before it).  No memory, LDS or VALU work inside the loop: its rate is what the
@@ -93,6 +122,20 @@ extern "C" int fm_debug_read(const void* src, int64_t nbytes, void* sink, void* 
   hipLaunchKernelGGL(read_probe_kernel, dim3(4096), dim3(256), 0, as_stream(stream), (const uint4*)src,
                      nbytes / 16, (uint32_t*)sink);
   return launch_status("fm_debug_read");
+}
+
+extern "C" int fm_debug_gather(const void* src, int64_t region_bytes, int passes, void* sink, void* stream) {
+  using namespace fm;
+  const int64_t rows = region_bytes / 256;
+  FM_REQUIRE(src && sink && passes >= 0 && rows >= (1 << 17) && rows <= (int64_t(1) << 31) && (rows & (rows - 1)) == 0 &&
+                 region_bytes % 256 == 0,
+             FM_ERR_ARG, "fm_debug_gather: region_bytes=%lld must be 256 x a power of two >= 2^17, passes=%d",
+             (long long)region_bytes, passes);
+  if (passes == 0) return FM_OK;
+  // 1024 workgroups x 16 groups x 8 rows = 2^17 rows per sweep of the grid
+  hipLaunchKernelGGL(gather_probe_kernel, dim3(1024), dim3(256), 0, as_stream(stream), (const uint4*)src,
+                     uint32_t(rows), passes, (uint32_t*)sink);
+  return launch_status("fm_debug_gather");
 }
 
 extern "C" int fm_debug_copy(void* dst, const void* src, int64_t nbytes, void* stream) {

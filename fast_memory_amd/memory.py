@@ -67,17 +67,19 @@ def compute_centroids(kq: torch.Tensor, centroids: torch.Tensor, n_hashes: int, 
 
 
 @torch.no_grad()
-def kmeans_spherical(X: torch.Tensor, init: torch.Tensor, iters: int):
+def kmeans_spherical(X: torch.Tensor, init: torch.Tensor, iters: int, normalize_rows: Optional[float] = None):
     """Spherical K-means (README.md:37-45): ``X [H,N,d]`` unit rows, ``init
     [H,C,d]`` -> centroids ``[H,C,d]`` (unit rows) and the labels of the last
-    assignment ``[H,N]`` int32."""
+    assignment ``[H,N]`` int32.  With ``normalize_rows=eps`` X holds rows of any length and the
+    result is that of K-means on ``x / max(|x|, eps)``: the assignment ``argmax_c c.x`` does not depend
+    on ``|x|``, and the update divides every member by its norm as it adds it."""
     cent = init.contiguous()
     C = cent.shape[1]
     labels = None
     for _ in range(iters):
         labels = ops.qhash(cent, X)
         groups = ops.group_queries(labels, C)
-        cent = ops.segment_mean(X, groups, cent)
+        cent = ops.segment_mean(X, groups, cent, normalize_rows)
     return cent, labels
 
 
@@ -87,12 +89,12 @@ def fit_projection(keys: torch.Tensor, n_buckets: int, iters: int = 2,
     L2-normalised keys ``[H,N,d]`` (README.md:33-45), starting from the
     reference's seeded random centroids, normalised."""
     H, N, d = keys.shape
-    X = ops.l2_normalize(keys.contiguous(), 1e-6)
     if init is None:
         c0 = init_centroids(n_buckets, d, keys.device, torch.float32)
         c0 = (c0 / c0.norm(dim=-1, keepdim=True)).to(keys.dtype)
         init = c0.unsqueeze(0).expand(H, -1, -1).contiguous()
-    cent, _ = kmeans_spherical(X, init, iters)
+    # no normalised copy of the keys is made: see kmeans_spherical
+    cent, _ = kmeans_spherical(keys.contiguous(), init, iters, normalize_rows=1e-6)
     return cent
 
 
@@ -228,6 +230,7 @@ class Memory:
         self.keys, self.values, self.A = keys, values, A
         self.Z = int(Z) if Z is not None else bucket_idx.shape[2]       # capacity; lists are shorter while N < Z
         self.key_order = bool(key_order)
+        self._build_status = None      # the status word of a build whose check was deferred (check_build)
         self._set_lists(bucket_idx, bucket_val)
 
     def _set_lists(self, bucket_idx: torch.Tensor, bucket_val: Optional[torch.Tensor]):
@@ -241,21 +244,45 @@ class Memory:
 
     @classmethod
     def build(cls, keys: torch.Tensor, values: torch.Tensor, A: torch.Tensor, Z: int,
-              workspace_bytes: int = 8 << 30, keep_values: bool = False, key_order: bool = True) -> "Memory":
+              workspace_bytes: int = 8 << 30, keep_values: bool = False, key_order: bool = True,
+              defer_check: bool = False) -> "Memory":
         """``keep_values`` also stores the projections of the listed keys (4 bytes per list entry), which
-        :meth:`append` needs; ``key_order`` as in the class description."""
+        :meth:`append` needs; ``key_order`` as in the class description.  The fused build's only host
+        synchronisation is the read-back of its status word; with ``defer_check`` the build returns without
+        it (build and attention can then be queued back to back, or recorded into one graph) and
+        :meth:`check_build` -- called by :meth:`append` and :meth:`save`, or by the caller at a point where
+        waiting costs nothing -- looks at the word and rebuilds the lists if rows were left unresolved."""
         keys, values, A = keys.contiguous(), values.contiguous(), A.contiguous()
         assert keys.shape == values.shape and A.shape[0] == keys.shape[0] and A.shape[2] == keys.shape[2]
-        if keep_values:
-            idx, val = ops.build_index(A, keys, Z, workspace_bytes, return_values=True)
-            return cls(keys, values, A, idx, val, Z, key_order)
-        return cls(keys, values, A, ops.build_index(A, keys, Z, workspace_bytes), None, Z, key_order)
+        res = ops.build_index(A, keys, Z, workspace_bytes, return_values=keep_values, defer_check=defer_check)
+        res = res if isinstance(res, tuple) else (res,)
+        status = res[-1] if defer_check else None
+        idx = res[0]
+        val = res[1] if keep_values else None
+        mem = cls(keys, values, A, idx, val, Z, key_order)
+        mem._build_status = status
+        mem._workspace_bytes = workspace_bytes
+        return mem
+
+    def check_build(self) -> bool:
+        """Reads the status word a deferred build left (synchronises with its stream).  ``True``: the lists
+        are final.  ``False``: rows had been left unresolved; the lists have now been rebuilt by the unfused
+        build, and results computed from them before this call are to be discarded."""
+        status, self._build_status = self._build_status, None
+        if status is None or status.unresolved() == 0:
+            return True
+        ops.build_index_unfused_(self.A, self.keys, self.Z, self.bucket_idx, self.bucket_val,
+                                 getattr(self, "_workspace_bytes", 8 << 30))
+        self._inverse = None
+        self._attn_idx = None
+        return False
 
     def append(self, new_keys: torch.Tensor, new_values: torch.Tensor, workspace_bytes: int = 8 << 30) -> "Memory":
         """Add keys/values ``[H,M,d]`` at the end of the memory and bring the bucket lists to what a rebuild
         over all keys would give, without projecting the old keys again (the reference rebuilds on every
         forward, memory.py:252-278).  Needs ``build(..., keep_values=True)``.  Returns ``self``."""
         assert self.bucket_val is not None, "Memory.build(..., keep_values=True) is needed to append"
+        self.check_build()
         new_keys, new_values = new_keys.contiguous(), new_values.contiguous()
         H, M, d = new_keys.shape
         assert new_values.shape == new_keys.shape and H == self.keys.shape[0] and d == self.keys.shape[2]
@@ -275,6 +302,7 @@ class Memory:
     def save(self, path: str) -> None:
         """Write the memory (keys, values, A, lists and, if kept, their values) as a safetensors file."""
         from safetensors.torch import save_file
+        self.check_build()
         t = {"keys": self.keys, "values": self.values, "A": self.A, "bucket_idx": self.bucket_idx}
         if self.bucket_val is not None:
             t["bucket_val"] = self.bucket_val

@@ -73,15 +73,37 @@ def argtopz(Y: torch.Tensor, Z: int, return_values: bool = False):
 last_build_info = {}
 
 
+class DeferredBuildStatus:
+    """Status word of a fused index build that has not been read back yet (``build_index(..., defer_check=True)``):
+    ``unresolved()`` synchronises with the build's stream and says whether rows were left for the unfused build."""
+
+    def __init__(self, status: Optional[torch.Tensor]):
+        self.status = status                 # int32 [2] on the device: rows repaired, rows unresolved; None = unfused
+        self._host = None
+
+    def read(self) -> Tuple[int, int]:
+        if self._host is None:
+            self._host = (0, 0) if self.status is None else tuple(self.status.tolist())
+            last_build_info.update(rows_repaired=self._host[0], rows_unresolved=self._host[1])
+        return self._host
+
+    def unresolved(self) -> int:
+        return self.read()[1]
+
+
 def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int = 8 << 30,
-                fused: Optional[bool] = None, return_values: bool = False):
+                fused: Optional[bool] = None, return_values: bool = False, defer_check: bool = False):
     """Bucket lists [H,C,min(Z,N)] int32 (memory.py:260-278 on one device); with ``return_values`` also
     the fp32 projections of the listed keys (what an index needs to be extended later).
 
     ``fused=None`` takes the fused build (no Y in memory) where the shape is
     eligible and the unfused one otherwise; both give identical lists.  The
-    fused build reports through a two-int status whether any row could not be
-    resolved on the device, in which case the unfused build runs instead."""
+    fused build reports through a two-int status on the device whether any row could not be
+    resolved there, in which case the unfused build runs instead.  Reading that word is the only
+    host synchronisation of the build: with ``defer_check`` it is left out, the lists come back with a
+    :class:`DeferredBuildStatus` as last element and the caller decides when to look (rows left
+    unresolved, more than 64 whose sampled threshold missed, hold keys ``0..Z-1`` until then: valid
+    indices, not the right ones)."""
     _dev(A, K)
     H, C, d = A.shape
     _, N, _ = K.shape
@@ -89,7 +111,13 @@ def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int =
     lib = _lib.load()
     out = torch.empty((H, C, min(int(Z), N)), dtype=torch.int32, device=A.device)
     vals = torch.empty(out.shape, dtype=torch.float32, device=A.device) if return_values else None
-    done = lambda: (out, vals) if return_values else out
+
+    def done(st=None):
+        res = (out, vals) if return_values else (out,)
+        if defer_check:
+            res = res + (DeferredBuildStatus(st),)
+        return res if len(res) > 1 else res[0]
+
     fws = lib.fm_build_index_fused_workspace(H, C, N, d, int(Z), _dt(A)) if fused is not False else 0
     if fused and not fws:
         raise ValueError("fused index build: shape not eligible (bf16, d=128, N>=65536, 64<=Z<=N/8)")
@@ -98,18 +126,29 @@ def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int =
         status = torch.empty(2, dtype=torch.int32, device=A.device)
         check(lib.fm_build_index_fused(_p(A), _p(K), _p(out), _p(vals), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(),
                                        _p(status), _stream(A)))
-        repaired, unresolved = status.tolist()          # one 8-byte read-back per build
-        last_build_info.update(path="fused", rows_repaired=repaired, rows_unresolved=unresolved)
         del ws
+        last_build_info.update(path="fused", rows_repaired=None, rows_unresolved=None)
+        if defer_check:
+            return done(status)
+        repaired, unresolved = status.tolist()          # one 8-byte read-back per build
+        last_build_info.update(rows_repaired=repaired, rows_unresolved=unresolved)
         if unresolved == 0:
             return done()
+    build_index_unfused_(A, K, Z, out, vals, workspace_bytes)
+    return done()
+
+
+def build_index_unfused_(A, K, Z: int, out: torch.Tensor, vals: Optional[torch.Tensor], workspace_bytes: int = 8 << 30):
+    """The unfused build (projection rows into a workspace, arg-top-Z from there) into ``out`` / ``vals``."""
+    H, C, d = A.shape
+    N = K.shape[1]
+    lib = _lib.load()
     last_build_info.update(path="unfused")
     full = lib.fm_build_index_workspace(H, C, N, d, int(Z), H * C)     # every row at once if the budget allows
     one = lib.fm_build_index_workspace(H, C, N, d, int(Z), 1)
     ws = _ws(max(one, min(full, int(workspace_bytes))), A)
     check(lib.fm_build_index(_p(A), _p(K), _p(out), _p(vals), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(),
                              _stream(A)))
-    return done()
 
 
 def index_append(A: torch.Tensor, K_new: torch.Tensor, n_old: int, idx: torch.Tensor, val: torch.Tensor, Z: int,
@@ -458,15 +497,24 @@ def topk_mean(Xn: torch.Tensor, top_idx: torch.Tensor, H: int, G: int, normalize
     return A
 
 
-def segment_mean(X: torch.Tensor, groups: QueryGroups, prev: torch.Tensor) -> torch.Tensor:
-    """Spherical K-means update: X [H,N,d] unit rows grouped by label -> centroids [H,C,d]."""
+def segment_mean(X: torch.Tensor, groups: QueryGroups, prev: torch.Tensor,
+                 normalize_rows: Optional[float] = None) -> torch.Tensor:
+    """Spherical K-means update: X [H,N,d] unit rows grouped by label -> centroids [H,C,d].  With
+    ``normalize_rows=eps`` the rows may have any length: a member contributes ``x / max(|x|, eps)``, so
+    no normalised copy of X is needed."""
     _dev(X, prev)
     H, N, d = X.shape
     _, C, _ = prev.shape
     assert prev.dtype == X.dtype
     out = torch.empty_like(prev)
-    check(_lib.load().fm_segment_mean(_p(X), _p(groups.q_perm), _p(groups.bin_off), _p(groups.bin_count),
-                                      _p(prev), _p(out), H, C, N, d, _dt(X), _stream(X)))
+    lib = _lib.load()
+    if normalize_rows is None:
+        check(lib.fm_segment_mean(_p(X), _p(groups.q_perm), _p(groups.bin_off), _p(groups.bin_count),
+                                  _p(prev), _p(out), H, C, N, d, _dt(X), _stream(X)))
+    else:
+        check(lib.fm_segment_mean_directions(_p(X), _p(groups.q_perm), _p(groups.bin_off), _p(groups.bin_count),
+                                             _p(prev), _p(out), H, C, N, d, float(normalize_rows), _dt(X),
+                                             _stream(X)))
     return out
 
 

@@ -133,8 +133,11 @@ int fm_bucket_offsets(const int32_t* cnt, int64_t n, int64_t* off_out, void* str
  *                           number of queries <= FM_QTILE}
  *   n_items   [1]      out  number of items written
  * max_items must be >= fm_group_max_items(H, C, Sq).  A query whose hash is outside
- * [0, C) belongs to no bucket: it is counted in no bin, is part of no item and
- * appears nowhere in q_perm (whose last slots then stay unwritten). */
+ * [0, C) belongs to no bucket: it is counted in no bin and is part of no item.  The
+ * grouped queries of all rows fill the first T slots of q_perm (T = bin_off +
+ * bin_count of the last bin); each query without a bucket leaves -(h*Sq + i) - 1 in
+ * one of the H*Sq - T slots behind them (in no particular order), which is where the
+ * attention entry points below find the rows that no work item writes. */
 typedef struct { int32_t row, bucket, q_start, n_q; } fm_item;
 int64_t fm_group_max_items(int H, int C, int Sq);
 size_t fm_group_queries_workspace(int H, int C, int Sq);
@@ -149,8 +152,8 @@ int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int32_t* q_per
  *   k_idx flat int32, bucket_off [H*C] int64, bucket_cnt [H*C] int32
  *   q_perm, items, n_items            from fm_group_queries
  *   out [H,Sq,d] (dtype of q), lse [H,Sq] fp32 natural log, original order.
- * A query whose bucket is empty gets out = 0, lse = -FLT_MAX.  Rows of queries that
- * are part of no item (hash outside [0, C), see fm_group_queries) are not written. */
+ * A query whose bucket is empty gets out = 0, lse = -FLT_MAX, and so does a query
+ * that is part of no item (hash outside [0, C), see fm_group_queries). */
 int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
                      const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                      const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
@@ -196,7 +199,8 @@ int fm_lists_key_order(const int32_t* k_idx, const int64_t* bucket_off, const in
  *   dout [H,Sq,d]                      gradient of the loss w.r.t. out
  *   dlse [H,Sq] fp32, may be NULL      gradient of the loss w.r.t. lse (a caller that merges
  *                                      partial results by their lse outside has one; NULL = 0)
- *   dq [H,Sq,d] (dtype of q)           written; a query whose bucket is empty gets 0
+ *   dq [H,Sq,d] (dtype of q)           written; a query whose bucket is empty, or that has no
+ *                                      bucket (hash outside [0, C)), gets 0
  *   dk, dv [H,N,d] fp32                ACCUMULATED into (atomic adds): zero them
  *                                      before the first call; several calls
  *                                      (key windows) may add into the same buffers.
@@ -320,7 +324,11 @@ int fm_lse_merge(float* out, float* lse, const void* block_out, const float* blo
  * fm_segment_mean: spherical K-means centroid update (README.md:41-43):
  *                  X [H,N,d] unit rows, perm/seg_off/seg_cnt from
  *                  fm_group_queries on the labels; an empty cluster keeps
- *                  prev; cent_out [H,C,d] in dtype, unit rows. */
+ *                  prev; cent_out [H,C,d] in dtype, unit rows.
+ * fm_segment_mean_directions: the same update on rows of any length: member x
+ *                  contributes x / max(||x||, eps), so K-means on the L2-normalised
+ *                  keys (README.md:33-45) never stores the normalised copy (the
+ *                  assignment argmax_c c.x does not depend on ||x||). */
 int fm_l2_normalize(const void* X, void* Xn, int64_t rows, int d, float eps, int dtype,
                     void* stream);
 int fm_topk_mean(const void* Xn, const int32_t* top_idx, void* A_out, int C, int H, int G, int N,
@@ -328,6 +336,9 @@ int fm_topk_mean(const void* Xn, const int32_t* top_idx, void* A_out, int C, int
 int fm_segment_mean(const void* X, const int32_t* perm, const int32_t* seg_off,
                     const int32_t* seg_cnt, const void* prev, void* cent_out, int H, int C, int N,
                     int d, int dtype, void* stream);
+int fm_segment_mean_directions(const void* X, const int32_t* perm, const int32_t* seg_off,
+                               const int32_t* seg_cnt, const void* prev, void* cent_out, int H, int C,
+                               int N, int d, float eps, int dtype, void* stream);
 
 /* ---- f3: extending an index by new keys -----------------------------------
  * The reference rebuilds the bucket lists from all keys on every forward

@@ -5,7 +5,7 @@
  * fm_debug_argtopz_exact_only, fm_debug_fused_filter, fm_debug_set_phase_events) are PROCESS-WIDE state, read by every call on
  * every stream: they exist so that tests can compare two implementations of one operator and so that the
  * benchmark can time the phases of the fused build; a production caller never touches them.  The probes
- * (fm_debug_copy, fm_debug_read, fm_debug_mfma) are plain kernels of known size.
+ * (fm_debug_copy, fm_debug_read, fm_debug_gather, fm_debug_mfma) are plain kernels of known size.
  */
 #ifndef FASTMEM_DEBUG_H
 #define FASTMEM_DEBUG_H
@@ -75,6 +75,14 @@ int fm_debug_copy(void* dst, const void* src, int64_t nbytes, void* stream);
  * nothing is written (sink: 4 bytes of device memory, left untouched).  Times the
  * read bandwidth a kernel reaches on the device. */
 int fm_debug_read(const void* src, int64_t nbytes, void* sink, void* stream);
+
+/* Diagnostic: `passes` sweeps over region_bytes (256 x a power of two >= 2^17) of device memory in which every
+ * 256-byte row is read exactly once per sweep, in a scattered order, by sixteen lanes with a 16-byte load each
+ * (the row fetch of the gathered attention); from one sweep to the next a row's reader moves behind another L2.
+ * With a region that the last-level cache holds and an L2 does not (say 64 MiB), the bytes of every sweep after the
+ * first come out of the last-level cache: region_bytes * passes / time is the rate the path from that cache into
+ * the L2s sustains for scattered rows.  Nothing is written (sink: 4 bytes, left untouched). */
+int fm_debug_gather(const void* src, int64_t region_bytes, int passes, void* sink, void* stream);
 
 /* Diagnostic: a register-resident stream of v_mfma_f32_32x32x16_bf16 (no memory, LDS or VALU work in
  * the loop) over the first 5120 bf16 values at `operands` (n_operands >= 5120): iters * 2^33 flops per call.

@@ -52,3 +52,66 @@ def test_hash_and_attention_replayed_from_a_graph(dtype):
         assert float(out_g.float().abs().sum()) > 0
     ref_out, ref_lse = ops.attention_hash_varlen_i32(q, k, v, kh, cnt, qh_e, scale)
     assert torch.equal(out_g.view(torch.int16), ref_out.view(torch.int16)) and torch.equal(lse_g, ref_lse)
+
+
+def test_build_hash_and_attention_in_one_graph():
+    """Index build and query path recorded together: fm_qhash -> fm_build_index_fused -> fm_lists_key_order ->
+    fm_attention_hash_varlen_static, all through the C ABI into one graph (kernels only: the build reads
+    nothing back, its status word stays on the device and is looked at after the replays).  Keys, values and
+    queries change between replays; every replay equals the eager run of the same calls bit for bit, and the
+    lists equal those of the Python wrapper that does check the status."""
+    dtype, dt = torch.bfloat16, 1
+    H, S, N, C, Z, d = 2, 3000, 65536, 40, 512, 128
+    g = gen(61)
+    mk = lambda *shape: (torch.randn(*shape, generator=g) * 0.5).to(dtype).cuda()
+    k, v, q, A = mk(H, N, d), mk(H, N, d), mk(H, S, d), mk(H, C, d)
+    scale = d ** -0.5
+    lib = _lib.load()
+    ws_bytes = lib.fm_build_index_fused_workspace(H, C, N, d, Z, dt)
+    assert ws_bytes > 0, "the shape must be one the fused build takes"
+    cnt = torch.full((H, C), Z, dtype=torch.int32, device="cuda")
+    off = (torch.arange(H * C, dtype=torch.int64, device="cuda") * Z)
+
+    def bufs():
+        return dict(ws=torch.empty(ws_bytes, dtype=torch.uint8, device="cuda"),
+                    idx=torch.zeros(H, C, Z, dtype=torch.int32, device="cuda"),
+                    idx_k=torch.zeros(H * C * Z, dtype=torch.int32, device="cuda"),
+                    status=torch.zeros(2, dtype=torch.int32, device="cuda"),
+                    qh=torch.zeros(H, S, dtype=torch.int32, device="cuda"), out=torch.zeros_like(q),
+                    lse=torch.zeros(H, S, dtype=torch.float32, device="cuda"))
+
+    def run(b):
+        st = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.fm_qhash(A.data_ptr(), q.data_ptr(), b["qh"].data_ptr(), None, H, C, S, d, dt, st))
+        _lib.check(lib.fm_build_index_fused(A.data_ptr(), k.data_ptr(), b["idx"].data_ptr(), None, H, C, N, d, Z, dt,
+                                            b["ws"].data_ptr(), ws_bytes, b["status"].data_ptr(), st))
+        _lib.check(lib.fm_lists_key_order(b["idx"].data_ptr(), off.data_ptr(), cnt.data_ptr(), H * C, N,
+                                          b["idx_k"].data_ptr(), None, st))
+        _lib.check(lib.fm_attention_hash_varlen_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), b["idx_k"].data_ptr(),
+                                                       cnt.data_ptr(), b["qh"].data_ptr(), b["out"].data_ptr(),
+                                                       b["lse"].data_ptr(), H, S, N, d, C, scale, dt, st))
+
+    e, gb = bufs(), bufs()
+    run(e)                               # first calls: kernel attributes, the static array's address
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(gb)
+    for rep in range(3):
+        if rep:
+            k.copy_(mk(H, N, d))
+            v.copy_(mk(H, N, d))
+            q.copy_(mk(H, S, d))
+        graph.replay()
+        torch.cuda.synchronize()
+        run(e)
+        torch.cuda.synchronize()
+        assert gb["status"].tolist()[1] == 0 and e["status"].tolist()[1] == 0
+        for name in ("qh", "idx", "idx_k"):
+            assert torch.equal(gb[name], e[name]), f"replay {rep}: {name} differs"
+        assert torch.equal(gb["out"].view(torch.int16), e["out"].view(torch.int16)), f"replay {rep}: out differs"
+        assert torch.equal(gb["lse"].view(torch.int32), e["lse"].view(torch.int32)), f"replay {rep}: lse differs"
+    assert torch.equal(gb["idx"], ops.build_index(A, k, Z, fused=True))
+    # the deferred check of the Python wrapper: same lists, nothing read back until asked
+    idx2, st2 = ops.build_index(A, k, Z, fused=True, defer_check=True)
+    assert st2.unresolved() == 0 and torch.equal(idx2, gb["idx"])

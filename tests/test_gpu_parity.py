@@ -507,7 +507,8 @@ def test_attention_with_listed_item_groups(ops, dtype):
         sync()
         res.append((out, lse))
     assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
-    assert bool((res[1][1][1, ::7] == 7.0).all())                            # rows of no bucket: untouched
+    # rows of no bucket: the result of an empty bucket
+    assert bool((res[1][1][1, ::7] < -1e30).all()) and bool((res[1][0][1, ::7] == 0).all())
     ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh.clamp(min=0), d ** -0.5)
     keep = qh >= 0
     assert_attn_close(res[1][0][keep], res[1][1][keep], ro[keep], rl[keep], dtype, "listed groups")
@@ -515,7 +516,7 @@ def test_attention_with_listed_item_groups(ops, dtype):
 
 def test_attention_a_launch_per_row_finds_every_rows_items(ops):
     """Eleven rows with very different numbers of work items, among them rows whose queries all carry a hash
-    outside [0, C) (no item at all; their output rows are never written): the per-row launches write exactly
+    outside [0, C) (no item at all; their rows get the result of an empty bucket): the per-row launches write exactly
     what the single launch writes."""
     H, S, N, C, Z, d = 11, 520, 700, 37, 90, 128
     q, k, v, kh, cnt, qh = make_attn_case(36, H, S, N, C, Z, d, torch.bfloat16, std=0.8)
@@ -546,7 +547,8 @@ def test_attention_a_launch_per_row_finds_every_rows_items(ops):
     assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
     assert torch.equal(res[2][0], res[3][0]) and torch.equal(res[2][1], res[3][1])
     for _, lse_r in res:
-        assert bool((lse_r[3] == 7.0).all()) and bool((lse_r[10] == 7.0).all())           # untouched rows
+        assert bool((lse_r[3] < -1e30).all()) and bool((lse_r[10] < -1e30).all())         # rows without a bucket
+        assert bool((lse_r[5, 40:] < -1e30).all())
         assert bool((lse_r[0] != 7.0).all())
 
 
@@ -710,10 +712,9 @@ def test_compute_centroids(ops, dtype):
     assert torch.allclose(A.float().norm(dim=-1), torch.ones(C, H), atol=1e-2)
     if dtype == torch.float32:
         assert torch.allclose(A, ref, atol=1e-5), (A - ref).abs().max()
-    else:
-        # bf16 scores: a near-tie at the k-th place may swap one of the G*k averaged rows
-        row_ok = ((A.float() - ref.float()).abs().amax(-1) < 1e-2).float().mean().item()
-        assert row_ok >= 0.9, row_ok
+    # bf16: a near-tie of the rounded scores at the k-th place may swap one of the averaged rows against
+    # the oracle's choice, so that case is held exactly elsewhere, on the GPU's own scores
+    # (test_gpu_strict.py::test_compute_centroids_bf16_exact); here its shape and unit rows are checked
 
 
 def test_kmeans_matches_oracle_fp32(ops):
@@ -758,6 +759,33 @@ def test_l2_normalize_and_segment_mean_bf16_d128(ops):
         lab = labels[h].cpu().long()
         rc = O.kmeans_update(Xn[h].float(), lab, init[h].float())
         assert torch.allclose(cent[h].float().cpu().double(), rc.double(), atol=4e-3, rtol=8e-3)
+
+
+@pytest.mark.parametrize("dtype,d,C", [(torch.bfloat16, 128, 37), (torch.float32, 64, 20), (torch.float16, 128, 11),
+                                       (torch.bfloat16, 64, 9)])
+def test_kmeans_on_unnormalised_rows(ops, dtype, d, C):
+    """K-means on the L2-normalised keys (README.md:33-45) without a normalised copy: the assignment on the
+    rows as stored (argmax_c c.x does not depend on |x|), the update dividing every member by its norm as it
+    adds it -- against the oracle's update on the fp64-normalised rows for the GPU's own labels, and against the
+    path that stores the normalised rows."""
+    from fast_memory_amd import kmeans_spherical
+    g = gen(704)
+    H, N = 2, 4000
+    X = (torch.randn(H, N, d, generator=g) * torch.exp(torch.randn(H, N, 1, generator=g))).to(dtype)
+    X[1, 11] = 0                                            # a zero row contributes nothing
+    init = O.l2_normalize(O.init_centroids(C, d)).to(dtype).unsqueeze(0).expand(H, -1, -1).contiguous()
+    cent, labels = kmeans_spherical(dev(X), dev(init), 1, normalize_rows=1e-6)
+    Xn = O.l2_normalize(X.double())
+    tol = 1e-5 if dtype == torch.float32 else 4e-3
+    for h in range(H):
+        lab = labels[h].cpu().long()
+        rc = O.kmeans_update(Xn[h], lab, init[h].double())
+        assert torch.allclose(cent[h].float().cpu().double(), rc, atol=tol, rtol=2 * tol)
+        # the labels are those of the normalised rows up to near-ties of the rounded scores
+        agree = (lab == O.kmeans_assign(Xn[h], init[h].double())).float().mean().item()
+        assert agree > (0.999 if dtype == torch.float32 else 0.97), agree
+    cent2, labels2 = kmeans_spherical(ops.l2_normalize(dev(X)), dev(init), 1)
+    assert (labels2 == labels).float().mean().item() > (0.999 if dtype == torch.float32 else 0.97)
 
 
 # ------------------------------------------------------------------ golden fixture (frozen oracle outputs)

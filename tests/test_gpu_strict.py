@@ -241,6 +241,46 @@ def test_out_of_range_query_hash_is_an_empty_bucket(ops, dtype, d):
     groups = ops.group_queries(dev(qh_bad.int()), 5)
     assert torch.equal(groups.bin_count.cpu().long(),
                        torch.stack([torch.bincount(qh[b][good[b]], minlength=5) for b in range(2)]))
+    # the grouped queries fill the first slots of q_perm, the three without a bucket the last ones, coded
+    # as -(flat query index) - 1
+    tail = sorted((-groups.q_perm.reshape(-1)[-3:].cpu().long() - 1).tolist())
+    assert tail == [3, 50, 90 + 89]
+    # every forward entry defines those rows, not only the one-call operator: poison the outputs' memory
+    # first (the caching allocator hands the same blocks out again)
+    off = ops.bucket_offsets(dev(cnt.int()))
+    for _ in range(2):
+        junk = torch.full((2, 90, d), float("nan"), dtype=dtype, device="cuda")
+        junk_l = torch.full((2, 90), float("nan"), device="cuda")
+        del junk, junk_l
+        o2, l2 = ops.hash_attn_fwd(*dev(q, k, v, kh.int()), off, dev(cnt.int()), groups, 0.2)
+        assert torch.equal(o2, out) and torch.equal(l2, lse)
+    # ... and so does the backward: dq = 0 for them, the other gradients as without them
+    from fast_memory_amd import attention_hash_varlen_op
+    g = gen(7601)
+    w = (torch.randn(2, 90, d, generator=g) * 0.5).to(dtype)
+    w0 = w.clone()
+    w0[bad] = 0                                            # "good" run: the three queries hashed, their d_out zero
+    grads = {}
+    for name, hashes, wt in (("bad", qh_bad, w), ("good", qh, w0)):
+        qd, kd, vd = (t.requires_grad_(True) for t in dev(q, k, v))
+        junk = torch.full((2, 90, d), float("nan"), dtype=dtype, device="cuda")
+        del junk
+        o3, _ = attention_hash_varlen_op(qd, kd, vd, *dev(kh, cnt, hashes), 0.2)
+        (o3.float() * dev(wt).float()).sum().backward()
+        grads[name] = (qd.grad, kd.grad, vd.grad)
+    assert bool((grads["bad"][0][dev(bad)] == 0).all()), "dq of a query without a bucket"
+    assert torch.equal(grads["bad"][0][dev(good)], grads["good"][0][dev(good)])
+    # dk / dv: a query with zero d_out contributes nothing, so the two runs agree up to the order of the
+    # fp32 atomic adds
+    for j in (1, 2):
+        a, b = grads["bad"][j].float(), grads["good"][j].float()
+        assert bool(torch.isfinite(a).all())
+        # (bf16 takes the form without atomics, whose per-bucket partial rows are bf16 sums over query tiles:
+        # three queries fewer in a row move the tile boundaries, and with them those roundings)
+        if dtype == torch.float32:
+            assert torch.allclose(a, b, atol=1e-5 * max(1.0, b.abs().max().item()), rtol=1e-4)
+        else:
+            assert (a - b).abs().max().item() <= 2e-2 * b.abs().max().item()
 
 
 # ------------------------------------------------------------------ a2 in the fused build: ties and long runs

@@ -582,6 +582,9 @@ def main():
     ap.add_argument("--list-order", default="key", choices=["key", "value"],
                     help="order of a bucket's list as the gathered attention reads it: ascending key index (the "
                          "copy Memory keeps for its attention) or descending score as torch.topk leaves it")
+    ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128, 256],
+                    help="run the configuration's shape with another head dimension (the reference kernel is "
+                         "generic in d_head); 0 keeps the configuration's own")
     ap.add_argument("--no-c4-build", action="store_true",
                     help="with --config c5: leave out the index build of c4 (the configuration the keys/s half of "
                          "the metric is quoted on), which otherwise runs after the c5 step and goes into the same line")
@@ -605,6 +608,9 @@ def main():
     if args.config == "tkperf":
         return bench_reference_harness(args)
     cfg = synth.CONFIGS[args.config]
+    if args.head_dim and args.head_dim != cfg.d:
+        import dataclasses
+        cfg = dataclasses.replace(cfg, d=args.head_dim, name=f"{cfg.name}-d{args.head_dim}")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     H, G, d, N, C, Z, S = cfg.H, cfg.G, cfg.d, cfg.N, cfg.C, cfg.Z, cfg.S
@@ -762,7 +768,7 @@ def main():
     attn_kernel = ops.hash_attn_fwd_kernel_name(H, Sq, N, d, C, cfg.dtype)     # what the library's dispatch took
     launches = ops.hash_attn_fwd_launches(H, Sq, N, d, C, cfg.dtype)           # one per row on large memories
     # fabric-side bytes per launch as the profiler counts them (L2 misses; HBM and the last-level cache answer)
-    traffic = hbm_traffic(attn_kernel, cfg.name, required=args.config != "c1")
+    traffic = hbm_traffic(attn_kernel, cfg.name, required=args.config != "c1" and not args.head_dim)
     avg_launch_ms = attn_ms / launches
     hit_mask = groups.bin_count > 0
     rows_per_launch = H / launches

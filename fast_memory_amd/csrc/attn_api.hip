@@ -46,6 +46,9 @@ extern "C" void fm_debug_force_generic(int on) { fm::g_force_generic.store(on, s
 extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype) {
   using namespace fm;
   if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype, N)) return "hash_attn_generic_kernel";
+  if (d == 64) return dtype == FM_F16 ? "hash_attn_staged_d_kernel<64, f16>" : "hash_attn_staged_d_kernel<64>";
+  if (d == 256) return dtype == FM_F16 ? "hash_attn_staged_d_kernel<256, f16>" : "hash_attn_staged_d_kernel<256>";
+  if (g_force_generic == 8) return dtype == FM_F16 ? "hash_attn_staged_d_kernel<128, f16>" : "hash_attn_staged_d_kernel<128>";
   const int choice = hash_attn_mfma_choice(H, Sq, N, C);
   if (choice && N > (1 << 24))
     return dtype == FM_F16 ? "hash_attn_staged_kernel<1, f16, 64-bit rows>" : "hash_attn_staged_kernel<1, 64-bit rows>";
@@ -62,7 +65,7 @@ extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int 
 
 extern "C" int fm_hash_attn_fwd_launches(int H, int Sq, int N, int d, int C, int dtype) {
   using namespace fm;
-  if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype, N)) return 1;
+  if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype, N) || d != 128 || g_force_generic == 8) return 1;
   int choice = hash_attn_mfma_choice(H, Sq, N, C);
   if (dtype == FM_F16 && choice == 0) choice = 1;
   return hash_attn_mfma_per_row(choice, H, Sq, N, C) ? H : 1;

@@ -470,9 +470,14 @@ int local_attn_decode(const void* q, const void* k, const void* v, void* out, fl
   return launch_status("fm_local_attn_fwd(decode)");
 }
 
+bool hash_attn_mfma_d_supported(int d, int N);  // attn_mfma_d.hip
+int hash_attn_mfma_d(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
+                     const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
+                     int64_t max_items, void* out, float* lse, int Sq, int N, int d, int C, float sm_scale, bool f16,
+                     hipStream_t st);
+
 bool hash_attn_mfma_supported(int d, int dtype, int N) {
-  (void)N;
-  return d == kD && (dtype == FM_BF16 || dtype == FM_F16);
+  return (d == kD || hash_attn_mfma_d_supported(d, N)) && (dtype == FM_BF16 || dtype == FM_F16);
 }
 
 int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const void* V_all,
@@ -558,7 +563,10 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
                    const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
                    float* lse, int H, int Sq, int N, int d, int C, float sm_scale, int dtype, void* ws, size_t ws_bytes,
                    hipStream_t st) {
-  (void)d;
+  // head dimensions 64 and 256, and 128 when a test asks for the kernel that takes every head dimension
+  if (d != kD || (g_force_generic == 8 && int64_t(N) * 2 * d < (int64_t(1) << 32)))
+    return hash_attn_mfma_d(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse, Sq,
+                            N, d, C, sm_scale, dtype == FM_F16, st);
   int choice = hash_attn_mfma_choice(H, Sq, N, C);
   if (dtype == FM_F16 && choice == 0) choice = 1;
   const bool per_row = hash_attn_mfma_per_row(choice, H, Sq, N, C);

@@ -471,6 +471,57 @@ def test_attention_grouped_forward_kernels(ops, which, case):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large"])
+def test_attention_mfma_forward_over_head_dimensions(ops, dtype, d, case):
+    """The reference kernel is generic in d_head (triton_kernel.py:141-147; its own test shapes run d = 16 and
+    d = 128, triton_kernel.py:500-505).  Head dimensions 64 and 256 take the MFMA kernel whose extents are
+    functions of the head dimension -- not the generic one -- and meet the oracle on the cases of the d = 128
+    kernels; instantiated for 128 it gives the bits of the kernels built for 128."""
+    if case == "ragged":
+        q, k, v, kh, cnt, qh = make_attn_case(131, 2, 900, 5000, 24, 333, d, dtype, std=0.7)
+    elif case == "full-items":
+        q, k, v, kh, cnt, qh = make_attn_case(132, 2, 700, 4096, 40, 300, d, dtype, window="all", std=1.0)
+        sizes = [1, 15, 16, 17, 63, 64, 65, 200]
+        pos = 0
+        for b, n in enumerate(sizes):
+            qh[0, pos:pos + n] = b
+            pos += n
+        qh[0, pos:] = torch.randint(len(sizes), 40, (700 - pos,), generator=gen(133))
+    else:
+        q, k, v, kh, cnt, qh = make_attn_case(120, 1, 2 * 2040, 1023 * 60, 512, 1024, d, dtype)
+        assert (cnt == 0).any()
+    H, S, N, C = q.shape[0], q.shape[1], k.shape[1], cnt.shape[1]
+    if d != 128:
+        name = ops.hash_attn_fwd_kernel_name(H, S, N, d, C, dtype)
+        assert name.startswith(f"hash_attn_staged_d_kernel<{d}"), name
+        out, lse = run_varlen(q, k, v, kh, cnt, qh, d ** -0.5)
+    else:
+        from fast_memory_amd import _lib
+        _lib.load().fm_debug_force_generic(8)               # the kernel of every head dimension, at 128
+        try:
+            assert ops.hash_attn_fwd_kernel_name(H, S, N, d, C, dtype).startswith("hash_attn_staged_d_kernel<128")
+            out, lse = run_varlen(q, k, v, kh, cnt, qh, d ** -0.5)
+        finally:
+            ops.grouped_forward_kernel(None)
+        ops.grouped_forward_kernel("staged")
+        try:
+            o1, l1 = run_varlen(q, k, v, kh, cnt, qh, d ** -0.5)
+        finally:
+            ops.grouped_forward_kernel(None)
+        assert torch.equal(out, o1) and torch.equal(lse, l1), "the 128-wide instantiation differs from the staged kernel"
+    ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, d ** -0.5)
+    assert_attn_close(out, lse, ro, rl, dtype, f"d={d} {case}")
+    # and against the generic kernel, which defines the numerics of every other shape
+    ops.force_generic_kernels(True)
+    try:
+        og, lg = run_varlen(q, k, v, kh, cnt, qh, d ** -0.5)
+    finally:
+        ops.force_generic_kernels(False)
+    assert_attn_close(out, lse, og.float().cpu(), lg.cpu(), dtype, f"d={d} {case} vs generic")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_attention_with_listed_item_groups(ops, dtype):
     """More than 64 queries per bucket on average: with its workspace the forward lists the groups of three
     items first (fm_hash_attn_fwd_ws), without it a workgroup is started per item and two of three return.  The

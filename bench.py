@@ -26,6 +26,10 @@ import time
 
 import torch
 
+# the phase markers of the fused build and the forced kernels of the controls are diagnostic switches of the
+# library, which take effect only in a process that asks for them before the library's first call
+os.environ.setdefault("FASTMEM_DEBUG_HOOKS", "1")
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 

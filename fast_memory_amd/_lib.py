@@ -17,6 +17,7 @@ FM_MAX_Z = 16384
 FM_MAX_D = 256
 FM_QTILE = 64
 FM_STATIC_SCRATCH_BYTES = 32 << 20
+FM_FUSED_STATUS_INTS = 66
 
 P = c_void_p
 
@@ -67,6 +68,7 @@ SIGNATURES = {
     "fm_index_append_workspace": (c_size_t, [c_int, c_int, c_int]),
     "fm_index_append": (c_int, [P, P, c_int, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, c_size_t, P, P]),
     "fm_segment_sum": (c_int, [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P]),
+    "fm_debug_hooks_enabled": (c_int, []),
     "fm_debug_force_generic": (None, [c_int]),
     "fm_hash_attn_fwd_kernel": (ctypes.c_char_p, [c_int] * 6),
     "fm_hash_attn_fwd_launches": (c_int, [c_int] * 6),

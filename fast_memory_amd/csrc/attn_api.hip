@@ -41,7 +41,9 @@ int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const 
 std::atomic<int> g_force_generic{0};
 }  // namespace fm
 
-extern "C" void fm_debug_force_generic(int on) { fm::g_force_generic.store(on, std::memory_order_relaxed); }
+extern "C" void fm_debug_force_generic(int on) {
+  if (fm::debug_hooks_enabled()) fm::g_force_generic.store(on, std::memory_order_relaxed);
+}
 
 extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype) {
   using namespace fm;

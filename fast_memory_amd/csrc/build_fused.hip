@@ -1052,10 +1052,16 @@ __global__ __launch_bounds__(256) void project_listed_rows_kernel(
   }
 }
 
-__global__ void fused_status_kernel(const int32_t* __restrict__ n_fail, int32_t* __restrict__ status) {
-  const int f = *n_fail;
-  status[0] = min(f, kMaxRepair);
-  status[1] = max(0, f - kMaxRepair);
+__global__ __launch_bounds__(64) void fused_status_kernel(const int32_t* __restrict__ n_fail,
+                                                          const int32_t* __restrict__ fail_rows,
+                                                          int32_t* __restrict__ status) {
+  const int f = *n_fail, t = threadIdx.x;
+  if (t == 0) {
+    status[0] = min(f, kMaxRepair);
+    status[1] = max(0, f - kMaxRepair);
+  }
+  static_assert(FM_FUSED_STATUS_INTS == 2 + kMaxRepair, "the status word names every repaired row");
+  status[2 + t] = t < min(f, kMaxRepair) ? fail_rows[t] : -1;  // the repaired (head * C + bucket) rows
 }
 
 // optional phase markers for profiling: events recorded after phases 0, 1, 2, 3
@@ -1071,9 +1077,12 @@ static inline void mark_phase(int i, hipStream_t st) {
 
 }  // namespace fm
 
-extern "C" void fm_debug_fused_filter(int form) { fm::g_fused_filter_form.store(form, std::memory_order_relaxed); }
+extern "C" void fm_debug_fused_filter(int form) {
+  if (fm::debug_hooks_enabled()) fm::g_fused_filter_form.store(form, std::memory_order_relaxed);
+}
 
 extern "C" void fm_debug_set_phase_events(void** events, int n) {
+  if (!fm::debug_hooks_enabled()) return;
   std::lock_guard<std::mutex> lk(fm::g_phase_mu);
   fm::g_phase_events = reinterpret_cast<hipEvent_t*>(events);
   fm::g_n_phase_events = events ? n : 0;
@@ -1182,7 +1191,7 @@ extern "C" int fm_build_index_fused(const void* A, const void* K, int32_t* idx_o
                        fail_rows, n_fail, Yf, C, N, p.ldy);
   rc = launch_argtopz(Yf, kMaxRepair, N, p.ldy, Zc, idx_out, val_out, fail_rows, n_fail, st);
   if (rc) return rc;
-  hipLaunchKernelGGL(fused_status_kernel, dim3(1), dim3(1), 0, st, n_fail, status_dev);
+  hipLaunchKernelGGL(fused_status_kernel, dim3(1), dim3(64), 0, st, n_fail, fail_rows, status_dev);
   mark_phase(4, st);
   return launch_status("fm_build_index_fused");
 }

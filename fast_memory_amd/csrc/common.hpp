@@ -13,6 +13,7 @@ namespace fm {
 // ---- host side: status + message ------------------------------------------
 void set_error(const char* fmt, ...);
 int launch_status(const char* what);  // FM_OK, or FM_ERR_LAUNCH with message
+bool debug_hooks_enabled();            // FASTMEM_DEBUG_HOOKS=1 was set when the library was first called
 
 #define FM_REQUIRE(cond, code, ...)   \
   do {                                \

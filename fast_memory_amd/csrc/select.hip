@@ -324,7 +324,9 @@ extern "C" size_t fm_argtopz_workspace(int64_t rows, int N, int Z) {
   return fm::argtopz_big_workspace(rows, Z < N ? Z : N);
 }
 
-extern "C" void fm_debug_argtopz_exact_only(int on) { fm::g_argtopz_exact_only = on != 0; }
+extern "C" void fm_debug_argtopz_exact_only(int on) {
+  if (fm::debug_hooks_enabled()) fm::g_argtopz_exact_only = on != 0;
+}
 
 extern "C" int fm_argtopz_f32(const float* Y, int64_t rows, int N, int64_t ldy, int Z,
                               int32_t* idx_out, float* val_out, void* ws, size_t ws_bytes, void* stream) {

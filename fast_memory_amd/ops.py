@@ -78,13 +78,14 @@ class DeferredBuildStatus:
     ``unresolved()`` synchronises with the build's stream and says whether rows were left for the unfused build."""
 
     def __init__(self, status: Optional[torch.Tensor]):
-        self.status = status                 # int32 [2] on the device: rows repaired, rows unresolved; None = unfused
+        self.status = status                 # the device status word of fm_build_index_fused; None = unfused
         self._host = None
 
     def read(self) -> Tuple[int, int]:
         if self._host is None:
-            self._host = (0, 0) if self.status is None else tuple(self.status.tolist())
-            last_build_info.update(rows_repaired=self._host[0], rows_unresolved=self._host[1])
+            st = [0, 0] if self.status is None else self.status.tolist()
+            self._host = (st[0], st[1])
+            last_build_info.update(rows_repaired=st[0], rows_unresolved=st[1], repaired_rows=[r for r in st[2:] if r >= 0])
         return self._host
 
     def unresolved(self) -> int:
@@ -123,15 +124,17 @@ def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int =
         raise ValueError("fused index build: shape not eligible (bf16, d=128, N>=65536, 64<=Z<=N/8)")
     if fws:
         ws = _ws(fws, A)
-        status = torch.empty(2, dtype=torch.int32, device=A.device)
+        status = torch.empty(_lib.FM_FUSED_STATUS_INTS, dtype=torch.int32, device=A.device)
         check(lib.fm_build_index_fused(_p(A), _p(K), _p(out), _p(vals), H, C, N, d, int(Z), _dt(A), _p(ws), ws.numel(),
                                        _p(status), _stream(A)))
         del ws
         last_build_info.update(path="fused", rows_repaired=None, rows_unresolved=None)
         if defer_check:
             return done(status)
-        repaired, unresolved = status.tolist()          # one 8-byte read-back per build
-        last_build_info.update(rows_repaired=repaired, rows_unresolved=unresolved)
+        st_host = status.tolist()                       # the one read-back of a build
+        repaired, unresolved = st_host[0], st_host[1]
+        last_build_info.update(rows_repaired=repaired, rows_unresolved=unresolved,
+                               repaired_rows=[r for r in st_host[2:] if r >= 0])
         if unresolved == 0:
             return done()
     build_index_unfused_(A, K, Z, out, vals, workspace_bytes)
@@ -531,9 +534,20 @@ def segment_sum(X: torch.Tensor, perm: torch.Tensor, seg_off: torch.Tensor, seg_
     return out
 
 
+def _debug_lib():
+    """The library, for a diagnostic switch: those take effect only in a process started with
+    FASTMEM_DEBUG_HOOKS=1 (the library reads it at its first call), so that no caller of a serving process can
+    reroute another caller's kernels; a switch flipped anywhere else would silently do nothing, hence the error."""
+    lib = _lib.load()
+    if not lib.fm_debug_hooks_enabled():
+        raise RuntimeError("libfastmem's diagnostic switches are off in this process: set FASTMEM_DEBUG_HOOKS=1 in "
+                           "the environment before the library is first called")
+    return lib
+
+
 def argtopz_exact_only(on: bool) -> None:
     """Diagnostic switch: dense arg-top-Z by exact radix passes only (no sampled one-pass form)."""
-    _lib.load().fm_debug_argtopz_exact_only(int(on))
+    _debug_lib().fm_debug_argtopz_exact_only(int(on))
 
 
 _generic_forced = False
@@ -543,7 +557,7 @@ def force_generic_kernels(on: bool) -> None:
     """Diagnostic switch: route attention through the generic kernels."""
     global _generic_forced
     _generic_forced = bool(on)
-    _lib.load().fm_debug_force_generic(int(on))
+    _debug_lib().fm_debug_force_generic(int(on))
 
 
 def generic_kernels_forced() -> bool:
@@ -578,5 +592,5 @@ def grouped_forward_kernel(which: Optional[str]) -> None:
     on average, else staged unless the launch has few and small work items)."""
     global _generic_forced
     _generic_forced = False
-    _lib.load().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4, "ring": 5,
+    _debug_lib().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4, "ring": 5,
                                          "staged-per-row": 6, "ring-per-row": 7}[which])

@@ -94,9 +94,14 @@ int fm_build_index(const void* A, const void* K, int32_t* idx_out, float* val_ou
  * bf16, d = 128, N >= 65536, 64 <= Z <= N/8; fm_build_index_fused_workspace
  * returns 0 for any other shape.  A per-row threshold taken from a sample of the
  * keys filters the MFMA output; rows whose threshold missed are recomputed
- * exactly on the device (up to 64 of them).  status_dev (device, 2 ints)
- * receives {rows repaired, rows left unresolved}; if the second is non-zero the
- * caller must rebuild with fm_build_index. */
+ * exactly on the device (up to 64 of them).  status_dev (device,
+ * FM_FUSED_STATUS_INTS ints) receives {rows repaired, rows left unresolved, then
+ * the repaired rows as head * C + bucket, -1 in the unused places}; if the
+ * second is non-zero the caller must rebuild with fm_build_index (until then the
+ * unresolved rows list keys 0 .. Z-1: valid indices, not the right ones).  The
+ * call reads nothing back: a caller may queue, or record into a graph, whatever
+ * reads the lists behind it and look at the status word later. */
+#define FM_FUSED_STATUS_INTS 66
 size_t fm_build_index_fused_workspace(int H, int C, int N, int d, int Z, int dtype);
 int fm_build_index_fused(const void* A, const void* K, int32_t* idx_out, float* val_out, int H, int C,
                          int N, int d, int Z, int dtype, void* ws, size_t ws_bytes, int32_t* status_dev,

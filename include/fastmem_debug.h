@@ -1,7 +1,10 @@
 /*
  * fastmem_debug.h -- test and measurement hooks of libfastmem.so.
  *
- * None of these has a counterpart in the reference.  The switches (fm_debug_force_generic,
+ * None of these has a counterpart in the reference.  The switches take effect only in a process whose
+ * environment held FASTMEM_DEBUG_HOOKS=1 when the library was first called (fm_debug_hooks_enabled() says
+ * whether it did); in any other process the setters do nothing, so no caller can reroute another caller's
+ * kernels.  The switches (fm_debug_force_generic,
  * fm_debug_argtopz_exact_only, fm_debug_fused_filter, fm_debug_set_phase_events) are PROCESS-WIDE state, read by every call on
  * every stream: they exist so that tests can compare two implementations of one operator and so that the
  * benchmark can time the phases of the fused build; a production caller never touches them.  The probes
@@ -16,6 +19,9 @@
 extern "C" {
 #endif
 
+/* 1 if the switches below take effect in this process (FASTMEM_DEBUG_HOOKS=1 at the first call), else 0. */
+int fm_debug_hooks_enabled(void);
+
 /* Diagnostic: 1 routes the attention entry points through the generic kernels
  * (used by tests to compare the two implementations), 0 restores dispatch.  For
  * fm_hash_attn_fwd on bf16 / fp16, d = 128 only: 2 = always the kernel that stages a
@@ -23,7 +29,9 @@ extern "C" {
  * same in one launch per row; 4 = the staged kernel with two work items per
  * workgroup; 5 = always the kernel that loads the rows straight into LDS (three
  * items per workgroup), in a single launch, 7 = the same in one launch per row;
- * 3 = always the kernel that gathers the rows into registers.  Dispatch: gather
+ * 3 = always the kernel that gathers the rows into registers; 8 = the kernel of the
+ * head dimensions 64 and 256 instantiated for 128 (tests compare it with the kernels
+ * built for 128).  Dispatch: gather
  * when H min(Sq, C) < 512 and Sq < 24 C; else the direct loads up to 2^24 keys and
  * the staged kernel beyond; one launch per row when K and V of all rows are 512 MB
  * or more, those of a row 32 MB or more, and a row has 1024 (staged kernel: 1536)

@@ -132,3 +132,29 @@ def test_grouped_forward_dispatch_rule():
     assert launches(8, 131072, 65536, 128, 1024, 2) == 1                              # reference harness
     assert launches(8, 32768, 1048576, 64, 2048, 0) == 1                              # generic kernels
     assert launches(1, 64, 1048576, 128, 64, 1) == 1                                  # few small items: gather kernel
+
+
+def test_diagnostic_switches_need_the_environment_flag():
+    """The process-wide switches of fastmem_debug.h take effect only where FASTMEM_DEBUG_HOOKS=1 was set before
+    the library's first call; elsewhere the setters do nothing and the Python wrappers refuse.  Checked through
+    a host-only query (which kernel fm_hash_attn_fwd would launch), in child processes with and without the flag."""
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "from fast_memory_amd import _lib, ops\n"
+            "lib = _lib.load()\n"
+            "lib.fm_debug_force_generic(1)\n"
+            "name = lib.fm_hash_attn_fwd_kernel(8, 8192, 32768, 128, 256, 1).decode()\n"
+            "try:\n"
+            "    ops.force_generic_kernels(True); refused = False\n"
+            "except RuntimeError:\n"
+            "    refused = True\n"
+            "print(lib.fm_debug_hooks_enabled(), name, refused)\n") % ROOT
+    for flag, want in ((None, "0 hash_attn_ring_kernel True"), ("0", "0 hash_attn_ring_kernel True"),
+                       ("1", "1 hash_attn_generic_kernel False")):
+        env = {k: v for k, v in os.environ.items() if k != "FASTMEM_DEBUG_HOOKS"}
+        if flag is not None:
+            env["FASTMEM_DEBUG_HOOKS"] = flag
+        out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+        assert out.returncode == 0, out.stderr
+        assert out.stdout.strip().splitlines()[-1] == want, (flag, out.stdout)

@@ -39,14 +39,18 @@ def check_lists_whole(idx, val, N):
     assert bool((rows[:, 1:][tie] > rows[:, :-1][tie]).all()), "equal values are not in ascending index order"
 
 
-def check_lists_sampled(ops, A, keys, idx, val, Z, rows_per_head=4, seed=0):
+def check_lists_sampled(ops, A, keys, idx, val, Z, rows_per_head=4, seed=0, also=()):
     """Sampled (head, bucket) rows against the definition: the first Z entries of a stable descending sort
     of the row of Y (bit-exact), with the list's values equal to Y at the listed keys; Y itself against
-    fp64 dot products."""
+    fp64 dot products.  ``also``: rows (head * C + bucket) to check beside the sampled ones."""
     H, C, d = A.shape
     g = torch.Generator().manual_seed(seed)
     for h in range(H):
-        rows = torch.randperm(C, generator=g)[:rows_per_head].to(A.device)
+        rows = torch.randperm(C, generator=g)[:rows_per_head]
+        extra = torch.tensor([r % C for r in also if r // C == h], dtype=torch.long)
+        rows = torch.cat([rows, extra]).to(A.device)
+        if rows.numel() == 0:
+            continue
         Y = ops.project(A[h:h + 1, rows].contiguous(), keys[h:h + 1].contiguous())[0]          # [r, N] fp32
         ref = torch.sort(Y, dim=1, descending=True, stable=True)
         assert torch.equal(idx[h, rows].long(), ref.indices[:, :Z]), f"head {h}: list differs from the stable sort"
@@ -127,7 +131,23 @@ def test_config5_one_million_keys_full_size(ops):
     A = fit_projection(wl.keys, C, iters=cfg.kmeans_iters)
     mem = Memory.build(wl.keys, wl.values, A, Z, keep_values=True)
     check_lists_whole(mem.bucket_idx, mem.bucket_val, N)
-    check_lists_sampled(ops, A, wl.keys, mem.bucket_idx, mem.bucket_val, Z, rows_per_head=2)
+    # six rows of every head, and every row whose sampled threshold missed and was recomputed on the device
+    # (about one row in 30 000 does: the status word of the build names them)
+    repaired = list(ops.last_build_info.get("repaired_rows", []))
+    assert ops.last_build_info["rows_repaired"] == len(repaired)
+    check_lists_sampled(ops, A, wl.keys, mem.bucket_idx, mem.bucket_val, Z, rows_per_head=6, also=repaired)
+    # the same build again with a tighter threshold rank would repair more rows; here the builds of four other
+    # seeds' projections are checked on the rows they repaired (a row is repaired in about every second build)
+    n_checked = len(repaired)
+    for it in range(4):
+        A2 = fit_projection(wl.keys[:, it::5].contiguous(), C, iters=1)
+        idx2, val2 = ops.build_index(A2, wl.keys, Z, return_values=True)
+        rep2 = list(ops.last_build_info.get("repaired_rows", []))
+        if rep2:
+            check_lists_sampled(ops, A2, wl.keys, idx2, val2, Z, rows_per_head=0, also=rep2)
+            n_checked += len(rep2)
+        del idx2, val2
+    print(f"c5: {n_checked} repaired rows checked against the stable sort")
     # the chunked build (projection to memory + the dense selection in its long-list form) on some rows of one head
     part = ops.build_index(A[5:6, 700:796].contiguous(), wl.keys[5:6].contiguous(), Z, fused=False)
     assert torch.equal(part, mem.bucket_idx[5:6, 700:796])

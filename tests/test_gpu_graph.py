@@ -76,7 +76,7 @@ def test_build_hash_and_attention_in_one_graph():
         return dict(ws=torch.empty(ws_bytes, dtype=torch.uint8, device="cuda"),
                     idx=torch.zeros(H, C, Z, dtype=torch.int32, device="cuda"),
                     idx_k=torch.zeros(H * C * Z, dtype=torch.int32, device="cuda"),
-                    status=torch.zeros(2, dtype=torch.int32, device="cuda"),
+                    status=torch.zeros(_lib.FM_FUSED_STATUS_INTS, dtype=torch.int32, device="cuda"),
                     qh=torch.zeros(H, S, dtype=torch.int32, device="cuda"), out=torch.zeros_like(q),
                     lse=torch.zeros(H, S, dtype=torch.float32, device="cuda"))
 

@@ -49,6 +49,8 @@ SIGNATURES = {
                                  c_int, c_float, c_int, P]),
     "fm_inverse_index_workspace": (c_size_t, [c_int64, c_int, c_int]),
     "fm_inverse_index": (c_int, [P, P, P, c_int, c_int, c_int, c_int64, P, P, P, c_size_t, P]),
+    "fm_inverse_index_key_order_workspace": (c_size_t, [c_int, c_int, c_int]),
+    "fm_inverse_index_key_order": (c_int, [P, P, P, c_int, c_int, c_int, c_int64, P, P, P, P, c_size_t, P]),
     "fm_hash_attn_bwd_staged_workspace": (c_size_t, [c_int64]),
     "fm_hash_attn_bwd_staged": (c_int, [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, c_int, c_int, c_int,
                                         c_int, c_int, P, c_float, c_int, P, c_size_t, P]),

@@ -222,15 +222,25 @@ class _ApproxCrossAttentionFunc(torch.autograd.Function):
         mo, ml = mem.attend(q3, sm_scale, q_hash=q_hashes)                                  # memory.py:319-321
         out, lse = update_out_and_lse(out.contiguous(), lse.contiguous(), mo, ml)           # memory.py:332
         out = out.to(q.dtype)
-        ctx.mem, ctx.sm_scale = mem, sm_scale
-        ctx.save_for_backward(q, k_self, v_self, q_hashes, out, lse.squeeze(-1))
+        ctx.sm_scale = sm_scale
+        # Everything the backward reads goes through save_for_backward (the reference keeps clones, k_og / v_og,
+        # memory.py:243-244): k and v themselves, so that an in-place update of the memory between forward and
+        # backward (a KV cache that is appended to or overwritten) is caught by autograd's version counter
+        # instead of silently giving gradients against the new contents, and the bucket lists with their
+        # key-ordered copy, from which the backward rebuilds a Memory view without building an index again.
+        attn_idx = mem._attn_idx if mem._attn_idx is not None else mem.bucket_idx.new_empty(0)
+        ctx.save_for_backward(q, k_self, v_self, q_hashes, out, lse.squeeze(-1), k, v, A, mem.bucket_idx, attn_idx)
         ctx.mark_non_differentiable(q_hashes)
         return out.reshape(q.shape), q_hashes
 
     @staticmethod
     def backward(ctx, dout, _d_hashes):
-        q, k_self, v_self, q_hashes, out, lse = ctx.saved_tensors
-        mem, sm_scale = ctx.mem, ctx.sm_scale
+        from .memory import Memory
+        q, k_self, v_self, q_hashes, out, lse, k, v, A, bucket_idx, attn_idx = ctx.saved_tensors
+        sm_scale = ctx.sm_scale
+        mem = Memory(k[0], v[0], A, bucket_idx)
+        if attn_idx.numel():
+            mem._attn_idx = attn_idx
         _, n_heads, seq_len, d_qkv = q.shape
         k_heads = k_self.shape[1]
         dout3 = dout[0].to(q.dtype).reshape(out.shape).contiguous()

@@ -26,8 +26,6 @@
 // depend on scheduling.
 #include <cstring>
 
-#include <rocprim/device/device_radix_sort.hpp>
-
 #include "common.hpp"
 
 namespace fm {
@@ -35,6 +33,7 @@ namespace fm {
 int launch_unlisted_rows(const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
                          const int32_t* bin_off, const int32_t* bin_count, int64_t n_bins, int64_t nq,
                          int row_bytes, void* rows, float* lse, hipStream_t st);  // group.hip
+int launch_fill(int32_t* p, int64_t n, int32_t v, hipStream_t st);  // group.hip
 int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, const int32_t* k_idx,
                                   const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                                   const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
@@ -56,7 +55,7 @@ __global__ __launch_bounds__(256) void inv_pairs_kernel(const int32_t* __restric
     const int64_t f = off + p;
     const int key = min(max(k_idx[f], 0), N - 1);
     keys[f] = uint32_t(row) * uint32_t(N) + uint32_t(key);
-    vals[f] = uint32_t(f);
+    if (vals) vals[f] = uint32_t(f);
   }
 }
 
@@ -76,18 +75,412 @@ __global__ __launch_bounds__(256) void inv_offsets_kernel(const uint32_t* __rest
   key_off[kk] = int32_t(lo);
 }
 
-static size_t sort_temp_bytes(int64_t T, int bits) {
-  size_t bytes = 0;
-  (void)rocprim::radix_sort_pairs(nullptr, bytes, static_cast<uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr),
-                                  static_cast<uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr), size_t(T), 0,
-                                  unsigned(bits), hipStream_t(nullptr));
-  return bytes;
-}
-
 static int key_bits(int64_t n_keys) {
   int bits = 1;
   while ((int64_t(1) << bits) < n_keys) ++bits;
   return bits;
+}
+
+// ---- stable radix sort of (key, position) pairs --------------------------------------
+// Least significant digit first, digits of up to 8 bits, three kernels a pass:
+//   radix_hist_kernel     a workgroup counts the digits of its tile of 4096 pairs; counts land digit-major
+//                         ([digit][tile]), so that their exclusive prefix sum is every (digit, tile)'s first
+//                         place in the output;
+//   radix_scan_kernel /   that prefix sum in chunks of 16384 counts (a workgroup each) and, by one workgroup,
+//   radix_scan_top_kernel over the chunks' totals;
+//   radix_scatter_kernel  the tile again: wave w takes pairs 1024 w .. 1024 w + 1023 of the tile, 64 consecutive
+//                         ones a step.  The lanes that hold the same digit find each other with one ballot per
+//                         digit bit; a pair's rank among the wave's earlier pairs of its digit is the wave's
+//                         counter of that digit plus the number of such lanes below it -- steps run in order and
+//                         lanes are in pair order, so equal digits keep their order (the sort is stable: a key's
+//                         positions come out ascending).  The waves' counters are then turned into their first
+//                         places inside the tile, the tile is put in order in LDS, and it leaves as runs of
+//                         consecutive places, one run per digit.
+// HBM-bound: a pass reads 12 bytes and writes 8 per pair (the first pass forms its keys from the lists).
+constexpr int kRsThreads = 256, kRsWaves = 4, kRsItems = 16;
+constexpr int kRsTile = kRsThreads * kRsItems;  // 4096 pairs per workgroup
+constexpr int kRsChunk = 16384;                 // counts per workgroup of the prefix sum
+
+__global__ __launch_bounds__(kRsThreads) void radix_hist_kernel(const uint32_t* __restrict__ keys, int64_t T,
+                                                                int shift, int nd, int64_t n_tiles,
+                                                                uint32_t* __restrict__ hist) {
+  __shared__ uint32_t h[256];
+  const int tid = threadIdx.x;
+  h[tid] = 0;
+  __syncthreads();
+  const int64_t base = int64_t(blockIdx.x) * kRsTile;
+#pragma unroll
+  for (int s = 0; s < kRsItems; ++s) {
+    const int64_t i = base + int64_t(s) * kRsThreads + tid;
+    if (i < T) atomicAdd(&h[(keys[i] >> shift) & uint32_t(nd - 1)], 1u);
+  }
+  __syncthreads();
+  if (tid < nd) hist[int64_t(tid) * n_tiles + blockIdx.x] = h[tid];
+}
+
+// exclusive prefix sums inside chunks of kRsChunk counts (in place) and the chunks' totals
+__global__ __launch_bounds__(1024) void radix_scan_kernel(uint32_t* __restrict__ hist, int64_t n,
+                                                          uint32_t* __restrict__ chunk_total) {
+  __shared__ int tmp[17];
+  const int64_t base = int64_t(blockIdx.x) * kRsChunk + int64_t(threadIdx.x) * 16;
+  uint32_t v[16];
+  int local = 0;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    v[j] = base + j < n ? hist[base + j] : 0u;
+    local += int(v[j]);
+  }
+  int total;
+  int run = block_excl_scan(local, tmp, &total);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    if (base + j < n) hist[base + j] = uint32_t(run);
+    run += int(v[j]);
+  }
+  if (threadIdx.x == 0) chunk_total[blockIdx.x] = uint32_t(total);
+}
+
+// exclusive prefix sum over the chunks' totals, one workgroup
+__global__ __launch_bounds__(1024) void radix_scan_top_kernel(uint32_t* __restrict__ chunk_total, int64_t n_chunks) {
+  __shared__ int tmp[17];
+  int carry = 0;
+  for (int64_t base = 0; base < n_chunks; base += 1024) {
+    const int64_t i = base + threadIdx.x;
+    const int v = i < n_chunks ? int(chunk_total[i]) : 0;
+    int total;
+    const int ex = block_excl_scan(v, tmp, &total);
+    if (i < n_chunks) chunk_total[i] = uint32_t(carry + ex);
+    carry += total;
+  }
+}
+
+// vals_in == nullptr: a pair's value is its index (the first pass).  The tile is put in order inside LDS first,
+// so that what goes to memory are runs of consecutive places (a digit's pairs of the tile), not 64 scattered
+// words per store.
+__global__ __launch_bounds__(kRsThreads) void radix_scatter_kernel(
+    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ keys_out,
+    uint32_t* __restrict__ vals_out, int64_t T, int shift, int nd, int n_bits, int64_t n_tiles,
+    const uint32_t* __restrict__ hist, const uint32_t* __restrict__ chunk_off) {
+  __shared__ uint32_t wcnt[kRsWaves][256];  // a wave's count of a digit, then its first place inside the tile
+  __shared__ uint32_t dstart[256];          // first place of a digit inside the tile
+  __shared__ uint32_t gfirst[256];          // ... in the output, minus dstart
+  __shared__ uint32_t sk[kRsTile], sv[kRsTile];
+  __shared__ int tmp[17];
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+  for (int d = tid; d < kRsWaves * 256; d += kRsThreads) (&wcnt[0][0])[d] = 0;
+  __syncthreads();
+  constexpr int kWaveItems = kRsTile / kRsWaves;  // 1024 pairs per wave, kRsItems steps of 64
+  const int64_t tile0 = int64_t(blockIdx.x) * kRsTile;
+  const int64_t base = tile0 + int64_t(w) * kWaveItems + l;
+  const uint64_t lt = (uint64_t(1) << l) - 1u;
+  uint32_t key[kRsItems], rank[kRsItems];
+#pragma unroll
+  for (int s = 0; s < kRsItems; ++s) {
+    const int64_t i = base + int64_t(s) * 64;
+    const bool valid = i < T;
+    key[s] = valid ? keys_in[i] : 0u;
+    const uint32_t digit = (key[s] >> shift) & uint32_t(nd - 1);
+    uint64_t peers = __ballot(valid);  // the lanes that hold this lane's digit
+    for (int b = 0; b < n_bits; ++b) {
+      const bool bit = (digit >> b) & 1u;
+      const uint64_t m = __ballot(bit);
+      peers &= bit ? m : ~m;
+    }
+    const uint32_t c0 = wcnt[w][digit];
+    rank[s] = c0 + uint32_t(__popcll(peers & lt));
+    if (valid && (peers & lt) == 0) wcnt[w][digit] = c0 + uint32_t(__popcll(peers));  // the group's first lane
+  }
+  __syncthreads();
+  // digit d: the tile's count -> its first place inside the tile and in the output; the waves' counts -> their
+  // first places inside the tile
+  {
+    uint32_t c[kRsWaves], tot = 0;
+#pragma unroll
+    for (int ww = 0; ww < kRsWaves; ++ww) {
+      c[ww] = tid < nd ? wcnt[ww][tid] : 0u;
+      tot += c[ww];
+    }
+    int total;
+    const int first = block_excl_scan(int(tot), tmp, &total);
+    if (tid < nd) {
+      const int64_t e = int64_t(tid) * n_tiles + blockIdx.x;
+      dstart[tid] = uint32_t(first);
+      gfirst[tid] = hist[e] + chunk_off[e / kRsChunk] - uint32_t(first);
+      uint32_t run = uint32_t(first);
+#pragma unroll
+      for (int ww = 0; ww < kRsWaves; ++ww) {
+        wcnt[ww][tid] = run;
+        run += c[ww];
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < kRsItems; ++s) {
+    const int64_t i = base + int64_t(s) * 64;
+    if (i < T) {
+      const uint32_t at = wcnt[w][(key[s] >> shift) & uint32_t(nd - 1)] + rank[s];
+      sk[at] = key[s];
+      sv[at] = vals_in ? vals_in[i] : uint32_t(i);
+    }
+  }
+  __syncthreads();
+  const int n_here = int(min<int64_t>(kRsTile, T - tile0));
+  for (int j = tid; j < n_here; j += kRsThreads) {
+    const uint32_t k = sk[j];
+    const uint32_t dest = gfirst[(k >> shift) & uint32_t(nd - 1)] + uint32_t(j);
+    keys_out[dest] = k;
+    vals_out[dest] = sv[j];
+  }
+}
+
+struct RadixPlan {
+  int passes, bits_per_pass;
+  int64_t n_tiles, n_counts, n_chunks;
+  size_t arr, off_hist, off_chunks, total;  // four arrays of T words, then the counts
+};
+static RadixPlan radix_plan(int64_t T, int bits) {
+  RadixPlan p;
+  p.passes = std::max(1, (bits + 7) / 8);
+  p.bits_per_pass = (bits + p.passes - 1) / p.passes;
+  p.n_tiles = ceil_div(T, kRsTile);
+  p.n_counts = p.n_tiles << p.bits_per_pass;
+  p.n_chunks = ceil_div(p.n_counts, kRsChunk);
+  p.arr = align_up(size_t(T) * sizeof(uint32_t), 256);
+  p.off_hist = 4 * p.arr;
+  p.off_chunks = p.off_hist + align_up(size_t(p.n_counts) * sizeof(uint32_t), 256);
+  p.total = p.off_chunks + align_up(size_t(p.n_chunks) * sizeof(uint32_t), 256) + 256;
+  return p;
+}
+
+// ---- inverse index of lists in ascending key order -----------------------------------
+// When every list is in strictly ascending key order (as fm_lists_key_order leaves them: the order the
+// attention and its backward read) the inverse is a transposition that needs no sort.  Keys are taken in
+// ranges of kIrRange; inside a sorted list the entries of a range are one contiguous run.
+//   inv_runs_kernel       per list: first the number of entries that break the order or lie outside [0, N);
+//                         for a list in order, where each range's run starts (a table [row][bucket][range]);
+//   inv_table_kernel      the table turned to [row][range][bucket], and the entries per (row, range), whose
+//                         prefix sum is the range's first place in inv_pos;
+//   inv_transpose_kernel  one workgroup per (row, range): the runs of all the row's buckets are counted per
+//                         (group of consecutive buckets, key) in LDS, a prefix over the groups and over the
+//                         keys gives every group its first place per key, and the groups then walk their
+//                         buckets again in ascending order handing out places -- so a key's positions come out
+//                         in ascending bucket order, which is ascending position order.  A group is 16 lanes
+//                         (a run is 4 entries on average at the benchmark shapes, a longer one takes further
+//                         rounds), its buckets go one after the other: a bucket lists a key once, so the
+//                         entries of a step never share a counter, and the steps of one wave reach LDS in
+//                         program order.  The bounds of 16 buckets are fetched by the group's lanes at once
+//                         (the next 16 while these are worked on), then their entries at once.  The places
+//                         are handed out into an LDS image of the range's part of inv_pos, written out in
+//                         whole lines afterwards: 4-byte stores in arrival order over thousands of ranges at
+//                         once leave the L2 as partial lines, which cost several times the index in traffic.
+// The counters are 16 bits wide: a key is in at most C <= 65535 lists.
+// Every index is clamped or checked, so lists that are not in order give no index but never an access
+// outside the buffers; the count of inv_runs_kernel tells the caller which it has, and the later kernels
+// end at once when it is not zero.
+constexpr int kIrShift = 8, kIrRange = 1 << kIrShift;  // keys per range
+constexpr int kIrGroups = 32;                          // groups of consecutive buckets per workgroup
+constexpr int kIrThreads = kIrGroups * 16;
+constexpr int kIrStage = 8320;  // entries of a range kept in LDS for the write-out (32.5 per key; more go direct)
+
+// S[(list) * (n_ranges + 1) + r] = first position of the list with key >= r * kIrRange
+__global__ __launch_bounds__(256) void inv_runs_kernel(const int32_t* __restrict__ k_idx,
+                                                       const int64_t* __restrict__ bucket_off,
+                                                       const int32_t* __restrict__ bucket_cnt, int N, int n_ranges,
+                                                       int32_t* __restrict__ S, int32_t* __restrict__ n_bad) {
+  const int64_t b = blockIdx.x;
+  const int32_t* p = k_idx + bucket_off[b];
+  const int cnt = bucket_cnt[b];
+  int32_t* Sb = S + b * (n_ranges + 1);
+  int bad = 0;
+  for (int base = 0; base < cnt; base += 2048) {
+    int here[8], prev[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {  // (the loads of a thread are in flight together)
+      const int i = base + u * 256 + int(threadIdx.x);
+      here[u] = i < cnt ? p[i] : N - 1;
+      prev[u] = i > 0 && i < cnt ? p[i - 1] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) bad += (here[u] < 0 || here[u] >= N) || prev[u] >= here[u];
+  }
+  bad = __syncthreads_count(bad != 0);
+  if (bad) {  // a list out of order: its table stays unwritten (no index comes out of this call)
+    if (threadIdx.x == 0) atomicAdd(n_bad, bad);
+    return;
+  }
+  for (int base = 0; base <= cnt; base += 1024) {
+    int here[4], prev[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = base + u * 256 + int(threadIdx.x);
+      here[u] = i < cnt ? p[i] : 0;
+      prev[u] = i > 0 && i <= cnt ? p[i - 1] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = base + u * 256 + int(threadIdx.x);
+      if (i > cnt) continue;
+      // ranges whose run starts at position i: those above the range of entry i - 1, up to the range of entry i
+      const int r_prev = i > 0 ? prev[u] >> kIrShift : -1;
+      const int r_here = i < cnt ? here[u] >> kIrShift : n_ranges;
+      for (int r = r_prev + 1; r <= r_here; ++r) Sb[r] = i;
+    }
+  }
+}
+
+// The table turned to [row][range][bucket] (what the workgroup of a range reads along the buckets), as flat
+// positions in k_idx (the list's offset added, clamped into the list), and the entries per (row, range)
+// added into totals (zero before).  One workgroup per (row, 64 ranges, 64 buckets), the tile through LDS.
+__global__ __launch_bounds__(256) void inv_table_kernel(const int32_t* __restrict__ S,
+                                                        const int64_t* __restrict__ bucket_off,
+                                                        const int32_t* __restrict__ bucket_cnt, int C, int n_ranges,
+                                                        const int32_t* __restrict__ n_bad, int32_t* __restrict__ St,
+                                                        uint32_t* __restrict__ totals) {
+  if (*n_bad) return;
+  __shared__ int tile[64][66];
+  const int row = blockIdx.z, r0 = blockIdx.x * 64, b0 = blockIdx.y * 64, w = threadIdx.x >> 6, l = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int bl = w + 4 * i, b = b0 + bl;
+    if (b < C) {
+      const int64_t list = int64_t(row) * C + b;
+      const int cnt = bucket_cnt[list], off = int(bucket_off[list]);
+      const int32_t* s = S + list * (n_ranges + 1);
+      if (r0 + l <= n_ranges) tile[bl][l] = off + min(max(s[r0 + l], 0), cnt);
+      if (l == 0 && r0 + 64 <= n_ranges) tile[bl][64] = off + min(max(s[r0 + 64], 0), cnt);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int rr = w + 4 * i, r = r0 + rr, b = b0 + l;
+    int t = 0;
+    if (r <= n_ranges && b < C) {
+      const int v = tile[l][rr];
+      St[(int64_t(row) * (n_ranges + 1) + r) * C + b] = v;
+      if (r < n_ranges) t = max(tile[l][rr + 1] - v, 0);
+    }
+    t = wave_sum_i(t);
+    if (l == 0 && r < n_ranges && t) atomicAdd(&totals[int64_t(row) * n_ranges + r], uint32_t(t));
+  }
+}
+
+__global__ __launch_bounds__(kIrThreads) void inv_transpose_kernel(
+    const int32_t* __restrict__ k_idx, const int32_t* __restrict__ St, const uint32_t* __restrict__ range_first,
+    const int32_t* __restrict__ n_bad, int n_rows, int C, int N, int n_ranges, int64_t T,
+    int32_t* __restrict__ key_off, int32_t* __restrict__ inv_pos) {
+  if (*n_bad) return;
+  __shared__ uint32_t cnt2[kIrGroups][kIrRange / 2];  // 16-bit counters, two to a word: [group][key of the range]
+  __shared__ uint32_t first[kIrRange];                // a key's first place within the range's part of inv_pos
+  __shared__ int32_t stage[kIrStage];
+  __shared__ __align__(16) int xst[kIrGroups][16];  // a group's 16 buckets in hand: first entry of the run ...
+  __shared__ __align__(16) uint8_t xlen[kIrGroups][16];  // ... and its length (17 = longer than the group)
+  __shared__ int tmp[17];
+  // Workgroups go to the 8 XCDs in turn: every XCD gets a contiguous span of (row, range) pairs, so that
+  // the ranges in flight on one L2 are neighbours (four consecutive ranges share a 64-byte line of a list).
+  const int64_t n_work = int64_t(n_rows) * n_ranges, per_xcd = (n_work + 7) / 8;
+  const int64_t work = int64_t(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if ((blockIdx.x >> 3) >= per_xcd || work >= n_work) return;
+  const int row = int(work / n_ranges), r = int(work - int64_t(row) * n_ranges), tid = threadIdx.x;
+  const int g = tid >> 4, gl = tid & 15;
+  for (int i = tid; i < kIrGroups * kIrRange / 2; i += kIrThreads) (&cnt2[0][0])[i] = 0;
+  __syncthreads();
+  const int per_group = (C + kIrGroups - 1) / kIrGroups;
+  const int b0 = min(C, g * per_group), b1 = min(C, b0 + per_group);
+  const int key0 = r << kIrShift;
+  const int32_t* s0 = St + (int64_t(row) * (n_ranges + 1) + r) * C;
+  // the run of this range in bucket bb + (lane of the group): flat position of its first entry, its length
+  auto bounds = [&](int bb, int& st, int& len) {
+    const int b = bb + gl;
+    st = 0, len = 0;
+    if (b < b1) {
+      st = s0[b];
+      len = max(s0[C + b] - st, 0);
+    }
+  };
+  // one pass over the group's buckets in ascending order: f(key index inside the range, flat list position)
+  // for every entry of the range.  The 16 lanes of a group fetch the bounds of 16 buckets, hand them to
+  // one another through LDS (the waves run on their own: a group's words are written and read by its own
+  // wave, in program order) and then take the buckets one by one, lane i the i-th entry of the run.
+  auto walk = [&](auto f) {
+    int st_n, len_n;
+    bounds(b0, st_n, len_n);
+    for (int bb = b0; bb < b1; bb += 16) {
+      const int st = st_n, len = len_n;
+      bounds(bb + 16, st_n, len_n);
+      __builtin_amdgcn_wave_barrier();
+      xst[g][gl] = st;
+      xlen[g][gl] = uint8_t(min(len, 17));
+      __builtin_amdgcn_wave_barrier();
+      const bool long_run = __any(len > 16);  // (the four groups of the wave step together)
+      int k[16], pos[16];
+      {
+        int s_u[16];
+        uint32_t l4[4];
+        *reinterpret_cast<int4*>(&s_u[0]) = *reinterpret_cast<const int4*>(&xst[g][0]);
+        *reinterpret_cast<int4*>(&s_u[4]) = *reinterpret_cast<const int4*>(&xst[g][4]);
+        *reinterpret_cast<int4*>(&s_u[8]) = *reinterpret_cast<const int4*>(&xst[g][8]);
+        *reinterpret_cast<int4*>(&s_u[12]) = *reinterpret_cast<const int4*>(&xst[g][12]);
+        *reinterpret_cast<uint4*>(&l4[0]) = *reinterpret_cast<const uint4*>(&xlen[g][0]);
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int l_u = int((l4[u >> 2] >> (8 * (u & 3))) & 0xffu);
+          pos[u] = s_u[u] + gl;
+          k[u] = gl < l_u ? k_idx[pos[u]] : -1;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int j = k[u] - key0;
+        if (k[u] >= 0 && j >= 0 && j < kIrRange) f(j, pos[u]);
+        if (long_run) {
+          const int l_u = __shfl(len, u, 16);
+          for (int p = gl + 16; __any(p < l_u); p += 16) {
+            if (p < l_u) {
+              const int jj = k_idx[pos[u] - gl + p] - key0;
+              if (jj >= 0 && jj < kIrRange) f(jj, pos[u] - gl + p);
+            }
+          }
+        }
+      }
+    }
+  };
+  walk([&](int j, int) { atomicAdd(&cnt2[g][j >> 1], 1u << (16 * (j & 1))); });
+  __syncthreads();
+  // keys 2 tid and 2 tid + 1 (one word of counters): counts of the groups -> the groups' first places within
+  // the key's entries; the keys' totals -> first
+  uint32_t tot0 = 0, tot1 = 0;
+  if (tid < kIrRange / 2)
+    for (int gg = 0; gg < kIrGroups; ++gg) {
+      const uint32_t w = cnt2[gg][tid];
+      cnt2[gg][tid] = (tot0 & 0xffffu) | (tot1 << 16);
+      tot0 += w & 0xffffu;
+      tot1 += w >> 16;
+    }
+  int total;
+  const int ex = block_excl_scan(int(tot0 + tot1), tmp, &total);
+  const uint32_t base = range_first[int64_t(row) * n_ranges + r];
+  if (tid < kIrRange / 2) {
+    const int j = 2 * tid;
+    first[j] = uint32_t(ex);
+    first[j + 1] = uint32_t(ex) + tot0;
+    if (key0 + j < N) key_off[int64_t(row) * N + key0 + j] = int32_t(base + uint32_t(ex));
+    if (key0 + j + 1 < N) key_off[int64_t(row) * N + key0 + j + 1] = int32_t(base + uint32_t(ex) + tot0);
+  }
+  if (tid == 0 && row == n_rows - 1 && r == n_ranges - 1) key_off[int64_t(n_rows) * N] = int32_t(T);
+  __syncthreads();
+  walk([&](int j, int pos) {
+    const uint32_t old = atomicAdd(&cnt2[g][j >> 1], 1u << (16 * (j & 1)));
+    const uint32_t at = first[j] + ((old >> (16 * (j & 1))) & 0xffffu);
+    if (at < uint32_t(kIrStage))
+      stage[at] = pos;
+    else if (uint64_t(base) + at < uint64_t(T))
+      inv_pos[uint64_t(base) + at] = pos;
+  });
+  __syncthreads();
+  const int n_stage = int(min<int64_t>(min(total, kIrStage), T - int64_t(base)));
+  for (int i = tid; i < n_stage; i += kIrThreads) inv_pos[uint64_t(base) + i] = stage[i];
 }
 
 // ---- step 2 ---------------------------------------------------------------------
@@ -155,8 +548,7 @@ __global__ __launch_bounds__(256) void bwd_reduce_kernel(const bf16_t* __restric
 
 extern "C" size_t fm_inverse_index_workspace(int64_t T, int H, int N) {
   if (T < 1 || H < 1 || N < 1) return 0;
-  const size_t arr = fm::align_up(size_t(T) * sizeof(uint32_t), 256);
-  return 3 * arr + fm::align_up(fm::sort_temp_bytes(T, fm::key_bits(int64_t(H) * N)), 256) + 256;
+  return fm::radix_plan(T, fm::key_bits(int64_t(H) * N)).total;
 }
 
 extern "C" int fm_inverse_index(const int32_t* k_idx, const int64_t* bucket_off, const int32_t* bucket_cnt, int H,
@@ -172,23 +564,94 @@ extern "C" int fm_inverse_index(const int32_t* k_idx, const int64_t* bucket_off,
   FM_REQUIRE(ws_bytes >= fm_inverse_index_workspace(T, H, N), FM_ERR_WORKSPACE, "fm_inverse_index: workspace %zu < %zu",
              ws_bytes, fm_inverse_index_workspace(T, H, N));
   hipStream_t st = as_stream(stream);
-  const size_t arr = align_up(size_t(T) * sizeof(uint32_t), 256);
-  char* base = static_cast<char*>(ws);
-  uint32_t* keys_in = reinterpret_cast<uint32_t*>(base);
-  uint32_t* keys_out = reinterpret_cast<uint32_t*>(base + arr);
-  uint32_t* vals_in = reinterpret_cast<uint32_t*>(base + 2 * arr);
-  void* temp = base + 3 * arr;
   const int bits = key_bits(int64_t(H) * N);
-  size_t temp_bytes = sort_temp_bytes(T, bits);
+  const RadixPlan p = radix_plan(T, bits);
+  char* base = static_cast<char*>(ws);
+  uint32_t* ka = reinterpret_cast<uint32_t*>(base);
+  uint32_t* va = reinterpret_cast<uint32_t*>(base + p.arr);
+  uint32_t* kb = reinterpret_cast<uint32_t*>(base + 2 * p.arr);
+  uint32_t* vb = reinterpret_cast<uint32_t*>(base + 3 * p.arr);
+  uint32_t* hist = reinterpret_cast<uint32_t*>(base + p.off_hist);
+  uint32_t* chunks = reinterpret_cast<uint32_t*>(base + p.off_chunks);
+  // the keys row * N + key of every list entry (the first pass takes a pair's position as its value)
   hipLaunchKernelGGL(inv_pairs_kernel, dim3(unsigned(int64_t(H) * C)), dim3(256), 0, st, k_idx, bucket_off, bucket_cnt,
-                     C, N, keys_in, vals_in);
-  hipError_t e = rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, vals_in,
-                                           reinterpret_cast<uint32_t*>(inv_pos), size_t(T), 0, unsigned(bits), st);
-  FM_REQUIRE(e == hipSuccess, FM_ERR_LAUNCH, "fm_inverse_index: sort: %s", hipGetErrorString(e));
+                     C, N, ka, static_cast<uint32_t*>(nullptr));
+  const uint32_t* kin = ka;
+  const uint32_t* vin = nullptr;
+  uint32_t* kout = kb;
+  for (int pass = 0; pass < p.passes; ++pass) {
+    const int shift = pass * p.bits_per_pass;
+    const int n_bits = std::min(p.bits_per_pass, std::max(bits - shift, 1));
+    const int nd = 1 << n_bits;
+    const bool last = pass + 1 == p.passes;
+    uint32_t* vout = last ? reinterpret_cast<uint32_t*>(inv_pos) : (kout == kb ? vb : va);
+    const int64_t n_counts = p.n_tiles * nd;
+    const int64_t n_chunks = ceil_div(n_counts, kRsChunk);
+    hipLaunchKernelGGL(radix_hist_kernel, dim3(unsigned(p.n_tiles)), dim3(kRsThreads), 0, st, kin, T, shift, nd,
+                       p.n_tiles, hist);
+    hipLaunchKernelGGL(radix_scan_kernel, dim3(unsigned(n_chunks)), dim3(1024), 0, st, hist, n_counts, chunks);
+    hipLaunchKernelGGL(radix_scan_top_kernel, dim3(1), dim3(1024), 0, st, chunks, n_chunks);
+    hipLaunchKernelGGL(radix_scatter_kernel, dim3(unsigned(p.n_tiles)), dim3(kRsThreads), 0, st, kin, vin, kout, vout,
+                       T, shift, nd, n_bits, p.n_tiles, hist, chunks);
+    kin = kout;
+    vin = vout;
+    kout = kout == kb ? ka : kb;
+  }
   const int64_t n_keys = int64_t(H) * N;
-  hipLaunchKernelGGL(inv_offsets_kernel, dim3(unsigned(ceil_div(n_keys + 1, int64_t(256)))), dim3(256), 0, st, keys_out,
+  hipLaunchKernelGGL(inv_offsets_kernel, dim3(unsigned(ceil_div(n_keys + 1, int64_t(256)))), dim3(256), 0, st, kin,
                      T, n_keys, key_off);
   return launch_status("fm_inverse_index");
+}
+
+namespace fm {
+struct KeyOrderPlan {
+  int n_ranges;
+  size_t off_turned, off_totals, total;
+};
+static KeyOrderPlan key_order_plan(int H, int C, int N) {
+  KeyOrderPlan p;
+  p.n_ranges = int(ceil_div(N, kIrRange));
+  p.off_turned = align_up(size_t(H) * (p.n_ranges + 1) * C * sizeof(int32_t), 256);
+  p.off_totals = 2 * p.off_turned;
+  p.total = p.off_totals + align_up(size_t(H) * p.n_ranges * sizeof(uint32_t), 256) + 256;
+  return p;
+}
+}  // namespace fm
+
+extern "C" size_t fm_inverse_index_key_order_workspace(int H, int C, int N) {
+  if (H < 1 || C < 1 || N < 1) return 0;
+  return fm::key_order_plan(H, C, N).total;
+}
+
+extern "C" int fm_inverse_index_key_order(const int32_t* k_idx, const int64_t* bucket_off, const int32_t* bucket_cnt,
+                                          int H, int C, int N, int64_t T, int32_t* key_off, int32_t* inv_pos,
+                                          int32_t* n_bad, void* ws, size_t ws_bytes, void* stream) {
+  using namespace fm;
+  FM_REQUIRE(H >= 1 && C >= 1 && N >= 1 && T >= 1, FM_ERR_ARG, "fm_inverse_index_key_order: H=%d C=%d N=%d T=%lld", H, C,
+             N, (long long)T);
+  FM_REQUIRE(k_idx && bucket_off && bucket_cnt && key_off && inv_pos && n_bad && ws, FM_ERR_ARG,
+             "fm_inverse_index_key_order: null pointer");
+  FM_REQUIRE(T <= 0x7fffffffLL && int64_t(H) * N < 0x7fffffffLL && H <= 65535 && C <= 65535,
+             FM_ERR_UNSUPPORTED, "fm_inverse_index_key_order: more than 2^31 list entries or keys, H > 65535 or C > 65535");
+  const KeyOrderPlan p = key_order_plan(H, C, N);
+  FM_REQUIRE(ws_bytes >= p.total, FM_ERR_WORKSPACE, "fm_inverse_index_key_order: workspace %zu < %zu", ws_bytes, p.total);
+  hipStream_t st = as_stream(stream);
+  int32_t* S = static_cast<int32_t*>(ws);
+  uint32_t* totals = reinterpret_cast<uint32_t*>(static_cast<char*>(ws) + p.off_totals);
+  int rc = launch_fill(n_bad, 1, 0, st);
+  if (rc) return rc;
+  hipLaunchKernelGGL(inv_runs_kernel, dim3(unsigned(int64_t(H) * C)), dim3(256), 0, st, k_idx, bucket_off, bucket_cnt, N,
+                     p.n_ranges, S, n_bad);
+  int32_t* St = reinterpret_cast<int32_t*>(static_cast<char*>(ws) + p.off_turned);
+  rc = launch_fill(reinterpret_cast<int32_t*>(totals), int64_t(H) * p.n_ranges, 0, st);
+  if (rc) return rc;
+  hipLaunchKernelGGL(inv_table_kernel, dim3(unsigned(ceil_div(p.n_ranges + 1, 64)), unsigned(ceil_div(C, 64)), unsigned(H)),
+                     dim3(256), 0, st, S, bucket_off, bucket_cnt, C, p.n_ranges, n_bad, St, totals);
+  hipLaunchKernelGGL(radix_scan_top_kernel, dim3(1), dim3(1024), 0, st, totals, int64_t(H) * p.n_ranges);
+  const int64_t per_xcd = ceil_div(int64_t(H) * p.n_ranges, 8);
+  hipLaunchKernelGGL(inv_transpose_kernel, dim3(unsigned(8 * per_xcd)), dim3(kIrThreads), 0, st, k_idx, St, totals, n_bad,
+                     H, C, N, p.n_ranges, T, key_off, inv_pos);
+  return launch_status("fm_inverse_index_key_order");
 }
 
 // behind the partial rows: 8 dump rows (stores past the end of a list land there) and alignment

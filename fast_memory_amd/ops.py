@@ -327,6 +327,9 @@ def _check_dlse(dlse: Optional[torch.Tensor], lse: torch.Tensor) -> Optional[tor
     return dlse.to(torch.float32).contiguous()
 
 
+last_inverse_info = {}
+
+
 class InverseIndex(NamedTuple):
     """For every key the flat list positions that name it (see ``fm_inverse_index``); depends on the bucket
     lists only, so it can be kept with them."""
@@ -338,25 +341,42 @@ class InverseIndex(NamedTuple):
 def inverse_index(k_idx: torch.Tensor, bucket_off: torch.Tensor, bucket_cnt: torch.Tensor, N: int) -> InverseIndex:
     """Inverse of the flat bucket lists ``k_idx`` (row-major (row, bucket) order, ``bucket_off`` / ``bucket_cnt``
     [H,C]) over keys 0..N-1 of every row.  ``k_idx`` may be longer than the lists (only
-    the first ``sum(bucket_cnt)`` entries are read).  Synchronises once (the rows' list boundaries are read back)."""
+    the first ``sum(bucket_cnt)`` entries are read).  Synchronises (the rows' list boundaries and the count of entries out of key order are read back)."""
     _dev(k_idx, bucket_off, bucket_cnt)
     H, C = bucket_cnt.shape
     assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and bucket_off.dtype == torch.int64
     # the listed entries are the first T of k_idx; a buffer from the window filter is longer (it has room
     # for every entry of the unfiltered lists) and its tail is not initialised
+    lib = _lib.load()
+    dev = k_idx.device
     starts = bucket_off[:, 0].cpu().tolist()
     T = int(bucket_off[-1, -1]) + int(bucket_cnt[-1, -1])
     assert 0 <= T <= k_idx.numel(), "k_idx is shorter than the lists bucket_off / bucket_cnt describe"
-    lib = _lib.load()
-    dev = k_idx.device
     key_off = torch.empty(H * N + 1, dtype=torch.int32, device=dev)
     inv_pos = torch.empty(T, dtype=torch.int32, device=dev)
-    ws = _ws(lib.fm_inverse_index_workspace(T, H, N), k_idx)
-    if T:
+    path = "none"
+    if not T:
+        key_off.zero_()
+    elif C > 65535:
+        ws = _ws(lib.fm_inverse_index_workspace(T, H, N), k_idx)
         check(lib.fm_inverse_index(_p(k_idx), _p(bucket_off), _p(bucket_cnt), H, C, int(N), T, _p(key_off),
                                    _p(inv_pos), _p(ws), ws.numel(), _stream(k_idx)))
+        path = "sort"
     else:
-        key_off.zero_()
+        # lists in strictly ascending key order (what Memory keeps for its attention) are inverted by a
+        # transposition, which also counts the entries out of order; any other lists by a sort
+        n_bad = torch.empty(1, dtype=torch.int32, device=dev)
+        ws = _ws(lib.fm_inverse_index_key_order_workspace(H, C, int(N)), k_idx)
+        check(lib.fm_inverse_index_key_order(_p(k_idx), _p(bucket_off), _p(bucket_cnt), H, C, int(N), T, _p(key_off),
+                                             _p(inv_pos), _p(n_bad), _p(ws), ws.numel(), _stream(k_idx)))
+        path = "transposition"
+        if int(n_bad.item()):
+            del ws
+            ws = _ws(lib.fm_inverse_index_workspace(T, H, N), k_idx)
+            check(lib.fm_inverse_index(_p(k_idx), _p(bucket_off), _p(bucket_cnt), H, C, int(N), T, _p(key_off),
+                                       _p(inv_pos), _p(ws), ws.numel(), _stream(k_idx)))
+            path = "sort"
+    last_inverse_info.update(path=path)
     row_pos = tuple(starts) + (T,)
     return InverseIndex(key_off, inv_pos, row_pos)
 

@@ -229,7 +229,7 @@ int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t*
  * still costs its rows (written as zeros and read back).
  *
  * fm_inverse_index: the inverse of the lists, which depends on the lists only and
- * can be kept with them.  T = number of list entries (the sum of bucket_cnt, the
+ * can be kept with them (lists in any order: a stable radix sort of (key, position) pairs).  T = number of list entries (the sum of bucket_cnt, the
  * length of k_idx; row-major (row, bucket) order as everywhere).
  *   key_off [H*N + 1] int32   entries of key (h, n): sorted positions
  *                              key_off[h*N + n] .. key_off[h*N + n + 1]
@@ -244,6 +244,16 @@ size_t fm_inverse_index_workspace(int64_t T, int H, int N);
 int fm_inverse_index(const int32_t* k_idx, const int64_t* bucket_off, const int32_t* bucket_cnt, int H,
                      int C, int N, int64_t T, int32_t* key_off, int32_t* inv_pos, void* ws, size_t ws_bytes,
                      void* stream);
+/* The same index without a sort, for lists in strictly ascending key order (every list as
+ * fm_lists_key_order leaves it, no key twice): a transposition by key ranges, several times
+ * faster (H, C <= 65535).  n_bad [1] (device) receives 0 when every list is in that order with
+ * all keys in [0, N), and a positive count otherwise: then key_off / inv_pos hold no index
+ * (every access still stays inside the buffers, and the call costs one pass over the lists)
+ * and fm_inverse_index is the one to call.  Workspace: two tables of H*C*(N/256+1) words. */
+size_t fm_inverse_index_key_order_workspace(int H, int C, int N);
+int fm_inverse_index_key_order(const int32_t* k_idx, const int64_t* bucket_off, const int32_t* bucket_cnt, int H,
+                               int C, int N, int64_t T, int32_t* key_off, int32_t* inv_pos, int32_t* n_bad,
+                               void* ws, size_t ws_bytes, void* stream);
 size_t fm_hash_attn_bwd_staged_workspace(int64_t max_row_entries);
 int fm_hash_attn_bwd_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
                             const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,

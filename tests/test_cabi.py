@@ -55,6 +55,7 @@ def test_argument_errors_are_status_codes():
     assert lib.fm_index_append(None, None, 1, 1, None, None, None, None, 1, 1, 1, 1, 1, None, 0, None, None) == 1
     assert b"fm_index_append" in lib.fm_last_error()
     assert lib.fm_inverse_index(None, None, None, 1, 1, 1, 1, None, None, None, 0, None) == 1
+    assert lib.fm_inverse_index_key_order(None, None, None, 1, 1, 1, 1, None, None, None, None, 0, None) == 1
     assert lib.fm_hash_attn_bwd(None, None, None, None, None, None, None, None, None, 1, None, None, None, None,
                                 None, None, None, 1, 1, 1, 8, 1, 1.0, 0, None) != 0
     assert lib.fm_hash_attn_bwd_staged(*([None] * 18), 1, 1, 1, 64, 1, None, 1.0, 1, None, 0, None) != 0   # d = 64
@@ -90,6 +91,9 @@ def test_workspace_queries():
     assert lib.fm_hash_attn_bwd_staged_workspace(1000) >= 1000 * 512         # two bf16 rows of 128 per list entry
     assert lib.fm_inverse_index_workspace(1000, 1, 100) >= 3 * 1000 * 4
     assert lib.fm_inverse_index_workspace(0, 1, 100) == 0
+    # two tables [H][C][N / 256 + 1] of words and the ranges' totals
+    assert lib.fm_inverse_index_key_order_workspace(2, 10, 1000) >= 2 * 2 * 10 * 5 * 4 + 2 * 4 * 4
+    assert lib.fm_inverse_index_key_order_workspace(0, 10, 1000) == 0
 
 
 def test_ops_refuse_cpu_tensors():

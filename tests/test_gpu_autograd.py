@@ -140,6 +140,24 @@ def test_module_forward_backward_against_joint_softmax():
         assert err <= 2e-4, f"{name}: max err {err:.3e}"
 
 
+def test_module_backward_notices_a_memory_changed_in_place():
+    """The keys and values of the memory reach the backward through save_for_backward (the reference keeps
+    clones, memory.py:243-244): overwriting them in place between forward and backward -- a KV cache that
+    moves on -- is an error autograd reports, not a gradient against the new contents."""
+    from fast_memory_amd import ring_cross_attention_approx
+    g = gen(8310)
+    H, G, S, N, d, C, Z, topk = 2, 2, 16, 300, 64, 4, 32, 8
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.6).cuda()
+    q, kq, ks, vs = mk(1, H * G, S, d).requires_grad_(True), mk(1, H * G, N, d), mk(1, H, S, d), mk(1, H, S, d)
+    k_leaf, v = mk(1, H, N, d).requires_grad_(True), mk(1, H, N, d)
+    k = k_leaf * 1.0                                    # a non-leaf that may be written in place
+    out = ring_cross_attention_approx(q, kq, ks, vs, k, v, dev(O.init_centroids(C, d, torch.float32)), d ** -0.5, C, Z,
+                                      centroid_topk=topk)
+    k.mul_(2.0)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        out.sum().backward()
+
+
 @pytest.mark.parametrize("S,L,chunk_entries", [(40, 56, None), (200, 200, 64 * 200)])   # one call; token chunks of 64
 def test_local_attention_backward_bf16(S, L, chunk_entries, monkeypatch):
     from fast_memory_amd import autograd as fm_autograd, local_attention_backward, ops as _ops

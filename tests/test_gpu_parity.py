@@ -1044,6 +1044,60 @@ def test_memory_attend_backward_against_autograd(ops):
     assert inv1 is not inv0 and inv1.key_off.numel() == H * (N + 50) + 1  # rebuilt for the longer memory
 
 
+def _inverse_by_stable_sort(flat_lists, rows, H, N):
+    flat = flat_lists.long() + rows * N
+    order = torch.sort(flat, stable=True).indices
+    key_off = torch.zeros(H * N + 1, dtype=torch.int64, device=flat.device)
+    key_off[1:] = torch.cumsum(torch.bincount(flat, minlength=H * N), 0)
+    return key_off.int(), order.int()
+
+
+@pytest.mark.parametrize("H,N,C,Z", [(2, 5000, 24, 333), (3, 700, 5, 40), (1, 256, 3, 256), (2, 70000, 130, 900),
+                                     (4, 131072, 64, 4096)])
+def test_inverse_index_by_transposition_and_by_sort(ops, H, N, C, Z):
+    """Lists in ascending key order are inverted by a transposition over key ranges, any others by a stable
+    radix sort; both equal a stable sort of (row, key) over the flat positions.  Ragged lists with empty
+    ones, runs of a key range longer than a group of lanes (Z = N), keys that no list names, N off the range
+    size; then the same lists out of order, and with one repeated key, which take the sort."""
+    g = torch.Generator(device="cuda").manual_seed(1700 + H)
+    # strictly ascending keys: a prefix sum of gaps >= 1 that stays below N
+    hi = max(1, 2 * (N // Z) - 1) if N > Z else 1
+    gaps = torch.randint(1, hi + 1, (H, C, Z), device="cuda", generator=g, dtype=torch.int32)
+    gaps[..., 0] = torch.randint(1, max(2, N // (4 * Z)) + 1, (H, C), device="cuda", generator=g, dtype=torch.int32)
+    lists = torch.cumsum(gaps, -1, dtype=torch.int32) - 1
+    lists = torch.minimum(lists, (N - Z + torch.arange(Z, device="cuda", dtype=torch.int32)).expand(H, C, Z))
+    assert int(lists.max()) < N and bool((lists[..., 1:] > lists[..., :-1]).all())
+    cnt = torch.randint(0, Z + 1, (H, C), device="cuda", generator=g, dtype=torch.int32)
+    cnt[0, 0] = 0
+    cnt[-1, -1] = Z
+    cnt[0, -1] = Z
+    off = ops.bucket_offsets(cnt)
+    mask = torch.arange(Z, device="cuda")[None, None, :] < cnt[..., None]
+    rows = torch.arange(H, device="cuda")[:, None, None].expand(H, C, Z)[mask]
+    flat_lists = lists[mask].contiguous()
+    inv = ops.inverse_index(flat_lists, off, cnt, N)
+    assert ops.last_inverse_info["path"] == "transposition"
+    ko, ip = _inverse_by_stable_sort(flat_lists, rows, H, N)
+    assert torch.equal(inv.key_off, ko) and torch.equal(inv.inv_pos, ip)
+    assert inv.row_pos == tuple(off[:, 0].tolist()) + (flat_lists.numel(),)
+    # the same entries in another order inside every list
+    shuffled = torch.where(mask, lists, torch.full_like(lists, N))               # unlisted entries sort last
+    perm = torch.rand(H, C, Z, device="cuda", generator=g).masked_fill(~mask, 2.0).argsort(-1)
+    flat_shuffled = torch.gather(shuffled, -1, perm)[mask].contiguous()
+    inv = ops.inverse_index(flat_shuffled, off, cnt, N)
+    assert ops.last_inverse_info["path"] == "sort"
+    ko, ip = _inverse_by_stable_sort(flat_shuffled, rows, H, N)
+    assert torch.equal(inv.key_off, ko) and torch.equal(inv.inv_pos, ip)
+    # one key twice in one list: not the order the transposition takes
+    twice = flat_lists.clone()
+    last = int(off[-1, -1])
+    twice[last + 1] = twice[last]
+    inv = ops.inverse_index(twice, off, cnt, N)
+    assert ops.last_inverse_info["path"] == "sort"
+    ko, ip = _inverse_by_stable_sort(twice, rows, H, N)
+    assert torch.equal(inv.key_off, ko) and torch.equal(inv.inv_pos, ip)
+
+
 def test_ring_attention_masked_backward_with_merged_result(ops):
     # memory part of a merged attention: out / lse passed to the backward are those of the softmax over
     # bucket keys and local keys together; checked against autograd through a dense fp64 evaluation

@@ -5,6 +5,7 @@
 // integer work with data-independent launch shapes: nothing here reads a count
 // back to the host.
 #include "common.hpp"
+#include "radix_sort.hpp"
 
 namespace fm {
 
@@ -166,6 +167,55 @@ __global__ __launch_bounds__(kGrpBlock) void group_scatter_kernel(
   q_perm[pos] = i;  // pos runs over the flattened [H*Sq] sorted axis
 }
 
+// ---- grouping of long rows ----------------------------------------------------------
+// The block table above is [H][Sq / 256][C] words: with a million entries a row (the keys of a K-means
+// assignment, grouped by centroid) it is hundreds of megabytes that are zeroed, scanned and read again.
+// From kGrpSortMin entries on the grouping is a stable radix sort of the keys row * C + bucket (H * C for an
+// entry without a bucket, which therefore sorts behind all others): the sorted positions are q_perm, the
+// bins' sizes come from the sorted keys.  Same q_perm, bin_off, bin_count and items as the block form.
+constexpr int64_t kGrpSortMin = int64_t(1) << 19;
+
+__global__ __launch_bounds__(256) void group_keys_kernel(const int32_t* __restrict__ q_hash, int64_t n, int C, int Sq,
+                                                         uint32_t no_bucket, uint32_t* __restrict__ keys) {
+  const int64_t f = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (f >= n) return;
+  const int b = q_hash[f];
+  keys[f] = b >= 0 && b < C ? uint32_t(f / Sq) * uint32_t(C) + uint32_t(b) : no_bucket;
+}
+
+__global__ __launch_bounds__(256) void group_bin_counts_kernel(const int32_t* __restrict__ off, int64_t n_bins,
+                                                               int32_t* __restrict__ bin_count) {
+  const int64_t g = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (g < n_bins) bin_count[g] = off[g + 1] - off[g];
+}
+
+// sorted flat positions -> q_perm: the entry's index inside its row, or -(flat position) - 1 without a bucket
+__global__ __launch_bounds__(256) void group_perm_kernel(const uint32_t* __restrict__ sorted_keys,
+                                                         const uint32_t* __restrict__ sorted_pos, int64_t n, int Sq,
+                                                         uint32_t no_bucket, int32_t* __restrict__ q_perm) {
+  const int64_t j = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (j >= n) return;
+  const uint32_t f = sorted_pos[j];
+  q_perm[j] = sorted_keys[j] == no_bucket ? -int32_t(f) - 1 : int32_t(f % uint32_t(Sq));
+}
+
+struct GroupSortPlan {
+  RadixPlan radix;
+  int bits;
+  size_t off_pos, off_off, total;
+};
+static GroupSortPlan group_sort_plan(int H, int C, int Sq) {
+  GroupSortPlan p;
+  const int64_t n = int64_t(H) * Sq;
+  p.bits = key_bits(int64_t(H) * C + 1);
+  p.radix = radix_plan(n, p.bits);
+  p.off_pos = p.radix.total;
+  p.off_off = p.off_pos + align_up(size_t(n) * sizeof(uint32_t), 256);
+  p.total = p.off_off + align_up((size_t(H) * C + 2) * sizeof(int32_t), 256);
+  return p;
+}
+static bool group_by_sort(int H, int Sq) { return int64_t(H) * Sq >= kGrpSortMin; }
+
 // ---- window filter ----------------------------------------------------------
 __global__ __launch_bounds__(256) void window_count_kernel(const int32_t* __restrict__ idx_in,
                                                            int64_t nb, int Z, int64_t lo,
@@ -263,6 +313,7 @@ extern "C" int64_t fm_group_max_items(int H, int C, int Sq) {
 }
 
 extern "C" size_t fm_group_queries_workspace(int H, int C, int Sq) {
+  if (H >= 1 && C >= 1 && Sq >= 1 && fm::group_by_sort(H, Sq)) return fm::group_sort_plan(H, C, Sq).total + 256;
   int64_t NB = fm::ceil_div(Sq, fm::kGrpBlock);
   return fm::align_up(size_t(H) * size_t(NB) * size_t(C) * sizeof(int32_t), 256) + 256;
 }
@@ -284,6 +335,26 @@ extern "C" int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int
   FM_REQUIRE(ws_bytes >= fm_group_queries_workspace(H, C, Sq), FM_ERR_WORKSPACE,
              "fm_group_queries: workspace %zu < %zu", ws_bytes, fm_group_queries_workspace(H, C, Sq));
   hipStream_t st = as_stream(stream);
+  if (group_by_sort(H, Sq)) {
+    const GroupSortPlan p = group_sort_plan(H, C, Sq);
+    const int64_t n = int64_t(H) * Sq, n_bins = int64_t(H) * C;
+    const uint32_t no_bucket = uint32_t(n_bins);
+    char* base = static_cast<char*>(ws);
+    uint32_t* pos = reinterpret_cast<uint32_t*>(base + p.off_pos);
+    int32_t* off = reinterpret_cast<int32_t*>(base + p.off_off);
+    int32_t* n_unlisted = reinterpret_cast<int32_t*>(base + p.total);  // (the items kernel zeroes it; unused here)
+    const unsigned blocks = unsigned(ceil_div(n, int64_t(256)));
+    hipLaunchKernelGGL(group_keys_kernel, dim3(blocks), dim3(256), 0, st, q_hash, n, C, Sq, no_bucket,
+                       reinterpret_cast<uint32_t*>(base));
+    const uint32_t* sorted = radix_sort_positions(ws, p.radix, n, p.bits, pos, st);
+    launch_sorted_offsets(sorted, n, n_bins, off, st);
+    hipLaunchKernelGGL(group_bin_counts_kernel, dim3(unsigned(ceil_div(n_bins, int64_t(256)))), dim3(256), 0, st, off,
+                       n_bins, bin_count);
+    hipLaunchKernelGGL(group_items_kernel, dim3(1), dim3(1024), 0, st, bin_count, n_bins, C, bin_off, items, n_items,
+                       max_items, n_unlisted);
+    hipLaunchKernelGGL(group_perm_kernel, dim3(blocks), dim3(256), 0, st, sorted, pos, n, Sq, no_bucket, q_perm);
+    return launch_status("fm_group_queries");
+  }
   const int NB = int(ceil_div(Sq, kGrpBlock));
   int32_t* block_hist = static_cast<int32_t*>(ws);
   // counter of the queries without a bucket: the spare 256 bytes behind the block table

@@ -243,6 +243,41 @@ def test_group_queries(ops, H, S, C):
     assert items.tolist() == exp
 
 
+@pytest.mark.parametrize("H,S,C", [(2, 300000, 37), (1, 600000, 2048), (5, 110000, 300)])
+def test_group_long_rows(ops, H, S, C):
+    """From half a million entries on the grouping is a stable radix sort instead of the table of block
+    counts: same permutation (stable: ascending entry index inside a bucket), bins and items; entries without
+    a bucket behind all others, as -(flat index) - 1."""
+    g = torch.Generator(device="cuda").manual_seed(402)
+    qh = torch.randint(0, C, (H, S), generator=g, device="cuda", dtype=torch.int32)
+    qh[0, : S // 3] = 3                                                  # a heavy bucket
+    qh[-1, 5::1000] = C + 7                                              # entries without a bucket
+    qh[0, 11::777] = -1
+    G = ops.group_queries(qh, C)
+    valid = (qh >= 0) & (qh < C)
+    key = torch.where(valid, qh.long() + torch.arange(H, device="cuda")[:, None] * C, torch.full_like(qh, H * C).long())
+    order = torch.sort(key.reshape(-1), stable=True).indices
+    n_valid = int(valid.sum())
+    exp = torch.where(torch.arange(H * S, device="cuda") < n_valid, order % S, -order - 1).int()
+    perm = G.q_perm.reshape(-1)
+    assert torch.equal(perm[:n_valid], exp[:n_valid])
+    assert torch.equal(torch.sort(perm[n_valid:]).values, torch.sort(exp[n_valid:]).values)
+    cnt = torch.bincount(key.reshape(-1), minlength=H * C + 1)[: H * C]
+    assert torch.equal(G.bin_count.reshape(-1).long(), cnt)
+    assert torch.equal(G.bin_off.reshape(-1).long(), torch.cumsum(cnt, 0) - cnt)
+    n = int(G.n_items.item())
+    items = G.items[:n].cpu().long()
+    tiles = (cnt + 63) // 64
+    assert n == int(tiles.sum())
+    first = (torch.cumsum(tiles, 0) - tiles).cpu()
+    bins = torch.repeat_interleave(torch.arange(H * C), tiles.cpu())
+    t_in = torch.arange(n) - first[bins]
+    off = (torch.cumsum(cnt, 0) - cnt).cpu()
+    exp_items = torch.stack([bins // C, bins % C, off[bins] + 64 * t_in,
+                             torch.minimum(torch.full_like(t_in, 64), cnt.cpu()[bins] - 64 * t_in)], 1)
+    assert torch.equal(items, exp_items)
+
+
 def test_bucket_offsets_and_window_filter(ops):
     g = gen(401)
     cnt = torch.randint(0, 50, (7, 300), generator=g).int()

@@ -161,7 +161,8 @@ def _causal_prefix_lists(H: int, t0: int, t1: int, S: int, L: int, causal: bool,
     return _prefix_lists[key]
 
 
-def local_attention_backward(d_out, q, k, v, out, lse, sm_scale: float, causal: bool = True):
+def local_attention_backward(d_out, q, k, v, out, lse, sm_scale: float, causal: bool = True,
+                             staged: Optional[bool] = None):
     """Gradients of the dense local attention (the ``attention_backward(dout, q, k_self, v_self, out, lse,
     sm_scale, True)`` call at memory.py:368, which the reference does not define).  ``q, out, d_out
     [H*G,S,d]``, ``k, v [H,L,d]``, ``lse [H*G,S]``; ``out`` / ``lse`` may be the merged result.  Returns
@@ -170,7 +171,14 @@ def local_attention_backward(d_out, q, k, v, out, lse, sm_scale: float, causal: 
     The causal prefix of every token is a list of keys, so this is the backward of the gathered attention
     with one bucket per token (shared by the G query heads of a KV head): no kernel of its own.  The lists
     hold S (L - S/2) entries per KV head, so the tokens are taken in chunks that keep a call's lists below
-    2^24 entries per head (one call up to S = L = 4096); dk and dv add up over the calls."""
+    2^24 entries per head (one call up to S = L = 4096); dk and dv add up over the calls.
+
+    ``staged`` is passed on to :func:`attention_hash_varlen_backward`: ``None`` (the default) takes the form
+    without atomics for bf16 with d = 128 (every bucket here receives queries; results do not depend on
+    scheduling) and the atomic adds otherwise or when its workspace does not fit.  Cost at H = 8, G = 8,
+    S = L = 4096, d = 128 bf16 on MI355X: 22 ms and 25 GiB of workspace (268 MB of lists, 34 GB of partial
+    rows taken a few KV heads at a time) staged, 51 ms and 0.7 GiB with atomic adds -- several times what a
+    kernel written for the dense causal case would take, which this library does not have."""
     HG, S, d = q.shape
     H, L, _ = k.shape
     G = HG // H
@@ -189,7 +197,7 @@ def local_attention_backward(d_out, q, k, v, out, lse, sm_scale: float, causal: 
         qh = t.repeat(H * G).reshape(H, G * n)                                                # query g*n + t -> t
         sl = lambda x: x[:, :, t0:t1].reshape(H, G * n, *x.shape[3:]).contiguous()
         dq_c, dk_c, dv_c = attention_hash_varlen_backward(
-            sl(do4), sl(q4), k, v, sl(o4).to(q.dtype), sl(l4).float(), flat, cnt, qh, sm_scale, staged=False)
+            sl(do4), sl(q4), k, v, sl(o4).to(q.dtype), sl(l4).float(), flat, cnt, qh, sm_scale, staged=staged)
         dq[:, :, t0:t1] = dq_c.reshape(H, G, n, d)
         dk, dv = (dk_c, dv_c) if dk is None else (dk + dk_c, dv + dv_c)
     return dq.reshape(HG, S, d), dk, dv

@@ -260,3 +260,29 @@ def test_reference_harness_shape_kernels_agree(ops):
         sel = torch.linspace(0, Sq - 1, 96).long().cuda()
         ro, rl = oracle_on_sample(q[b, sel], qh[b, sel].long(), lists[b], k[b], v[b], scale)
         assert_attn_close(out[b, sel][None], lse[b, sel][None], ro, rl, torch.bfloat16, f"row {b} sampled queries")
+
+
+def test_local_attention_backward_full_size(ops):
+    """The backward of the dense causal local attention at the c5 shape (8 KV heads x 8 query heads, 4096
+    tokens, d = 128 bf16), which runs as a gathered backward with one bucket per token.  The reference calls
+    ``attention_backward`` (memory.py:368) without defining it, so parity with it is unpinned: the check is
+    against autograd through the textbook definition in fp32, for KV head 0 and its eight query heads, and
+    the form without atomics gives the same bits twice."""
+    from fast_memory_amd import local_attention_backward
+    H, G, S, L, d = 8, 8, 4096, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(9100)
+    mk = lambda *s: (torch.randn(*s, generator=g, device="cuda") * 0.6).to(torch.bfloat16)
+    q, k, v, w = mk(H * G, S, d), mk(H, L, d), mk(H, L, d), mk(H * G, S, d)
+    out, lse = ops.local_attn_fwd(q, k, v, d ** -0.5, True)
+    dq, dk, dv = local_attention_backward(w, q, k, v, out, lse, d ** -0.5, True)
+    dq2, dk2, dv2 = local_attention_backward(w, q, k, v, out, lse, d ** -0.5, True)
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+    qf = q.float().view(H, G, S, d)[:1].cpu().requires_grad_()
+    kf, vf = k.float()[:1].cpu().requires_grad_(), v.float()[:1].cpu().requires_grad_()
+    s = torch.einsum("hgid,hjd->hgij", qf, kf) * d ** -0.5
+    mask = torch.arange(L)[None, :] > torch.arange(S)[:, None]
+    o = torch.einsum("hgij,hjd->hgid", torch.softmax(s.masked_fill(mask, float("-inf")), -1), vf)
+    (o * w.float().view(H, G, S, d)[:1].cpu()).sum().backward()
+    for got, want, name in ((dq.view(H, G, S, d)[:1], qf.grad, "dq"), (dk[:1], kf.grad, "dk"), (dv[:1], vf.grad, "dv")):
+        err = (got.float().cpu() - want).abs().max().item()
+        assert err <= 2e-2 * max(1.0, want.abs().max().item()), f"{name}: {err:.3e}"

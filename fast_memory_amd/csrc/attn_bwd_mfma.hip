@@ -34,6 +34,7 @@ typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bbf16x2;
 typedef __attribute__((__vector_size__(2 * sizeof(float)))) float bf32x2;
 
 constexpr int kBD = 128;
+constexpr int kPartLd = 2 * kBD;  // a list position's partial rows lie side by side: [dK row | dV row], 512 bytes
 
 __device__ __forceinline__ bf16x8 b_as_bf16x8(uint4 u) {
   union {
@@ -297,7 +298,7 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
             const int pos = kp0 + 16 * kt + rr;
             const bool ok = pos < cnt;
             bf16_t* base = mat == 0 ? dvp : dkp;
-            uint4* px = reinterpret_cast<uint4*>((ok ? base + int64_t(pos) * kBD : dump + (4 * mat + g) * kBD) + 8 * c);
+            uint4* px = reinterpret_cast<uint4*>((ok ? base + int64_t(pos) * kPartLd : dump + (4 * mat + g) * kBD) + 8 * c);
             if (!FIRST_TILE) x = add_bf16x8(x, *px);
             *px = x;
           }
@@ -316,7 +317,7 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
             const int pos = kp0 + 16 * kt + rr;
             const bool ok = pos < cnt;
             bf16_t* base = tw == 0 ? dvp : dkp;
-            uint4* px = reinterpret_cast<uint4*>((ok ? base + int64_t(pos) * kBD : dump + (4 * tw + g) * kBD) + 8 * c);
+            uint4* px = reinterpret_cast<uint4*>((ok ? base + int64_t(pos) * kPartLd : dump + (4 * tw + g) * kBD) + 8 * c);
             if (!FIRST_TILE) x = add_bf16x8(x, *px);
             *px = x;
           }
@@ -330,8 +331,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
           uint4 xk = *reinterpret_cast<const uint4*>(slab + (16 + rr) * kStLd + 8 * c);
           const int pos = kp0 + 16 * kt + rr;
           const bool ok = pos < cnt;
-          uint4* pv = reinterpret_cast<uint4*>((ok ? dvp + int64_t(pos) * kBD : dump + g * kBD) + 8 * c);
-          uint4* pk = reinterpret_cast<uint4*>((ok ? dkp + int64_t(pos) * kBD : dump + (4 + g) * kBD) + 8 * c);
+          uint4* pv = reinterpret_cast<uint4*>((ok ? dvp + int64_t(pos) * kPartLd : dump + g * kBD) + 8 * c);
+          uint4* pk = reinterpret_cast<uint4*>((ok ? dkp + int64_t(pos) * kPartLd : dump + (4 + g) * kBD) + 8 * c);
           if (!FIRST_TILE) {  // (compile time: a load here, even skipped, would make every store wait)
             xv = add_bf16x8(xv, *pv);
             xk = add_bf16x8(xk, *pk);
@@ -483,7 +484,8 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
 }
 
 // grid (C, rows): one workgroup per (row, bucket) takes the bucket's query tiles one after the other;
-// dK, dV partial rows of the bucket go to dkp / dvp at (flat list position - pos0); dump: 8 rows of
+// dK, dV partial rows of the bucket go to dkp / dvp + (flat list position - pos0) * kPartLd (dvp = dkp + kBD:
+// the two rows of a position are 512 contiguous bytes, which the reduction reads together); dump: 8 rows of
 // 128 bf16 that take the stores of a block's positions past the end of a list.
 // MAXT: the most tiles a pass takes (2 or 4).  The four-tile form costs registers in every path of the
 // kernel that holds it, so it is only launched where buckets receive more than 24 queries on average.
@@ -509,18 +511,17 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
   const int nq = bin_count[bkt];
   const int64_t off = bucket_off[bkt];
   if (nq <= 0) {  // nobody hashed here: the bucket contributes zero rows
-    const int64_t n16 = int64_t(bucket_cnt[bkt]) * (kBD * sizeof(bf16_t) / 16);
-    uint4* zk = reinterpret_cast<uint4*>(dkp + (off - pos0) * kBD);
-    uint4* zv = reinterpret_cast<uint4*>(dvp + (off - pos0) * kBD);
-    for (int64_t i = threadIdx.x; i < n16; i += 256) zk[i] = zv[i] = make_uint4(0, 0, 0, 0);
+    const int64_t n16 = int64_t(bucket_cnt[bkt]) * (kPartLd * sizeof(bf16_t) / 16);
+    uint4* z = reinterpret_cast<uint4*>(dkp + (off - pos0) * kPartLd);
+    for (int64_t i = threadIdx.x; i < n16; i += 256) z[i] = make_uint4(0, 0, 0, 0);
     return;
   }
   const int32_t* ql = q_perm + bin_off[bkt];
   const bf16_t* Kb = k + int64_t(row) * N * kBD;
   const bf16_t* Vb = v + int64_t(row) * N * kBD;
   const int cnt = bucket_cnt[bkt];
-  bf16_t* dkb = dkp + (off - pos0) * kBD;
-  bf16_t* dvb = dvp + (off - pos0) * kBD;
+  bf16_t* dkb = dkp + (off - pos0) * kPartLd;
+  bf16_t* dvb = dvp + (off - pos0) * kPartLd;
   // the first pass stores the bucket's partial rows, the others add to them; a pass takes up to MAXT tiles.
   // The partial rows are bf16 and every pass after the first rounds them again, so only the first
   // kStagedMaxQ queries of a bucket go through them; a bucket that receives more (a heavily skewed hash)

@@ -6,8 +6,8 @@
 // sustain a fraction of the HBM rate; here the contributions are staged:
 //   1. hash_attn_bwd_staged_kernel (attn_bwd_mfma.hip): one workgroup per
 //      (row, bucket) writes the bucket's own dK, dV partial rows, one bf16 row of
-//      128 per listed key, at the key's flat list position -- plain coalesced
-//      stores, 2 x 256 B per (bucket, key) pair; dQ is complete after this step;
+//      128 per listed key each, side by side at the key's flat list position --
+//      plain coalesced stores, 512 B per (bucket, key) pair; dQ is complete after this step;
 //   2. bwd_reduce_kernel: one wave per key sums the key's partial rows over the
 //      list positions that name it, in ascending position order, and adds the
 //      fp32 sums into dK, dV.
@@ -321,8 +321,8 @@ __global__ __launch_bounds__(256) void bwd_reduce_kernel(const bf16_t* __restric
     xk = xv = make_uint4(0, 0, 0, 0);
     if (j < j1) {
       const int64_t f = uint32_t(inv_pos[j]);
-      xk = *reinterpret_cast<const uint4*>(dkp + (f - pos0) * 128 + 8 * c);
-      xv = *reinterpret_cast<const uint4*>(dvp + (f - pos0) * 128 + 8 * c);
+      xk = *reinterpret_cast<const uint4*>(dkp + (f - pos0) * 256 + 8 * c);
+      xv = *reinterpret_cast<const uint4*>(dvp + (f - pos0) * 256 + 8 * c);
     }
   };
   for (int j = j0 + g; j < j1; j += 16) {  // four rows per lane group in flight, added in ascending j
@@ -478,8 +478,8 @@ extern "C" int fm_hash_attn_bwd_staged(const void* q, const void* k, const void*
     const int64_t pos0 = row_pos_host[h0], n_pos = row_pos_host[h1] - pos0;
     if (n_pos > 0) {
       bf16_t* dkp = static_cast<bf16_t*>(ws);
-      bf16_t* dvp = dkp + size_t(n_pos) * 128;
-      bf16_t* dump = dvp + size_t(n_pos) * 128;
+      bf16_t* dvp = dkp + 128;  // a position's rows side by side: [dK | dV]
+      bf16_t* dump = dkp + size_t(n_pos) * 256;
       int rc = hash_attn_bwd_staged_partials(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, bin_off, bin_count, out,
                                              lse, dout, dlse, dq, dkp, dvp, dump, pos0, h0, h1 - h0, Sq, N, C, sm_scale, dk, dv, st);
       if (rc) return rc;

@@ -170,10 +170,13 @@ __global__ __launch_bounds__(kGrpBlock) void group_scatter_kernel(
 // ---- grouping of long rows ----------------------------------------------------------
 // The block table above is [H][Sq / 256][C] words: with a million entries a row (the keys of a K-means
 // assignment, grouped by centroid) it is hundreds of megabytes that are zeroed, scanned and read again.
-// From kGrpSortMin entries on the grouping is a stable radix sort of the keys row * C + bucket (H * C for an
-// entry without a bucket, which therefore sorts behind all others): the sorted positions are q_perm, the
-// bins' sizes come from the sorted keys.  Same q_perm, bin_off, bin_count and items as the block form.
-constexpr int64_t kGrpSortMin = int64_t(1) << 19;
+// From kGrpSortMinTable words of block table on the grouping is a stable radix sort of the keys row * C + bucket
+// (H * C for an entry without a bucket, which therefore sorts behind all others): the sorted positions are
+// q_perm, the bins' sizes come from the sorted keys.  Same q_perm, bin_off, bin_count and items as the block
+// form.  (8 rows of 131072 queries over 1024 buckets, 4 M words of table: 0.11 ms by blocks, 0.13 by sort;
+// 8 rows of 262144 keys over 1024 centroids, 8 M words: 0.19 against 0.15 ms; 8 rows of a million keys over
+// 2048, 67 M words: 0.8 against 0.25 ms.)
+constexpr int64_t kGrpSortMinTable = int64_t(1) << 23;
 
 __global__ __launch_bounds__(256) void group_keys_kernel(const int32_t* __restrict__ q_hash, int64_t n, int C, int Sq,
                                                          uint32_t no_bucket, uint32_t* __restrict__ keys) {
@@ -214,7 +217,9 @@ static GroupSortPlan group_sort_plan(int H, int C, int Sq) {
   p.total = p.off_off + align_up((size_t(H) * C + 2) * sizeof(int32_t), 256);
   return p;
 }
-static bool group_by_sort(int H, int Sq) { return int64_t(H) * Sq >= kGrpSortMin; }
+static bool group_by_sort(int H, int C, int Sq) {
+  return int64_t(H) * ceil_div(Sq, kGrpBlock) * C >= kGrpSortMinTable;
+}
 
 // ---- window filter ----------------------------------------------------------
 __global__ __launch_bounds__(256) void window_count_kernel(const int32_t* __restrict__ idx_in,
@@ -313,7 +318,7 @@ extern "C" int64_t fm_group_max_items(int H, int C, int Sq) {
 }
 
 extern "C" size_t fm_group_queries_workspace(int H, int C, int Sq) {
-  if (H >= 1 && C >= 1 && Sq >= 1 && fm::group_by_sort(H, Sq)) return fm::group_sort_plan(H, C, Sq).total + 256;
+  if (H >= 1 && C >= 1 && Sq >= 1 && fm::group_by_sort(H, C, Sq)) return fm::group_sort_plan(H, C, Sq).total + 256;
   int64_t NB = fm::ceil_div(Sq, fm::kGrpBlock);
   return fm::align_up(size_t(H) * size_t(NB) * size_t(C) * sizeof(int32_t), 256) + 256;
 }
@@ -335,7 +340,7 @@ extern "C" int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int
   FM_REQUIRE(ws_bytes >= fm_group_queries_workspace(H, C, Sq), FM_ERR_WORKSPACE,
              "fm_group_queries: workspace %zu < %zu", ws_bytes, fm_group_queries_workspace(H, C, Sq));
   hipStream_t st = as_stream(stream);
-  if (group_by_sort(H, Sq)) {
+  if (group_by_sort(H, C, Sq)) {
     const GroupSortPlan p = group_sort_plan(H, C, Sq);
     const int64_t n = int64_t(H) * Sq, n_bins = int64_t(H) * C;
     const uint32_t no_bucket = uint32_t(n_bins);

@@ -243,10 +243,9 @@ def test_group_queries(ops, H, S, C):
     assert items.tolist() == exp
 
 
-@pytest.mark.parametrize("H,S,C", [(2, 300000, 37), (1, 600000, 2048), (5, 110000, 300)])
+@pytest.mark.parametrize("H,S,C", [(2, 300000, 3700), (1, 1100000, 2048), (5, 110000, 4000)])
 def test_group_long_rows(ops, H, S, C):
-    """From half a million entries on the grouping is a stable radix sort instead of the table of block
-    counts: same permutation (stable: ascending entry index inside a bucket), bins and items; entries without
+    """Where the table of block counts would take 2^23 words or more the grouping is a stable radix sort instead: same permutation (stable: ascending entry index inside a bucket), bins and items; entries without
     a bucket behind all others, as -(flat index) - 1."""
     g = torch.Generator(device="cuda").manual_seed(402)
     qh = torch.randint(0, C, (H, S), generator=g, device="cuda", dtype=torch.int32)

@@ -23,9 +23,14 @@
 //
 // Roofline: the atomic traffic, 2 * d * 4 bytes per gathered (item tile, key)
 // pair, on top of the forward's gather traffic.
+#include <atomic>
+
 #include "common.hpp"
+#include "attn_ring.hpp"
 
 namespace fm {
+
+extern std::atomic<int> g_force_generic;  // attn_api.hip; 9: the staged backward loads its blocks into registers
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4s;
@@ -112,7 +117,13 @@ __device__ __forceinline__ void bwd_load_block(BwdBlock& r, const bf16_t* __rest
 // a block's partial rows is summed through the waves' LDS slabs before it is stored, so the bucket's K
 // and V rows are gathered and its partial rows written once for all the tiles of the pass.  The sums are
 // those of single-tile passes in tile order (bf16 rows added and rounded one by one).
-template <bool STAGED, bool FIRST_TILE, int TILES = 1>
+//
+// LDSBLK (two-tile staged form, first pass only): a block's K and V rows do not come into registers straight
+// from memory when the block is needed; they are requested a block ahead with loads that write LDS directly
+// (no registers in between), and the waves fill their operand registers from there.  The gather then runs
+// beside the arithmetic and the stores of the block before it.  blk: 32 KB, [block parity][K | V][32 rows of 256 B],
+// 16-byte chunk q of row r at position q ^ f(r) (no padding, no bank conflicts for either read pattern).
+template <bool STAGED, bool FIRST_TILE, int TILES = 1, bool LDSBLK = false>
 __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ out,
                                          const float* __restrict__ lse, const bf16_t* __restrict__ dout,
                                          const float* __restrict__ dlse, const int32_t* __restrict__ q_list, int n_q, int64_t qbase,
@@ -120,7 +131,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
                                          const int32_t* __restrict__ idx, int cnt, int N, float sm_scale,
                                          bf16_t* __restrict__ dq, float* __restrict__ dKb, float* __restrict__ dVb,
                                          bf16_t* dkp, bf16_t* dvp, bf16_t* dump, float* red, int* q_rows,
-                                         bf16_t* stage) {
+                                         bf16_t* stage, unsigned char* blk = nullptr) {
+  static_assert(!LDSBLK || (STAGED && FIRST_TILE && TILES == 2), "the LDS block form is the first two-tile pass");
   if (threadIdx.x < 16 * TILES) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_list[threadIdx.x] : -1;
   __syncthreads();
   const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -380,6 +392,69 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
         bwd_load_block(ra, Kb, Vb, rows, g, c);
         compute(ra, b);
       }
+    } else if (PAIR && LDSBLK) {
+      const int par = w & 1;  // the parity of this wave's blocks; waves par and par + 2 walk them together
+      const lds_char_t* const blk_l = (lds_char_t*)blk;
+      const uint32_t blk0 = __builtin_amdgcn_readfirstlane(uint32_t(uintptr_t(blk_l)));
+      const uint32_t kbuf = uint32_t(par) * 16384u, vbuf = kbuf + 8192u;  // byte offsets inside blk
+      // wave par brings the K rows of a block, wave par + 2 its V rows: 8 loads of 4 rows each
+      const bf16_t* src = ring_uniform_ptr(w < 2 ? Kb : Vb);
+      const uint32_t dst = blk0 + (w < 2 ? kbuf : vbuf);
+      auto swz = [](int r) { return ((r & 7) << 1) | ((r >> 3) & 1); };
+      auto issue = [&](int rows) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int r = 4 * j + g;  // row of the block this lane's 16 bytes belong to; its position in the row: c
+          const uint32_t key = uint32_t(__shfl(rows, r));
+          ring_load16(dst + uint32_t(j) * 1024u, key * 256u + uint32_t((c ^ swz(r & 15)) * 16), src);
+        }
+      };
+      auto rd = [&](uint32_t a) {
+        const ring_u32x4 x = *reinterpret_cast<const __attribute__((address_space(3))) ring_u32x4*>(blk_l + a);
+        return make_uint4(x.x, x.y, x.z, x.w);
+      };
+      auto fill = [&](BwdBlock& r, int rows) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+          const uint32_t row = uint32_t(kt * 16 + c) * 256u;
+          const int f = swz(c);
+#pragma unroll
+          for (int s2 = 0; s2 < 4; ++s2) {
+            const uint32_t at = row + uint32_t(((4 * s2 + g) ^ f) * 16);
+            r.k[kt][s2] = rd(kbuf + at);
+            r.vk[kt][s2] = rd(vbuf + at);
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int r2 = kt * 16 + 4 * g + j;
+            r.kc[kt][j] = rd(kbuf + uint32_t(r2) * 256u + uint32_t((c ^ swz(r2 & 15)) * 16));
+          }
+          r.rk[kt] = __shfl(rows, kt * 16 + c);
+        }
+      };
+      const int nb2 = (nblk + 1) & ~1;
+      int rows_nx = rows_of(par + 2);
+      {
+        const int rows0 = rows_of(par);
+        issue(rows0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        ring_barrier();
+        fill(ra, rows0);
+      }
+      for (int b = par; b < nb2; b += 2) {
+        const int rows_nx2 = rows_of(b + 4);  // (an ordinary load: older than the block's loads below)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's operands have left LDS ...
+        ring_barrier();                                      // ... and so have the other waves'
+        issue(rows_nx);  // block b + 2 (past the end: clamped rows, never used)
+        compute(ra, b);
+        // the block's loads are older than the eight partial-row stores of compute(): they have landed once at
+        // most eight operations are outstanding (a wave's vector memory operations complete in order)
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        ring_barrier();
+        fill(ra, rows_nx);
+        rows_nx = rows_nx2;
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     } else if (PAIR) {
       // every wave makes the same number of trips (the barriers inside): a block past the end is
       // clamped, contributes zeros and stores to the dump rows
@@ -491,7 +566,10 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
 // kernel that holds it, so it is only launched where buckets receive more than 24 queries on average.
 constexpr int kStagedMaxQ = 256;  // queries of a bucket that go through its bf16 partial rows
 
-template <int MAXT>
+#ifndef FM_LDSBLK_MIN
+#define FM_LDSBLK_MIN 16
+#endif
+template <int MAXT, bool LDSBLK>
 __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
@@ -504,6 +582,7 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
   __shared__ __attribute__((aligned(16))) unsigned char lds_buf[4 * 2 * 16 * kStLd * sizeof(bf16_t)];
   static_assert(sizeof(lds_buf) >= 4 * 8 * 4 * 64 * sizeof(float), "dQ partials fit the staging slabs");
   __shared__ int q_rows[16 * MAXT];
+  __shared__ __attribute__((aligned(16))) unsigned char blk[LDSBLK ? 32768 : 16];
   float* red = reinterpret_cast<float*>(lds_buf);
   bf16_t* stage = reinterpret_cast<bf16_t*>(lds_buf);
   const int row = row0 + blockIdx.y;
@@ -538,6 +617,11 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
         FM_BWD_PASS(true, MAXT);  // (MAXT, not 4: the two-tile kernel does not instantiate this form)
       else
         FM_BWD_PASS(false, MAXT);
+    } else if (LDSBLK && q0 == 0 && left > FM_LDSBLK_MIN) {
+      // the first pass of a bucket, up to 32 queries (with 16 or fewer the second tile is empty and adds zeros:
+      // the same bits as the one-tile form), its rows through LDS
+      bwd_tile<true, true, 2, LDSBLK>(q, out, lse, dout, dlse, ql, min(32, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,
+                                      cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage, blk);
     } else if (left > 16) {
       if (q0 == 0)
         FM_BWD_PASS(true, 2);
@@ -597,15 +681,17 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
                                   const void* dout, const float* dlse, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0,
                                   int row0, int rows, int Sq, int N, int C, float sm_scale, float* dk, float* dv,
                                   hipStream_t st) {
-#define FM_BWD_STAGED(MAXT)                                                                                        \
-  hipLaunchKernelGGL(hash_attn_bwd_staged_kernel<MAXT>, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,       \
+#define FM_BWD_STAGED(MAXT, LB)                                                                                    \
+  hipLaunchKernelGGL((hash_attn_bwd_staged_kernel<MAXT, LB>), dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st, \
                      (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,  \
                      bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, (bf16_t*)dkp,  \
                      (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale)
   if (int64_t(Sq) > 24 * int64_t(C))  // more than 24 queries per bucket on average
-    FM_BWD_STAGED(4);
+    FM_BWD_STAGED(4, false);
+  else if (N < (1 << 24) && g_force_generic != 9)  // (rows addressed by 32-bit byte offsets in the loads that write LDS)
+    FM_BWD_STAGED(2, true);
   else
-    FM_BWD_STAGED(2);
+    FM_BWD_STAGED(2, false);
 #undef FM_BWD_STAGED
   if (Sq > kStagedMaxQ)  // some bucket may hold more queries than go through its partial rows
     hipLaunchKernelGGL(hash_attn_bwd_excess_kernel, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,

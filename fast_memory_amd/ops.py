@@ -607,10 +607,12 @@ def grouped_forward_kernel(which: Optional[str]) -> None:
     launch, ``"staged-per-row"`` the same in one launch per row, ``"staged-pairs"`` the same kernel with two
     work items per workgroup, ``"ring"`` the kernel whose rows go from global memory straight into LDS (three
     items per workgroup) in a single launch, ``"ring-per-row"`` the same in one launch per row, ``"gather"``
-    always the kernel that gathers the rows into registers, ``None`` restores the dispatch (the direct loads
+    always the kernel that gathers the rows into registers, ``"bwd-register-blocks"`` (backward only) makes the
+    two-tile pass of the staged backward load its key blocks into registers instead of through LDS a block
+    ahead, ``None`` restores the dispatch (the direct loads
     per row where a row's K and V outgrow the last-level cache, the direct loads from 24 queries per bucket
     on average, else staged unless the launch has few and small work items)."""
     global _generic_forced
     _generic_forced = False
     _debug_lib().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4, "ring": 5,
-                                         "staged-per-row": 6, "ring-per-row": 7}[which])
+                                         "staged-per-row": 6, "ring-per-row": 7, "bwd-register-blocks": 9}[which])

@@ -31,7 +31,9 @@ int fm_debug_hooks_enabled(void);
  * items per workgroup), in a single launch, 7 = the same in one launch per row;
  * 3 = always the kernel that gathers the rows into registers; 8 = the kernel of the
  * head dimensions 64 and 256 instantiated for 128 (tests compare it with the kernels
- * built for 128).  Dispatch: gather
+ * built for 128); 9 = (backward) the two-tile pass of fm_hash_attn_bwd_staged
+ * loads its key blocks into registers as its other passes do, instead of through
+ * LDS a block ahead (tests compare the two, which give the same bits).  Dispatch: gather
  * when H min(Sq, C) < 512 and Sq < 24 C; else the direct loads up to 2^24 keys and
  * the staged kernel beyond; one launch per row when K and V of all rows are 512 MB
  * or more, those of a row 32 MB or more, and a row has 1024 (staged kernel: 1536)

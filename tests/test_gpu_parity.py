@@ -1078,6 +1078,41 @@ def test_memory_attend_backward_against_autograd(ops):
     assert inv1 is not inv0 and inv1.key_off.numel() == H * (N + 50) + 1  # rebuilt for the longer memory
 
 
+def test_backward_staged_blocks_through_lds_same_bits(ops):
+    """The first pass of the staged backward over a bucket with 17 to 32 queries takes its key blocks through
+    LDS, requested a block ahead; the same pass with the blocks loaded into registers (the diagnostic switch)
+    gives the same bits.  Lists of many blocks, ragged and empty ones, lengths that are no multiple of a block or
+    of a pair of blocks; buckets of 1 to 40 queries (below 17 and above 32 other passes run); twice in a row."""
+    B, S, N, C, Z, d = 2, 900, 9000, 40, 1999, 128
+    q, k, v, kh, cnt, qh = make_attn_case(1610, B, S, N, C, Z, d, torch.bfloat16, window="ref", std=0.7)
+    cnt[0, 3], cnt[0, 4], cnt[1, 5], cnt[1, 6] = 0, 1, 33, 64
+    dout = (torch.randn(B, S, d, generator=gen(1611)) * 0.5).to(torch.bfloat16)
+    sm = d ** -0.5
+    qd, kd, vd, khd, cntd, qhd = dev(q, k, v, kh, cnt, qh)
+    from fast_memory_amd import attention_hash_varlen
+    out, lse = attention_hash_varlen(qd, kd, vd, khd, cntd, qhd, sm)
+    lists, counts = khd.int().contiguous(), cntd.int().contiguous()
+    off = ops.bucket_offsets(counts)
+    groups = ops.group_queries(qhd.int().contiguous(), C)
+    per_bucket = groups.bin_count.reshape(-1)
+    assert int(((per_bucket > 16) & (per_bucket <= 32)).sum()) >= 10 and int((per_bucket > 32).sum()) >= 1
+    inv = ops.inverse_index(lists, off, counts, N)
+    run = lambda: ops.hash_attn_bwd_staged(qd, kd, vd, lists, off, counts, groups, inv, out, lse, dev(dout), sm)
+    a, b = run(), run()
+    ops.grouped_forward_kernel("bwd-register-blocks")
+    try:
+        c = run()
+    finally:
+        ops.grouped_forward_kernel(None)
+    for x, y, z, name in zip(a, b, c, ("dq", "dk", "dv")):
+        assert torch.equal(x, y), name + ": two runs differ"
+        assert torch.equal(x, z), name + ": blocks through LDS and blocks in registers differ"
+    rq, rk, rv = O.hashed_attention_backward_gather(q.float(), k.float(), v.float(), kh, cnt, qh, out.float().cpu(),
+                                                    lse.cpu(), dout.float(), sm)
+    for got, ref, name in ((a[0], rq, "dq"), (a[1], rk, "dk"), (a[2], rv, "dv")):
+        _assert_grad_close(got, ref, torch.bfloat16, name)
+
+
 def _inverse_by_stable_sort(flat_lists, rows, H, N):
     flat = flat_lists.long() + rows * N
     order = torch.sort(flat, stable=True).indices

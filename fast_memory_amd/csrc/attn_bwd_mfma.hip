@@ -688,7 +688,10 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
                      (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale)
   if (int64_t(Sq) > 24 * int64_t(C))  // more than 24 queries per bucket on average
     FM_BWD_STAGED(4, false);
-  else if (N < (1 << 24) && g_force_generic != 9)  // (rows addressed by 32-bit byte offsets in the loads that write LDS)
+  else if (N < (1 << 24) && int64_t(Sq) > 12 * int64_t(C) && g_force_generic != 9)
+    // rows addressed by 32-bit byte offsets in the loads that write LDS; and enough buckets with more than 16
+    // queries to pay for the registers the extra form costs the others (12 queries per bucket on average: a
+    // fifth of the buckets of evenly hashed queries; at 8 the form costs 2 %, at 16 it gains 8 %)
     FM_BWD_STAGED(2, true);
   else
     FM_BWD_STAGED(2, false);

@@ -1095,6 +1095,7 @@ def test_backward_staged_blocks_through_lds_same_bits(ops):
     off = ops.bucket_offsets(counts)
     groups = ops.group_queries(qhd.int().contiguous(), C)
     per_bucket = groups.bin_count.reshape(-1)
+    assert S > 12 * C                                           # the launch takes the form with the LDS blocks
     assert int(((per_bucket > 16) & (per_bucket <= 32)).sum()) >= 10 and int((per_bucket > 32).sum()) >= 1
     inv = ops.inverse_index(lists, off, counts, N)
     run = lambda: ops.hash_attn_bwd_staged(qd, kd, vd, lists, off, counts, groups, inv, out, lse, dev(dout), sm)

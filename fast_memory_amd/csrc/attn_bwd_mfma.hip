@@ -566,11 +566,11 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
 // kernel that holds it, so it is only launched where buckets receive more than 24 queries on average.
 constexpr int kStagedMaxQ = 256;  // queries of a bucket that go through its bf16 partial rows
 
-#ifndef FM_LDSBLK_MIN
-#define FM_LDSBLK_MIN 16
-#endif
+// LDSBLK: the kernel whose two-tile first pass takes its blocks through LDS.  It has a compute unit to itself
+// (one workgroup of four waves, all the registers a lane can have, nothing spilled): with two workgroups at 256
+// registers each its 138 spilled registers cost more than the second workgroup hides (c5: 94.5 against 91.8 ms).
 template <int MAXT, bool LDSBLK>
-__global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
+__global__ __launch_bounds__(256, LDSBLK ? 1 : 2) void hash_attn_bwd_staged_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
     const int32_t* __restrict__ q_perm, const int32_t* __restrict__ bin_off, const int32_t* __restrict__ bin_count,
@@ -617,9 +617,8 @@ __global__ __launch_bounds__(256, 2) void hash_attn_bwd_staged_kernel(
         FM_BWD_PASS(true, MAXT);  // (MAXT, not 4: the two-tile kernel does not instantiate this form)
       else
         FM_BWD_PASS(false, MAXT);
-    } else if (LDSBLK && q0 == 0 && left > FM_LDSBLK_MIN) {
-      // the first pass of a bucket, up to 32 queries (with 16 or fewer the second tile is empty and adds zeros:
-      // the same bits as the one-tile form), its rows through LDS
+    } else if (LDSBLK && q0 == 0 && left > 16) {
+      // the first pass of a bucket with 17 to 32 queries, its rows through LDS
       bwd_tile<true, true, 2, LDSBLK>(q, out, lse, dout, dlse, ql, min(32, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,
                                       cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage, blk);
     } else if (left > 16) {

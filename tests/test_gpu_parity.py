@@ -1079,9 +1079,9 @@ def test_memory_attend_backward_against_autograd(ops):
 
 
 def test_backward_staged_blocks_through_lds_same_bits(ops):
-    """The first pass of the staged backward over a bucket with 17 to 32 queries takes its key blocks through
-    LDS, requested a block ahead; the same pass with the blocks loaded into registers (the diagnostic switch)
-    gives the same bits.  Lists of many blocks, ragged and empty ones, lengths that are no multiple of a block or
+    """The first pass of the staged backward over a bucket (up to 32 queries) takes its key blocks through LDS,
+    requested a block ahead; the same pass with the blocks loaded into registers (the diagnostic switch) gives
+    the same bits.  Lists of many blocks, ragged and empty ones, lengths that are no multiple of a block or
     of a pair of blocks; buckets of 1 to 40 queries (below 17 and above 32 other passes run); twice in a row."""
     B, S, N, C, Z, d = 2, 900, 9000, 40, 1999, 128
     q, k, v, kh, cnt, qh = make_attn_case(1610, B, S, N, C, Z, d, torch.bfloat16, window="ref", std=0.7)

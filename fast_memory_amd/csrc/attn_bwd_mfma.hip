@@ -566,11 +566,13 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
 // kernel that holds it, so it is only launched where buckets receive more than 24 queries on average.
 constexpr int kStagedMaxQ = 256;  // queries of a bucket that go through its bf16 partial rows
 
-// LDSBLK: the kernel whose two-tile first pass takes its blocks through LDS.  It has a compute unit to itself
-// (one workgroup of four waves, all the registers a lane can have, nothing spilled): with two workgroups at 256
-// registers each its 138 spilled registers cost more than the second workgroup hides (c5: 94.5 against 91.8 ms).
+// LDSBLK: the kernel whose two-tile first pass takes its blocks through LDS.  The two-tile kernels have a compute
+// unit to themselves (one workgroup of four waves, all the registers a lane can have, nothing spilled): with two
+// workgroups at 256 registers each their 96 / 138 spilled registers cost more than the second workgroup hides
+// (c5: 94.5 against 91.8 ms; c4: 11.4 against 10.9 ms).  The four-tile kernel keeps two workgroups per CU
+// (c2: 1.3 against 1.6 ms).
 template <int MAXT, bool LDSBLK>
-__global__ __launch_bounds__(256, LDSBLK ? 1 : 2) void hash_attn_bwd_staged_kernel(
+__global__ __launch_bounds__(256, MAXT == 4 ? 2 : 1) void hash_attn_bwd_staged_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
     const int32_t* __restrict__ q_perm, const int32_t* __restrict__ bin_off, const int32_t* __restrict__ bin_count,

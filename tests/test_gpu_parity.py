@@ -34,6 +34,9 @@ def sync():
     (torch.float32, 2, 5, 130, 16),
     (torch.bfloat16, 2, 256, 1000, 128),
     (torch.bfloat16, 1, 130, 257, 64),
+    (torch.bfloat16, 2, 200, 700, 256),     # the MFMA kernel for any head dimension that is a multiple of 16
+    (torch.float16, 2, 96, 513, 64),
+    (torch.float16, 1, 70, 300, 256),
     (torch.bfloat16, 3, 7, 33, 24),         # d not a multiple of 16: generic kernel
 ])
 def test_project(ops, dtype, H, C, N, d):
@@ -157,6 +160,9 @@ def test_build_index_matches_project_then_select(ops):
     (torch.float32, 1, 64, 512, 64),
     (torch.bfloat16, 2, 256, 1000, 128),
     (torch.bfloat16, 2, 300, 77, 64),
+    (torch.bfloat16, 2, 150, 333, 256),
+    (torch.float16, 1, 90, 200, 64),
+    (torch.float16, 2, 257, 129, 256),
     (torch.float32, 3, 9, 40, 16),
 ])
 def test_qhash(ops, dtype, H, C, S, d):

@@ -139,25 +139,33 @@ _prefix_lists = {}
 
 
 _PREFIX_CHUNK_ENTRIES = 1 << 24   # list entries per KV head and call of the gathered backward (64 MiB of int32)
+_PREFIX_BLOCK = 8                 # tokens that share a bucket: with G query heads a bucket has 8 G queries
 
 
-def _causal_prefix_lists(H: int, t0: int, t1: int, S: int, L: int, causal: bool, device):
-    """Bucket lists that express the dense local attention of tokens t0 .. t1-1 as a gathered one: token t of
-    every query head is "hashed" to bucket t - t0, whose list is the keys it may see, 0 .. t + (L - S) (all L
-    keys without the causal mask, one bucket).  The last one built is kept."""
-    key = (H, t0, t1, S, L, bool(causal), str(device))
+def _causal_prefix_lists(H: int, t0: int, t1: int, S: int, L: int, device):
+    """Bucket lists that express the causal local attention of tokens t0 .. t1-1 (t0 a multiple of the token
+    block) as two gathered ones.  Token t sees keys 0 .. t + (L - S).  *Blocks*: the tokens of a block of
+    ``_PREFIX_BLOCK`` share bucket (t - t0) // block, whose list is what the block's first token sees -- keys
+    every token of the block sees.  *Diagonal*: token t alone in bucket t - t0, whose list is the rest of its
+    keys, the at most block - 1 keys between its block's first token and itself.  The last pair built is kept."""
+    key = (H, t0, t1, S, L, str(device))
     if key not in _prefix_lists:
-        if causal:
-            lim = (torch.arange(t0, t1, device=device) + (L - S + 1)).clamp(min=0, max=L)    # keys seen by token t
-            j = torch.arange(L, device=device)
-            flat1 = j.expand(t1 - t0, L)[j[None, :] < lim[:, None]].to(torch.int32)          # row-major (t, key)
-            cnt = lim.to(torch.int32).unsqueeze(0).expand(H, t1 - t0).contiguous()
-        else:
-            flat1 = torch.arange(L, device=device, dtype=torch.int32)
-            cnt = torch.full((H, 1), L, dtype=torch.int32, device=device)
-        flat = flat1.repeat(H)
+        P = _PREFIX_BLOCK
+        off = L - S
+        j = torch.arange(L, device=device)
+        first = torch.arange(t0, t1, P, device=device)                                       # a block's first token
+        lim_b = (first + off + 1).clamp(min=0, max=L)                                        # keys seen by it
+        flat_b = j.expand(first.numel(), L)[j[None, :] < lim_b[:, None]].to(torch.int32)     # row-major (block, key)
+        cnt_b = lim_b.to(torch.int32).unsqueeze(0).expand(H, first.numel()).contiguous()
+        t = torch.arange(t0, t1, device=device)
+        lo = ((t - t0) // P * P + t0 + off + 1).clamp(min=0, max=L)                          # first key not in the block's list
+        hi = (t + off + 1).clamp(min=0, max=L)
+        w = torch.arange(P, device=device)
+        keys_d = lo[:, None] + w[None, :]
+        flat_d = keys_d[keys_d < hi[:, None]].to(torch.int32)
+        cnt_d = (hi - lo).clamp(min=0).to(torch.int32).unsqueeze(0).expand(H, t.numel()).contiguous()
         _prefix_lists.clear()                                                                # one shape at a time
-        _prefix_lists[key] = (flat, cnt)
+        _prefix_lists[key] = (flat_b.repeat(H), cnt_b, flat_d.repeat(H), cnt_d)
     return _prefix_lists[key]
 
 
@@ -168,17 +176,17 @@ def local_attention_backward(d_out, q, k, v, out, lse, sm_scale: float, causal: 
     [H*G,S,d]``, ``k, v [H,L,d]``, ``lse [H*G,S]``; ``out`` / ``lse`` may be the merged result.  Returns
     ``(dq [H*G,S,d], dk, dv [H,L,d] fp32)``.
 
-    The causal prefix of every token is a list of keys, so this is the backward of the gathered attention
-    with one bucket per token (shared by the G query heads of a KV head): no kernel of its own.  The lists
-    hold S (L - S/2) entries per KV head, so the tokens are taken in chunks that keep a call's lists below
-    2^24 entries per head (one call up to S = L = 4096); dk and dv add up over the calls.
+    No kernel of its own: given ``out`` and ``lse`` the backward is a sum over keys, so the causal case is two
+    backwards of the gathered attention whose key sets partition every token's prefix.  In the first, blocks of
+    8 tokens (with all their G query heads: 8 G queries) share a bucket that lists the keys all of them see; in
+    the second every token has a bucket of its own with the up to 7 keys left.  The lists of the first hold
+    S L / 16 entries per KV head at S = L (one sixteenth of a list per token), taken in token chunks that keep a
+    call below 2^24 entries per head; dk and dv add up over the calls, dq is the sum of the two parts (each
+    rounded to q's dtype, added in fp32).  Without the causal mask one bucket lists all keys.
 
     ``staged`` is passed on to :func:`attention_hash_varlen_backward`: ``None`` (the default) takes the form
-    without atomics for bf16 with d = 128 (every bucket here receives queries; results do not depend on
-    scheduling) and the atomic adds otherwise or when its workspace does not fit.  Cost at H = 8, G = 8,
-    S = L = 4096, d = 128 bf16 on MI355X: 22 ms and 25 GiB of workspace (268 MB of lists, 34 GB of partial
-    rows taken a few KV heads at a time) staged, 51 ms and 0.7 GiB with atomic adds -- several times what a
-    kernel written for the dense causal case would take, which this library does not have."""
+    without atomics for bf16 with d = 128 where a call has at least as many queries as buckets (results do not
+    depend on scheduling) and the atomic adds otherwise or when its workspace does not fit."""
     HG, S, d = q.shape
     H, L, _ = k.shape
     G = HG // H
@@ -186,20 +194,36 @@ def local_attention_backward(d_out, q, k, v, out, lse, sm_scale: float, causal: 
     q4, do4 = q.reshape(H, G, S, d), d_out.reshape(H, G, S, d)
     o4, l4 = out.reshape(H, G, S, d), lse.reshape(H, G, S)
     k, v = k.contiguous(), v.contiguous()
-    T = S if not causal else max(64, min(S, _PREFIX_CHUNK_ENTRIES // max(L, 1)))
+    if not causal:
+        flat = torch.arange(L, device=dev, dtype=torch.int32).repeat(H)
+        cnt = torch.full((H, 1), L, dtype=torch.int32, device=dev)
+        qh = torch.zeros(H, G * S, dtype=torch.int32, device=dev)
+        flat3 = lambda x: x.reshape(H, G * S, *x.shape[3:]).contiguous()
+        dq, dk, dv = attention_hash_varlen_backward(flat3(do4), flat3(q4), k, v, flat3(o4).to(q.dtype), flat3(l4).float(),
+                                                    flat, cnt, qh, sm_scale, staged=staged)
+        return dq.reshape(HG, S, d), dk, dv
+    P = _PREFIX_BLOCK
+    T = max(64, min(S, _PREFIX_CHUNK_ENTRIES * P // max(L, 1))) // P * P        # tokens per chunk, whole blocks
     dq = torch.empty((H, G, S, d), dtype=q.dtype, device=dev)
     dk = dv = None
     for t0 in range(0, S, T):
         t1 = min(S, t0 + T)
         n = t1 - t0
-        flat, cnt = _causal_prefix_lists(H, t0, t1, S, L, causal, dev)
-        t = torch.arange(n, device=dev, dtype=torch.int32) if causal else torch.zeros(n, dtype=torch.int32, device=dev)
-        qh = t.repeat(H * G).reshape(H, G * n)                                                # query g*n + t -> t
+        flat_b, cnt_b, flat_d, cnt_d = _causal_prefix_lists(H, t0, t1, S, L, dev)
+        t = torch.arange(n, device=dev, dtype=torch.int32)
         sl = lambda x: x[:, :, t0:t1].reshape(H, G * n, *x.shape[3:]).contiguous()
-        dq_c, dk_c, dv_c = attention_hash_varlen_backward(
-            sl(do4), sl(q4), k, v, sl(o4).to(q.dtype), sl(l4).float(), flat, cnt, qh, sm_scale, staged=staged)
-        dq[:, :, t0:t1] = dq_c.reshape(H, G, n, d)
-        dk, dv = (dk_c, dv_c) if dk is None else (dk + dk_c, dv + dv_c)
+        args = (sl(do4), sl(q4), k, v, sl(o4).to(q.dtype), sl(l4).float())
+        dq_c = None
+        for flat, cnt, bucket_of in ((flat_b, cnt_b, t // P), (flat_d, cnt_d, t)):
+            if flat.numel() == 0:                                                   # a single token has no diagonal
+                continue
+            qh = bucket_of.repeat(H * G).reshape(H, G * n)                         # query g*n + t -> its bucket
+            dq_p, dk_p, dv_p = attention_hash_varlen_backward(*args, flat, cnt, qh, sm_scale, staged=staged)
+            dq_c = dq_p.float() if dq_c is None else dq_c + dq_p.float()
+            dk, dv = (dk_p, dv_p) if dk is None else (dk + dk_p, dv + dv_p)
+        dq[:, :, t0:t1] = 0 if dq_c is None else dq_c.to(q.dtype).reshape(H, G, n, d)
+    if dk is None:                                                                  # no token sees a key
+        dk, dv = (torch.zeros((H, L, d), dtype=torch.float32, device=dev) for _ in range(2))
     return dq.reshape(HG, S, d), dk, dv
 
 

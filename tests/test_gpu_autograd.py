@@ -158,7 +158,8 @@ def test_module_backward_notices_a_memory_changed_in_place():
         out.sum().backward()
 
 
-@pytest.mark.parametrize("S,L,chunk_entries", [(40, 56, None), (200, 200, 64 * 200)])   # one call; token chunks of 64
+@pytest.mark.parametrize("S,L,chunk_entries", [(40, 56, None), (37, 61, None), (1, 9, None),   # one chunk; a last block of 5; decode
+                                               (200, 200, 8 * 200), (203, 230, 8 * 230)])   # token chunks of 64
 def test_local_attention_backward_bf16(S, L, chunk_entries, monkeypatch):
     from fast_memory_amd import autograd as fm_autograd, local_attention_backward, ops as _ops
     if chunk_entries:

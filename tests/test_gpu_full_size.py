@@ -264,7 +264,7 @@ def test_reference_harness_shape_kernels_agree(ops):
 
 def test_local_attention_backward_full_size(ops):
     """The backward of the dense causal local attention at the c5 shape (8 KV heads x 8 query heads, 4096
-    tokens, d = 128 bf16), which runs as a gathered backward with one bucket per token.  The reference calls
+    tokens, d = 128 bf16), which runs as two gathered backwards (blocks of 8 tokens, then single tokens).  The reference calls
     ``attention_backward`` (memory.py:368) without defining it, so parity with it is unpinned: the check is
     against autograd through the textbook definition in fp32, for KV head 0 and its eight query heads, and
     the form without atomics gives the same bits twice."""

@@ -660,12 +660,12 @@ __global__ __launch_bounds__(512) void fused_filter_wide_kernel(
 // A writer is a key split, so a row has n_splits segments; records carry the same key codes as above, the
 // selection does not see which form ran.
 constexpr int kFPDumpLd = 36;   // floats per lane in the dump: 32 accumulator registers + 4 (bank spread of the 16-byte stores)
-constexpr int kFPQueue = 448;   // queue places of a group's candidates (64 lanes x at most 7 rounds); lanes without one write behind it
+constexpr int kFPQueue = 448;   // queue places of a group's candidates (64 lanes x at most 7 rounds)
 
 struct FpShared {
   bf16_t keys[2][kFKeys * kFLd];
   float dump[kFWaves][64 * kFPDumpLd];
-  uint32_t queue[kFWaves][kFPQueue + 64];
+  uint32_t queue[kFWaves][kFPQueue];
   uint32_t cursor[kFWaves][128 + 64];  // a bucket's candidate count so far; lanes without a candidate add behind them
 };
 
@@ -697,10 +697,10 @@ __global__ __launch_bounds__(512) void fused_filter_ping_kernel(
 
   // staging: chunks tid and tid + 512 of a tile's 1024 16-byte chunks (rows tid/16 and 32 + tid/16)
   uint4 st0, st1;
-  auto fetch = [&](int i) {
+  auto fetch = [&](int i) {  // rows past the last key repeat it (no branch): the emission drops keys >= N
     const int64_t key0 = (int64_t(sk) + int64_t(i) * n_splits) * kFKeys + (tid >> 4);
-    st0 = key0 < N ? reinterpret_cast<const uint4*>(Kh + key0 * kFD)[tid & 15] : make_uint4(0, 0, 0, 0);
-    st1 = key0 + 32 < N ? reinterpret_cast<const uint4*>(Kh + (key0 + 32) * kFD)[tid & 15] : make_uint4(0, 0, 0, 0);
+    st0 = reinterpret_cast<const uint4*>(Kh + min(key0, int64_t(N) - 1) * kFD)[tid & 15];
+    st1 = reinterpret_cast<const uint4*>(Kh + min(key0 + 32, int64_t(N) - 1) * kFD)[tid & 15];
   };
   auto stash = [&](int buf) {
     *reinterpret_cast<uint4*>(&sm.keys[buf][(tid >> 4) * kFLd + (tid & 15) * 8]) = st0;
@@ -741,6 +741,8 @@ __global__ __launch_bounds__(512) void fused_filter_ping_kernel(
   uint4 af[2];      // A fragment of a k-step, [k-step parity]
   uint32_t msk = 0, msk0 = 0;
   int n_mine = 0, base = 0, base0 = 0, total = 0;
+  bool more = false;
+  uint32_t* my_queue = queue;
   // dense passes in flight: descriptor, value, bucket, slot of lane j's candidate
   uint32_t d_desc[ND], d_slot[ND];
   float d_val[ND];
@@ -775,13 +777,15 @@ __global__ __launch_bounds__(512) void fused_filter_ping_kernel(
         if constexpr (bt == 0) {
           if constexpr (ks < 3)
             af[(ks + 1) & 1] = *reinterpret_cast<const uint4*>(fp + (ks + 1) * 32);
-          else if (fp_next)
-            af[0] = *reinterpret_cast<const uint4*>(fp_next);
+          else
+            af[0] = *reinterpret_cast<const uint4*>(fp_next);  // always a readable address: a branch here would
+                                                                // make the waits behind it count a read that may not have been issued
         }
         acc[P][bt] = Mma<F16>::m16(af[ks & 1], bfrag[bt][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[P][bt]);
       }
       if constexpr (DO_EPI) {
         constexpr int Q = 1 - P;
+        constexpr int kTS = 8;  // slots of the threshold test
         if constexpr (S < 8) {
           // the four registers of bucket tile S: mask bit 31 - (4 bt + i)
           if constexpr (S == 0) msk = 0;
@@ -794,27 +798,25 @@ __global__ __launch_bounds__(512) void fused_filter_ping_kernel(
                        : "vcc");
           *reinterpret_cast<float4*>(&dump[l * kFPDumpLd + 4 * S]) =
               make_float4(acc[Q][S][0], acc[Q][S][1], acc[Q][S][2], acc[Q][S][3]);
-        } else if constexpr (S == 8) {
+        } else if constexpr (S == kTS) {
           msk0 = msk;
           n_mine = __popc(msk);
           base = wave_incl_scan_dpp(min(n_mine, NR));  // the queue takes a lane's first NR candidates
-        } else if constexpr (S == 9) {
+        } else if constexpr (S == kTS + 1) {
           total = __builtin_amdgcn_readlane(base, 63);
           base -= min(n_mine, NR);
           base0 = base;
-        } else if constexpr (S < 10 + NR) {
-          // a round: one candidate per lane to its place in the queue
-          // (a lane's places are below 64 NR; msk & (msk - 1) leaves an empty mask empty, and what a lane
-          // without a candidate writes behind the queue is read by nobody)
+          more = __ballot(n_mine > NR) != 0ull || total > ND * 64;  // candidates the rounds or the passes do not reach
+          my_queue = queue + base;
+        } else if constexpr (S < kTS + 2 + NR) {
+          // a round: one candidate per lane to its place in the queue (a lane's places are below 64 NR)
           static_assert(NR * 64 <= kFPQueue, "every lane's NR places are inside the queue");
-          const bool has = msk != 0u;
-          const uint32_t p = uint32_t(__ffs(int(msk)) - 1);
-          queue[has ? base : kFPQueue + l] = (uint32_t(l) << 5) | (p & 31u);
-          base += has ? 1 : 0;
-          msk &= msk - 1u;
+          constexpr int k = S - (kTS + 2);
+          if (msk != 0u) my_queue[k] = (uint32_t(l) << 5) | uint32_t(__builtin_ctz(msk));
+          msk &= msk - 1u;  // leaves an empty mask empty
         } else {
           // dense passes: three stages a pass, staggered by one slot from pass to pass
-          constexpr int S0 = 10 + NR + 1;  // first stage of pass 0 (a slot after the last round)
+          constexpr int S0 = kTS + 2 + NR + 1;  // first stage of pass 0 (a slot after the last round)
           constexpr int gap = (31 - S0 - (ND - 1)) / 2;  // as far apart as the step allows: each stage waits for LDS
           fp_static_for<ND>([&](auto D_) {
             constexpr int D = decltype(D_)::value;
@@ -846,21 +848,23 @@ __global__ __launch_bounds__(512) void fused_filter_ping_kernel(
       // rounds left in its mask: appended here, a lane a round (keys that cluster make this less rare than even
       // rates would: a bucket then takes most keys of a group).
       static_assert(ND * 64 <= kFPQueue, "the passes read what the queue holds");
-      while (__ballot(msk != 0u)) {
-        const bool has = msk != 0u;
-        const uint32_t e = 31u - uint32_t(__builtin_ctz(msk | 0x80000000u));
-        emit_one(has, uint32_t(l), e, dump[l * kFPDumpLd + e], key0_old);
-        msk = has ? (msk & (msk - 1u)) : msk;
-      }
-      // ... and the candidates whose place in the queue lies beyond the passes' ND * 64 (a group with more than
-      // that many candidates in all): the lanes that hold them go through their first NR again
-      if (total > ND * 64) {
-        uint32_t m = msk0;
-        for (int k = 0; k < NR; ++k) {
-          const bool has = m != 0u;
-          const uint32_t e = 31u - uint32_t(__builtin_ctz(m | 0x80000000u));
-          emit_one(has && base0 + k >= ND * 64, uint32_t(l), e, dump[l * kFPDumpLd + e], key0_old);
-          m = has ? (m & (m - 1u)) : m;
+      if (more) {
+        while (__ballot(msk != 0u)) {
+          const bool has = msk != 0u;
+          const uint32_t e = 31u - uint32_t(__builtin_ctz(msk | 0x80000000u));
+          emit_one(has, uint32_t(l), e, dump[l * kFPDumpLd + e], key0_old);
+          msk = has ? (msk & (msk - 1u)) : msk;
+        }
+        // ... and the candidates whose place in the queue lies beyond the passes' ND * 64 (a group with more than
+        // that many candidates in all): the lanes that hold them go through their first NR again
+        if (total > ND * 64) {
+          uint32_t m = msk0;
+          for (int k = 0; k < NR; ++k) {
+            const bool has = m != 0u;
+            const uint32_t e = 31u - uint32_t(__builtin_ctz(m | 0x80000000u));
+            emit_one(has && base0 + k >= ND * 64, uint32_t(l), e, dump[l * kFPDumpLd + e], key0_old);
+            m = has ? (m & (m - 1u)) : m;
+          }
         }
       }
     }
@@ -888,7 +892,7 @@ __global__ __launch_bounds__(512) void fused_filter_ping_kernel(
         group_step(B0{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 0), frag_ptr(buf, 1), key0_prev);
       group_step(B1{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 1), frag_ptr(buf, 2), kbase);
       group_step(B0{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 2), frag_ptr(buf, 3), kbase + 16u);
-      group_step(B1{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 3), nullptr, kbase + 32u);
+      group_step(B1{}, std::true_type{}, std::true_type{}, frag_ptr(buf, 3), frag_ptr(buf, 0), kbase + 32u);
       key0_prev = kbase + 48u;
     }
     __syncthreads();

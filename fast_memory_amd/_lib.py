@@ -73,6 +73,7 @@ SIGNATURES = {
     "fm_debug_hooks_enabled": (c_int, []),
     "fm_debug_force_generic": (None, [c_int]),
     "fm_hash_attn_fwd_kernel": (ctypes.c_char_p, [c_int] * 6),
+    "fm_local_attn_fwd_kernel": (ctypes.c_char_p, [c_int] * 5),
     "fm_hash_attn_fwd_launches": (c_int, [c_int] * 6),
     "fm_build_index_fused_kernel": (ctypes.c_char_p, [c_int] * 6),
     "fm_debug_argtopz_exact_only": (None, [c_int]),

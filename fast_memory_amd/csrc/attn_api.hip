@@ -24,7 +24,7 @@ int hash_attn_mfma_choice(int H, int Sq, int N, int C);
 bool hash_attn_mfma_per_row(int choice, int H, int Sq, int N, int C);
 bool local_attn_mfma_supported(int d, int dtype);
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
-                    int S, int L, int d, float sm_scale, int causal, hipStream_t st);
+                    int S, int L, int d, int dtype, float sm_scale, int causal, hipStream_t st);
 
 int launch_unlisted_rows(const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
                          const int32_t* bin_off, const int32_t* bin_count, int64_t n_bins, int64_t nq,
@@ -63,6 +63,15 @@ extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int 
     case 3: return "hash_attn_ring_kernel";
     default: return "hash_attn_mfma_kernel";
   }
+}
+
+extern "C" const char* fm_local_attn_fwd_kernel(int G, int S, int L, int d, int dtype) {
+  using namespace fm;
+  if (g_force_generic == 1 || !local_attn_mfma_supported(d, dtype)) return "local_attn_generic_kernel";
+  if (S == 1 && G <= 16 && L >= 1 && d == 128 && dtype == FM_BF16) return "local_attn_decode_kernel";
+  if (d == 64) return dtype == FM_F16 ? "local_attn_dense_kernel<f16, 64>" : "local_attn_dense_kernel<bf16, 64>";
+  if (d == 128) return dtype == FM_F16 ? "local_attn_dense_kernel<f16, 128>" : "local_attn_dense_kernel<bf16, 128>";
+  return dtype == FM_F16 ? "local_attn_dense_kernel<f16, 256>" : "local_attn_dense_kernel<bf16, 256>";
 }
 
 extern "C" int fm_hash_attn_fwd_launches(int H, int Sq, int N, int d, int C, int dtype) {
@@ -275,7 +284,7 @@ extern "C" int fm_local_attn_fwd(const void* q, const void* k, const void* v, vo
   FM_REQUIRE(S <= 65535 * 128, FM_ERR_UNSUPPORTED, "fm_local_attn_fwd: S=%d > 65535 * 128", S);
   hipStream_t st = as_stream(stream);
   if (g_force_generic != 1 && local_attn_mfma_supported(d, dtype))
-    return local_attn_mfma(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, st);
+    return local_attn_mfma(q, k, v, out, lse, H, G, S, L, d, dtype, sm_scale, causal, st);
   return local_attn_generic(q, k, v, out, lse, H, G, S, L, d, sm_scale, causal, dtype, st);
 }
 

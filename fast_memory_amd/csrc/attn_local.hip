@@ -1,4 +1,4 @@
-// Dense local attention for bf16, head dimension 128 (gfx950): the attention over
+// Dense local attention for bf16 / fp16, head dimensions 64, 128 and 256 (gfx950): the attention over
 // the most recent keys that the memory's output is merged with (call site
 // memory.py:302; the reference leaves `attention_forward` undefined, the contract
 // here is softmax(q.k^T * scale) v with a causal mask aligned bottom-right, output
@@ -8,7 +8,7 @@
 // per wave.  K and V tiles of 64 keys go global -> registers -> LDS, double buffered;
 // V is transposed on the way ( Vt[d][key] ) because both MFMA operands want the
 // contraction index contiguous per lane.
-//   S^T = K.Q^T    v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q^T fragments
+//   S^T = K.Q^T    v_mfma_f32_32x32x16_{bf16,f16}, A = K rows from LDS, B = Q^T fragments
 //                  resident in registers.  Lane (query l%32, half l/32) ends up with
 //                  the scores of keys 8*(r/4) + 4*(l/32) + r%4 of each 32-key block:
 //                  one query per lane column, so the softmax statistics are per-lane
@@ -19,49 +19,40 @@
 //                  with its key columns in that order, so neither P nor V is shuffled.
 // Softmax as in the gather kernel (triton_kernel.py:248-263): base 2 with
 // sm_scale*log2(e), fp32 running max and denominator, denominator from unrounded p,
-// p rounded to bf16 before P.V; the running maximum is followed lazily (see kLazy).
+// p rounded to the input type before P.V; the running maximum is followed lazily (see kLazy: p stays below
+// 2^8, far inside fp16).  Head dimension 256 runs one workgroup per CU (141 KB of LDS, 128 output registers).
 //
 // Roofline: MFMA (4*d flops per visible query-key pair); the per-element softmax
 // VALU work is of the same order as the MFMA time and does not overlap with it.
 #include "common.hpp"
+#include "mma16.hpp"
 
 namespace fm {
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
-typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 
-constexpr int kLD = 128;    // head dimension
 constexpr int kLQ = 128;    // queries per workgroup
 constexpr int kLK = 64;     // keys per tile
-constexpr int kLKld = 136;  // K tile row stride in LDS (elements)
 constexpr int kLVld = 72;   // Vt row stride in LDS (elements): 64 keys + 8
 constexpr float kLazy = 8.f;  // growth of a running maximum (in powers of two) that is left unfollowed
 
-__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
-  f32x2 x = {lo, hi};
-  bf16x2 y = __builtin_convertvector(x, bf16x2);  // v_cvt_pk_bf16_f32, round to nearest even
-  return *reinterpret_cast<uint32_t*>(&y);
-}
-
-__device__ __forceinline__ bf16x8 u4_as_bf16x8(uint4 u) {
-  union {
-    uint4 u;
-    bf16x8 b;
-  } x;
-  x.u = u;
-  return x.b;
-}
-
-struct LocalTileRegs {
-  uint4 k[4];  // K rows tid/16 + 16u, 16-byte chunk tid%16
-  uint4 v[4];  // V rows 4j..4j+3 (j = lane/4), chunk c = 4*wave + lane%4
-};
-
-__global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
+// F16: the 16-bit type is fp16 (else bf16); D: head dimension.  A row has CP = D / 8 16-byte chunks.  K: thread
+// tid takes chunk tid % CP of rows tid / CP + (256 / CP) u.  V: a unit is (chunk c, four consecutive keys 4j..4j+3),
+// 16 CP of them in a tile; unit u has c = u % 4 + 4 (u / 64), j = (u / 4) % 16 (four neighbouring lanes read 64
+// contiguous bytes), thread tid takes units tid + 256 i.
+template <bool F16, int D>
+__global__ __launch_bounds__(256, D == 256 ? 1 : 2) void local_attn_dense_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     bf16_t* __restrict__ out, float* __restrict__ lse, int G, int S, int L, float scale2, int causal) {
+  constexpr int kLD = D;
+  constexpr int kLKld = D + 8;            // K tile row stride in LDS (elements)
+  constexpr int CP = D / 8;               // 16-byte chunks of a row
+  constexpr int KU = kLK * CP / 256;      // K chunks per thread
+  constexpr int KR = 256 / CP;            // rows between a thread's K chunks
+  constexpr int VUNITS = 16 * CP;         // (chunk, four keys) units of a V tile
+  constexpr int VU = (VUNITS + 255) / 256;
+  constexpr int NKS = D / 16, NDT = D / 32;
+  using M = Mma<F16>;
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][kLK * kLKld];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][kLD * kLVld];
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
@@ -91,75 +82,96 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
   const int wave_lim_hi = lim_of(min(S - 1, wq0 + 31));  // most keys any query of the wave sees
   const int wave_lim_lo = (wq0 + 31 < S) ? lim_of(wq0) : 0;  // fewest
 
-  bf16x8 qf[8];
+  uint4 qf[NKS];
   {
     const uint4* pq = reinterpret_cast<const uint4*>(q + (qrow0 + (q_ok ? iq : 0)) * kLD + hb * 8);
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = u4_as_bf16x8(q_ok ? pq[2 * ks] : make_uint4(0, 0, 0, 0));
+    for (int ks = 0; ks < NKS; ++ks) qf[ks] = q_ok ? pq[2 * ks] : make_uint4(0, 0, 0, 0);
   }
   // The compiler's wait-count pass cannot see that these loads have landed by the time the loop starts (the path
   // that skips the first tile has no wait) and would otherwise wait, in front of every tile's first MFMA, for
   // all loads in flight: the next tile's, whose latency the double buffering is there to hide.  The empty
   // statements read the registers (the pass waits for the loads here, once) and count as their last writers.
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
-  f32x16 O[4];
+  for (int ks = 0; ks < NKS; ++ks)
+    asm volatile("" : "+v"(qf[ks].x), "+v"(qf[ks].y), "+v"(qf[ks].z), "+v"(qf[ks].w));
+  f32x16 O[NDT];
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
+  for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) O[dt][r] = 0.f;
   float m = -INFINITY, lsum = 0.f;
 
-  LocalTileRegs tr;
-  const int vj = l >> 2, vc = 4 * w + (l & 3);
-  const uint4* pk0 = reinterpret_cast<const uint4*>(Kh + int64_t(tid >> 4) * kLD) + (tid & 15);
-  const uint4* pv0 = reinterpret_cast<const uint4*>(Vh + int64_t(4 * vj) * kLD) + vc;
+  uint4 trk[KU];      // K rows tid / CP + KR u, chunk tid % CP
+  uint4 trv[VU][4];   // V unit tid + 256 i: rows 4j..4j+3, chunk c
+  const int krow = tid / CP, kch = tid % CP;
+  auto unit_c = [&](int i) { const int u = tid + 256 * i; return (u & 3) + 4 * (u >> 6); };
+  auto unit_j = [&](int i) { return ((tid + 256 * i) >> 2) & 15; };
+  auto unit_ok = [&](int i) { return VUNITS % 256 == 0 || tid + 256 * i < VUNITS; };
+  const uint4* pk0 = reinterpret_cast<const uint4*>(Kh + int64_t(krow) * kLD) + kch;
+  const uint4* pv0[VU];
+#pragma unroll
+  for (int i = 0; i < VU; ++i) pv0[i] = reinterpret_cast<const uint4*>(Vh + int64_t(4 * unit_j(i)) * kLD) + unit_c(i);
   auto load_tile = [&](int t) {
     const int kp0 = t * kLK;
     if (kp0 + kLK <= L) {  // a whole tile: no row of it lies past the keys
-      const uint4* pk = pk0 + int64_t(kp0) * (kLD / 8);
-      const uint4* pv = pv0 + int64_t(kp0) * (kLD / 8);
+      const uint4* pk = pk0 + int64_t(kp0) * CP;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) tr.k[u] = pk[16 * u * (kLD / 8)];
+      for (int u = 0; u < KU; ++u) trk[u] = pk[KR * u * CP];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) tr.v[kk] = pv[kk * (kLD / 8)];
+      for (int i = 0; i < VU; ++i) {
+        if (!unit_ok(i)) continue;
+        const uint4* pv = pv0[i] + int64_t(kp0) * CP;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) trv[i][kk] = pv[kk * CP];
+      }
       return;
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int row = kp0 + (tid >> 4) + 16 * u;
-      tr.k[u] = row < L ? reinterpret_cast<const uint4*>(Kh + int64_t(row) * kLD)[tid & 15] : make_uint4(0, 0, 0, 0);
+    for (int u = 0; u < KU; ++u) {
+      const int row = kp0 + krow + KR * u;
+      trk[u] = row < L ? reinterpret_cast<const uint4*>(Kh + int64_t(row) * kLD)[kch] : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int row = kp0 + 4 * vj + kk;
-      tr.v[kk] = row < L ? reinterpret_cast<const uint4*>(Vh + int64_t(row) * kLD)[vc] : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < VU; ++i) {
+      if (!unit_ok(i)) continue;
+      const int c = unit_c(i), j = unit_j(i);
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const int row = kp0 + 4 * j + kk;
+        trv[i][kk] = row < L ? reinterpret_cast<const uint4*>(Vh + int64_t(row) * kLD)[c] : make_uint4(0, 0, 0, 0);
+      }
     }
   };
   auto stash_tile = [&](int buf) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-      *reinterpret_cast<uint4*>(&sK[buf][((tid >> 4) + 16 * u) * kLKld + (tid & 15) * 8]) = tr.k[u];
+    for (int u = 0; u < KU; ++u)
+      *reinterpret_cast<uint4*>(&sK[buf][(krow + KR * u) * kLKld + kch * 8]) = trk[u];
     // keys 4j..4j+3 of the tile keep their order; the groups of four inside each 16 are
     // stored in the order 0, 2, 1, 3
-    const int a = vj >> 2, g4 = vj & 3;
-    const int pos0 = 16 * a + 4 * ((g4 & 1) * 2 + (g4 >> 1));
-    const uint32_t w0[4] = {tr.v[0].x, tr.v[0].y, tr.v[0].z, tr.v[0].w};
-    const uint32_t w1[4] = {tr.v[1].x, tr.v[1].y, tr.v[1].z, tr.v[1].w};
-    const uint32_t w2[4] = {tr.v[2].x, tr.v[2].y, tr.v[2].z, tr.v[2].w};
-    const uint32_t w3[4] = {tr.v[3].x, tr.v[3].y, tr.v[3].z, tr.v[3].w};
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int wi = e >> 1;
-      uint2 o;
-      if (e & 1) {
-        o.x = (w0[wi] >> 16) | (w1[wi] & 0xffff0000u);
-        o.y = (w2[wi] >> 16) | (w3[wi] & 0xffff0000u);
-      } else {
-        o.x = (w0[wi] & 0xffffu) | (w1[wi] << 16);
-        o.y = (w2[wi] & 0xffffu) | (w3[wi] << 16);
+    for (int i = 0; i < VU; ++i) {
+      if (!unit_ok(i)) continue;
+      const int vc = unit_c(i), vj = unit_j(i);
+      const int a = vj >> 2, g4 = vj & 3;
+      const int pos0 = 16 * a + 4 * ((g4 & 1) * 2 + (g4 >> 1));
+      const uint32_t w0[4] = {trv[i][0].x, trv[i][0].y, trv[i][0].z, trv[i][0].w};
+      const uint32_t w1[4] = {trv[i][1].x, trv[i][1].y, trv[i][1].z, trv[i][1].w};
+      const uint32_t w2[4] = {trv[i][2].x, trv[i][2].y, trv[i][2].z, trv[i][2].w};
+      const uint32_t w3[4] = {trv[i][3].x, trv[i][3].y, trv[i][3].z, trv[i][3].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int wi = e >> 1;
+        uint2 o;
+        if (e & 1) {
+          o.x = (w0[wi] >> 16) | (w1[wi] & 0xffff0000u);
+          o.y = (w2[wi] >> 16) | (w3[wi] & 0xffff0000u);
+        } else {
+          o.x = (w0[wi] & 0xffffu) | (w1[wi] << 16);
+          o.y = (w2[wi] & 0xffffu) | (w3[wi] << 16);
+        }
+        *reinterpret_cast<uint2*>(&sVt[buf][(8 * vc + e) * kLVld + pos0]) = o;
       }
-      *reinterpret_cast<uint2*>(&sVt[buf][(8 * vc + e) * kLVld + pos0]) = o;
     }
   };
 
@@ -176,11 +188,10 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
       const bf16_t* pa = &sK[buf][col * kLKld + hb * 8];
       // the two 32-key blocks in turn: neighbouring MFMAs do not wait for each other's sums
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
+      for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb)
-          s[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              *reinterpret_cast<const bf16x8*>(pa + sb * 32 * kLKld + ks * 16), qf[ks], s[sb], 0, 0, 0);
+          s[sb] = M::m32(*reinterpret_cast<const uint4*>(pa + sb * 32 * kLKld + ks * 16), qf[ks], s[sb]);
     }
     // ---- mask (only tiles that reach past what some query of the wave sees; the empty statement keeps the
     // compiler from turning the branch into per-lane selects that every tile would execute) ----
@@ -212,13 +223,13 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
       const float alpha = __builtin_amdgcn_exp2f(m - m_to);
       lsum *= alpha;
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
+      for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) O[dt][r] *= alpha;
       m = m_new;
     }
     const float m_sub = (m == -INFINITY) ? 0.f : m;  // a query that sees no key yet
-    bf16x8 pf[2][2];
+    uint4 pf[2][2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       float p[16];
@@ -229,8 +240,8 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
       }
 #pragma unroll
       for (int st = 0; st < 2; ++st)
-        pf[sb][st] = u4_as_bf16x8(make_uint4(cvt_pk_bf16(p[8 * st + 0], p[8 * st + 1]), cvt_pk_bf16(p[8 * st + 2], p[8 * st + 3]),
-                                             cvt_pk_bf16(p[8 * st + 4], p[8 * st + 5]), cvt_pk_bf16(p[8 * st + 6], p[8 * st + 7])));
+        pf[sb][st] = make_uint4(M::pack2(p[8 * st + 0], p[8 * st + 1]), M::pack2(p[8 * st + 2], p[8 * st + 3]),
+                                M::pack2(p[8 * st + 4], p[8 * st + 5]), M::pack2(p[8 * st + 6], p[8 * st + 7]));
     }
     // ---- O^T += Vt.P^T (the four 32-row blocks of the output in turn, for the same reason) ----
 #pragma unroll
@@ -238,10 +249,9 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
 #pragma unroll
       for (int st = 0; st < 2; ++st)
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
+        for (int dt = 0; dt < NDT; ++dt) {
           const bf16_t* pv = &sVt[buf][(dt * 32 + col) * kLVld + hb * 8];
-          O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(pv + sb * 32 + st * 16),
-                                                          pf[sb][st], O[dt], 0, 0, 0);
+          O[dt] = M::m32(*reinterpret_cast<const uint4*>(pv + sb * 32 + st * 16), pf[sb][st], O[dt]);
         }
   };
 
@@ -264,23 +274,40 @@ __global__ __launch_bounds__(256, 2) void local_attn_dense_kernel(
   if (q_ok) {
     bf16_t* po = out + (qrow0 + iq) * kLD;
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
         uint2 o;
-        o.x = cvt_pk_bf16(O[dt][4 * rq + 0] * inv, O[dt][4 * rq + 1] * inv);
-        o.y = cvt_pk_bf16(O[dt][4 * rq + 2] * inv, O[dt][4 * rq + 3] * inv);
+        o.x = M::pack2(O[dt][4 * rq + 0] * inv, O[dt][4 * rq + 1] * inv);
+        o.y = M::pack2(O[dt][4 * rq + 2] * inv, O[dt][4 * rq + 3] * inv);
         *reinterpret_cast<uint2*>(po + dt * 32 + 8 * rq + 4 * hb) = o;
       }
     if (hb == 0) lse[qrow0 + iq] = empty ? -FLT_MAX : (m + __builtin_amdgcn_logf(ltot)) * kLn2;
   }
 }
 
-int local_attn_dense(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G, int S,
-                     int L, float sm_scale, int causal, hipStream_t st) {
+template <bool F16, int D>
+static void launch_local_dense(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G, int S,
+                               int L, float sm_scale, int causal, hipStream_t st) {
   dim3 grid = dim3(unsigned(H * G), unsigned(ceil_div(S, kLQ)));
-  hipLaunchKernelGGL(local_attn_dense_kernel, grid, dim3(256), 0, st, (const bf16_t*)q, (const bf16_t*)k,
+  hipLaunchKernelGGL((local_attn_dense_kernel<F16, D>), grid, dim3(256), 0, st, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, (bf16_t*)out, lse, G, S, L, sm_scale * kLog2e, causal);
+}
+
+bool local_attn_dense_supported(int d, int dtype) {
+  return (d == 64 || d == 128 || d == 256) && (dtype == FM_BF16 || dtype == FM_F16);
+}
+
+int local_attn_dense(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G, int S,
+                     int L, int d, bool f16, float sm_scale, int causal, hipStream_t st) {
+#define FM_LOCAL_DENSE(F, DD) launch_local_dense<F, DD>(q, k, v, out, lse, H, G, S, L, sm_scale, causal, st)
+  if (d == 64)
+    f16 ? FM_LOCAL_DENSE(true, 64) : FM_LOCAL_DENSE(false, 64);
+  else if (d == 128)
+    f16 ? FM_LOCAL_DENSE(true, 128) : FM_LOCAL_DENSE(false, 128);
+  else
+    f16 ? FM_LOCAL_DENSE(true, 256) : FM_LOCAL_DENSE(false, 256);
+#undef FM_LOCAL_DENSE
   return launch_status("fm_local_attn_fwd(dense)");
 }
 

@@ -494,7 +494,8 @@ int decode_hash_attn(const void* q, const void* A_all, const void* K_all, const 
                      scores_out);
   return launch_status("fm_decode_hash_attn");
 }
-bool local_attn_mfma_supported(int d, int dtype) { return d == kD && dtype == FM_BF16; }
+bool local_attn_dense_supported(int d, int dtype);  // attn_local.hip
+bool local_attn_mfma_supported(int d, int dtype) { return local_attn_dense_supported(d, dtype); }
 
 int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int32_t* k_idx,
                           const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
@@ -586,13 +587,13 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
 }
 
 int local_attn_dense(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G, int S,
-                     int L, float sm_scale, int causal, hipStream_t st);
+                     int L, int d, bool f16, float sm_scale, int causal, hipStream_t st);
 
 int local_attn_mfma(const void* q, const void* k, const void* v, void* out, float* lse, int H, int G,
-                    int S, int L, int d, float sm_scale, int causal, hipStream_t st) {
-  (void)d;
-  if (S == 1 && G <= 16 && L >= 1) return local_attn_decode(q, k, v, out, lse, H, G, L, sm_scale, st);
-  return local_attn_dense(q, k, v, out, lse, H, G, S, L, sm_scale, causal, st);
+                    int S, int L, int d, int dtype, float sm_scale, int causal, hipStream_t st) {
+  if (S == 1 && G <= 16 && L >= 1 && d == kD && dtype == FM_BF16)
+    return local_attn_decode(q, k, v, out, lse, H, G, L, sm_scale, st);
+  return local_attn_dense(q, k, v, out, lse, H, G, S, L, d, dtype == FM_F16, sm_scale, causal, st);
 }
 
 }  // namespace fm

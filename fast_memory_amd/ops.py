@@ -595,6 +595,11 @@ def hash_attn_fwd_kernel_name(H: int, Sq: int, N: int, d: int, C: int, dtype: to
     return _lib.load().fm_hash_attn_fwd_kernel(H, Sq, N, d, C, _DT[dtype]).decode()
 
 
+def local_attn_fwd_kernel_name(G: int, S: int, L: int, d: int, dtype: torch.dtype) -> str:
+    """Name of the kernel :func:`local_attn_fwd` launches for these extents."""
+    return _lib.load().fm_local_attn_fwd_kernel(G, S, L, d, _DT[dtype]).decode()
+
+
 def hash_attn_fwd_launches(H: int, Sq: int, N: int, d: int, C: int, dtype: torch.dtype) -> int:
     """Number of launches of that kernel one :func:`hash_attn_fwd` call makes (one per row where a row's K
     and V outgrow the last-level cache)."""

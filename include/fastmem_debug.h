@@ -49,6 +49,12 @@ void fm_debug_force_generic(int on);
  * memories of more than 2^24 keys.  bench.py names its roofline kernel with it. */
 const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int C, int dtype);
 
+/* Diagnostic: name of the kernel fm_local_attn_fwd launches for these extents (a static
+ * string): "local_attn_dense_kernel<bf16|f16, 64|128|256>" (MFMA, a workgroup per 128
+ * queries of a head), "local_attn_decode_kernel" (bf16, d = 128, one query per head) or
+ * "local_attn_generic_kernel" (fp32 and other head dimensions). */
+const char* fm_local_attn_fwd_kernel(int G, int S, int L, int d, int dtype);
+
 /* Diagnostic: number of launches of that kernel one fm_hash_attn_fwd call makes for
  * these extents: 1, or H where the kernel goes out once per row (see above).  bench.py
  * divides its event time and the algorithmic bytes by it. */

@@ -103,6 +103,20 @@ def test_ops_refuse_cpu_tensors():
         ops.project(torch.zeros(1, 2, 8), torch.zeros(1, 4, 8))
 
 
+def test_local_attention_dispatch_rule():
+    # host-only: which kernel fm_local_attn_fwd would launch (G, S, L, d, dtype; FM_F32 = 0, FM_BF16 = 1, FM_F16 = 2)
+    lib = _lib.load()
+    name = lambda *a: lib.fm_local_attn_fwd_kernel(*a).decode()
+    assert name(8, 4096, 4096, 128, 1) == "local_attn_dense_kernel<bf16, 128>"
+    assert name(8, 4096, 4096, 128, 2) == "local_attn_dense_kernel<f16, 128>"
+    assert name(8, 4096, 4096, 64, 1) == "local_attn_dense_kernel<bf16, 64>"
+    assert name(8, 4096, 4096, 256, 2) == "local_attn_dense_kernel<f16, 256>"
+    assert name(8, 1, 4096, 128, 1) == "local_attn_decode_kernel"
+    assert name(8, 1, 4096, 128, 2) == "local_attn_dense_kernel<f16, 128>"
+    assert name(8, 4096, 4096, 96, 1) == "local_attn_generic_kernel"
+    assert name(8, 4096, 4096, 128, 0) == "local_attn_generic_kernel"
+
+
 def test_grouped_forward_dispatch_rule():
     # host-only: which kernel fm_hash_attn_fwd would launch (H, Sq, N, d, C, dtype)
     lib = _lib.load()

@@ -752,6 +752,20 @@ def test_lse_merge(ops):
     (torch.bfloat16, 1, 1, 260, 100, 128, True),        # more queries than keys: the first 160 see nothing
     (torch.bfloat16, 1, 1, 128, 64, 128, False),        # exactly one tile
     (torch.bfloat16, 2, 2, 129, 257, 128, True),
+    # the MFMA kernel's other types and head dimensions
+    (torch.float16, 2, 4, 200, 200, 128, True),
+    (torch.float16, 1, 2, 300, 1000, 128, True),
+    (torch.float16, 2, 4, 1, 512, 128, True),
+    (torch.bfloat16, 2, 2, 200, 200, 64, True),
+    (torch.bfloat16, 1, 2, 300, 1000, 64, True),
+    (torch.float16, 1, 2, 70, 130, 64, False),
+    (torch.float16, 1, 1, 260, 100, 64, True),
+    (torch.bfloat16, 1, 1, 1, 77, 64, True),
+    (torch.bfloat16, 2, 2, 200, 200, 256, True),
+    (torch.bfloat16, 1, 2, 300, 1000, 256, True),
+    (torch.float16, 1, 2, 70, 130, 256, False),
+    (torch.float16, 2, 2, 129, 257, 256, True),
+    (torch.float16, 1, 3, 1, 300, 256, True),
 ])
 def test_local_attention(ops, dtype, H, G, S, L, d, causal):
     g = gen(600)
@@ -761,6 +775,10 @@ def test_local_attention(ops, dtype, H, G, S, L, d, causal):
     out, lse = ops.local_attn_fwd(dev(q[0]), dev(k[0]), dev(v[0]), d ** -0.5, causal)
     ro, rl = O.local_attention(q, k, v, d ** -0.5, causal)
     assert_attn_close(out, lse, ro[0], rl[0], dtype, "local")
+    name = ops.local_attn_fwd_kernel_name(G, S, L, d, dtype)
+    mfma = dtype in (torch.bfloat16, torch.float16) and d in (64, 128, 256)
+    assert name.startswith("local_attn_dense_kernel") or name == "local_attn_decode_kernel" if mfma \
+        else name == "local_attn_generic_kernel", name
 
 
 def test_memory_plus_local_equals_joint_softmax(ops):

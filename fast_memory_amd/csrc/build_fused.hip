@@ -59,6 +59,20 @@ constexpr int kMaxRepair = 64;
 // builds of 16384 rows, and ~18 % more candidates than Z are kept at mu = 512 (six would keep 27 %).
 constexpr double kRankSigmas = 4.0;
 
+// Rank (from the top) of the sample value that serves as a row's threshold.  The share of a row's keys above
+// the sample's r-th largest value spreads around r / ns by sqrt(r) / ns, so the threshold keeps fewer than Z
+// keys (the row is then repaired) with the probability of (r - mu) / sqrt(r) standard deviations, mu = Z ns / N.
+// The rank is mu + 4 sqrt(mu) + 3, raised where that is not enough for the build's rows: with small mu the
+// 4 sqrt(mu) are fewer than 3.5 deviations of sqrt(r), and a build of many rows needs more of them to leave
+// the expected number of repaired rows at about four (64 can be repaired).
+static int threshold_rank(double mu, double rows) {
+  const double base = mu + kRankSigmas * sqrt(mu) + 3.0;
+  const double lp = 2.0 * log(std::max(rows, 64.0) / 4.0);                       // tail 4 / rows
+  const double z = std::min(6.0, std::max(3.0, sqrt(lp - log(lp) - 1.8379)));    // its normal quantile
+  const double need = mu + 0.5 * z * z + z * sqrt(mu + 0.25 * z * z);            // (r - mu) / sqrt(r) = z
+  return int(std::max(base, need));
+}
+
 constexpr int kCandRegs = 28;       // candidates a thread of the selection holds, 1024 threads per row
 constexpr int kCandRegsSmall = 32;  // ... with 256 or 512 threads per row
 
@@ -102,12 +116,12 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
     // long one with long lists the 16 K sample that keeps fewer candidates.
     double best = 0;
     int best_ns = 0, best_nt = 0;
-    for (int ns_try : {4096, 8192, 16384, 32768}) {
+    for (int ns_try : {4096, 8192, 16384, 32768, 65536, 131072}) {  // the last two for memories of millions of keys
       const int stride = N / ns_try;
       if (stride < 1) continue;
       const int ns = N / stride;
       const double mu = double(Z) * ns / N;
-      const int rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
+      const int rank = threshold_rank(mu, double(H) * C);
       if (rank * 4 > ns) continue;
       const double m = double(rank) * N / ns;
       const double per_w = m / p.n_writers;
@@ -129,7 +143,7 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
     p.stride = std::max(1, N / ns_take);
     p.ns = N / p.stride;
     const double mu = double(Z) * p.ns / N;
-    p.rank = int(mu + kRankSigmas * sqrt(mu) + 3.0);
+    p.rank = threshold_rank(mu, double(H) * C);
     if (p.rank * 4 > p.ns) return false;
     m_exp = double(p.rank) * N / p.ns;
     p.sel_threads = found ? best_nt : kSelThreads;
@@ -150,7 +164,14 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
     if (!p.ping) p.n_writers = 2 * p.n_splits;
   }
   if (!p.ping && !search()) return false;
-  p.cap_w = int(1.35 * m_exp / p.n_writers) + 64;  // > 16: the overflow guard keeps 16 slots free
+  // A writer's segment: its share of the expected candidates with room for five standard deviations (the
+  // threshold's noise, a relative 1 / sqrt(rank) of all of a row's candidates, plus the spread of a share);
+  // the overflow guard keeps 16 slots free.  With a small rank 1.35 times the share is less than that.
+  {
+    const double per_w = m_exp / p.n_writers;
+    const double sd_w = sqrt(pow(double(N) / p.ns * sqrt(double(p.rank)) / p.n_writers, 2) + per_w);
+    p.cap_w = int(std::max(1.35 * per_w + 64.0, per_w + 5.0 * sd_w + 16.0));
+  }
   p.ld_s = (int64_t(p.ns) + 3) / 4 * 4;
   p.ldy = (int64_t(N) + 3) / 4 * 4;
   size_t o = 0;

@@ -1362,6 +1362,20 @@ def test_fused_build_shapes(ops, H, C, N, Z):
     assert torch.equal(fused, unfused) and torch.equal(fv.view(torch.int32), uv.view(torch.int32))
 
 
+def test_fused_build_many_rows_with_short_lists(ops):
+    """32 768 rows whose thresholds come from few sample values (rank 61 of a 4096-key sample): a threshold
+    that spreads by a relative 1 / sqrt(rank) must neither overflow the candidate segments nor leave more rows
+    to repair than can be repaired -- the build stays on the fused path and gives the unfused lists."""
+    H, C, N, Z = 8, 4096, 262144, 2048
+    g = torch.Generator(device="cuda").manual_seed(915)
+    K = (torch.randn(H, N, 128, generator=g, device="cuda") * 0.6).to(torch.bfloat16)
+    A = torch.nn.functional.normalize(torch.randn(H, C, 128, generator=g, device="cuda"), dim=-1).to(torch.bfloat16)
+    fused = ops.build_index(A, K, Z, fused=True)
+    info = dict(ops.last_build_info)
+    assert info["path"] == "fused" and info["rows_unresolved"] == 0 and info["rows_repaired"] <= 24, info
+    assert torch.equal(fused, ops.build_index(A, K, Z, fused=False))
+
+
 @pytest.mark.parametrize("dtype,H,C,N,Z,runs", [
     (torch.bfloat16, 2, 1024, 65536 + 77, 1100, False),   # pass rate ~2 %: four rounds, one pass; a ragged key tile
     (torch.bfloat16, 1, 900, 131072, 6000, False),        # ~6 %: seven rounds, three passes; a partial last wave

@@ -102,7 +102,7 @@ bool hash_attn_bwd_mfma_supported(int d, int dtype);
 int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                        const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
                        int64_t max_items, const void* out, const float* lse, const void* dout, const float* dlse, void* dq,
-                       float* dk, float* dv, int Sq, int N, int C, float sm_scale, hipStream_t st);
+                       float* dk, float* dv, int Sq, int N, int C, float sm_scale, bool f16, hipStream_t st);
 
 int launch_unlisted_rows(const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
                          const int32_t* bin_off, const int32_t* bin_count, int64_t n_bins, int64_t nq,
@@ -131,7 +131,7 @@ extern "C" int fm_hash_attn_bwd(const void* q, const void* k, const void* v, con
   if (rc) return rc;
   if (g_force_generic != 1 && hash_attn_bwd_mfma_supported(d, dtype))
     return hash_attn_bwd_mfma(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse,
-                              dout, dlse, dq, dk, dv, Sq, N, C, sm_scale, st);
+                              dout, dlse, dq, dk, dv, Sq, N, C, sm_scale, dtype == FM_F16, st);
   if (dtype == FM_F32)
     hipLaunchKernelGGL(hash_attn_bwd_generic_kernel<float>, dim3(unsigned(max_items)), dim3(256), 0, st,
                        (const float*)q, (const float*)k, (const float*)v, k_idx, bucket_off, bucket_cnt, q_perm, items,

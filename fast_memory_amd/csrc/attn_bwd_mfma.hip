@@ -27,6 +27,7 @@
 
 #include "common.hpp"
 #include "attn_ring.hpp"
+#include "mma16.hpp"
 
 namespace fm {
 
@@ -123,7 +124,7 @@ __device__ __forceinline__ void bwd_load_block(BwdBlock& r, const bf16_t* __rest
 // (no registers in between), and the waves fill their operand registers from there.  The gather then runs
 // beside the arithmetic and the stores of the block before it.  blk: 32 KB, [block parity][K | V][32 rows of 256 B],
 // 16-byte chunk q of row r at position q ^ f(r) (no padding, no bank conflicts for either read pattern).
-template <bool STAGED, bool FIRST_TILE, int TILES = 1, bool LDSBLK = false>
+template <bool STAGED, bool FIRST_TILE, int TILES = 1, bool LDSBLK = false, bool F16 = false>
 __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ out,
                                          const float* __restrict__ lse, const bf16_t* __restrict__ dout,
                                          const float* __restrict__ dlse, const int32_t* __restrict__ q_list, int n_q, int64_t qbase,
@@ -133,6 +134,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
                                          bf16_t* dkp, bf16_t* dvp, bf16_t* dump, float* red, int* q_rows,
                                          bf16_t* stage, unsigned char* blk = nullptr) {
   static_assert(!LDSBLK || (STAGED && FIRST_TILE && TILES == 2), "the LDS block form is the first two-tile pass");
+  static_assert(!(F16 && STAGED), "the partial rows of the staged form are bf16: fp16 takes the atomic form");
+  using M = Mma<F16>;  // the 16-bit type of q, k, v, out, dout and dq (F16: fp16, else bf16)
   if (threadIdx.x < 16 * TILES) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_list[threadIdx.x] : -1;
   __syncthreads();
   const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -166,8 +169,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
       const uint32_t ow[4] = {o4.x, o4.y, o4.z, o4.w};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        Dc = fmaf(__uint_as_float(dw[e] << 16), __uint_as_float(ow[e] << 16), Dc);
-        Dc = fmaf(__uint_as_float(dw[e] & 0xffff0000u), __uint_as_float(ow[e] & 0xffff0000u), Dc);
+        Dc = fmaf(M::lo(dw[e]), M::lo(ow[e]), Dc);
+        Dc = fmaf(M::hi(dw[e]), M::hi(ow[e]), Dc);
       }
     }
   }
@@ -240,10 +243,10 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
       f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0, p0 = s0, p1 = s0;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_as_bf16x8(kv.k[0][s]), b_as_bf16x8(qf[s]), s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_as_bf16x8(kv.k[1][s]), b_as_bf16x8(qf[s]), s1, 0, 0, 0);
-        p0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_as_bf16x8(kv.vk[0][s]), b_as_bf16x8(dof[s]), p0, 0, 0, 0);
-        p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_as_bf16x8(kv.vk[1][s]), b_as_bf16x8(dof[s]), p1, 0, 0, 0);
+        s0 = M::m16(kv.k[0][s], qf[s], s0);
+        s1 = M::m16(kv.k[1][s], qf[s], s1);
+        p0 = M::m16(kv.vk[0][s], dof[s], p0);
+        p1 = M::m16(kv.vk[1][s], dof[s], p1);
       }
       float ds[8];
 #pragma unroll
@@ -253,10 +256,10 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
         ds[r] = pa * (p0[r] - Dc) * sm_scale;
         ds[4 + r] = pb * (p1[r] - Dc) * sm_scale;
       }
-      const uint4 pf = make_uint4(b_pack(ds[0], ds[1]), b_pack(ds[2], ds[3]), b_pack(ds[4], ds[5]), b_pack(ds[6], ds[7]));
+      const uint4 pf = make_uint4(M::pack2(ds[0], ds[1]), M::pack2(ds[2], ds[3]), M::pack2(ds[4], ds[5]), M::pack2(ds[6], ds[7]));
 #pragma unroll
       for (int t = 0; t < 8; ++t)
-        dQ[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_as_bf16x8(kf[t]), b_as_bf16x8(pf), dQ[t], 0, 0, 0);
+        dQ[t] = M::m16(kf[t], pf, dQ[t]);
     }
     // ---- queries on rows: S, dP -> P, dS -> dV, dK tiles, added to the keys' rows ----
 #pragma unroll
@@ -264,8 +267,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
       f32x4 sN = {0.f, 0.f, 0.f, 0.f}, pN = sN;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        sN = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_as_bf16x8(qf[s]), b_as_bf16x8(kv.k[kt][s]), sN, 0, 0, 0);
-        pN = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_as_bf16x8(dof[s]), b_as_bf16x8(kv.vk[kt][s]), pN, 0, 0, 0);
+        sN = M::m16(qf[s], kv.k[kt][s], sN);
+        pN = M::m16(dof[s], kv.vk[kt][s], pN);
       }
       const bool key_ok = kp0 + 16 * kt + c < cnt;
       float pr[4], dsr[4];
@@ -277,8 +280,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
       // P and dS as the A operand (lane (g,c): row = key c, contraction = queries 4g..4g+3), dO^T and
       // Q^T fragments as B: the output tile has keys on rows and d on columns, so that one atomic
       // instruction covers, per lane group, 16 consecutive floats (a 64-byte line) of one key's row
-      const bf16x4s pA = b_as_bf16x4(make_uint2(b_pack(pr[0], pr[1]), b_pack(pr[2], pr[3])));
-      const bf16x4s dsA = b_as_bf16x4(make_uint2(b_pack(dsr[0], dsr[1]), b_pack(dsr[2], dsr[3])));
+      const uint2 pA = make_uint2(M::pack2(pr[0], pr[1]), M::pack2(pr[2], pr[3]));
+      const uint2 dsA = make_uint2(M::pack2(dsr[0], dsr[1]), M::pack2(dsr[2], dsr[3]));
       if (STAGED) {
         // The transposed tiles (the same registers with the operands swapped): lane (g,c) holds key c and
         // the four consecutive columns 16t + 4g .. +3.  They go through a slab of LDS private to the wave
@@ -288,8 +291,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
           const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-          const f32x4 tv = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(b_as_bf16x4(doT[t]), pA, z, 0, 0, 0);
-          const f32x4 tk = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(b_as_bf16x4(qT[t]), dsA, z, 0, 0, 0);
+          const f32x4 tv = M::m16k16(doT[t], pA, z);
+          const f32x4 tk = M::m16k16(qT[t], dsA, z);
           *reinterpret_cast<uint2*>(slab + c * kStLd + 16 * t + 4 * g) =
               make_uint2(b_pack(tv[0], tv[1]), b_pack(tv[2], tv[3]));
           *reinterpret_cast<uint2*>(slab + (16 + c) * kStLd + 16 * t + 4 * g) =
@@ -365,8 +368,8 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
           const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-          const f32x4 tv = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pA, b_as_bf16x4(doT[t]), z, 0, 0, 0);
-          const f32x4 tk = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(dsA, b_as_bf16x4(qT[t]), z, 0, 0, 0);
+          const f32x4 tv = M::m16k16(pA, doT[t], z);
+          const f32x4 tk = M::m16k16(dsA, qT[t], z);
 #pragma unroll
           for (int r = 0; r < 4; ++r)
             if (rok[r]) {
@@ -505,7 +508,7 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
       for (int t = 0; t < 8; ++t) o[t] = red[((w * 8 + t) * 4 + r) * 64 + l];
       if (myq >= 0)
         *reinterpret_cast<uint4*>(dq + (qbase + myq) * kBD + 32 * g + 8 * r) =
-            make_uint4(b_pack(o[0], o[1]), b_pack(o[2], o[3]), b_pack(o[4], o[5]), b_pack(o[6], o[7]));
+            make_uint4(M::pack2(o[0], o[1]), M::pack2(o[2], o[3]), M::pack2(o[4], o[5]), M::pack2(o[6], o[7]));
     }
     return;
   }
@@ -520,7 +523,7 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
         o[t] = red[(((2 * tw) * 8 + t) * 4 + r) * 64 + l] + red[(((2 * tw + 1) * 8 + t) * 4 + r) * 64 + l];
       if (myq >= 0)
         *reinterpret_cast<uint4*>(dq + (qbase + myq) * kBD + 32 * g + 8 * r) =
-            make_uint4(b_pack(o[0], o[1]), b_pack(o[2], o[3]), b_pack(o[4], o[5]), b_pack(o[6], o[7]));
+            make_uint4(M::pack2(o[0], o[1]), M::pack2(o[2], o[3]), M::pack2(o[4], o[5]), M::pack2(o[6], o[7]));
     }
     return;
   }
@@ -535,10 +538,12 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
   }
   if (myq >= 0)
     *reinterpret_cast<uint4*>(dq + (qbase + myq) * kBD + 32 * g + 8 * w) =
-        make_uint4(b_pack(o[0], o[1]), b_pack(o[2], o[3]), b_pack(o[4], o[5]), b_pack(o[6], o[7]));
+        make_uint4(M::pack2(o[0], o[1]), M::pack2(o[2], o[3]), M::pack2(o[4], o[5]), M::pack2(o[6], o[7]));
 }
 
 // grid (items, FM_QTILE / 16): one workgroup per (work item, 16-query tile); dK, dV by atomic adds.
+// F16: q, k, v, out, dout and dq are fp16 (else bf16).
+template <bool F16>
 __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
@@ -552,7 +557,7 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_mfma_kernel(
   const int q0 = int(blockIdx.y) * 16;  // this workgroup's query tile inside the item
   if (q0 >= it.n_q) return;
   const int64_t bkt = int64_t(it.row) * C + it.bucket;
-  bwd_tile<false, true>(q, out, lse, dout, dlse, q_perm + it.q_start + q0, min(16, it.n_q - q0), int64_t(it.row) * Sq,
+  bwd_tile<false, true, 1, false, F16>(q, out, lse, dout, dlse, q_perm + it.q_start + q0, min(16, it.n_q - q0), int64_t(it.row) * Sq,
                   k + int64_t(it.row) * N * kBD, v + int64_t(it.row) * N * kBD, k_idx + bucket_off[bkt],
                   bucket_cnt[bkt], N, sm_scale, dq, dk + int64_t(it.row) * N * kBD, dv + int64_t(it.row) * N * kBD,
                   nullptr, nullptr, nullptr, red, q_rows, nullptr);
@@ -663,16 +668,21 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_excess_kernel(
   }
 }
 
-bool hash_attn_bwd_mfma_supported(int d, int dtype) { return d == kBD && dtype == FM_BF16; }
+bool hash_attn_bwd_mfma_supported(int d, int dtype) { return d == kBD && (dtype == FM_BF16 || dtype == FM_F16); }
 
 int hash_attn_bwd_mfma(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                        const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items, const int32_t* n_items,
                        int64_t max_items, const void* out, const float* lse, const void* dout, const float* dlse, void* dq,
-                       float* dk, float* dv, int Sq, int N, int C, float sm_scale, hipStream_t st) {
+                       float* dk, float* dv, int Sq, int N, int C, float sm_scale, bool f16, hipStream_t st) {
   dim3 grid = dim3(unsigned(max_items), unsigned(FM_QTILE / 16));
-  hipLaunchKernelGGL(hash_attn_bwd_mfma_kernel, grid, dim3(256), 0, st, (const bf16_t*)q, (const bf16_t*)k,
-                     (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, (const bf16_t*)out, lse,
-                     (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, Sq, N, C, sm_scale);
+  if (f16)
+    hipLaunchKernelGGL(hash_attn_bwd_mfma_kernel<true>, grid, dim3(256), 0, st, (const bf16_t*)q, (const bf16_t*)k,
+                       (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, (const bf16_t*)out, lse,
+                       (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, Sq, N, C, sm_scale);
+  else
+    hipLaunchKernelGGL(hash_attn_bwd_mfma_kernel<false>, grid, dim3(256), 0, st, (const bf16_t*)q, (const bf16_t*)k,
+                       (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, (const bf16_t*)out, lse,
+                       (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, Sq, N, C, sm_scale);
   return launch_status("fm_hash_attn_bwd(mfma)");
 }
 

@@ -31,6 +31,28 @@ struct Mma {
     else
       return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(b8, a), __builtin_bit_cast(b8, b), c, 0, 0, 0);
   }
+  // v_mfma_f32_16x16x16_{bf16_1k,f16}: four elements per operand
+  __device__ static __forceinline__ f4 m16k16(uint2 a, uint2 b, f4 c) {
+    typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s4;
+    typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 h4;
+    if constexpr (F16)
+      return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a), __builtin_bit_cast(h4, b), c, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s4, a), __builtin_bit_cast(s4, b), c, 0, 0, 0);
+  }
+  // the two elements of a packed word as floats
+  __device__ static __forceinline__ float lo(uint32_t w) {
+    if constexpr (F16)
+      return float(__builtin_bit_cast(_Float16, uint16_t(w & 0xffffu)));
+    else
+      return __uint_as_float(w << 16);
+  }
+  __device__ static __forceinline__ float hi(uint32_t w) {
+    if constexpr (F16)
+      return float(__builtin_bit_cast(_Float16, uint16_t(w >> 16)));
+    else
+      return __uint_as_float(w & 0xffff0000u);
+  }
   // two floats rounded to nearest even and packed (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32)
   __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
     f2 x = {lo, hi};

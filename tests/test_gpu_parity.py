@@ -978,6 +978,9 @@ def _assert_grad_close(got, ref, dtype, what):
     (torch.float32, 1, 24, 1024, 8, 16, 16),             # the reference's small test shape (tk:500)
     (torch.bfloat16, 2, 200, 2000, 12, 150, 128),
     (torch.bfloat16, 1, 130, 700, 3, 333, 128),          # more than 64 queries per bucket: several items
+    (torch.float16, 2, 200, 2000, 12, 150, 128),         # fp16 on the MFMA kernel
+    (torch.float16, 1, 130, 700, 3, 333, 128),
+    (torch.float16, 2, 70, 300, 6, 40, 64),              # fp16 on the generic kernel
 ])
 def test_hash_attention_backward(ops, dtype, B, S, N, C, Z, d):
     from fast_memory_amd import attention_hash_varlen, attention_hash_varlen_backward
@@ -999,11 +1002,12 @@ def test_hash_attention_backward(ops, dtype, B, S, N, C, Z, d):
     assert (dq.float().cpu()[empty] == 0).all()
 
 
-def test_backward_mfma_and_generic_agree(ops):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_backward_mfma_and_generic_agree(ops, dtype):
     from fast_memory_amd import attention_hash_varlen, attention_hash_varlen_backward
-    q, k, v, kh, cnt, qh = make_attn_case(1500, 2, 300, 3000, 9, 500, 128, torch.bfloat16, window="ref", std=0.7)
+    q, k, v, kh, cnt, qh = make_attn_case(1500, 2, 300, 3000, 9, 500, 128, dtype, window="ref", std=0.7)
     qh[0, :150] = 2                                             # a bucket with several 16-query tiles and items
-    dout = (torch.randn(2, 300, 128, generator=gen(1501)) * 0.5).to(torch.bfloat16)
+    dout = (torch.randn(2, 300, 128, generator=gen(1501)) * 0.5).to(dtype)
     args = dev(q, k, v, kh, cnt, qh)
     out, lse = attention_hash_varlen(*args, 128 ** -0.5)
     call = lambda: attention_hash_varlen_backward(dev(dout), args[0], args[1], args[2], out, lse, args[3], args[4],

@@ -307,9 +307,10 @@ __device__ __forceinline__ void collect_sort_write(Source& src, uint64_t cut, in
 // Returns false, with nothing written, when a bin is longer than kSelMaxBin (many equal or nearly equal
 // values): the caller then takes the radix select and the sorting network.
 // (Measured at 16384-entry lists, 16384 rows: 8192 bins instead of 4096 and four bin members fetched per
-// round of the counting loop take the selection from 2.55 to 2.32 ms; the counting loop is bound by the bank
-// conflicts of its scattered 8-byte LDS reads.  A second level of bins that splits the dense ones into
-// sub-bins of about 8 members costs more in its extra passes, 0.4 ms, than it saves.)
+// round of the counting loop take the selection from 2.55 to 2.32 ms; rounds that read past the end of their
+// bin without clamping or masking -- what lies there compares as smaller -- to 1.88 ms, of which the counting
+// loop is 0.55 ms, the read of the candidates 0.63 ms.  A second level of bins that splits the dense ones
+// into sub-bins of about 8 members costs more in its extra passes, 0.4 ms, than it saves.)
 constexpr int kSelBinBits = 13;
 constexpr int kSelBins = 1 << kSelBinBits;
 constexpr int kSelMaxBin = 256;
@@ -400,11 +401,12 @@ __device__ __forceinline__ bool binned_select_write(Source& src, int Zc, uint64_
         pack = uint32_t(running);
       running += h[j];
     }
-    if (longest > kSelMaxBin) atomicMax(&bs.max_bin, longest);
+    if (longest > kSelMaxBin - 4) atomicMax(&bs.max_bin, longest);  // (four places stay free behind the kept ones)
   }
   __syncthreads();
   const int cut_bin = bs.cut_bin, n_keep = bs.n_keep;
-  if (cut_bin < 0 || bs.max_bin > kSelMaxBin) return false;  // fewer than Zc candidates, or a long bin
+  if (cut_bin < 0 || bs.max_bin > kSelMaxBin - 4) return false;  // fewer than Zc candidates, or a long bin
+  if (tid < 4) buf[n_keep + tid] = 0;  // smaller than any composite: what a rank round reads past the last bin
   src([&](float y, uint32_t i) {
     const int d = dbin(float_key(y));
     if (d <= cut_bin) {
@@ -421,15 +423,15 @@ __device__ __forceinline__ bool binned_select_write(Source& src, int Zc, uint64_
     const int s0 = d ? half_of(d - 1) : 0, e0 = half_of(d);
     int rank = s0;
     // rank += (c < o) for the bin's members o: the borrow of the 64-bit subtraction c - o, two full-rate
-    // instructions.  Four members per round, fetched before the first is used.  (A round's reads past the
-    // bin's end are clamped to its last member and counted as c itself, for which c < c is false.)
+    // instructions.  Four members per round, fetched before the first is used.  A round's reads past the
+    // bin's end need no mask: what follows in the buffer are the members of the bins after it, all smaller
+    // than c, and behind the last bin four zeros.
     for (int q = s0; q < e0; q += 4) {
       uint64_t o[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = buf[min(q + i, e0 - 1)];
+      for (int i = 0; i < 4; ++i) o[i] = buf[q + i];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        if (q + i >= e0) o[i] = c;
         uint32_t t;
         asm("v_sub_co_u32 %0, vcc, %2, %4\n\t"
             "v_subb_co_u32 %0, vcc, %3, %5, vcc\n\t"

@@ -45,6 +45,16 @@ def ev_pair():
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
 
+def settle(fn, seconds=0.25):
+    """Runs fn() for a quarter of a second before the warm-up steps.  The first process on a fresh machine has
+    been seen to stall once, for some 40 ms, within its first launches of a kernel sequence; in a configuration
+    whose step takes 0.1 ms that one stall, landing inside the timed steps, was most of their time."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        fn()
+        torch.cuda.synchronize()
+
+
 def timed(fn, reps=1, warm=1):
     """Average milliseconds of fn() over `reps` runs, HIP events on the current stream."""
     for _ in range(warm):
@@ -362,6 +372,7 @@ def bench_decode_batch(args):
             evs.append((a, b))
         return out, lse, h
 
+    settle(lambda: step(False))
     for _ in range(args.warmup):
         step(False)
     torch.cuda.synchronize()
@@ -483,6 +494,7 @@ def bench_reference_harness(args):
     attn_ms, (mo, ml) = timed(lambda: ops.hash_attn_fwd(q, k, v, flat, off, cnt, groups, sm_scale), reps=5, warm=2)
 
     step = lambda: attention_hash(q, k, v, centroids, Z, sm_scale)
+    settle(step)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -701,6 +713,7 @@ def main():
                 part_events["merge"].append((l1, m1))
         return out, lse, qh, groups, mo, ml
 
+    settle(lambda: step(record=False))
     for _ in range(args.warmup):
         step(record=False)
     torch.cuda.synchronize()

@@ -24,6 +24,21 @@ def _p(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
+_no_entries = {}
+
+
+def _pl(k_idx: torch.Tensor):
+    """Pointer to flat bucket lists.  Lists without a single entry (every count zero: all buckets empty, e.g.
+    behind a window that no key passes) are an empty tensor, whose data pointer is null, which the library
+    refuses; it reads no entry of such lists, so any valid address serves."""
+    if k_idx.numel() > 0:
+        return k_idx.data_ptr()
+    dev_key = (k_idx.device.type, k_idx.device.index)
+    if dev_key not in _no_entries:
+        _no_entries[dev_key] = torch.zeros(4, dtype=torch.int32, device=k_idx.device)
+    return _no_entries[dev_key].data_ptr()
+
+
 def _stream(t: torch.Tensor):
     return torch.cuda.current_stream(t.device).cuda_stream
 
@@ -268,7 +283,7 @@ def hash_attn_fwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, s
     lse = torch.empty((H, Sq), dtype=torch.float32, device=q.device)
     lib = _lib.load()
     ws = torch.empty(int(lib.fm_hash_attn_fwd_workspace(groups.max_items)), dtype=torch.uint8, device=q.device)
-    check(lib.fm_hash_attn_fwd_ws(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
+    check(lib.fm_hash_attn_fwd_ws(_p(q), _p(k), _p(v), _pl(k_idx), _p(bucket_off), _p(bucket_cnt),
                                   _p(groups.q_perm), _p(groups.items), _p(groups.n_items),
                                   groups.max_items, _p(out), _p(lse), H, Sq, N, d, C,
                                   float(sm_scale), _dt(q), _p(ws), ws.numel(), _stream(q)))
@@ -287,7 +302,7 @@ def lists_key_order(k_idx, bucket_off, bucket_cnt, N: int, return_unsorted: bool
     assert bucket_off.numel() == bucket_cnt.numel()
     out = torch.empty_like(k_idx)
     n_uns = torch.empty(1, dtype=torch.int32, device=k_idx.device) if return_unsorted else None
-    check(_lib.load().fm_lists_key_order(_p(k_idx), _p(bucket_off), _p(bucket_cnt), bucket_cnt.numel(), int(N),
+    check(_lib.load().fm_lists_key_order(_pl(k_idx), _p(bucket_off), _p(bucket_cnt), bucket_cnt.numel(), int(N),
                                          _p(out), _p(n_uns) if n_uns is not None else None, _stream(k_idx)))
     return (out, n_uns) if return_unsorted else out
 
@@ -313,7 +328,7 @@ def hash_attn_bwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, o
     if dv is None:
         dv = torch.zeros((H, N, d), dtype=torch.float32, device=q.device)
     assert dk.dtype == dv.dtype == torch.float32 and dk.shape == dv.shape == (H, N, d)
-    check(_lib.load().fm_hash_attn_bwd(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
+    check(_lib.load().fm_hash_attn_bwd(_p(q), _p(k), _p(v), _pl(k_idx), _p(bucket_off), _p(bucket_cnt),
                                        _p(groups.q_perm), _p(groups.items), _p(groups.n_items), groups.max_items,
                                        _p(out), _p(lse), _p(dout), _p(dlse), _p(dq), _p(dk), _p(dv), H, Sq, N, d, C,
                                        float(sm_scale), _dt(q), _stream(q)))
@@ -408,7 +423,7 @@ def hash_attn_bwd_staged(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGr
     need_all = lib.fm_hash_attn_bwd_staged_workspace(total)
     ws = _ws(min(need_all, max(int(workspace_bytes), lib.fm_hash_attn_bwd_staged_workspace(longest))), q)
     row_pos = (ctypes.c_int64 * (H + 1))(*inv.row_pos)
-    check(lib.fm_hash_attn_bwd_staged(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_off), _p(bucket_cnt),
+    check(lib.fm_hash_attn_bwd_staged(_p(q), _p(k), _p(v), _pl(k_idx), _p(bucket_off), _p(bucket_cnt),
                                       _p(groups.q_perm), _p(groups.bin_off), _p(groups.bin_count), _p(out), _p(lse),
                                       _p(dout), _p(dlse), _p(inv.key_off), _p(inv.inv_pos), _p(dq), _p(dk),
                                       _p(dv), H, Sq, N, d, C, ctypes.cast(row_pos, ctypes.c_void_p), float(sm_scale),
@@ -427,7 +442,7 @@ def attention_hash_varlen_i32(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: floa
     ws = _ws(lib.fm_attention_hash_varlen_workspace(H, C, Sq), q)
     out = torch.empty_like(q)
     lse = torch.empty((H, Sq), dtype=torch.float32, device=q.device)
-    check(lib.fm_attention_hash_varlen(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_cnt), _p(q_hash), _p(out),
+    check(lib.fm_attention_hash_varlen(_p(q), _p(k), _p(v), _pl(k_idx), _p(bucket_cnt), _p(q_hash), _p(out),
                                        _p(lse), H, Sq, N, d, C, float(sm_scale), _dt(q), _p(ws),
                                        ws.numel(), _stream(q)))
     return out, lse
@@ -445,7 +460,7 @@ def attention_hash_varlen_static_(q, k, v, k_idx, bucket_cnt, q_hash, sm_scale: 
     C = bucket_cnt.shape[-1]
     assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and q_hash.dtype == torch.int32
     assert out.shape == q.shape and out.dtype == q.dtype and lse.shape == (H, Sq) and lse.dtype == torch.float32
-    check(_lib.load().fm_attention_hash_varlen_static(_p(q), _p(k), _p(v), _p(k_idx), _p(bucket_cnt), _p(q_hash),
+    check(_lib.load().fm_attention_hash_varlen_static(_p(q), _p(k), _p(v), _pl(k_idx), _p(bucket_cnt), _p(q_hash),
                                                       _p(out), _p(lse), H, Sq, N, d, C, float(sm_scale), _dt(q),
                                                       _stream(q)))
     return out, lse

@@ -112,3 +112,137 @@ def test_local_attention_random_extents(dt, H, G, S, L, d, causal, seed):
     out, lse = ops.local_attn_fwd(dev(q[0]), dev(k[0]), dev(v[0]), d ** -0.5, causal)
     ro, rl = O.local_attention(q, k, v, d ** -0.5, causal)
     assert_attn_close(out, lse, ro[0], rl[0], dtype, "local")
+
+
+def _memory_cases(n, seed):
+    rnd = random.Random(seed)
+    out = []
+    for i in range(n):
+        dt = rnd.choice(["f32", "bf16", "bf16", "f16"])
+        d = rnd.choice([64, 128, 128] if dt != "f32" else [16, 64])
+        H, G = rnd.randint(1, 2), rnd.choice([1, 2, 4])
+        N0 = rnd.choice([10, 300, 2000, 66000])
+        M = rnd.choice([1, 7, 100, 700])
+        C = rnd.choice([1, 4, 13, 40])
+        Z = rnd.choice([1, 16, 100, 512])
+        S = rnd.choice([1, 5, 40])
+        L = rnd.choice([1, 40, 70])
+        out.append(pytest.param(dt, H, G, N0, M, C, Z, S, L, d, 7000 + i,
+                                id=f"{dt}-H{H}-G{G}-N{N0}+{M}-C{C}-Z{Z}-S{S}-L{L}-d{d}"))
+    return out
+
+
+@pytest.mark.parametrize("dt,H,G,N0,M,C,Z,S,L,d,seed", _memory_cases(24, 20263))
+def test_memory_build_append_attend_random_extents(dt, H, G, N0, M, C, Z, S, L, d, seed):
+    """A memory through its life: built (lists shorter than Z while it holds fewer than Z keys), extended, asked
+    with local keys -- the lists against the oracle's arg-top-Z of the device's scores, the merged attention
+    against one softmax over the hashed bucket's keys and the visible local keys."""
+    from fast_memory_amd import Memory, ops
+    dtype = _DT[dt]
+    g = gen(seed)
+    K = (torch.randn(H, N0 + M, d, generator=g) * 0.5).to(dtype)
+    V = (torch.randn(H, N0 + M, d, generator=g) * 0.5).to(dtype)
+    A = torch.randn(H, C, d, generator=g).to(dtype)
+    q = (torch.randn(H, G * S, d, generator=g) * 0.5).to(dtype)
+    kl = (torch.randn(H, L, d, generator=g) * 0.5).to(dtype)
+    vl = (torch.randn(H, L, d, generator=g) * 0.5).to(dtype)
+    Kd, Vd, Ad, qd = dev(K, V, A, q)
+    mem = Memory.build(Kd[:, :N0].contiguous(), Vd[:, :N0].contiguous(), Ad, Z, keep_values=True)
+    mem.append(Kd[:, N0:].contiguous(), Vd[:, N0:].contiguous())
+    N = N0 + M
+    Zl = min(Z, N)                                            # a memory of fewer than Z keys lists them all
+    Y = ops.project(Ad, Kd).cpu()
+    want = O.argtopz(Y, Zl)
+    cnt = mem.bucket_cnt.cpu()
+    assert (cnt == Zl).all()
+    assert torch.equal(mem.bucket_idx.cpu().long()[..., :Zl], want)
+    sm = d ** -0.5
+    out, lse = mem.attend_with_local(qd, *dev(kl, vl), sm, n_groups=G, causal=True)
+    qh = mem.hash(qd).cpu().long()
+    o64, l64 = out.cpu().double(), lse.cpu().double()
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    for h in range(H):
+        for i in range(0, G * S, max(1, (G * S) // 7)):
+            t = i % S                                          # token of query i inside its query head
+            vis = min(L, max(0, t + (L - S) + 1))              # local keys it sees (mask aligned bottom-right)
+            idx = want[h, qh[h, i]]
+            kk = torch.cat([K[h, idx], kl[h, :vis]]).double()
+            vv = torch.cat([V[h, idx], vl[h, :vis]]).double()
+            s = kk @ q[h, i].double() * sm
+            assert abs(torch.logsumexp(s, 0).item() - l64[h, i].item()) < 1e-3
+            assert torch.allclose(torch.softmax(s, 0) @ vv, o64[h, i], atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("seed", [8001, 8002, 8003, 8004, 8005, 8006])
+def test_decode_batch_random_extents(seed):
+    """Batched decode over memories of random lengths, bucket counts and list lengths (one token per query
+    head), hashes against the first argmax of the returned scores, attention against the oracle."""
+    from fast_memory_amd import Memory, MemoryBatch
+    rnd = random.Random(seed)
+    g = gen(seed)
+    H, G, d = rnd.randint(1, 3), rnd.choice([1, 2, 4, 8, 16]), 128
+    n_seq = rnd.randint(1, 6)
+    shapes = []
+    for _ in range(n_seq):
+        N = rnd.choice([1, 50, 700, 3000, 9000])
+        C = rnd.choice([1, 3, 26, 64, 95])
+        shapes.append((N, C, rnd.randint(1, min(N, 400))))
+    mems, cpu = [], []
+    for N, C, Z in shapes:
+        K = torch.randn(H, N, d, generator=g).to(torch.bfloat16)
+        V = torch.randn(H, N, d, generator=g).to(torch.bfloat16)
+        A = torch.randn(H, C, d, generator=g).to(torch.bfloat16)
+        mems.append(Memory.build(*dev(K, V, A), Z))
+        cpu.append((K, V, A))
+    batch = MemoryBatch(mems)
+    q = (torch.randn(n_seq, H, G, d, generator=g) * 1.5).to(torch.bfloat16)
+    out, lse, h, scores = batch.attend(dev(q), d ** -0.5, return_scores=True)
+    out, lse, h, scores = out.cpu(), lse.cpu(), h.cpu().long(), scores.cpu()
+    a_off = 0
+    for s, ((N, C, Z), (K, V, A), mem) in enumerate(zip(shapes, cpu, mems)):
+        for hh in range(H):
+            sc = scores[a_off:a_off + C].T
+            assert torch.equal(h[s, hh], O.argmax_first(sc)), f"seq {s} head {hh}: hash"
+            a_off += C
+        lists = mem.bucket_idx.cpu().long()
+        ro, rl = O.hashed_attention_gather(q[s], K, V, lists.reshape(-1), torch.full((H, C), Z), h[s], d ** -0.5)
+        assert_attn_close(out[s], lse[s], ro, rl, torch.bfloat16, f"decode batch seq {s} {shapes[s]}")
+
+
+def _window_cases(n, seed):
+    rnd = random.Random(seed)
+    out = []
+    for i in range(n):
+        dt = rnd.choice(["f32", "bf16", "f16"])
+        d = rnd.choice([64, 128] if dt != "f32" else [16, 64])
+        B = rnd.randint(1, 2)
+        N = rnd.choice([500, 3000, 70000])
+        C = rnd.choice([2, 9, 30])
+        Z = rnd.choice([8, 64, 300])
+        S = rnd.choice([3, 50, 400])
+        lo = rnd.choice([0, 0, N // 3, N - 5])
+        hi = rnd.choice([N, lo + 1, lo + max(1, (N - lo) // 2), lo])       # the last: an empty window
+        out.append(pytest.param(dt, B, S, N, C, Z, d, lo, hi, 9000 + i, id=f"{dt}-B{B}-S{S}-N{N}-C{C}-Z{Z}-d{d}-w{lo}:{hi}"))
+    return out
+
+
+@pytest.mark.parametrize("dt,B,S,N,C,Z,d,lo,hi,seed", _window_cases(20, 20264))
+def test_attention_hash_with_window_random_extents(dt, B, S, N, C, Z, d, lo, hi, seed):
+    """The composite (build + hash + attention, triton_kernel.py:275-286) with a window of key indices as the
+    reference hard-codes one (triton_kernel.py:283), including windows no listed key falls into."""
+    from fast_memory_amd import attention_hash, ops
+    dtype = _DT[dt]
+    g = gen(seed)
+    q = (torch.randn(B, S, d, generator=g) * 0.5).to(dtype)
+    k = (torch.randn(B, N, d, generator=g) * 0.5).to(dtype)
+    v = (torch.randn(B, N, d, generator=g) * 0.5).to(dtype)
+    cen = torch.randn(B, C, d, generator=g).to(dtype)
+    qd, kd, vd, cd = dev(q, k, v, cen)
+    sm = d ** -0.5
+    out, lse = attention_hash(qd, kd, vd, cd, Z, sm, window=(lo, hi))
+    lists = O.argtopz(ops.project(cd, kd).cpu(), Z)
+    qh, sc = ops.qhash(cd, qd, return_scores=True)
+    assert torch.equal(qh.cpu().long(), O.argmax_first(sc.cpu()))
+    mask = (lists >= lo) & (lists < hi)
+    ro, rl = O.hashed_attention_gather(q, k, v, lists[mask], mask.sum(-1), qh.cpu().long(), sm)
+    assert_attn_close(out, lse, ro, rl, dtype, "attention_hash with a window")

@@ -246,3 +246,58 @@ def test_attention_hash_with_window_random_extents(dt, B, S, N, C, Z, d, lo, hi,
     mask = (lists >= lo) & (lists < hi)
     ro, rl = O.hashed_attention_gather(q, k, v, lists[mask], mask.sum(-1), qh.cpu().long(), sm)
     assert_attn_close(out, lse, ro, rl, dtype, "attention_hash with a window")
+
+
+def _dispatch_cases(n, seed):
+    rnd = random.Random(seed)
+    out = []
+    for i in range(n):
+        dt = rnd.choice(["bf16", "f16"])
+        d = rnd.choice([64, 128, 128, 128, 256])
+        B = rnd.randint(1, 3)
+        N = rnd.choice([5000, 40000, 300000])
+        C = rnd.choice([1, 8, 64, 700])
+        Z = rnd.choice([1, 64, 700, 3000])
+        S = rnd.choice([10, 700, 9000])
+        skew = rnd.random() < 0.3
+        out.append(pytest.param(dt, B, S, N, C, Z, d, skew, 9500 + i, id=f"{dt}-B{B}-S{S}-N{N}-C{C}-Z{Z}-d{d}{'-skew' if skew else ''}"))
+    return out
+
+
+@pytest.mark.parametrize("dt,B,S,N,C,Z,d,skew,seed", _dispatch_cases(48, 20265))
+def test_mfma_kernels_against_generic_random_extents(dt, B, S, N, C, Z, d, skew, seed):
+    """Whatever kernel the dispatch takes for the extents (rows gathered into registers, staged in LDS, loaded
+    straight into LDS; one launch or one per row; forward and backward) against the generic kernels on the same
+    device inputs -- at sizes the CPU oracle would take minutes for.  ``skew``: a third of the queries in one
+    bucket (several work items and workgroups for it)."""
+    from fast_memory_amd import attention_hash_varlen, attention_hash_varlen_backward, ops
+    dtype = _DT[dt]
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    mk = lambda *s: (torch.randn(*s, generator=g, device="cuda") * 0.6).to(dtype)
+    q, k, v, dout = mk(B, S, d), mk(B, N, d), mk(B, N, d), mk(B, S, d)
+    lists = torch.randint(0, N, (B, C, Z), generator=g, device="cuda", dtype=torch.int32)
+    cnt = torch.randint(0, Z + 1, (B, C), generator=g, device="cuda", dtype=torch.int32)       # ragged, some empty
+    keep = torch.arange(Z, device="cuda")[None, None, :] < cnt[..., None]
+    flat = lists[keep].contiguous()
+    qh = torch.randint(0, C, (B, S), generator=g, device="cuda", dtype=torch.int32)
+    if skew:
+        qh[:, : S // 3] = C // 2
+    sm = d ** -0.5
+    run = lambda: attention_hash_varlen(q, k, v, flat, cnt, qh, sm, lse_dtype=torch.float32)
+    bwd = lambda o, l: attention_hash_varlen_backward(dout, q, k, v, o, l, flat, cnt, qh, sm)
+    o1, l1 = run()
+    g1 = bwd(o1, l1)
+    ops.force_generic_kernels(True)
+    try:
+        o2, l2 = run()
+        g2 = bwd(o1, l1)                                                   # the same out / lse into both backwards
+    finally:
+        ops.force_generic_kernels(False)
+    empty = l2 < -1e30
+    assert torch.equal(l1 < -1e30, empty)
+    assert torch.allclose(o1.float(), o2.float(), atol=2e-2, rtol=1e-2)
+    assert (l1[~empty] - l2[~empty]).abs().max().item() < 1e-3 if (~empty).any() else True
+    for a, b, name in zip(g1, g2, ("dq", "dk", "dv")):
+        a, b = a.float(), b.float()
+        assert torch.allclose(a, b, atol=2e-2 * max(1.0, b.abs().max().item()), rtol=2e-2), \
+            f"{name}: {(a - b).abs().max().item():.3e} vs max {b.abs().max().item():.3e}"

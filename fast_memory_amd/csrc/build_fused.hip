@@ -65,6 +65,11 @@ constexpr double kRankSigmas = 4.0;
 // The rank is mu + 4 sqrt(mu) + 3, raised where that is not enough for the build's rows: with small mu the
 // 4 sqrt(mu) are fewer than 3.5 deviations of sqrt(r), and a build of many rows needs more of them to leave
 // the expected number of repaired rows at about four (64 can be repaired).
+// Room, in standard deviations, for the number of candidates a threshold of that rank lets through: five, and
+// more for a small rank, whose count (a Gamma variable of that shape) has a long upper tail (at rank 11 one row
+// in a thousand exceeded five deviations).
+static double room_sigmas(int rank) { return 5.0 + 6.0 / sqrt(double(std::max(rank, 1))); }
+
 static int threshold_rank(double mu, double rows) {
   const double base = mu + kRankSigmas * sqrt(mu) + 3.0;
   const double lp = 2.0 * log(std::max(rows, 64.0) / 4.0);                       // tail 4 / rows
@@ -101,7 +106,7 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   // selection must hold in registers (R per thread, T = NT / n_writers threads per writer segment,
   // whose share of m spreads by another sqrt).  The sort keeps 16 keys per thread, so P/16 threads
   // are all it can use; fewer threads per row let several rows share a CU.  Of the samples that leave
-  // five standard deviations of room (each with the fewest threads that do), take the one with the
+  // five standard deviations of room or more (room_sigmas; each with the fewest threads that do), take the one with the
   // least expected work; if none does, the large sample with 1024 threads (rows that do not fit are
   // repaired).
   const int P = next_pow2(Z);
@@ -128,7 +133,8 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
       const double sd_w = sqrt(pow(double(N) / ns * sqrt(double(rank)) / p.n_writers, 2) + per_w);
       int nt_ok = 0;
       for (int nt = 256; nt <= kSelThreads && !nt_ok; nt *= 2)
-        if (nt * 16 >= P && (nt / p.n_writers) * (nt < kSelThreads ? kCandRegsSmall : kCandRegs) >= per_w + 5.0 * sd_w)
+        if (nt * 16 >= P &&
+            (nt / p.n_writers) * (nt < kSelThreads ? kCandRegsSmall : kCandRegs) >= per_w + room_sigmas(rank) * sd_w)
           nt_ok = nt;
       if (!nt_ok) continue;
       const double cost = 2.7 * ns + 10.0 * m;
@@ -155,22 +161,33 @@ static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& 
   // standard deviations of a group's candidates fit the passes.
   const int forced = g_fused_filter_form.load(std::memory_order_relaxed);  // 1: not this form; 2, 3, 4: its ND = 1, 2, 3
   if (p.wide && forced != 1) {
-    p.n_writers = p.n_splits;
-    if (search()) {
-      const double per_group = 2048.0 * m_exp / N;
-      const int nd = forced >= 2 && forced <= 4 ? forced - 1 : int(ceil((per_group + 3.5 * sqrt(per_group)) / 64.0));
-      if (nd >= 1 && nd <= 3) p.ping = nd;
+    // With few rows (one or two KV heads: a GPU's share of a model sharded by head) 32 key splits leave most
+    // compute units without a workgroup: up to 64 then, a writer each, where the selection's registers still
+    // hold a writer's candidates with room (found); otherwise the splits chosen above.
+    const int base_splits = p.n_splits;
+    const int more_splits = int(std::max<int64_t>(1, std::min<int64_t>(64, std::min(ceil_div(256, int64_t(H) * p.slabs), ntiles))));
+    for (int attempt = more_splits > base_splits ? 0 : 1; attempt < 2 && !p.ping; ++attempt) {
+      p.n_splits = attempt == 0 ? more_splits : base_splits;
+      p.n_writers = p.n_splits;
+      if (search() && (found || attempt == 1)) {
+        const double per_group = 2048.0 * m_exp / N;
+        const int nd = forced >= 2 && forced <= 4 ? forced - 1 : int(ceil((per_group + 3.5 * sqrt(per_group)) / 64.0));
+        if (nd >= 1 && nd <= 3) p.ping = nd;
+      }
     }
-    if (!p.ping) p.n_writers = 2 * p.n_splits;
+    if (!p.ping) {
+      p.n_splits = base_splits;
+      p.n_writers = 2 * p.n_splits;
+    }
   }
   if (!p.ping && !search()) return false;
-  // A writer's segment: its share of the expected candidates with room for five standard deviations (the
+  // A writer's segment: its share of the expected candidates with room for five or more standard deviations (the
   // threshold's noise, a relative 1 / sqrt(rank) of all of a row's candidates, plus the spread of a share);
   // the overflow guard keeps 16 slots free.  With a small rank 1.35 times the share is less than that.
   {
     const double per_w = m_exp / p.n_writers;
     const double sd_w = sqrt(pow(double(N) / p.ns * sqrt(double(p.rank)) / p.n_writers, 2) + per_w);
-    p.cap_w = int(std::max(1.35 * per_w + 64.0, per_w + 5.0 * sd_w + 16.0));
+    p.cap_w = int(std::max(1.35 * per_w + 64.0, per_w + room_sigmas(p.rank) * sd_w + 16.0));
   }
   p.ld_s = (int64_t(p.ns) + 3) / 4 * 4;
   p.ldy = (int64_t(N) + 3) / 4 * 4;

@@ -91,7 +91,7 @@ struct FusedPlan {
 
 static bool fused_plan(int H, int C, int N, int d, int Z, int dtype, FusedPlan& p) {
   if ((dtype != FM_BF16 && dtype != FM_F16) || d != kFD) return false;
-  if (N < 65536 || int64_t(Z) * 8 > N || Z > FM_MAX_Z || Z < 64) return false;
+  if (N < 16384 || int64_t(Z) * 8 > N || Z > FM_MAX_Z || Z < 64) return false;  // (the smallest sample is a quarter of 16384 keys)
   // the wide form wherever its 1024-bucket slabs are at least three quarters full
   p.wide = C >= 768 && (C % 1024 == 0 || C % 1024 >= 768 || C >= 4096);
   p.slabs = int(ceil_div(C, p.wide ? 1024 : kFSlab));

@@ -113,7 +113,7 @@ def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int =
     the fp32 projections of the listed keys (what an index needs to be extended later).
 
     ``fused=None`` takes the fused build (no Y in memory) where the shape is
-    eligible and the unfused one otherwise; both give identical lists.  The
+    eligible and H * C * N is at least 2^24, and the unfused one otherwise; both give identical lists.  The
     fused build reports through a two-int status on the device whether any row could not be
     resolved there, in which case the unfused build runs instead.  Reading that word is the only
     host synchronisation of the build: with ``defer_check`` it is left out, the lists come back with a
@@ -136,7 +136,9 @@ def build_index(A: torch.Tensor, K: torch.Tensor, Z: int, workspace_bytes: int =
 
     fws = lib.fm_build_index_fused_workspace(H, C, N, d, int(Z), _dt(A)) if fused is not False else 0
     if fused and not fws:
-        raise ValueError("fused index build: shape not eligible (bf16, d=128, N>=65536, 64<=Z<=N/8)")
+        raise ValueError("fused index build: shape not eligible (bf16 / fp16, d=128, N>=16384, 64<=Z<=N/8)")
+    if fused is None and H * C * N < (1 << 24):
+        fws = 0          # a small build: the fixed cost of the fused form's four phases is more than it saves
     if fws:
         ws = _ws(fws, A)
         status = torch.empty(_lib.FM_FUSED_STATUS_INTS, dtype=torch.int32, device=A.device)

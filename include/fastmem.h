@@ -91,8 +91,10 @@ int fm_build_index(const void* A, const void* K, int32_t* idx_out, float* val_ou
 /* ---- a1+a2 fused: the same lists without ever writing Y to memory ------------
  * (memory.py:260-278; the selection sees exactly the fp32 values fm_project
  * would produce, so the lists are bit-identical to fm_build_index).  Built for
- * bf16, d = 128, N >= 65536, 64 <= Z <= N/8; fm_build_index_fused_workspace
- * returns 0 for any other shape.  A per-row threshold taken from a sample of the
+ * bf16 / fp16, d = 128, N >= 16384, 64 <= Z <= N/8; fm_build_index_fused_workspace
+ * returns 0 for any other shape.  (It pays from about H * C * N = 2^24 on: 8 x
+ * 256 x 32768 builds in 0.16 ms against 0.36 ms, 8 x 64 x 8192 in 0.095 ms
+ * against 0.068 ms.)  A per-row threshold taken from a sample of the
  * keys filters the MFMA output; rows whose threshold missed are recomputed
  * exactly on the device (up to 64 of them).  status_dev (device,
  * FM_FUSED_STATUS_INTS ints) receives {rows repaired, rows left unresolved, then

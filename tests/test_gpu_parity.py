@@ -1354,7 +1354,10 @@ def test_fused_build_bit_identical_to_unfused(ops):
 @pytest.mark.parametrize("H,C,N,Z", [(1, 513, 65536 + 31, 64),        # one bucket past a 512-bucket slab, ragged key tile
                                      (3, 1024, 98304, 4096),           # three splits' worth of whole tiles
                                      (2, 600, 131072 + 1, 2000),       # Z not a power of two, one key past a tile
-                                     (1, 64, 65536, 8192)])            # the longest list N/8 allows here
+                                     (1, 64, 65536, 8192),             # the longest list N/8 allows here
+                                     (8, 256, 32768, 1024),            # the prefill chunk's extents
+                                     (2, 130, 16384, 2048),            # the shortest memory the fused build takes, Z = N/8
+                                     (3, 1024, 20001, 64)])            # ... a ragged one, the shortest lists
 def test_fused_build_shapes(ops, H, C, N, Z):
     g = gen(910 + C)
     K = _clustered_keys(g, H, N, 128)

@@ -70,7 +70,7 @@ def _build_cases(n, seed):
 @pytest.mark.parametrize("dt,H,N,C,Z,S,d,seed", _build_cases(30, 20261))
 def test_build_and_hash_random_extents(dt, H, N, C, Z, S, d, seed):
     """Lists and hashes bit-exact against the oracle on the device's own fp32 scores (whichever build path the
-    extents take: fused for bf16 / fp16 at d = 128 with 65 536 keys or more, chunked otherwise)."""
+    extents take: fused for bf16 / fp16 at d = 128 with 16 384 keys or more and enough rows, chunked otherwise)."""
     from fast_memory_amd import ops
     dtype = _DT[dt]
     g = gen(seed)

@@ -151,7 +151,8 @@ __global__ __launch_bounds__(256) void segment_mean_kernel(
 // the sixteen partial sums are then added in group order, so the result does not depend on
 // scheduling.  HBM-bound on the gathered rows (256 bytes per member).
 // NORM as in segment_mean_kernel: a row's squared norm is summed inside its group of 16 lanes.
-template <bool NORM>
+// F16: the rows are fp16 (else bf16); bf16_t and f16_t are both 16-bit words here.
+template <bool NORM, bool F16 = false>
 __global__ __launch_bounds__(256) void segment_mean_bf16_d128_kernel(
     const bf16_t* __restrict__ X, const int32_t* __restrict__ perm, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_cnt, const bf16_t* __restrict__ prev, bf16_t* __restrict__ out, int C,
@@ -177,7 +178,16 @@ __global__ __launch_bounds__(256) void segment_mean_bf16_d128_kernel(
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       float f[8];
-      cent_unpack8(u[k], f);
+      if constexpr (F16) {
+        const uint32_t w4[4] = {u[k].x, u[k].y, u[k].z, u[k].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          f[2 * i] = float(__builtin_bit_cast(_Float16, uint16_t(w4[i] & 0xffffu)));
+          f[2 * i + 1] = float(__builtin_bit_cast(_Float16, uint16_t(w4[i] >> 16)));
+        }
+      } else {
+        cent_unpack8(u[k], f);
+      }
       if constexpr (NORM) {
         float ss = 0.f;
 #pragma unroll
@@ -208,7 +218,7 @@ __global__ __launch_bounds__(256) void segment_mean_bf16_d128_kernel(
     if (cnt == 0 || nrm < 1e-12f)
       out[hc * 128 + t] = prev[hc * 128 + t];
     else
-      out[hc * 128 + t] = f32_to_bf16(v / nrm);
+      out[hc * 128 + t] = F16 ? bf16_t(__builtin_bit_cast(uint16_t, _Float16(v / nrm))) : f32_to_bf16(v / nrm);
   }
 }
 
@@ -324,6 +334,13 @@ static int segment_mean_any(const char* name, bool norm, const void* X, const in
     else
       hipLaunchKernelGGL(segment_mean_bf16_d128_kernel<false>, grid, dim3(256), 0, st, (const bf16_t*)X, perm, seg_off,
                          seg_cnt, (const bf16_t*)prev, (bf16_t*)cent_out, C, N, eps);
+  } else if (dtype == FM_F16 && d == 128) {
+    if (norm)
+      hipLaunchKernelGGL((segment_mean_bf16_d128_kernel<true, true>), grid, dim3(256), 0, st, (const bf16_t*)X, perm,
+                         seg_off, seg_cnt, (const bf16_t*)prev, (bf16_t*)cent_out, C, N, eps);
+    else
+      hipLaunchKernelGGL((segment_mean_bf16_d128_kernel<false, true>), grid, dim3(256), 0, st, (const bf16_t*)X, perm,
+                         seg_off, seg_cnt, (const bf16_t*)prev, (bf16_t*)cent_out, C, N, eps);
   } else if (dtype == FM_F32) {
     if (norm) FM_SEGMEAN(float, true); else FM_SEGMEAN(float, false);
   } else if (dtype == FM_BF16) {

@@ -324,6 +324,19 @@ def hash_attn_bwd(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGroups, o
     assert k.shape == v.shape and out.shape == q.shape and dout.shape == q.shape and lse.shape == (H, Sq)
     assert q.dtype == k.dtype == v.dtype == out.dtype == dout.dtype and lse.dtype == torch.float32
     assert k_idx.dtype == torch.int32 and bucket_cnt.dtype == torch.int32 and bucket_off.dtype == torch.int64
+    if d == 64 and q.dtype in (torch.bfloat16, torch.float16) and not generic_kernels_forced():
+        # The MFMA backward is built for d = 128; at d = 64 the generic kernel (an atomic add per query, key and
+        # dimension) is twenty times slower than that kernel on rows padded with zeros, which add nothing to
+        # any dot product: the same sums, on copies twice the size.
+        pad = lambda t: torch.nn.functional.pad(t, (0, 64))
+        dq, dk2, dv2 = hash_attn_bwd(pad(q), pad(k), pad(v), k_idx, bucket_off, bucket_cnt, groups, pad(out), lse,
+                                     pad(dout), sm_scale, dlse=dlse)
+        dk2, dv2 = dk2[..., :64], dv2[..., :64]
+        if dk is not None:
+            dk2 = dk.add_(dk2)
+        if dv is not None:
+            dv2 = dv.add_(dv2)
+        return dq[..., :64].contiguous(), dk2.contiguous(), dv2.contiguous()
     dq = torch.empty_like(q)
     if dk is None:
         dk = torch.zeros((H, N, d), dtype=torch.float32, device=q.device)

@@ -134,8 +134,7 @@ __device__ __forceinline__ void bwd_tile(const bf16_t* __restrict__ q, const bf1
                                          bf16_t* dkp, bf16_t* dvp, bf16_t* dump, float* red, int* q_rows,
                                          bf16_t* stage, unsigned char* blk = nullptr) {
   static_assert(!LDSBLK || (STAGED && FIRST_TILE && TILES == 2), "the LDS block form is the first two-tile pass");
-  static_assert(!(F16 && STAGED), "the partial rows of the staged form are bf16: fp16 takes the atomic form");
-  using M = Mma<F16>;  // the 16-bit type of q, k, v, out, dout and dq (F16: fp16, else bf16)
+  using M = Mma<F16>;  // the 16-bit type of q, k, v, out, dout and dq (F16: fp16, else bf16); partial rows are bf16
   if (threadIdx.x < 16 * TILES) q_rows[threadIdx.x] = threadIdx.x < n_q ? q_list[threadIdx.x] : -1;
   __syncthreads();
   const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -576,7 +575,7 @@ constexpr int kStagedMaxQ = 256;  // queries of a bucket that go through its bf1
 // workgroups at 256 registers each their 96 / 138 spilled registers cost more than the second workgroup hides
 // (c5: 94.5 against 91.8 ms; c4: 11.4 against 10.9 ms).  The four-tile kernel keeps two workgroups per CU
 // (c2: 1.3 against 1.6 ms).
-template <int MAXT, bool LDSBLK>
+template <int MAXT, bool LDSBLK, bool F16 = false>
 __global__ __launch_bounds__(256, MAXT == 4 ? 2 : 1) void hash_attn_bwd_staged_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
@@ -617,7 +616,7 @@ __global__ __launch_bounds__(256, MAXT == 4 ? 2 : 1) void hash_attn_bwd_staged_k
     if (q0) __syncthreads();  // red and q_rows are reused
     const int left = nq_staged - q0;
 #define FM_BWD_PASS(FIRST, NT)                                                                                        \
-  bwd_tile<true, FIRST, NT>(q, out, lse, dout, dlse, ql + q0, min(16 * NT, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,  \
+  bwd_tile<true, FIRST, NT, false, F16>(q, out, lse, dout, dlse, ql + q0, min(16 * NT, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,  \
                             cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage)
     if (MAXT == 4 && left > 32) {
       if (q0 == 0)
@@ -626,7 +625,7 @@ __global__ __launch_bounds__(256, MAXT == 4 ? 2 : 1) void hash_attn_bwd_staged_k
         FM_BWD_PASS(false, MAXT);
     } else if (LDSBLK && q0 == 0 && left > 16) {
       // the first pass of a bucket with 17 to 32 queries, its rows through LDS
-      bwd_tile<true, true, 2, LDSBLK>(q, out, lse, dout, dlse, ql, min(32, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,
+      bwd_tile<true, true, 2, LDSBLK, F16>(q, out, lse, dout, dlse, ql, min(32, left), int64_t(row) * Sq, Kb, Vb, k_idx + off,
                                       cnt, N, sm_scale, dq, nullptr, nullptr, dkb, dvb, dump, red, q_rows, stage, blk);
     } else if (left > 16) {
       if (q0 == 0)
@@ -645,6 +644,7 @@ __global__ __launch_bounds__(256, MAXT == 4 ? 2 : 1) void hash_attn_bwd_staged_k
 
 // grid (C, rows): the queries of a bucket beyond the first kStagedMaxQ, 16 at a time, with atomic adds into
 // dK / dV; a workgroup whose bucket has no such query (nearly all of them) reads one word and leaves.
+template <bool F16>
 __global__ __launch_bounds__(256) void hash_attn_bwd_excess_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off, const int32_t* __restrict__ bucket_cnt,
@@ -661,7 +661,7 @@ __global__ __launch_bounds__(256) void hash_attn_bwd_excess_kernel(
   const int32_t* ql = q_perm + bin_off[bkt];
   for (int q0 = kStagedMaxQ; q0 < nq; q0 += 16) {
     if (q0 > kStagedMaxQ) __syncthreads();  // red and q_rows are reused
-    bwd_tile<false, true>(q, out, lse, dout, dlse, ql + q0, min(16, nq - q0), int64_t(row) * Sq,
+    bwd_tile<false, true, 1, false, F16>(q, out, lse, dout, dlse, ql + q0, min(16, nq - q0), int64_t(row) * Sq,
                           k + int64_t(row) * N * kBD, v + int64_t(row) * N * kBD, k_idx + bucket_off[bkt],
                           bucket_cnt[bkt], N, sm_scale, dq, dk + int64_t(row) * N * kBD, dv + int64_t(row) * N * kBD,
                           nullptr, nullptr, nullptr, red, q_rows, nullptr);
@@ -691,12 +691,20 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
                                   const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
                                   const void* dout, const float* dlse, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0,
                                   int row0, int rows, int Sq, int N, int C, float sm_scale, float* dk, float* dv,
-                                  hipStream_t st) {
+                                  bool f16, hipStream_t st) {
 #define FM_BWD_STAGED(MAXT, LB)                                                                                    \
-  hipLaunchKernelGGL((hash_attn_bwd_staged_kernel<MAXT, LB>), dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st, \
+  do {                                                                                                             \
+  if (f16)                                                                                                         \
+    hipLaunchKernelGGL((hash_attn_bwd_staged_kernel<MAXT, LB, true>), dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st, \
+                       (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,  \
+                       bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, (bf16_t*)dkp,  \
+                       (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale);                                  \
+  else                                                                                                             \
+  hipLaunchKernelGGL((hash_attn_bwd_staged_kernel<MAXT, LB, false>), dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st, \
                      (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,  \
                      bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, (bf16_t*)dkp,  \
-                     (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale)
+                     (bf16_t*)dvp, (bf16_t*)dump, pos0, row0, Sq, N, C, sm_scale);                                    \
+  } while (0)
   if (int64_t(Sq) > 24 * int64_t(C))  // more than 24 queries per bucket on average
     FM_BWD_STAGED(4, false);
   else if (N < (1 << 24) && int64_t(Sq) > 12 * int64_t(C) && g_force_generic != 9)
@@ -707,11 +715,18 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
   else
     FM_BWD_STAGED(2, false);
 #undef FM_BWD_STAGED
-  if (Sq > kStagedMaxQ)  // some bucket may hold more queries than go through its partial rows
-    hipLaunchKernelGGL(hash_attn_bwd_excess_kernel, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,
-                       (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
-                       bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, row0,
-                       Sq, N, C, sm_scale);
+  if (Sq > kStagedMaxQ) {  // some bucket may hold more queries than go through its partial rows
+    if (f16)
+      hipLaunchKernelGGL(hash_attn_bwd_excess_kernel<true>, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,
+                         (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
+                         bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, row0,
+                         Sq, N, C, sm_scale);
+    else
+      hipLaunchKernelGGL(hash_attn_bwd_excess_kernel<false>, dim3(unsigned(C), unsigned(rows)), dim3(256), 0, st,
+                         (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, bucket_off, bucket_cnt, q_perm,
+                         bin_off, bin_count, (const bf16_t*)out, lse, (const bf16_t*)dout, dlse, (bf16_t*)dq, dk, dv, row0,
+                         Sq, N, C, sm_scale);
+  }
   return launch_status("fm_hash_attn_bwd_staged(partials)");
 }
 

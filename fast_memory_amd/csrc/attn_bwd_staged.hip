@@ -40,7 +40,7 @@ int hash_attn_bwd_staged_partials(const void* q, const void* k, const void* v, c
                                   const int32_t* bin_off, const int32_t* bin_count, const void* out, const float* lse,
                                   const void* dout, const float* dlse, void* dq, void* dkp, void* dvp, void* dump, int64_t pos0,
                                   int row0, int rows, int Sq, int N, int C, float sm_scale, float* dk, float* dv,
-                                  hipStream_t st);  // attn_bwd_mfma.hip
+                                  bool f16, hipStream_t st);  // attn_bwd_mfma.hip
 
 // ---- inverse index ------------------------------------------------------------
 // One workgroup per (row, bucket): sort keys row * N + key, values = flat positions.
@@ -453,7 +453,8 @@ extern "C" int fm_hash_attn_bwd_staged(const void* q, const void* k, const void*
   using namespace fm;
   FM_REQUIRE(H >= 1 && Sq >= 1 && N >= 1 && C >= 1, FM_ERR_ARG, "fm_hash_attn_bwd_staged: H=%d Sq=%d N=%d C=%d", H, Sq,
              N, C);
-  FM_REQUIRE(dtype == FM_BF16 && d == 128, FM_ERR_UNSUPPORTED, "fm_hash_attn_bwd_staged: bf16 with d=128 only");
+  FM_REQUIRE((dtype == FM_BF16 || dtype == FM_F16) && d == 128, FM_ERR_UNSUPPORTED,
+             "fm_hash_attn_bwd_staged: bf16 or fp16 with d=128 only");
   FM_REQUIRE(q && k && v && k_idx && bucket_off && bucket_cnt && q_perm && bin_off && bin_count && out && lse && dout &&
                  key_off && inv_pos && dq && dk && dv && row_pos_host && ws,
              FM_ERR_ARG, "fm_hash_attn_bwd_staged: null pointer");
@@ -481,7 +482,7 @@ extern "C" int fm_hash_attn_bwd_staged(const void* q, const void* k, const void*
       bf16_t* dvp = dkp + 128;  // a position's rows side by side: [dK | dV]
       bf16_t* dump = dkp + size_t(n_pos) * 256;
       int rc = hash_attn_bwd_staged_partials(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, bin_off, bin_count, out,
-                                             lse, dout, dlse, dq, dkp, dvp, dump, pos0, h0, h1 - h0, Sq, N, C, sm_scale, dk, dv, st);
+                                             lse, dout, dlse, dq, dkp, dvp, dump, pos0, h0, h1 - h0, Sq, N, C, sm_scale, dk, dv, dtype == FM_F16, st);
       if (rc) return rc;
       const int64_t n_keys = int64_t(h1 - h0) * N;
       hipLaunchKernelGGL(bwd_reduce_kernel, dim3(unsigned(ceil_div(n_keys, int64_t(4)))), dim3(256), 0, st, dkp, dvp,

@@ -415,7 +415,7 @@ def hash_attn_bwd_staged(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGr
                          dout, sm_scale: float, dk: Optional[torch.Tensor] = None,
                          dv: Optional[torch.Tensor] = None, workspace_bytes: int = 24 << 30,
                          dlse: Optional[torch.Tensor] = None):
-    """:func:`hash_attn_bwd` without atomics (bf16, d = 128): per-bucket partial rows in a workspace, then a
+    """:func:`hash_attn_bwd` without atomics (bf16 or fp16, d = 128): per-bucket bf16 partial rows in a workspace, then a
     sum per key over the list positions that name it (``inv`` from :func:`inverse_index`).  Same results to
     rounding (the partial rows are bf16), in a fixed summation order."""
     _dev(q, k, v, k_idx, bucket_off, bucket_cnt, out, lse, dout)
@@ -424,7 +424,7 @@ def hash_attn_bwd_staged(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGr
     _, N, _ = k.shape
     C = bucket_cnt.shape[-1]
     assert k.shape == v.shape and out.shape == q.shape and dout.shape == q.shape and lse.shape == (H, Sq)
-    assert q.dtype == k.dtype == v.dtype == out.dtype == dout.dtype == torch.bfloat16 and d == 128
+    assert q.dtype == k.dtype == v.dtype == out.dtype == dout.dtype and q.dtype in (torch.bfloat16, torch.float16) and d == 128
     assert len(inv.row_pos) == H + 1 and inv.key_off.numel() == H * N + 1
     dq = torch.zeros_like(q)                                  # queries of an empty bucket keep 0
     if dk is None:

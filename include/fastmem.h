@@ -220,7 +220,8 @@ int fm_hash_attn_bwd(const void* q, const void* k, const void* v, const int32_t*
                      int Sq, int N, int d, int C, float sm_scale, int dtype, void* stream);
 
 /* ---- f1, dense query sets: backward without atomics ---------------------------
- * Same gradients as fm_hash_attn_bwd (bf16, d = 128 only).  A key's dk and dv rows
+ * Same gradients as fm_hash_attn_bwd (bf16 or fp16, d = 128 only; the partial rows
+ * are bf16 for both).  A key's dk and dv rows
  * collect contributions from every bucket that lists it; here each (row, bucket)
  * workgroup writes the bucket's own partial rows (bf16, one per listed key, in the
  * workspace) and a second kernel sums, per key, the partial rows of the list

@@ -120,7 +120,7 @@ def test_composite_local_merge_and_backward_fp16(ops):
     eo, el = O.lse_merge_closed_form(lo.reshape(H, G * S, d).float(), ll.reshape(H, G * S), ro.float(), rl)
     assert torch.allclose(mo.cpu().double(), eo.double(), atol=4e-3, rtol=1e-2)
     assert float((ml.cpu().double() - el.double()).abs().max()) < 2e-3
-    # backward (the MFMA kernel with atomic adds: the partial rows of the form without atomics are bf16)
+    # backward (the MFMA kernels; the partial rows of the form without atomics are bf16 for fp16 inputs too)
     dout = (torch.randn(H, G * S, d, generator=g) * 0.5).to(F16)
     dq, dk, dv = mem.attend_backward(dev(dout), qd, out, lse, d ** -0.5, q_hash=qh)
     rq, rk, rv = O.hashed_attention_backward_gather(q.float(), keys.float(), vals.float(), lists.reshape(-1), cnt,

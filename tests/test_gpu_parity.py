@@ -1024,20 +1024,21 @@ def test_backward_mfma_and_generic_agree(ops, dtype):
             f"{name}: {(a - b).abs().max().item():.3e} vs max {b.abs().max().item():.3e}"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("ws_bytes,C", [(24 << 30, 10), (1 << 20, 10),    # everything in one pass; one row per pass
                                         (24 << 30, 16)])                   # fewer queries per bucket: the two-tile kernel
-def test_backward_staged_equals_atomic_and_oracle(ops, ws_bytes, C):
+def test_backward_staged_equals_atomic_and_oracle(ops, ws_bytes, C, dtype):
     """The backward without atomics (per-bucket partial rows, then a sum per key over the inverted lists)
     against the atomic path and the oracle: buckets with several query tiles (passes of one, two and four
     tiles; the launch takes the four-tile kernel above 24 queries per bucket on average), buckets nobody
     hashed to, ragged and empty lists, keys listed by no bucket."""
     from fast_memory_amd import attention_hash_varlen
     B, S, N, Z, d = 3, 260, 1500, 200, 128
-    q, k, v, kh, cnt, qh = make_attn_case(1600, B, S, N, C, Z, d, torch.bfloat16, window="ref", std=0.7)
+    q, k, v, kh, cnt, qh = make_attn_case(1600, B, S, N, C, Z, d, dtype, window="ref", std=0.7)
     qh[0, :120] = 2                                             # 120 queries in one bucket: 8 tiles
     qh[qh == 7] = 8                                             # bucket 7 receives no query
     qh[1] = 4                                                   # one row hashes everything to one bucket
-    dout = (torch.randn(B, S, d, generator=gen(1601)) * 0.5).to(torch.bfloat16)
+    dout = (torch.randn(B, S, d, generator=gen(1601)) * 0.5).to(dtype)
     sm = d ** -0.5
     qd, kd, vd, khd, cntd, qhd = dev(q, k, v, kh, cnt, qh)
     out, lse = attention_hash_varlen(qd, kd, vd, khd, cntd, qhd, sm)
@@ -1059,8 +1060,8 @@ def test_backward_staged_equals_atomic_and_oracle(ops, ws_bytes, C):
     rq, rk, rv = O.hashed_attention_backward_gather(q.float(), k.float(), v.float(), kh, cnt, qh, out.float().cpu(),
                                                     lse.cpu(), dout.float(), sm)
     for got, other, ref, name in ((dq1, dq2, rq, "dq"), (dk1, dk2, rk, "dk"), (dv1, dv2, rv, "dv")):
-        _assert_grad_close(got, ref, torch.bfloat16, name + " (staged vs oracle)")
-        _assert_grad_close(got, other.float().cpu(), torch.bfloat16, name + " (staged vs atomic)")
+        _assert_grad_close(got, ref, dtype, name + " (staged vs oracle)")
+        _assert_grad_close(got, other.float().cpu(), dtype, name + " (staged vs atomic)")
     # a fixed summation order: bit-identical from run to run, and when the rows go through one at a time
     dq3, dk3, dv3 = ops.hash_attn_bwd_staged(qd, kd, vd, lists, off, counts, groups, inv, out, lse, dev(dout), sm,
                                              workspace_bytes=24 << 30)

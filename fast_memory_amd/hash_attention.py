@@ -140,12 +140,12 @@ def attention_hash_varlen_backward(d_out: torch.Tensor, q: torch.Tensor, k: torc
     off = ops.bucket_offsets(counts)
     groups = ops.group_queries(hashes, n_buckets)
     lists = _as_i32(k_hashes).contiguous()
-    can_stage = q.dtype in (torch.bfloat16, torch.float16) and d_head == 128 and lists.numel() > 0
+    can_stage = q.dtype in (torch.bfloat16, torch.float16) and d_head in (64, 128) and lists.numel() > 0
     auto = staged is None
     if auto:
         staged = can_stage and q_seq_len >= n_buckets and not ops.generic_kernels_forced()
     if staged:
-        assert can_stage, "the staged backward takes bf16 or fp16 with d_head = 128"
+        assert can_stage, "the staged backward takes bf16 or fp16 with d_head = 64 or 128"
         try:
             inv = inverse_index if inverse_index is not None else ops.inverse_index(lists, off, counts, k.shape[1])
             if inv.row_pos[-1] > 0:        # no listed entry at all: nothing to stage, the other form handles it

@@ -363,7 +363,7 @@ class Memory:
             q_hash = self.hash(q)
         groups = ops.group_queries(q_hash, self.n_buckets)
         lists = self.attention_lists(q.shape[1])
-        can_stage = q.dtype in (torch.bfloat16, torch.float16) and q.shape[2] == 128
+        can_stage = q.dtype in (torch.bfloat16, torch.float16) and q.shape[2] in (64, 128)
         auto = staged is None
         if auto:
             staged = can_stage and q.shape[1] >= self.n_buckets and not ops.generic_kernels_forced()

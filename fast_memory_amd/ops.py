@@ -424,7 +424,18 @@ def hash_attn_bwd_staged(q, k, v, k_idx, bucket_off, bucket_cnt, groups: QueryGr
     _, N, _ = k.shape
     C = bucket_cnt.shape[-1]
     assert k.shape == v.shape and out.shape == q.shape and dout.shape == q.shape and lse.shape == (H, Sq)
-    assert q.dtype == k.dtype == v.dtype == out.dtype == dout.dtype and q.dtype in (torch.bfloat16, torch.float16) and d == 128
+    assert q.dtype == k.dtype == v.dtype == out.dtype == dout.dtype and q.dtype in (torch.bfloat16, torch.float16)
+    if d == 64:      # on rows padded with zeros, as in hash_attn_bwd
+        pad = lambda t: torch.nn.functional.pad(t, (0, 64))
+        dq, dk2, dv2 = hash_attn_bwd_staged(pad(q), pad(k), pad(v), k_idx, bucket_off, bucket_cnt, groups, inv, pad(out),
+                                            lse, pad(dout), sm_scale, workspace_bytes=workspace_bytes, dlse=dlse)
+        dk2, dv2 = dk2[..., :64], dv2[..., :64]
+        if dk is not None:
+            dk2 = dk.add_(dk2)
+        if dv is not None:
+            dv2 = dv.add_(dv2)
+        return dq[..., :64].contiguous(), dk2.contiguous(), dv2.contiguous()
+    assert d == 128
     assert len(inv.row_pos) == H + 1 and inv.key_off.numel() == H * N + 1
     dq = torch.zeros_like(q)                                  # queries of an empty bucket keep 0
     if dk is None:

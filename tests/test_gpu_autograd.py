@@ -95,19 +95,26 @@ def test_reference_operator_schema():
     assert qs.grad is not None and bool(torch.isfinite(qs.grad).all()) and float(qs.grad.abs().sum()) > 0
 
 
-def test_module_forward_backward_against_joint_softmax():
+@pytest.mark.parametrize("dtype,H,G,S,N,d,C,Z,topk", [
+    (torch.float32, 2, 2, 24, 600, 64, 6, 40, 8),
+    (torch.float32, 1, 3, 9, 70, 16, 3, 70, 5),            # every key in every list; three query heads per KV head
+    (torch.float32, 2, 1, 33, 300, 128, 11, 7, 3),
+    (torch.bfloat16, 2, 2, 20, 500, 128, 5, 60, 8),        # the MFMA kernels, forward and backward
+    (torch.float16, 1, 4, 17, 400, 128, 7, 33, 6),
+    (torch.bfloat16, 2, 2, 12, 300, 64, 4, 50, 8),         # head dimension 64: the backward on padded rows
+])
+def test_module_forward_backward_against_joint_softmax(dtype, H, G, S, N, d, C, Z, topk):
     """ring_cross_attention_approx (memory.py:421-425, one device): the output is the softmax over the
     union of each query's bucket and its causal local prefix, and loss.backward() gives the gradients of
     exactly that function w.r.t. q, k_self, v_self, k and v (fp64 autograd on the GPU's own lists and
     hashes)."""
     from fast_memory_amd import compute_centroids, ops, ring_cross_attention_approx
-    g = gen(8300)
-    H, G, S, N, d, C, Z, topk = 2, 2, 24, 600, 64, 6, 40, 8
+    g = gen(8300 + S)
     sm = d ** -0.5
-    mk = lambda *s: (torch.randn(*s, generator=g) * 0.6)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.6).to(dtype)
     q, kq, ks, vs, k, v = mk(1, H * G, S, d), mk(1, H * G, N, d), mk(1, H, S, d), mk(1, H, S, d), mk(1, H, N, d), mk(1, H, N, d)
     w = mk(1, H * G, S, d)
-    cent0 = O.init_centroids(C, d, torch.float32)
+    cent0 = O.init_centroids(C, d, dtype)
     leaves = [t.requires_grad_(True) for t in dev(q, ks, vs, k, v)]
     qd, ksd, vsd, kd, vd = leaves
     out, hashes = ring_cross_attention_approx(qd, dev(kq), ksd, vsd, kd, vd, dev(cent0), sm, C, Z, centroid_topk=topk,
@@ -133,11 +140,13 @@ def test_module_forward_backward_against_joint_softmax():
         ref[0, hq, t] = o.detach()
         loss = loss + (o * w[0, hq, t].double()).sum()
     loss.backward()
-    assert torch.allclose(out.detach().cpu().double(), ref, atol=1e-4, rtol=1e-4)
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(out.detach().cpu().double(), ref, atol=tol, rtol=tol)
     for got, want, name in ((qd.grad, q64.grad, "dq"), (ksd.grad, ks64.grad, "dk_self"), (vsd.grad, vs64.grad, "dv_self"),
                             (kd.grad, k64.grad, "dk"), (vd.grad, v64.grad, "dv")):
         err = (got.cpu().double() - want).abs().max().item()
-        assert err <= 2e-4, f"{name}: max err {err:.3e}"
+        bound = 2e-4 if dtype == torch.float32 else 2e-2 * max(1.0, want.abs().max().item())
+        assert err <= bound, f"{name}: max err {err:.3e} (bound {bound:.1e})"
 
 
 def test_module_backward_notices_a_memory_changed_in_place():

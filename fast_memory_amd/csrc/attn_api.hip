@@ -54,6 +54,7 @@ extern "C" const char* fm_hash_attn_fwd_kernel(int H, int Sq, int N, int d, int 
   const int choice = hash_attn_mfma_choice(H, Sq, N, C);
   if (choice && N > (1 << 24))
     return dtype == FM_F16 ? "hash_attn_staged_kernel<1, f16, 64-bit rows>" : "hash_attn_staged_kernel<1, 64-bit rows>";
+  if (choice == 4) return dtype == FM_F16 ? "hash_attn_wave_kernel<f16>" : "hash_attn_wave_kernel";
   if (dtype == FM_F16)
     return choice == 3 ? "hash_attn_ring_kernel<f16>"
                        : choice == 2 ? "hash_attn_staged_kernel<2, f16>" : "hash_attn_staged_kernel<1, f16>";

@@ -502,6 +502,10 @@ int hash_attn_mfma_staged(const void* q, const void* k, const void* v, const int
                           const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
                           float* lse, int H, int Sq, int N, int C, float sm_scale, bool pairs, bool f16, bool per_row,
                           hipStream_t st);
+int hash_attn_mfma_wave(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
+                        const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items,
+                        const int32_t* n_items, int64_t max_items, void* out, float* lse, int Sq, int N, int C,
+                        float sm_scale, bool f16, int H, bool per_row, hipStream_t st);
 int hash_attn_mfma_ring(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                         const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items,
                         const int32_t* n_items, int64_t max_items, void* out, float* lse, int Sq, int N, int C,
@@ -510,7 +514,8 @@ extern std::atomic<int> g_force_generic;
 
 // Which grouped forward kernel a launch takes: 0 = rows gathered into registers (this file), 1 = rows
 // staged in LDS through registers, one work item per workgroup, 2 = the same, two items per workgroup,
-// 3 = rows loaded straight into LDS, three items per workgroup (attn_ring.hpp).  Measured rule: a kernel
+// 3 = rows loaded straight into LDS, three items per workgroup (attn_ring.hpp), 4 = the same loads, a wave
+// per work item (attn_wave.hpp; its rule stands further down).  Measured rule: a kernel
 // that shares a bucket's rows through LDS is at least as fast as the register-gather one wherever the launch
 // has work items enough to fill the chip (at least 512, taking min(Sq, C) per row as their number) or buckets
 // receive 24 queries or more on average; with few and small items the four waves of the gather kernel, which
@@ -536,7 +541,24 @@ extern std::atomic<int> g_force_generic;
 // 60 us is mostly start and tail; rows of 32 MB, 32 of them with 1024 buckets of 3072: 4.58 against 5.23.)
 static bool row_launches_pay(int choice, int H, int Sq, int N, int C) {
   return H > 1 && int64_t(H) * N * kD * 4 >= (int64_t(512) << 20) && int64_t(N) * kD * 4 >= (int64_t(32) << 20) &&
-         (C < Sq ? C : Sq) >= (choice == 3 ? 1024 : 1536);
+         (C < Sq ? C : Sq) >= (choice >= 3 ? 1024 : 1536);
+}
+
+// Form 4 (attn_wave.hpp: a wave per work item, eight buckets swept per compute unit instead of two) where the
+// launches go per row and a bucket receives few queries: there a launch is bound by the requests that miss the
+// L2s, and four times as many buckets in flight behind an L2 meet at more rows (requests answered by an L2,
+// 2^20 keys, 2048 buckets of 16384, 16 queries each: 32 % -> 42 %).  Its tile is 16 keys and a wave's MFMA and
+// softmax work grows with the queries of its item, so it loses from two tiles of queries per item on.  Measured
+// against form 3, both per row, lists in key order, queries assigned to buckets at random, per step (ms):
+//   8 rows of 2^20 keys, 2048 buckets of 16384; 4 / 8 / 16 / 24 / 32 queries per bucket on average:
+//     12.65 / 12.35 / 13.08 / 13.23 / 13.25 against 10.90 / 10.94 / 12.46 / 13.10 / 18.45
+//   8 rows of 2^20 keys, 4096 buckets of 4096; 4 / 8 / 16 / 24 / 32: 8.55 / 8.68 / 8.74 / 8.78 / 8.81 against
+//     6.94 / 7.03 / 7.37 / 7.47 / 9.00
+//   8 rows of 2^18 keys, 1024 buckets of 4096; 4 / 8 / 16: 1.54 / 1.51 / 1.52 against 1.26 / 1.44 / 1.60
+//   16 rows of 2^19 keys, 1024 buckets of 8192; 4 / 8 / 16: 5.83 / 5.83 / 5.89 against 4.90 / 5.49 / 6.29
+//   (with exactly 16 queries in every bucket, the first shape: 12.47 against 10.89)
+static bool wave_per_item_pays(int H, int Sq, int N, int C) {
+  return row_launches_pay(4, H, Sq, N, C) && int64_t(Sq) <= int64_t(C >= 2048 ? 16 : 8) * C;
 }
 
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
@@ -545,17 +567,19 @@ int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
   if (force == 2 || force == 6) return 1;
   if (force == 4) return N <= (1 << 24) ? 2 : 1;
   if (force == 5 || force == 7) return N <= (1 << 24) ? 3 : 1;
+  if (force >= 10 && force <= 12) return N <= (1 << 24) ? 4 : 1;
   const bool many_items = int64_t(H) * (Sq < C ? Sq : C) >= 512;
   const bool dense = Sq >= 24 * int64_t(C);
   if (!many_items && !dense) return 0;
-  return N <= (1 << 24) ? 3 : 1;
+  if (N > (1 << 24)) return 1;
+  return wave_per_item_pays(H, Sq, N, C) ? 4 : 3;
 }
 
-// One launch per row (forms 1 and 3 only).
+// One launch per row (forms 1, 3 and 4 only).
 bool hash_attn_mfma_per_row(int choice, int H, int Sq, int N, int C) {
   const int force = g_force_generic;
-  if ((choice != 1 && choice != 3) || force == 2 || force == 5) return false;
-  if (force == 6 || force == 7) return true;
+  if ((choice != 1 && choice != 3 && choice != 4) || force == 2 || force == 5 || force == 11) return false;
+  if (force == 6 || force == 7 || force == 12) return true;
   return row_launches_pay(choice, H, Sq, N, C);
 }
 
@@ -571,6 +595,9 @@ int hash_attn_mfma(const void* q, const void* k, const void* v, const int32_t* k
   int choice = hash_attn_mfma_choice(H, Sq, N, C);
   if (dtype == FM_F16 && choice == 0) choice = 1;
   const bool per_row = hash_attn_mfma_per_row(choice, H, Sq, N, C);
+  if (choice == 4)
+    return hash_attn_mfma_wave(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse, Sq,
+                               N, C, sm_scale, dtype == FM_F16, H, per_row, st);
   if (choice == 3)
     return hash_attn_mfma_ring(q, k, v, k_idx, bucket_off, bucket_cnt, q_perm, items, n_items, max_items, out, lse, Sq,
                                N, C, sm_scale, dtype == FM_F16, H, per_row, ws, ws_bytes, st);

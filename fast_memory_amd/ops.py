@@ -652,7 +652,9 @@ def grouped_forward_kernel(which: Optional[str]) -> None:
     kernel that shares a bucket's rows among its waves through LDS, one work item per workgroup, in a single
     launch, ``"staged-per-row"`` the same in one launch per row, ``"staged-pairs"`` the same kernel with two
     work items per workgroup, ``"ring"`` the kernel whose rows go from global memory straight into LDS (three
-    items per workgroup) in a single launch, ``"ring-per-row"`` the same in one launch per row, ``"gather"``
+    items per workgroup) in a single launch, ``"ring-per-row"`` the same in one launch per row, ``"wave"`` the kernel that
+    gives every work item a wave of its own in a single launch, ``"wave-per-row"`` the same in one launch per
+    row, ``"wave-auto"`` the same with the dispatch's own choice between the two, ``"gather"``
     always the kernel that gathers the rows into registers, ``"bwd-register-blocks"`` (backward only) makes the
     two-tile pass of the staged backward load its key blocks into registers instead of through LDS a block
     ahead, ``None`` restores the dispatch (the direct loads
@@ -661,4 +663,5 @@ def grouped_forward_kernel(which: Optional[str]) -> None:
     global _generic_forced
     _generic_forced = False
     _debug_lib().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4, "ring": 5,
-                                         "staged-per-row": 6, "ring-per-row": 7, "bwd-register-blocks": 9}[which])
+                                         "staged-per-row": 6, "ring-per-row": 7, "bwd-register-blocks": 9,
+                                         "wave-auto": 10, "wave": 11, "wave-per-row": 12}[which])

@@ -82,7 +82,7 @@ def test_attention_forward_fp16_many_queries_per_bucket(ops):
     qh[0, pos:] = 7
     ro, rl = O.hashed_attention_gather(q, k, v, kh, cnt, qh, 128 ** -0.5)
     outs = {}
-    for which in ("staged-pairs", "ring", "ring-per-row", "staged-per-row"):
+    for which in ("staged-pairs", "ring", "ring-per-row", "staged-per-row", "wave", "wave-per-row"):
         ops.grouped_forward_kernel(which)
         try:
             out, lse = attention_hash_varlen(*dev(q, k, v, kh, cnt, qh), 128 ** -0.5)
@@ -93,6 +93,9 @@ def test_attention_forward_fp16_many_queries_per_bucket(ops):
     assert torch.equal(outs["ring"][0], outs["staged-pairs"][0]) and torch.equal(outs["ring"][1], outs["staged-pairs"][1])
     for which in ("ring-per-row", "staged-per-row"):          # a launch per row: the same items, the same bits
         assert torch.equal(outs[which][0], outs["ring"][0]) and torch.equal(outs[which][1], outs["ring"][1])
+    # (the kernel with a wave per item takes its softmax in steps of 16 keys, not 64: other roundings than the
+    # rest, the same in both of its launch forms)
+    assert torch.equal(outs["wave-per-row"][0], outs["wave"][0]) and torch.equal(outs["wave-per-row"][1], outs["wave"][1])
 
 
 def test_composite_local_merge_and_backward_fp16(ops):

@@ -463,7 +463,8 @@ def test_attention_dense_buckets(dtype, d):
     assert_attn_close(out, lse, ro, rl, dtype, f"dense d={d}")
 
 
-@pytest.mark.parametrize("which", ["staged", "staged-per-row", "staged-pairs", "ring", "ring-per-row", "gather"])
+@pytest.mark.parametrize("which", ["staged", "staged-per-row", "staged-pairs", "ring", "ring-per-row", "wave",
+                                   "wave-per-row", "gather"])
 @pytest.mark.parametrize("case", ["ragged", "full-items", "reference-large", "heavy-bucket"])
 def test_attention_grouped_forward_kernels(ops, which, case):
     # the bf16 d=128 forward kernels (rows shared through LDS, one or two work items per workgroup / rows
@@ -617,7 +618,7 @@ def test_attention_a_launch_per_row_finds_every_rows_items(ops):
     qh[5, :40] = torch.arange(40) % C           # the rest of row 5 in no bucket
     qh[5, 40:] = -1
     res = []
-    for which in ("staged", "staged-per-row", "ring", "ring-per-row"):
+    for which in ("staged", "staged-per-row", "ring", "ring-per-row", "wave", "wave-per-row"):
         ops.grouped_forward_kernel(which)
         try:
             qd, kd, vd, khd, cntd, qhd = dev(q, k, v, kh, cnt, qh)
@@ -637,13 +638,14 @@ def test_attention_a_launch_per_row_finds_every_rows_items(ops):
             ops.grouped_forward_kernel(None)
     assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
     assert torch.equal(res[2][0], res[3][0]) and torch.equal(res[2][1], res[3][1])
+    assert torch.equal(res[4][0], res[5][0]) and torch.equal(res[4][1], res[5][1])
     for _, lse_r in res:
         assert bool((lse_r[3] < -1e30).all()) and bool((lse_r[10] < -1e30).all())         # rows without a bucket
         assert bool((lse_r[5, 40:] < -1e30).all())
         assert bool((lse_r[0] != 7.0).all())
 
 
-@pytest.mark.parametrize("which", ["staged", "staged-pairs", "ring", "gather", "generic"])
+@pytest.mark.parametrize("which", ["staged", "staged-pairs", "ring", "wave", "gather", "generic"])
 def test_attention_out_of_range_list_entries_are_clamped(ops, which):
     # the contract of every entry point: key indices outside [0, N) are clamped, never dereferenced
     # (negative -> key 0, >= N -> key N-1); lists here hold such entries in every bucket, and lists

@@ -107,14 +107,14 @@ def cpu_timed(fn, reps=3):
 
 def no_reuse_control(dev, reps=3, list_order="key", force=None):
     """fm_hash_attn_fwd on lists that name every key and value row exactly once: H = 8 rows of N = 2^24 keys,
-    C = 1024 buckets of Z = 16384 keys = a seeded permutation of the keys, 16 queries per bucket (c5's
-    average).  K and V are 69 GB, far beyond the 256 MB last-level cache, and no row is listed twice, so
+    C = 2048 buckets (c5's number) of Z = 8192 keys = a seeded permutation of the keys, 16 queries per bucket
+    (c5's average).  K and V are 69 GB, far beyond the 256 MB last-level cache, and no row is listed twice, so
     every gathered byte comes from HBM: the rate the gather kernel reaches here is an HBM rate, which the
     c5 figure (every key listed in ~32 buckets) is not.  Timed with the lists in the order the step reads
     them (``list_order``) and, beside it, in the other one.  ``force`` (a name :func:`ops.grouped_forward_kernel`
     takes) overrides the library's dispatch, which takes the kernel and the launch per row of c5 here too."""
     from fast_memory_amd import ops
-    H, C, Z, d, per_bucket = 8, 1024, 16384, 128, 16
+    H, C, Z, d, per_bucket = 8, 2048, 8192, 128, 16
     N, Sq = C * Z, per_bucket * C
     k = torch.empty((H, N, d), dtype=torch.bfloat16, device=dev).normal_()
     v = torch.empty((H, N, d), dtype=torch.bfloat16, device=dev).normal_()

@@ -33,15 +33,20 @@ int fm_debug_hooks_enabled(void);
  * head dimensions 64 and 256 instantiated for 128 (tests compare it with the kernels
  * built for 128); 9 = (backward) the two-tile pass of fm_hash_attn_bwd_staged
  * loads its key blocks into registers as its other passes do, instead of through
- * LDS a block ahead (tests compare the two, which give the same bits).  Dispatch: gather
+ * LDS a block ahead (tests compare the two, which give the same bits); 10 = the
+ * kernel with a wave per work item, launched as dispatch would launch it, 11 = that
+ * kernel in a single launch, 12 = in one launch per row.  Dispatch: gather
  * when H min(Sq, C) < 512 and Sq < 24 C; else the direct loads up to 2^24 keys and
  * the staged kernel beyond; one launch per row when K and V of all rows are 512 MB
  * or more, those of a row 32 MB or more, and a row has 1024 (staged kernel: 1536)
- * or more buckets and queries. */
+ * or more buckets and queries; where the launches go per row, a row has 2048 or
+ * more buckets and queries and a bucket receives 16 queries or fewer on average,
+ * the kernel with a wave per work item in place of the direct loads. */
 void fm_debug_force_generic(int on);
 
 /* Diagnostic: name of the kernel fm_hash_attn_fwd launches for these extents
- * (a static string): "hash_attn_generic_kernel", "hash_attn_mfma_kernel" (rows
+ * (a static string): "hash_attn_generic_kernel", "hash_attn_wave_kernel" (a wave per work item),
+ * "hash_attn_mfma_kernel" (rows
  * gathered into registers), "hash_attn_staged_kernel<1>" or "...<2>" (rows staged
  * in LDS through registers, one or two work items per workgroup),
  * "hash_attn_ring_kernel" (rows loaded straight into LDS, three work items per

@@ -126,8 +126,9 @@ def test_grouped_forward_dispatch_rule():
     assert name(8, 32769, 1048576, 128, 2048, 1) == "hash_attn_ring_kernel"           # ... more than 16
     assert name(1, 32768, 1048576, 128, 2048, 1) == "hash_attn_ring_kernel"           # ... a single row (one launch)
     assert name(8, 16384, 262144, 128, 1024, 1) == "hash_attn_ring_kernel"            # 256 K keys, 16 queries / bucket
-    assert name(8, 8192, 262144, 128, 1024, 1) == "hash_attn_wave_kernel"             # ... 8 queries / bucket
-    assert name(8, 8192, 262144, 128, 512, 1) == "hash_attn_ring_kernel"              # ... too few buckets per row
+    assert name(8, 8192, 262144, 128, 1024, 1) == "hash_attn_ring_kernel"             # ... 8 / bucket: too few buckets per row
+    assert name(8, 16384, 1048576, 128, 4096, 1) == "hash_attn_wave_kernel"           # 4096 buckets, 4 queries / bucket
+    assert name(8, 2047, 1048576, 128, 4096, 1) == "hash_attn_ring_kernel"            # ... too few queries per row
     assert name(8, 32768, (1 << 24) + 64, 128, 2048, 1) == "hash_attn_staged_kernel<1, 64-bit rows>"
     assert name(8, 8192, 32768, 128, 256, 1) == "hash_attn_ring_kernel"               # prefill chunk, 32 / bucket
     assert name(8, 131072, 65536, 128, 1024, 1) == "hash_attn_ring_kernel"       # reference harness, 128 / bucket

@@ -188,6 +188,7 @@ __device__ __forceinline__ void attend_ring(const bf16_t* __restrict__ Qb, const
           s[qt][kt] = Mma<F16>::m16(a, qf[qt][st], st == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[qt][kt]);
       }
     }
+    mfma_settle_scores<T>(s);  // (a branch follows: see mma16.hpp)
     const int kp0 = t * 64;
     if (kp0 + 64 > cnt) {  // the bucket's last, ragged tile
 #pragma unroll

@@ -208,6 +208,7 @@ __device__ __forceinline__ void attend_staged(
           s[qt][kt] = Mma<F16>::m16(a, qf[qt][st], st == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[qt][kt]);
       }
     }
+    mfma_settle_scores<NQW>(s);  // (a branch follows: see mma16.hpp)
     if (kp0 + kSK > cnt) {  // the bucket's last, ragged tile
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)

@@ -159,6 +159,10 @@ __device__ __forceinline__ void attend_staged_d(const bf16_t* __restrict__ Qb, c
         s[kt] = Mma<F16>::m16(a, qf[st], st == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[kt]);
       }
     }
+    {  // (a branch follows: see mfma_settle in mma16.hpp)
+      f32x4(&s1)[1][4] = reinterpret_cast<f32x4(&)[1][4]>(s);
+      mfma_settle_scores<1>(s1);
+    }
     if (kp0 + 64 > cnt) {  // the bucket's last, ragged tile
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)

@@ -33,21 +33,16 @@ constexpr int kWTileBytes = 16 * 256;                  // 16 rows of 128 two-byt
 constexpr int kWWaveBytes = 512 + 4 * kWTileBytes;     // two buffers of list entries, two tiles of K and V
 constexpr size_t kWaveLdsBytes = size_t(4) * kWWaveBytes;
 
-// A vector instruction may read what an MFMA of 8 passes wrote 11 issue slots after it at the earliest.  The
-// compiler counts them within a basic block and fills up with s_nop, but not across a branch: with the branch
-// around the masking of a ragged tile between the last MFMA of S^T and the row maxima, the maxima were taken
-// from registers the MFMA had not written yet (the results still met the oracle, the softmax being the same
-// for any running maximum, but the rounding of P changed from run to run).  The slots are spent here, in a
-// statement that the values pass through.
+// (the slots an MFMA's result needs before a vector instruction may touch it: mfma_settle in mma16.hpp)
 template <int T>
 __device__ __forceinline__ void wave_mfma_settle(f32x4 (&x)[T]) {
   static_assert(T >= 1 && T <= 3, "one to three accumulators");
   if constexpr (T == 1)
-    asm volatile("s_nop 7\n\ts_nop 3" : "+v"(x[0]));
+    mfma_settle(x[0]);
   else if constexpr (T == 2)
-    asm volatile("s_nop 7\n\ts_nop 3" : "+v"(x[0]), "+v"(x[1]));
+    mfma_settle(x[0], x[1]);
   else
-    asm volatile("s_nop 7\n\ts_nop 3" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]));
+    mfma_settle(x[0], x[1], x[2]);
 }
 
 // The attention of n_q <= 16 NQW queries (rows q_rows[0..n_q) of Qb / Ob / Lb) over the cnt keys idx[0..cnt)

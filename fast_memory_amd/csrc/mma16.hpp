@@ -63,4 +63,35 @@ struct Mma {
   }
 };
 
+// A vector instruction may touch what an MFMA of 8 passes wrote 11 issue slots after it at the earliest.  The
+// compiler counts the slots within a basic block and fills up with s_nop, but not across a branch -- and the
+// attention kernels have one, around the masking of a ragged tile, between the last MFMAs of the scores and
+// the row maxima.  Read too early, a maximum comes from a register the MFMA has not written yet: the online
+// softmax gives the same result for any running maximum, so results still meet the oracle, but the rounding
+// of P, and with it the output bits, then depend on timing (seen with one slot between: outputs differing in
+// the last bit from run to run).  These statements spend the slots (other waves of the SIMD issue meanwhile)
+// and take the accumulators through, so that every later use of them comes after.
+#define FM_MFMA_SETTLE "s_nop 7\n\ts_nop 3"
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float settle_f4;
+__device__ __forceinline__ void mfma_settle(settle_f4& a) { asm volatile(FM_MFMA_SETTLE : "+v"(a)); }
+__device__ __forceinline__ void mfma_settle(settle_f4& a, settle_f4& b) { asm volatile(FM_MFMA_SETTLE : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void mfma_settle(settle_f4& a, settle_f4& b, settle_f4& c) {
+  asm volatile(FM_MFMA_SETTLE : "+v"(a), "+v"(b), "+v"(c));
+}
+// the accumulators of T query tiles x 4 key tiles
+template <int T, int NQW>
+__device__ __forceinline__ void mfma_settle_scores(settle_f4 (&s)[NQW][4]) {
+  static_assert(T >= 1 && T <= 3 && T <= NQW, "one to three query tiles");
+  if constexpr (T == 1)
+    asm volatile(FM_MFMA_SETTLE : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[0][2]), "+v"(s[0][3]));
+  else if constexpr (T == 2)
+    asm volatile(FM_MFMA_SETTLE
+                 : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[0][2]), "+v"(s[0][3]), "+v"(s[1][0]), "+v"(s[1][1]), "+v"(s[1][2]),
+                   "+v"(s[1][3]));
+  else
+    asm volatile(FM_MFMA_SETTLE
+                 : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[0][2]), "+v"(s[0][3]), "+v"(s[1][0]), "+v"(s[1][1]), "+v"(s[1][2]),
+                   "+v"(s[1][3]), "+v"(s[2][0]), "+v"(s[2][1]), "+v"(s[2][2]), "+v"(s[2][3]));
+}
+
 }  // namespace fm

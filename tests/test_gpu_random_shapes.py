@@ -301,3 +301,55 @@ def test_mfma_kernels_against_generic_random_extents(dt, B, S, N, C, Z, d, skew,
         a, b = a.float(), b.float()
         assert torch.allclose(a, b, atol=2e-2 * max(1.0, b.abs().max().item()), rtol=2e-2), \
             f"{name}: {(a - b).abs().max().item():.3e} vs max {b.abs().max().item():.3e}"
+
+
+def _forced_cases(n, seed):
+    rng = random.Random(seed)
+    out = []
+    for i in range(n):
+        which = ("wave", "wave-per-row", "ring", "ring-per-row", "staged", "staged-pairs")[i % 6]
+        dt = rng.choice(["bf16", "f16"])
+        B = rng.choice([1, 2, 3])
+        N = rng.randint(40, 6000)
+        C = rng.randint(1, 48)
+        Z = rng.randint(1, min(N, 700))
+        S = rng.randint(1, 1500)
+        out.append(pytest.param(which, dt, B, S, N, C, Z, rng.random() < 0.4, seed + i, id=f"{i}-{which}-{dt}-B{B}-S{S}-N{N}-C{C}-Z{Z}"))
+    return out
+
+
+@pytest.mark.parametrize("which,dt,B,S,N,C,Z,skew,seed", _forced_cases(48, 20266))
+def test_forced_forward_kernels_against_generic_and_themselves_random_extents(which, dt, B, S, N, C, Z, skew, seed):
+    """Each d = 128 forward kernel forced on shapes dispatch would never give it (a wave per work item on short
+    lists and on items of 49-64 queries, which it sweeps twice; three items per workgroup on single-query
+    buckets, ...): against the generic kernel on the same device inputs, and twice in a row with the same bits
+    (a result may not depend on timing)."""
+    from fast_memory_amd import attention_hash_varlen, ops
+    dtype = _DT[dt]
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    mk = lambda *s: (torch.randn(*s, generator=g, device="cuda") * 0.6).to(dtype)
+    q, k, v = mk(B, S, 128), mk(B, N, 128), mk(B, N, 128)
+    lists = torch.randint(0, N, (B, C, Z), generator=g, device="cuda", dtype=torch.int32).sort(-1).values
+    cnt = torch.randint(0, Z + 1, (B, C), generator=g, device="cuda", dtype=torch.int32)       # ragged, some empty
+    keep = torch.arange(Z, device="cuda")[None, None, :] < cnt[..., None]
+    flat = lists[keep].contiguous()
+    qh = torch.randint(0, C, (B, S), generator=g, device="cuda", dtype=torch.int32)
+    if skew:
+        qh[:, : S // 3] = C // 2
+    run = lambda: attention_hash_varlen(q, k, v, flat, cnt, qh, 128 ** -0.5, lse_dtype=torch.float32)
+    ops.grouped_forward_kernel(which)
+    try:
+        o1, l1 = run()
+        o1b, l1b = run()
+    finally:
+        ops.grouped_forward_kernel(None)
+    assert torch.equal(o1, o1b) and torch.equal(l1, l1b), "two runs of one kernel on the same inputs differ"
+    ops.force_generic_kernels(True)
+    try:
+        o2, l2 = run()
+    finally:
+        ops.force_generic_kernels(False)
+    empty = l2 < -1e30
+    assert torch.equal(l1 < -1e30, empty)
+    assert torch.allclose(o1.float(), o2.float(), atol=2e-2, rtol=1e-2)
+    assert (l1[~empty] - l2[~empty]).abs().max().item() < 1e-3 if (~empty).any() else True

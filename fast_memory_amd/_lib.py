@@ -42,6 +42,7 @@ SIGNATURES = {
     "fm_hash_attn_fwd": (c_int, [P, P, P, P, P, P, P, P, P, c_int64, P, P, c_int, c_int, c_int, c_int,
                                  c_int, c_float, c_int, P]),
     "fm_hash_attn_fwd_workspace": (c_size_t, [c_int64]),
+    "fm_debug_wave_pace_state": (c_int, [c_int, c_int, c_int, c_void_p, c_int, c_void_p]),
     "fm_hash_attn_fwd_ws": (c_int, [P, P, P, P, P, P, P, P, P, c_int64, P, P, c_int, c_int, c_int, c_int,
                                     c_int, c_float, c_int, P, c_size_t, P]),
     "fm_lists_key_order": (c_int, [P, P, P, c_int64, c_int, P, P, P]),

@@ -75,6 +75,14 @@ extern "C" const char* fm_local_attn_fwd_kernel(int G, int S, int L, int d, int 
   return dtype == FM_F16 ? "local_attn_dense_kernel<f16, 256>" : "local_attn_dense_kernel<bf16, 256>";
 }
 
+namespace fm {
+int wave_pace_state(int N, int C, int Sq, const void* lists, int row, float* out);
+}
+extern "C" int fm_debug_wave_pace_state(int N, int C, int Sq, const void* k_idx, int row, float* out6) {
+  if (!out6) return FM_ERR_ARG;
+  return fm::wave_pace_state(N, C, Sq, k_idx, row, out6);
+}
+
 extern "C" int fm_hash_attn_fwd_launches(int H, int Sq, int N, int d, int C, int dtype) {
   using namespace fm;
   if (g_force_generic == 1 || !hash_attn_mfma_supported(d, dtype, N) || d != 128 || g_force_generic == 8) return 1;

@@ -572,7 +572,7 @@ int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
   if (force == 2 || force == 6) return 1;
   if (force == 4) return N <= (1 << 24) ? 2 : 1;
   if (force == 5 || force == 7) return N <= (1 << 24) ? 3 : 1;
-  if (force >= 10 && force <= 12) return N <= (1 << 24) ? 4 : 1;
+  if (force >= 10 && force <= 13) return N <= (1 << 24) ? 4 : 1;
   const bool many_items = int64_t(H) * (Sq < C ? Sq : C) >= 512;
   const bool dense = Sq >= 24 * int64_t(C);
   if (!many_items && !dense) return 0;
@@ -584,7 +584,7 @@ int hash_attn_mfma_choice(int H, int Sq, int N, int C) {
 bool hash_attn_mfma_per_row(int choice, int H, int Sq, int N, int C) {
   const int force = g_force_generic;
   if ((choice != 1 && choice != 3 && choice != 4) || force == 2 || force == 5 || force == 11) return false;
-  if (force == 6 || force == 7 || force == 12) return true;
+  if (force == 6 || force == 7 || force == 12 || force == 13) return true;
   return row_launches_pay(choice, H, Sq, N, C);
 }
 

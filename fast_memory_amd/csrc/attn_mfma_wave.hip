@@ -1,9 +1,86 @@
 // Launch of the bucket-gathered attention that gives every work item a wave of its own (attn_wave.hpp): four
 // items per workgroup of 256 threads, two workgroups per compute unit, no barriers.  The form for long lists
 // with few queries each on a memory whose key rows are listed in many buckets.
+#include <atomic>
+#include <mutex>
+#include <unordered_map>
+
 #include "attn_wave.hpp"
 
 namespace fm {
+
+extern std::atomic<int> g_force_generic;  // attn_api.hip; 13: a launch per row with the sweeps unpaced
+
+// The schedule of a paced launch (WaveClock in attn_wave.hpp) is found by trying, launch after launch, for
+// every (memory, lists, row) the library sees: a table of the library's own in device memory, one copy per
+// GPU, a slot per (N, C, Sq, the lists' address, the row) -- the host hands the slots out (the 1024 keys seen
+// last have one each).  The last wave of a launch to finish
+// (every wave counts itself out) compares the launch's duration with its schedule and sets the next one:
+//   * no schedule yet: the launch ran unpaced; the next gets 0.9 x its duration;
+//   * schedule kept (duration <= 1.02 x schedule + 15 us): unless held, try one 2 % faster;
+//   * schedule missed while trying a faster one: back to 1.01 x the last one kept, held for 256 launches;
+//   * schedule missed at one that had been kept: 3 % slower, held for 256 launches; after 8 misses in a row or
+//     beyond 1.1 x the unpaced duration the slot gives up for 512 launches (unpaced), then starts again.
+// A missed schedule costs that launch up to a third of its time, a kept one saves a fifth; once settled a
+// slot misses one launch in about 256.  Calls that use a slot at the same time (two streams on one memory and
+// row; two keys on one slot) mix their measurements: the schedule may then be a poor one, nothing else.
+struct WavePaceSlot {
+  unsigned long long key;   // whose slot this is (0: nobody's)
+  unsigned long long t0;    // start of the launch in flight (0: none has started)
+  unsigned int done;        // waves of it that have finished
+  int mode;                 // 0 the next launch runs unpaced and is measured, 1 paced, 2 given up (hold counts down)
+  float tpk;                // ticks per key of the next launch
+  float good;               // the fastest schedule kept so far (0: none)
+  float base;               // ticks per key of the unpaced launch
+  int hold;                 // launches until the next try of a faster schedule / of pacing at all
+  int misses;               // schedules missed in a row
+  int pad[3];
+};
+constexpr int kWavePaceSlots = 1024;
+static __device__ __align__(256) WavePaceSlot g_wave_pace[kWavePaceSlots];
+
+// What the last wave of a launch does with the slot (one lane).  elapsed: ticks since the launch's first wave
+// started; tpk_used: the schedule the launch ran on (0: unpaced).
+__device__ inline void wave_pace_update(WavePaceSlot* s, unsigned long long key, float elapsed, float tpk_used, int N) {
+  if (s->key != key) {  // (first use, or another memory's slot: start over)
+    s->key = key;
+    s->mode = 0;
+    s->good = 0.f;
+    s->hold = 0;
+    s->misses = 0;
+  }
+  if (tpk_used <= 0.f) {
+    if (s->mode == 2 && --s->hold > 0) {
+      s->tpk = 0.f;
+    } else {
+      s->base = elapsed / float(N);
+      s->tpk = 0.9f * s->base;
+      s->mode = 1;
+      s->good = 0.f;
+      s->hold = 0;
+      s->misses = 0;
+    }
+  } else if (elapsed <= 1.02f * tpk_used * float(N) + 1500.f) {
+    s->good = tpk_used;
+    s->misses = 0;
+    if (s->hold > 0)
+      --s->hold;
+    else
+      s->tpk = fmaxf(0.98f * tpk_used, 0.4f * s->base);
+  } else {
+    ++s->misses;
+    // a faster schedule than the last one kept was being tried: back to just above that one; else the one
+    // held has stopped working: a little slower
+    s->tpk = (s->good > 0.f && tpk_used < 0.995f * s->good) ? 1.01f * s->good : 1.03f * tpk_used;
+    s->good = s->tpk;
+    s->hold = 256;
+    if (s->misses > 8 || s->tpk > 1.1f * s->base) {
+      s->mode = 2;
+      s->hold = 512;
+      s->tpk = 0.f;
+    }
+  }
+}
 
 template <bool F16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void hash_attn_wave_kernel(
@@ -11,7 +88,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int32_t* __restrict__ k_idx, const int64_t* __restrict__ bucket_off,
     const int32_t* __restrict__ bucket_cnt, const int32_t* __restrict__ q_perm,
     const fm_item* __restrict__ items, const int32_t* __restrict__ n_items,
-    bf16_t* __restrict__ out, float* __restrict__ lse, int Sq, int N, int C, float scale2, int only_row) {
+    bf16_t* __restrict__ out, float* __restrict__ lse, int Sq, int N, int C, float scale2, int only_row,
+    WavePaceSlot* __restrict__ pace, unsigned long long pace_key) {
   extern __shared__ __attribute__((aligned(16))) bf16_t wave_lds[];
   int n_it = *n_items;
   int first = 0;
@@ -25,42 +103,152 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const fm_item it = items[me];
   const int64_t bkt = int64_t(it.row) * C + it.bucket;
   const int64_t qbase = int64_t(it.row) * Sq;
-  // (an item has up to FM_QTILE = 64 queries, a sweep takes 48: the few items with more are swept twice)
-  for (int q0 = 0; q0 < it.n_q; q0 += 48)
+  // The launch's schedule and start (WaveClock): the first wave to come sets the start.
+  WaveClock clk{0, 0.f};
+  float tpk_used = 0.f;
+  if (pace) {
+    unsigned long long t0 = 0;
+    float tpk = 0.f;
+    if ((threadIdx.x & 63) == 0) {
+      const unsigned long long now = __builtin_amdgcn_s_memrealtime();
+      unsigned long long old = atomicCAS(&pace->t0, 0ull, now);
+      if (old && now - old > (1ull << 28)) {  // a start 2.7 s old: a launch never counted itself out (two calls
+        // mixed on the slot with different numbers of waves); start over
+        if (atomicCAS(&pace->t0, old, now) == old) atomicExch(&pace->done, 0u);
+        old = 0;
+      }
+      t0 = old ? old : now;
+      tpk = pace->key == pace_key && pace->mode == 1 ? pace->tpk : 0.f;
+    }
+    t0 = (uint64_t(__builtin_amdgcn_readfirstlane(uint32_t(t0 >> 32))) << 32) | __builtin_amdgcn_readfirstlane(uint32_t(t0));
+    tpk_used = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, tpk)));
+    clk = WaveClock{t0, tpk_used};
+  }
+  // (an item has up to FM_QTILE = 64 queries, a sweep takes 48: the few items with more are swept twice, the
+  // second time unpaced)
+  for (int q0 = 0; q0 < it.n_q; q0 += 48) {
     attend_wave<3, F16>(q + qbase * kSD, q_perm + it.q_start + q0, min(it.n_q - q0, 48), k + int64_t(it.row) * N * kSD,
                         v + int64_t(it.row) * N * kSD, k_idx + bucket_off[bkt], bucket_cnt[bkt], N, scale2,
-                        out + qbase * kSD, lse + qbase, (lds_char_t*)wave_lds + w * kWWaveBytes);
+                        out + qbase * kSD, lse + qbase, (lds_char_t*)wave_lds + w * kWWaveBytes, clk);
+    clk.ticks_per_key = 0.f;
+  }
+  // Every wave counts itself out; the last one sets the next launch's schedule and clears the way for it.
+  if (pace && (threadIdx.x & 63) == 0) {
+    const unsigned int n_waves = unsigned(n_it - first);
+    if (atomicAdd(&pace->done, 1u) + 1u == n_waves) {
+      const unsigned long long now = __builtin_amdgcn_s_memrealtime();
+      const unsigned long long t0 = atomicAdd(&pace->t0, 0ull);
+      wave_pace_update(pace, pace_key, float(now - t0), tpk_used, N);
+      __threadfence();
+      pace->done = 0u;
+      atomicExch(&pace->t0, 0ull);
+    }
+  }
+}
+
+// The table's address on the current device (in host code its name only stands for the symbol).
+static WavePaceSlot* wave_pace_table() {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static WavePaceSlot* table[kMaxDevices];
+  static bool asked[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!asked[dev]) {
+    asked[dev] = true;
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_wave_pace)) == hipSuccess)
+      table[dev] = static_cast<WavePaceSlot*>(p);
+    else
+      (void)hipGetLastError();
+  }
+  return table[dev];
+}
+
+// The slot of a key: the keys in use have a slot each; the 1025th new key takes over the slot handed out
+// longest ago (the kernel sees another key in it and starts that slot over).
+static int wave_pace_slot(unsigned long long key) {
+  static std::mutex mu;
+  static std::unordered_map<unsigned long long, int> slot_of;
+  static unsigned long long owner[kWavePaceSlots];
+  static int next = 0;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = slot_of.find(key);
+  if (it != slot_of.end()) return it->second;
+  const int s = next;
+  next = (next + 1) % kWavePaceSlots;
+  if (owner[s]) slot_of.erase(owner[s]);
+  owner[s] = key;
+  slot_of[key] = s;
+  return s;
+}
+
+static unsigned long long wave_pace_key(int N, int C, int Sq, const void* lists, int row) {
+  unsigned long long x = (unsigned long long)(uintptr_t)lists ^ ((unsigned long long)N << 40) ^ ((unsigned long long)C << 20) ^
+                         ((unsigned long long)Sq * 0x9E3779B97F4A7C15ull) ^ ((unsigned long long)(row + 1) * 0xC2B2AE3D27D4EB4Full);
+  x ^= x >> 30; x *= 0xBF58476D1CE4E5B9ull;
+  x ^= x >> 27; x *= 0x94D049BB133111EBull;
+  x ^= x >> 31;
+  return x | 1ull;
 }
 
 int hash_attn_mfma_wave(const void* q, const void* k, const void* v, const int32_t* k_idx, const int64_t* bucket_off,
                         const int32_t* bucket_cnt, const int32_t* q_perm, const fm_item* items,
                         const int32_t* n_items, int64_t max_items, void* out, float* lse, int Sq, int N, int C,
                         float sm_scale, bool f16, int H, bool per_row, hipStream_t st) {
+  // paced sweeps for the launches per row (a single launch over all rows has no common sweep to pace)
+  WavePaceSlot* const table = per_row && g_force_generic != 13 ? wave_pace_table() : nullptr;
 #define FM_WAVE_LAUNCH(F16, ITEMS, ROW)                                                                           \
   do {                                                                                                            \
     FM_ALLOW_LDS((hash_attn_wave_kernel<F16>), kWaveLdsBytes, "fm_hash_attn_fwd: lds");                           \
     hipLaunchKernelGGL((hash_attn_wave_kernel<F16>), dim3(unsigned(ceil_div(int64_t(ITEMS), int64_t(4)))),        \
                        dim3(256), kWaveLdsBytes, st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, k_idx, \
                        bucket_off, bucket_cnt, q_perm, items, n_items, (bf16_t*)out, lse, Sq, N, C,               \
-                       sm_scale * kLog2e, ROW);                                                                   \
+                       sm_scale * kLog2e, ROW, pace_slot, pace_key);                                              \
   } while (0)
   if (per_row) {
     // One launch per row, in row order, for the reason given in attn_mfma_ring.hip: the waves of a launch start
     // together and sweep the row's K and V at about the same pace.
     const int64_t row_items = std::min<int64_t>(max_items, int64_t(C < Sq ? C : Sq) + Sq / FM_QTILE + 1);
     for (int row = 0; row < H; ++row) {
+      const unsigned long long pace_key = wave_pace_key(N, C, Sq, k_idx, row);
+      WavePaceSlot* const pace_slot = table ? table + wave_pace_slot(pace_key) : nullptr;
       if (f16)
         FM_WAVE_LAUNCH(true, row_items, row);
       else
         FM_WAVE_LAUNCH(false, row_items, row);
     }
-  } else if (f16) {
-    FM_WAVE_LAUNCH(true, max_items, -1);
   } else {
-    FM_WAVE_LAUNCH(false, max_items, -1);
+    const unsigned long long pace_key = 0;
+    WavePaceSlot* const pace_slot = nullptr;
+    if (f16)
+      FM_WAVE_LAUNCH(true, max_items, -1);
+    else
+      FM_WAVE_LAUNCH(false, max_items, -1);
   }
 #undef FM_WAVE_LAUNCH
   return launch_status("fm_hash_attn_fwd(mfma, wave)");
+}
+
+// out[0..5] = mode, ticks per key of the next launch, the fastest schedule kept, ticks per key unpaced, hold,
+// misses of the slot of (N, C, Sq, lists, row); all zero where there is none yet.  A synchronous copy.
+int wave_pace_state(int N, int C, int Sq, const void* lists, int row, float* out) {
+  for (int i = 0; i < 6; ++i) out[i] = 0.f;
+  WavePaceSlot* const table = wave_pace_table();
+  if (!table) return FM_ERR_LAUNCH;
+  const unsigned long long key = wave_pace_key(N, C, Sq, lists, row);
+  WavePaceSlot h;
+  if (hipMemcpy(&h, table + wave_pace_slot(key), sizeof(h), hipMemcpyDeviceToHost) != hipSuccess) {
+    (void)hipGetLastError();
+    return FM_ERR_LAUNCH;
+  }
+  if (h.key != key) return FM_OK;
+  out[0] = float(h.mode); out[1] = h.tpk; out[2] = h.good; out[3] = h.base; out[4] = float(h.hold); out[5] = float(h.misses);
+  return FM_OK;
 }
 
 }  // namespace fm

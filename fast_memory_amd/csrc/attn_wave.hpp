@@ -33,6 +33,30 @@ constexpr int kWTileBytes = 16 * 256;                  // 16 rows of 128 two-byt
 constexpr int kWWaveBytes = 512 + 4 * kWTileBytes;     // two buffers of list entries, two tiles of K and V
 constexpr size_t kWaveLdsBytes = size_t(4) * kWWaveBytes;
 
+// Pacing of the sweeps.  The requests of two buckets for one row meet in the L2 only while that row is still
+// there, and the 4 MB of an L2 hold the rows of about 8000 consecutive keys: the waves behind one L2 have to
+// sweep the key range within that distance of each other.  Left alone they do not -- entry i of a sorted list
+// lies where the list's own density puts it (a standard deviation of 4000 keys in the middle of 16384 entries
+// among 2^20 keys), and a wave with more queries takes longer per tile.  Talking to each other costs the waves
+// more than it wins (a line that 256 waves read and write).  They share a clock, though (s_memrealtime, 100
+// MHz, the same for every wave of the device): a launch has a schedule, key x is due t0 + x * ticks_per_key,
+// and a wave asks for a tile only once its first key is due (less a margin).  Waves that are behind run free,
+// waves that are ahead wait, and if the schedule is one the launch can keep, all of them sweep the key range
+// together and the launch ends on schedule -- sooner than it ends unpaced (2^20 keys, 2048 buckets of 16384:
+// 1.32 ms per launch unpaced, 1.05 ms on a schedule of 1.0 ms; on a schedule it cannot keep, 1.43 ms).  Which
+// schedule a launch can keep is found by trying (WavePaceSlot).  A wait ends after kWaveGateTicks at the
+// latest and a wave stops pacing after kWaveLongWaits such waits or kWaveSpinLimit looks at the clock in all
+// (lists that do not ascend; a clock that stands still), so every wave ends whatever the clock says.  The
+// clock only delays loads: results do not depend on it.
+struct WaveClock {
+  uint64_t t0;          // the launch's start
+  float ticks_per_key;  // 0: unpaced
+};
+constexpr int kWaveMarginKeys = 2048;   // how far ahead of the schedule a wave may ask
+constexpr int kWaveGateTicks = 2000;    // 20 us: the longest single wait
+constexpr int kWaveLongWaits = 4;
+constexpr int kWaveSpinLimit = 40000;
+
 // (the slots an MFMA's result needs before a vector instruction may touch it: mfma_settle in mma16.hpp)
 template <int T>
 __device__ __forceinline__ void wave_mfma_settle(f32x4 (&x)[T]) {
@@ -52,7 +76,7 @@ template <int NQW, bool F16>
 __device__ __forceinline__ void attend_wave(const bf16_t* __restrict__ Qb, const int* __restrict__ q_rows, int n_q,
                                             const bf16_t* Kb, const bf16_t* Vb, const int32_t* idx, int cnt, int N,
                                             float scale2, bf16_t* __restrict__ Ob, float* __restrict__ Lb,
-                                            lds_char_t* lds) {
+                                            lds_char_t* lds, const WaveClock clk) {
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane(uint32_t(uintptr_t(lds)));
   const int l = threadIdx.x & 63;
   const int g = l >> 4, c = l & 15;
@@ -101,13 +125,33 @@ __device__ __forceinline__ void attend_wave(const bf16_t* __restrict__ Qb, const
     ring_load4(lds0 + uint32_t(b & 1) * 256u, uint32_t(kp) * 4u, idx);
   };
   uint32_t rows[4];  // byte offsets of this lane's four rows of a tile
+  int first_key = 0;  // the tile's first key (lane 0 reads entry 0 of the tile)
   auto read_rows = [&](int t) {
     const lds_char_t* p = lds + ((t >> 2) & 1) * 256 + (t & 3) * 64 + la * 4;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int a = *reinterpret_cast<const __attribute__((address_space(3))) int*>(p + 16 * u);
+      const int a = min(max(*reinterpret_cast<const __attribute__((address_space(3))) int*>(p + 16 * u), 0), N - 1);
       const uint32_t cu = uint32_t(((u & 1) << 3) | (u >> 1)) << 4;
-      rows[u] = (uint32_t(min(max(a, 0), N - 1)) << 8) | (ld_chunk ^ cu);  // (a list may hold any int: clamp)
+      rows[u] = (uint32_t(a) << 8) | (ld_chunk ^ cu);  // (a list may hold any int: clamp)
+      if (u == 0) first_key = __builtin_amdgcn_readfirstlane(a);
+    }
+  };
+  // ---- pacing (see WaveClock): wait until the tile's first key is due ----
+  int looks_left = clk.ticks_per_key > 0.f ? kWaveSpinLimit : 0, long_waits = 0;
+  auto gate = [&]() {
+    if (looks_left > 0) {
+      const uint64_t due = clk.t0 + uint64_t(float(max(first_key - kWaveMarginKeys, 0)) * clk.ticks_per_key);
+      uint64_t now = __builtin_amdgcn_s_memrealtime();
+      const uint64_t give_up = now + kWaveGateTicks;
+      while (now < due) {
+        if (now >= give_up) {
+          if (++long_waits >= kWaveLongWaits) looks_left = 0;
+          break;
+        }
+        if (--looks_left <= 0) break;
+        __builtin_amdgcn_s_sleep(8);
+        now = __builtin_amdgcn_s_memrealtime();
+      }
     }
   };
   // K and V of a tile into buffer `par`
@@ -132,6 +176,7 @@ __device__ __forceinline__ void attend_wave(const bf16_t* __restrict__ Qb, const
       if (nblk > 1) issue_ids(1);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       read_rows(0);
+      gate();
       issue_tile(0);
       // two tiles per round, so that the buffers are compile-time constants
       for (int t0 = 0; t0 < ntiles; t0 += 2) {
@@ -142,6 +187,7 @@ __device__ __forceinline__ void attend_wave(const bf16_t* __restrict__ Qb, const
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tile t is in place, and every list entry asked for so far
           if (t + 1 < ntiles) {
             read_rows(t + 1);
+            gate();
             // block b + 1 of the list entries takes the buffer of block b - 1, last read for tile 4 b - 1 (in round 4 b - 2)
             if (par == 0 && (t & 3) == 0 && t > 0 && (t >> 2) + 1 < nblk) issue_ids((t >> 2) + 1);
             issue_tile(1 - par);

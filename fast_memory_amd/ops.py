@@ -641,6 +641,17 @@ def local_attn_fwd_kernel_name(G: int, S: int, L: int, d: int, dtype: torch.dtyp
     return _lib.load().fm_local_attn_fwd_kernel(G, S, L, d, _DT[dtype]).decode()
 
 
+def wave_pace_state(N: int, C: int, Sq: int, k_idx: torch.Tensor, row: int) -> dict:
+    """Where the schedule of the paced per-row launches of ``hash_attn_wave_kernel`` stands for one row of a
+    memory (diagnostic; synchronises): mode 0 measuring / 1 paced / 2 given up for a while, and the 100 MHz ticks
+    per key of the next launch, of the fastest schedule kept and of the unpaced launch."""
+    import ctypes
+    out = (ctypes.c_float * 6)()
+    check(_lib.load().fm_debug_wave_pace_state(N, C, Sq, _p(k_idx), row, ctypes.cast(out, ctypes.c_void_p)))
+    return {"mode": int(out[0]), "ticks_per_key": out[1], "kept": out[2], "unpaced": out[3], "hold": int(out[4]),
+            "misses": int(out[5])}
+
+
 def hash_attn_fwd_launches(H: int, Sq: int, N: int, d: int, C: int, dtype: torch.dtype) -> int:
     """Number of launches of that kernel one :func:`hash_attn_fwd` call makes (one per row where a row's K
     and V outgrow the last-level cache)."""
@@ -654,7 +665,7 @@ def grouped_forward_kernel(which: Optional[str]) -> None:
     work items per workgroup, ``"ring"`` the kernel whose rows go from global memory straight into LDS (three
     items per workgroup) in a single launch, ``"ring-per-row"`` the same in one launch per row, ``"wave"`` the kernel that
     gives every work item a wave of its own in a single launch, ``"wave-per-row"`` the same in one launch per
-    row, ``"wave-auto"`` the same with the dispatch's own choice between the two, ``"gather"``
+    row (its sweeps paced against the device's clock), ``"wave-per-row-unpaced"`` that without the pacing, ``"wave-auto"`` the same with the dispatch's own choice between the two, ``"gather"``
     always the kernel that gathers the rows into registers, ``"bwd-register-blocks"`` (backward only) makes the
     two-tile pass of the staged backward load its key blocks into registers instead of through LDS a block
     ahead, ``None`` restores the dispatch (the direct loads
@@ -664,4 +675,5 @@ def grouped_forward_kernel(which: Optional[str]) -> None:
     _generic_forced = False
     _debug_lib().fm_debug_force_generic({None: 0, "staged": 2, "gather": 3, "staged-pairs": 4, "ring": 5,
                                          "staged-per-row": 6, "ring-per-row": 7, "bwd-register-blocks": 9,
-                                         "wave-auto": 10, "wave": 11, "wave-per-row": 12}[which])
+                                         "wave-auto": 10, "wave": 11, "wave-per-row": 12,
+                                         "wave-per-row-unpaced": 13}[which])

@@ -35,7 +35,8 @@ int fm_debug_hooks_enabled(void);
  * loads its key blocks into registers as its other passes do, instead of through
  * LDS a block ahead (tests compare the two, which give the same bits); 10 = the
  * kernel with a wave per work item, launched as dispatch would launch it, 11 = that
- * kernel in a single launch, 12 = in one launch per row.  Dispatch: gather
+ * kernel in a single launch, 12 = in one launch per row, 13 = the same with its
+ * sweeps unpaced.  Dispatch: gather
  * when H min(Sq, C) < 512 and Sq < 24 C; else the direct loads up to 2^24 keys and
  * the staged kernel beyond; one launch per row when K and V of all rows are 512 MB
  * or more, those of a row 32 MB or more, and a row has 1024 (staged kernel: 1536)
@@ -43,6 +44,13 @@ int fm_debug_hooks_enabled(void);
  * more buckets and queries and a bucket receives 16 queries or fewer on average,
  * the kernel with a wave per work item in place of the direct loads. */
 void fm_debug_force_generic(int on);
+
+/* Diagnostic: where the schedule of the paced launches of "hash_attn_wave_kernel" stands for row `row` of a
+ * memory of N keys, C buckets, Sq queries per row and the lists at k_idx (device pointer, as passed to
+ * fm_hash_attn_fwd): out6 = { mode (0 measuring, 1 paced, 2 given up for a while), 100 MHz ticks per key of the
+ * next launch, of the fastest schedule kept, of the unpaced launch, launches until the next try, schedules
+ * missed in a row }; zeros before the first launch.  Copies from the device (synchronous). */
+int fm_debug_wave_pace_state(int N, int C, int Sq, const void* k_idx, int row, float* out6);
 
 /* Diagnostic: name of the kernel fm_hash_attn_fwd launches for these extents
  * (a static string): "hash_attn_generic_kernel", "hash_attn_wave_kernel" (a wave per work item),

@@ -78,9 +78,9 @@ extern "C" const char* fm_local_attn_fwd_kernel(int G, int S, int L, int d, int 
 namespace fm {
 int wave_pace_state(int N, int C, int Sq, const void* lists, int row, float* out);
 }
-extern "C" int fm_debug_wave_pace_state(int N, int C, int Sq, const void* k_idx, int row, float* out6) {
-  if (!out6) return FM_ERR_ARG;
-  return fm::wave_pace_state(N, C, Sq, k_idx, row, out6);
+extern "C" int fm_debug_wave_pace_state(int N, int C, int Sq, const void* k_idx, int row, float* out8) {
+  if (!out8) return FM_ERR_ARG;
+  return fm::wave_pace_state(N, C, Sq, k_idx, row, out8);
 }
 
 extern "C" int fm_hash_attn_fwd_launches(int H, int Sq, int N, int d, int C, int dtype) {

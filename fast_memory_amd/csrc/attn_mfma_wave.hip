@@ -14,27 +14,39 @@ extern std::atomic<int> g_force_generic;  // attn_api.hip; 13: a launch per row 
 // The schedule of a paced launch (WaveClock in attn_wave.hpp) is found by trying, launch after launch, for
 // every (memory, lists, row) the library sees: a table of the library's own in device memory, one copy per
 // GPU, a slot per (N, C, Sq, the lists' address, the row) -- the host hands the slots out (the 1024 keys seen
-// last have one each).  The last wave of a launch to finish
-// (every wave counts itself out) compares the launch's duration with its schedule and sets the next one:
-//   * no schedule yet: the launch ran unpaced; the next gets 0.9 x its duration;
-//   * schedule kept (duration <= 1.02 x schedule + 15 us): unless held, try one 2 % faster;
-//   * schedule missed while trying a faster one: back to 1.01 x the last one kept, held for 256 launches;
-//   * schedule missed at one that had been kept: 3 % slower, held for 256 launches; after 8 misses in a row or
-//     beyond 1.1 x the unpaced duration the slot gives up for 512 launches (unpaced), then starts again.
-// A missed schedule costs that launch up to a third of its time, a kept one saves a fifth; once settled a
-// slot misses one launch in about 256.  Calls that use a slot at the same time (two streams on one memory and
-// row; two keys on one slot) mix their measurements: the schedule may then be a poor one, nothing else.
+// last have one each).  The last wave of a launch to finish (every wave counts itself out) takes the launch's
+// duration and sets the next launch's schedule -- a descent on the duration itself, which is what counts:
+//   * no schedule yet: the launch ran unpaced; the one after the second such launch (the first on a memory is
+//     a cold one) gets 0.92 x its duration;
+//   * the launch was no slower than the best so far (within 1 %): it is the best now, and unless the schedule is
+//     being held the next one is 2 % faster;
+//   * it was slower: back to the best schedule, held for 16 launches the first time and twice as long after
+//     every such step back, up to 256 (while a schedule is held, the best duration follows what the launches
+//     at it take);
+//   * while a schedule is held, every 33rd launch runs unpaced and renews the unpaced duration;
+//   * the best is no better than 0.97 x the unpaced duration, or four launches in a row were slower than the
+//     unpaced one: the slot gives up for 1024 launches (they run unpaced and cost nothing), then starts again.
+// A schedule that a launch cannot keep costs that launch up to a third of its time; one it can keep saves up to
+// a quarter; once settled a slot tries a faster one every 256 launches.  Calls that use a slot at the same time
+// (two streams on one memory and row) mix their measurements: the schedule may then be a poor one, nothing
+// else.
 struct WavePaceSlot {
   unsigned long long key;   // whose slot this is (0: nobody's)
   unsigned long long t0;    // start of the launch in flight (0: none has started)
   unsigned int done;        // waves of it that have finished
   int mode;                 // 0 the next launch runs unpaced and is measured, 1 paced, 2 given up (hold counts down)
-  float tpk;                // ticks per key of the next launch
-  float good;               // the fastest schedule kept so far (0: none)
+  float tpk;                // ticks per key of the next launch's schedule
+  float best_tpk;           // the schedule of the shortest launch so far, and that launch's ticks per key
+  float best;
   float base;               // ticks per key of the unpaced launch
-  int hold;                 // launches until the next try of a faster schedule / of pacing at all
-  int misses;               // schedules missed in a row
-  int pad[3];
+  int hold;                 // launches until a faster schedule is tried again / until pacing is tried again
+  int hold_len;             // how long the next hold lasts
+  int slow;                 // launches in a row slower than the unpaced one
+  float last_elapsed;       // the last launch: its ticks per key and the schedule it ran on (diagnostics)
+  float last_tpk;
+  int refresh;              // 1: the next launch runs unpaced although the slot paces, to measure the unpaced duration again
+  int since_refresh;        // paced launches since the last such measurement
+  int measured;             // unpaced launches measured since the slot (re)started
 };
 constexpr int kWavePaceSlots = 1024;
 static __device__ __align__(256) WavePaceSlot g_wave_pace[kWavePaceSlots];
@@ -42,43 +54,70 @@ static __device__ __align__(256) WavePaceSlot g_wave_pace[kWavePaceSlots];
 // What the last wave of a launch does with the slot (one lane).  elapsed: ticks since the launch's first wave
 // started; tpk_used: the schedule the launch ran on (0: unpaced).
 __device__ inline void wave_pace_update(WavePaceSlot* s, unsigned long long key, float elapsed, float tpk_used, int N) {
+  const float e = elapsed / float(N);  // ticks per key of this launch
   if (s->key != key) {  // (first use, or another memory's slot: start over)
     s->key = key;
     s->mode = 0;
-    s->good = 0.f;
     s->hold = 0;
-    s->misses = 0;
+    s->measured = 0;
+    s->refresh = 0;
   }
+  s->last_elapsed = e;
+  s->last_tpk = tpk_used;
   if (tpk_used <= 0.f) {
-    if (s->mode == 2 && --s->hold > 0) {
+    if (s->mode == 1) {  // the unpaced duration measured again beside the paced launches
+      s->base = 0.7f * s->base + 0.3f * e;
+      s->refresh = 0;
+      s->since_refresh = 0;
+    } else if (s->mode == 2 && --s->hold > 0) {
       s->tpk = 0.f;
+      s->measured = 0;
+    } else if (++s->measured < 2) {  // (the first launch on a memory is a cold one: the second counts)
+      s->mode = 0;
     } else {
-      s->base = elapsed / float(N);
-      s->tpk = 0.9f * s->base;
+      s->base = e;
+      s->tpk = 0.92f * e;
       s->mode = 1;
-      s->good = 0.f;
+      s->best = 0.f;
+      s->best_tpk = 0.f;
       s->hold = 0;
-      s->misses = 0;
+      s->hold_len = 16;
+      s->slow = 0;
+      s->refresh = 0;
+      s->since_refresh = 0;
     }
-  } else if (elapsed <= 1.02f * tpk_used * float(N) + 1500.f) {
-    s->good = tpk_used;
-    s->misses = 0;
+    if (s->mode == 1 && s->hold > 0 && s->best > 0.97f * s->base) {
+      s->mode = 2;
+      s->hold = 1024;
+      s->tpk = 0.f;
+      s->measured = 0;
+    }
+    return;
+  }
+  if (++s->since_refresh >= 32 && s->hold > 0) s->refresh = 1;
+  s->slow = e > s->base ? s->slow + 1 : 0;
+  if (s->best <= 0.f || e <= 1.01f * s->best) {
+    if (s->best <= 0.f || e < s->best || tpk_used == s->best_tpk) {
+      s->best = (tpk_used == s->best_tpk && s->best > 0.f) ? 0.8f * s->best + 0.2f * e : e;
+      s->best_tpk = tpk_used;
+    }
     if (s->hold > 0)
       --s->hold;
     else
-      s->tpk = fmaxf(0.98f * tpk_used, 0.4f * s->base);
+      s->tpk = fmaxf(0.98f * s->best_tpk, 0.4f * s->base);
+  } else if (tpk_used == s->best_tpk) {  // the best schedule itself has become slower: follow it
+    s->best = 0.8f * s->best + 0.2f * e;
+    if (s->hold > 0) --s->hold;
   } else {
-    ++s->misses;
-    // a faster schedule than the last one kept was being tried: back to just above that one; else the one
-    // held has stopped working: a little slower
-    s->tpk = (s->good > 0.f && tpk_used < 0.995f * s->good) ? 1.01f * s->good : 1.03f * tpk_used;
-    s->good = s->tpk;
-    s->hold = 256;
-    if (s->misses > 8 || s->tpk > 1.1f * s->base) {
-      s->mode = 2;
-      s->hold = 512;
-      s->tpk = 0.f;
-    }
+    s->tpk = s->best_tpk;
+    s->hold = s->hold_len;
+    s->hold_len = s->hold_len < 128 ? 2 * s->hold_len : 256;
+  }
+  if (s->slow >= 4 || (s->hold > 0 && s->best > 0.97f * s->base)) {
+    s->mode = 2;
+    s->hold = 1024;
+    s->tpk = 0.f;
+    s->measured = 0;
   }
 }
 
@@ -118,7 +157,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         old = 0;
       }
       t0 = old ? old : now;
-      tpk = pace->key == pace_key && pace->mode == 1 ? pace->tpk : 0.f;
+      tpk = pace->key == pace_key && pace->mode == 1 && !pace->refresh ? pace->tpk : 0.f;
     }
     t0 = (uint64_t(__builtin_amdgcn_readfirstlane(uint32_t(t0 >> 32))) << 32) | __builtin_amdgcn_readfirstlane(uint32_t(t0));
     tpk_used = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, tpk)));
@@ -234,10 +273,11 @@ int hash_attn_mfma_wave(const void* q, const void* k, const void* v, const int32
   return launch_status("fm_hash_attn_fwd(mfma, wave)");
 }
 
-// out[0..5] = mode, ticks per key of the next launch, the fastest schedule kept, ticks per key unpaced, hold,
-// misses of the slot of (N, C, Sq, lists, row); all zero where there is none yet.  A synchronous copy.
+// out[0..7] = mode, ticks per key of the next launch's schedule, of the best schedule and of the launch that
+// ran on it, of the unpaced launch, launches until the next try, the last launch's ticks per key and the
+// schedule it ran on, of the slot of (N, C, Sq, lists, row); all zero where there is none yet.  A synchronous copy.
 int wave_pace_state(int N, int C, int Sq, const void* lists, int row, float* out) {
-  for (int i = 0; i < 6; ++i) out[i] = 0.f;
+  for (int i = 0; i < 8; ++i) out[i] = 0.f;
   WavePaceSlot* const table = wave_pace_table();
   if (!table) return FM_ERR_LAUNCH;
   const unsigned long long key = wave_pace_key(N, C, Sq, lists, row);
@@ -247,7 +287,8 @@ int wave_pace_state(int N, int C, int Sq, const void* lists, int row, float* out
     return FM_ERR_LAUNCH;
   }
   if (h.key != key) return FM_OK;
-  out[0] = float(h.mode); out[1] = h.tpk; out[2] = h.good; out[3] = h.base; out[4] = float(h.hold); out[5] = float(h.misses);
+  out[0] = float(h.mode); out[1] = h.tpk; out[2] = h.best_tpk; out[3] = h.best; out[4] = h.base; out[5] = float(h.hold);
+  out[6] = h.last_elapsed; out[7] = h.last_tpk;
   return FM_OK;
 }
 

@@ -643,13 +643,14 @@ def local_attn_fwd_kernel_name(G: int, S: int, L: int, d: int, dtype: torch.dtyp
 
 def wave_pace_state(N: int, C: int, Sq: int, k_idx: torch.Tensor, row: int) -> dict:
     """Where the schedule of the paced per-row launches of ``hash_attn_wave_kernel`` stands for one row of a
-    memory (diagnostic; synchronises): mode 0 measuring / 1 paced / 2 given up for a while, and the 100 MHz ticks
-    per key of the next launch, of the fastest schedule kept and of the unpaced launch."""
+    memory (diagnostic; synchronises): mode 0 measuring / 1 paced / 2 given up for a while, and, in 100 MHz ticks
+    per key, the next launch's schedule, the best schedule so far and what the launch on it took, the unpaced
+    launch, the last launch and its schedule."""
     import ctypes
-    out = (ctypes.c_float * 6)()
+    out = (ctypes.c_float * 8)()
     check(_lib.load().fm_debug_wave_pace_state(N, C, Sq, _p(k_idx), row, ctypes.cast(out, ctypes.c_void_p)))
-    return {"mode": int(out[0]), "ticks_per_key": out[1], "kept": out[2], "unpaced": out[3], "hold": int(out[4]),
-            "misses": int(out[5])}
+    return {"mode": int(out[0]), "ticks_per_key": out[1], "best_schedule": out[2], "best_launch": out[3], "unpaced": out[4],
+            "hold": int(out[5]), "last_launch": out[6], "last_schedule": out[7]}
 
 
 def hash_attn_fwd_launches(H: int, Sq: int, N: int, d: int, C: int, dtype: torch.dtype) -> int:

@@ -826,6 +826,17 @@ def main():
         f"{attn_ms:.2f} ms = {achieved:.0f} GB/s algorithmic ({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak); "
         f"parts {parts_ms}")
 
+    if attn_kernel.startswith("hash_attn_wave_kernel") and launches > 1:
+        # where the schedules of the paced per-row launches stand (100 MHz ticks per key; see fastmem_debug.h)
+        pace = [ops.wave_pace_state(N, C, Sq, attn_lists, r) for r in range(H)]
+        roofline["paced_sweeps"] = {
+            "rows_paced": sum(1 for p in pace if p["mode"] == 1),
+            "rows_given_up": sum(1 for p in pace if p["mode"] == 2),
+            "schedule_us_per_launch": [round(p["ticks_per_key"] * N / 100.0, 1) for p in pace],
+            "unpaced_us_per_launch": [round(p["unpaced"] * N / 100.0, 1) for p in pace],
+            "last_launch_us": [round(p["last_launch"] * N / 100.0, 1) for p in pace]}
+        log(f"[bench] paced sweeps: {roofline['paced_sweeps']}")
+
     # read bandwidth a plain streaming-read kernel reaches on this device, for scale beside the published peak
     probe = torch.empty(4 << 30, dtype=torch.uint8, device=dev).fill_(1)
     sink = torch.zeros(1, dtype=torch.int32, device=dev)

@@ -14,39 +14,39 @@ extern std::atomic<int> g_force_generic;  // attn_api.hip; 13: a launch per row 
 // The schedule of a paced launch (WaveClock in attn_wave.hpp) is found by trying, launch after launch, for
 // every (memory, lists, row) the library sees: a table of the library's own in device memory, one copy per
 // GPU, a slot per (N, C, Sq, the lists' address, the row) -- the host hands the slots out (the 1024 keys seen
-// last have one each).  The last wave of a launch to finish (every wave counts itself out) takes the launch's
-// duration and sets the next launch's schedule -- a descent on the duration itself, which is what counts:
-//   * no schedule yet: the launch ran unpaced; the one after the second such launch (the first on a memory is
-//     a cold one) gets 0.92 x its duration;
-//   * the launch was no slower than the best so far (within 1 %): it is the best now, and unless the schedule is
-//     being held the next one is 2 % faster;
-//   * it was slower: back to the best schedule, held for 16 launches the first time and twice as long after
-//     every such step back, up to 256 (while a schedule is held, the best duration follows what the launches
-//     at it take);
-//   * while a schedule is held, every 33rd launch runs unpaced and renews the unpaced duration;
-//   * the best is no better than 0.97 x the unpaced duration, or four launches in a row were slower than the
-//     unpaced one: the slot gives up for 1024 launches (they run unpaced and cost nothing), then starts again.
-// A schedule that a launch cannot keep costs that launch up to a third of its time; one it can keep saves up to
-// a quarter; once settled a slot tries a faster one every 256 launches.  Calls that use a slot at the same time
-// (two streams on one memory and row) mix their measurements: the schedule may then be a poor one, nothing
-// else.
+// last have one each).  A one-thread kernel behind every launch (wave_pace_step_kernel) takes the launch's
+// duration and sets the next launch's schedule.  A launch either keeps its schedule (it ends within 10 % of
+// it) or falls off it: the waves that get behind the others no longer find their rows in the L2, get further
+// behind, and the launch takes a fifth to a half longer than unpaced.  So:
+//   * no schedule yet: the launch runs unpaced; the second such launch (the first on a memory is a cold one)
+//     gives the unpaced duration, and the next launch a schedule of 0.92 x that;
+//   * searching: a kept schedule is followed by one 2 % faster; the first one missed ends the search -- the
+//     slot holds the fastest schedule kept + 4 % (if none was kept: 5 % slower and on with the search);
+//   * holding, for 16 launches the first time and twice as long after every search, up to 256: a launch that
+//     misses the held schedule makes it 3 % slower; every 33rd launch runs unpaced and renews the unpaced
+//     duration; then the search goes on from the held schedule;
+//   * the held schedule's launches take more than 0.97 x the unpaced duration on average, or a schedule would
+//     have to be slower than that: the slot gives up for 1024 launches (they run unpaced and cost nothing),
+//     then starts again.
+// Calls that use a slot at the same time (two streams on one memory and row) mix their measurements: the
+// schedule may then be a poor one, nothing else.
 struct WavePaceSlot {
   unsigned long long key;   // whose slot this is (0: nobody's)
-  unsigned long long t0;    // start of the launch in flight (0: none has started)
-  unsigned int done;        // waves of it that have finished
+  unsigned long long t0;    // start of the launch in flight (0: none, or one without a work item)
+  float tpk_used;           // the schedule it runs on (0: unpaced)
   int mode;                 // 0 the next launch runs unpaced and is measured, 1 paced, 2 given up (hold counts down)
   float tpk;                // ticks per key of the next launch's schedule
-  float best_tpk;           // the schedule of the shortest launch so far, and that launch's ticks per key
-  float best;
+  float good;               // the fastest schedule kept in the current search (0: none yet)
+  float held;               // mean ticks per key of the launches on the held schedule
   float base;               // ticks per key of the unpaced launch
-  int hold;                 // launches until a faster schedule is tried again / until pacing is tried again
+  int hold;                 // launches until the search goes on / until pacing is tried again
   int hold_len;             // how long the next hold lasts
-  int slow;                 // launches in a row slower than the unpaced one
   float last_elapsed;       // the last launch: its ticks per key and the schedule it ran on (diagnostics)
   float last_tpk;
-  int refresh;              // 1: the next launch runs unpaced although the slot paces, to measure the unpaced duration again
+  int refresh;              // 1: the next launch runs unpaced although the slot paces, to renew the unpaced duration
   int since_refresh;        // paced launches since the last such measurement
   int measured;             // unpaced launches measured since the slot (re)started
+  int pad;
 };
 constexpr int kWavePaceSlots = 1024;
 static __device__ __align__(256) WavePaceSlot g_wave_pace[kWavePaceSlots];
@@ -64,61 +64,61 @@ __device__ inline void wave_pace_update(WavePaceSlot* s, unsigned long long key,
   }
   s->last_elapsed = e;
   s->last_tpk = tpk_used;
+  auto give_up = [&]() {
+    s->mode = 2;
+    s->hold = 1024;
+    s->tpk = 0.f;
+    s->measured = 0;
+  };
   if (tpk_used <= 0.f) {
     if (s->mode == 1) {  // the unpaced duration measured again beside the paced launches
       s->base = 0.7f * s->base + 0.3f * e;
       s->refresh = 0;
       s->since_refresh = 0;
+      if (s->hold > 0 && s->held > 0.97f * s->base) give_up();
     } else if (s->mode == 2 && --s->hold > 0) {
       s->tpk = 0.f;
       s->measured = 0;
-    } else if (++s->measured < 2) {  // (the first launch on a memory is a cold one: the second counts)
+    } else if (++s->measured < 2) {
       s->mode = 0;
     } else {
       s->base = e;
       s->tpk = 0.92f * e;
       s->mode = 1;
-      s->best = 0.f;
-      s->best_tpk = 0.f;
+      s->good = 0.f;
+      s->held = 0.f;
       s->hold = 0;
       s->hold_len = 16;
-      s->slow = 0;
       s->refresh = 0;
       s->since_refresh = 0;
     }
-    if (s->mode == 1 && s->hold > 0 && s->best > 0.97f * s->base) {
-      s->mode = 2;
-      s->hold = 1024;
-      s->tpk = 0.f;
-      s->measured = 0;
-    }
     return;
   }
-  if (++s->since_refresh >= 32 && s->hold > 0) s->refresh = 1;
-  s->slow = e > s->base ? s->slow + 1 : 0;
-  if (s->best <= 0.f || e <= 1.01f * s->best) {
-    if (s->best <= 0.f || e < s->best || tpk_used == s->best_tpk) {
-      s->best = (tpk_used == s->best_tpk && s->best > 0.f) ? 0.8f * s->best + 0.2f * e : e;
-      s->best_tpk = tpk_used;
+  const bool kept = e <= 1.10f * tpk_used;
+  if (s->hold == 0) {  // searching
+    if (kept) {
+      s->good = tpk_used;
+      s->tpk = fmaxf(0.98f * tpk_used, 0.4f * s->base);
+    } else if (s->good > 0.f) {
+      s->tpk = 1.04f * s->good;
+      s->held = 1.02f * s->tpk;  // (what a launch on it should take; the launches will tell)
+      s->good = 0.f;
+      s->hold = s->hold_len;
+      s->hold_len = s->hold_len < 128 ? 2 * s->hold_len : 256;
+    } else {
+      s->tpk = 1.05f * tpk_used;
     }
-    if (s->hold > 0)
-      --s->hold;
-    else
-      s->tpk = fmaxf(0.98f * s->best_tpk, 0.4f * s->base);
-  } else if (tpk_used == s->best_tpk) {  // the best schedule itself has become slower: follow it
-    s->best = 0.8f * s->best + 0.2f * e;
-    if (s->hold > 0) --s->hold;
-  } else {
-    s->tpk = s->best_tpk;
-    s->hold = s->hold_len;
-    s->hold_len = s->hold_len < 128 ? 2 * s->hold_len : 256;
+  } else {  // holding
+    s->held = 0.8f * s->held + 0.2f * e;
+    if (kept) {
+      if (--s->hold == 0) s->good = 0.f;
+    } else {
+      s->tpk = 1.03f * tpk_used;
+    }
+    if (++s->since_refresh >= 32) s->refresh = 1;
+    if (s->held > 0.97f * s->base) give_up();
   }
-  if (s->slow >= 4 || (s->hold > 0 && s->best > 0.97f * s->base)) {
-    s->mode = 2;
-    s->hold = 1024;
-    s->tpk = 0.f;
-    s->measured = 0;
-  }
+  if (s->mode == 1 && s->tpk > 0.97f * s->base) give_up();
 }
 
 template <bool F16>
@@ -142,26 +142,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const fm_item it = items[me];
   const int64_t bkt = int64_t(it.row) * C + it.bucket;
   const int64_t qbase = int64_t(it.row) * Sq;
-  // The launch's schedule and start (WaveClock): the first wave to come sets the start.
+  // The launch's schedule (WaveClock).  Every wave takes its own start for the launch's: the waves of a launch
+  // start within a microsecond or two of each other (measured), while 2048 of them agreeing on one start through
+  // an atomic on one word took the last of them 100 us, which put those behind the schedule before they began.
   WaveClock clk{0, 0.f};
-  float tpk_used = 0.f;
   if (pace) {
-    unsigned long long t0 = 0;
-    float tpk = 0.f;
-    if ((threadIdx.x & 63) == 0) {
-      const unsigned long long now = __builtin_amdgcn_s_memrealtime();
-      unsigned long long old = atomicCAS(&pace->t0, 0ull, now);
-      if (old && now - old > (1ull << 28)) {  // a start 2.7 s old: a launch never counted itself out (two calls
-        // mixed on the slot with different numbers of waves); start over
-        if (atomicCAS(&pace->t0, old, now) == old) atomicExch(&pace->done, 0u);
-        old = 0;
-      }
-      t0 = old ? old : now;
-      tpk = pace->key == pace_key && pace->mode == 1 && !pace->refresh ? pace->tpk : 0.f;
+    const unsigned long long now = __builtin_amdgcn_s_memrealtime();
+    const float tpk = pace->key == pace_key && pace->mode == 1 && !pace->refresh ? pace->tpk : 0.f;
+    clk = WaveClock{now, __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, tpk)))};
+    if (blockIdx.x == 0 && threadIdx.x == 0) {  // for wave_pace_step_kernel, which follows the launch
+      pace->t0 = now;
+      pace->tpk_used = tpk;
     }
-    t0 = (uint64_t(__builtin_amdgcn_readfirstlane(uint32_t(t0 >> 32))) << 32) | __builtin_amdgcn_readfirstlane(uint32_t(t0));
-    tpk_used = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, tpk)));
-    clk = WaveClock{t0, tpk_used};
   }
   // (an item has up to FM_QTILE = 64 queries, a sweep takes 48: the few items with more are swept twice, the
   // second time unpaced)
@@ -171,18 +163,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         out + qbase * kSD, lse + qbase, (lds_char_t*)wave_lds + w * kWWaveBytes, clk);
     clk.ticks_per_key = 0.f;
   }
-  // Every wave counts itself out; the last one sets the next launch's schedule and clears the way for it.
-  if (pace && (threadIdx.x & 63) == 0) {
-    const unsigned int n_waves = unsigned(n_it - first);
-    if (atomicAdd(&pace->done, 1u) + 1u == n_waves) {
-      const unsigned long long now = __builtin_amdgcn_s_memrealtime();
-      const unsigned long long t0 = atomicAdd(&pace->t0, 0ull);
-      wave_pace_update(pace, pace_key, float(now - t0), tpk_used, N);
-      __threadfence();
-      pace->done = 0u;
-      atomicExch(&pace->t0, 0ull);
-    }
-  }
+}
+
+// One thread, launched behind every paced launch on its stream: the launch's duration (from the start its
+// first wave noted to now) sets the next launch's schedule.
+__global__ void wave_pace_step_kernel(WavePaceSlot* __restrict__ pace, unsigned long long pace_key, int N) {
+  const unsigned long long now = __builtin_amdgcn_s_memrealtime(), t0 = pace->t0;
+  if (t0 == 0 || now <= t0) return;  // (the launch had no work item: nothing was measured)
+  wave_pace_update(pace, pace_key, float(now - t0), pace->tpk_used, N);
+  pace->t0 = 0;
 }
 
 // The table's address on the current device (in host code its name only stands for the symbol).
@@ -260,6 +249,7 @@ int hash_attn_mfma_wave(const void* q, const void* k, const void* v, const int32
         FM_WAVE_LAUNCH(true, row_items, row);
       else
         FM_WAVE_LAUNCH(false, row_items, row);
+      if (pace_slot) hipLaunchKernelGGL(wave_pace_step_kernel, dim3(1), dim3(1), 0, st, pace_slot, pace_key, N);
     }
   } else {
     const unsigned long long pace_key = 0;
@@ -273,9 +263,9 @@ int hash_attn_mfma_wave(const void* q, const void* k, const void* v, const int32
   return launch_status("fm_hash_attn_fwd(mfma, wave)");
 }
 
-// out[0..7] = mode, ticks per key of the next launch's schedule, of the best schedule and of the launch that
-// ran on it, of the unpaced launch, launches until the next try, the last launch's ticks per key and the
-// schedule it ran on, of the slot of (N, C, Sq, lists, row); all zero where there is none yet.  A synchronous copy.
+// out[0..7] = mode, ticks per key of the next launch's schedule, of the fastest schedule kept in the current
+// search, of the launches on the held schedule (mean), of the unpaced launch, launches the hold still lasts, the
+// last launch's ticks per key and the schedule it ran on, of the slot of (N, C, Sq, lists, row); all zero where there is none yet.  A synchronous copy.
 int wave_pace_state(int N, int C, int Sq, const void* lists, int row, float* out) {
   for (int i = 0; i < 8; ++i) out[i] = 0.f;
   WavePaceSlot* const table = wave_pace_table();
@@ -287,7 +277,7 @@ int wave_pace_state(int N, int C, int Sq, const void* lists, int row, float* out
     return FM_ERR_LAUNCH;
   }
   if (h.key != key) return FM_OK;
-  out[0] = float(h.mode); out[1] = h.tpk; out[2] = h.best_tpk; out[3] = h.best; out[4] = h.base; out[5] = float(h.hold);
+  out[0] = float(h.mode); out[1] = h.tpk; out[2] = h.good; out[3] = h.held; out[4] = h.base; out[5] = float(h.hold);
   out[6] = h.last_elapsed; out[7] = h.last_tpk;
   return FM_OK;
 }

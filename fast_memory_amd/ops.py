@@ -644,12 +644,12 @@ def local_attn_fwd_kernel_name(G: int, S: int, L: int, d: int, dtype: torch.dtyp
 def wave_pace_state(N: int, C: int, Sq: int, k_idx: torch.Tensor, row: int) -> dict:
     """Where the schedule of the paced per-row launches of ``hash_attn_wave_kernel`` stands for one row of a
     memory (diagnostic; synchronises): mode 0 measuring / 1 paced / 2 given up for a while, and, in 100 MHz ticks
-    per key, the next launch's schedule, the best schedule so far and what the launch on it took, the unpaced
-    launch, the last launch and its schedule."""
+    per key, the next launch's schedule, the fastest schedule kept in the current search, the mean of the launches
+    on the held schedule, the unpaced launch, the last launch and its schedule."""
     import ctypes
     out = (ctypes.c_float * 8)()
     check(_lib.load().fm_debug_wave_pace_state(N, C, Sq, _p(k_idx), row, ctypes.cast(out, ctypes.c_void_p)))
-    return {"mode": int(out[0]), "ticks_per_key": out[1], "best_schedule": out[2], "best_launch": out[3], "unpaced": out[4],
+    return {"mode": int(out[0]), "ticks_per_key": out[1], "kept_in_search": out[2], "held_launches": out[3], "unpaced": out[4],
             "hold": int(out[5]), "last_launch": out[6], "last_schedule": out[7]}
 
 

@@ -48,9 +48,9 @@ void fm_debug_force_generic(int on);
 /* Diagnostic: where the schedule of the paced launches of "hash_attn_wave_kernel" stands for row `row` of a
  * memory of N keys, C buckets, Sq queries per row and the lists at k_idx (device pointer, as passed to
  * fm_hash_attn_fwd): out8 = { mode (0 measuring, 1 paced, 2 given up for a while), then in 100 MHz ticks per key:
- * the next launch's schedule, the best schedule so far, what the launch on it took, what the unpaced launch
- * took; launches until the next try; ticks per key of the last launch and of its schedule }; zeros before the
- * first launch.  Copies from the device (synchronous). */
+ * the next launch's schedule, the fastest schedule kept in the current search, the mean of the launches on the
+ * held schedule, the unpaced launch; launches the hold still lasts; ticks per key of the last launch and of its
+ * schedule }; zeros before the first launch.  Copies from the device (synchronous). */
 int fm_debug_wave_pace_state(int N, int C, int Sq, const void* k_idx, int row, float* out8);
 
 /* Diagnostic: name of the kernel fm_hash_attn_fwd launches for these extents

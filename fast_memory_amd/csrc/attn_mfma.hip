@@ -544,26 +544,26 @@ static bool row_launches_pay(int choice, int H, int Sq, int N, int C) {
          (C < Sq ? C : Sq) >= (choice >= 3 ? 1024 : 1536);
 }
 
-// Form 4 (attn_wave.hpp: a wave per work item, eight buckets swept per compute unit instead of two) where the
-// launches go per row, a row has 2048 buckets and queries or more (one item per wave: fewer do not fill the
-// device) and a bucket receives 16 queries or fewer on average: there a launch is bound by the requests that
-// miss the L2s, and four times as many buckets in flight behind an L2 meet at more rows (requests answered by
-// an L2, 2^20 keys, 2048 buckets of 16384, 16 queries each: 32 % -> 42 %).  Its tile is 16 keys and a wave's
-// MFMA and softmax work grows with the queries of its item, so it loses from two tiles of queries per item on.
-// Measured against form 3, both per row, lists in key order, per step (ms):
+// Form 4 (attn_wave.hpp: a wave per work item, eight buckets swept per compute unit instead of two, the sweeps
+// of a launch paced against the device's clock) where the launches go per row, a row has 2048 buckets and
+// queries or more (one item per wave: fewer do not fill the device) and a bucket receives 24 queries or fewer
+// on average: there a launch is bound by the requests that miss the L2s, and waves that sweep the key range
+// together find most of their rows in the L2.  Its tile is 16 keys and a wave's MFMA and softmax work grows
+// with the queries of its item, so it loses from two tiles of queries per item on.  Measured against form 3,
+// both per row, lists in key order, per step (ms), form 4 unpaced and paced (after its schedules have settled):
 //   8 rows of 2^20 keys, 2048 buckets of 16384, the queries of the 1 M-key benchmark workload (16 per bucket on
-//     average, as its hash deals them): 12.24 against 10.60
+//     average, as its hash deals them): 12.2 against 10.6 and 8.0
 //   the same memory, queries assigned to buckets at random; 4 / 8 / 16 / 24 / 32 per bucket on average:
-//     12.65 / 12.35 / 13.08 / 13.23 / 13.25 against 10.90 / 10.94 / 12.46 / 13.10 / 18.45
-//   8 rows of 2^20 keys, 4096 buckets of 4096; 4 / 8 / 16 / 24 / 32: 8.55 / 8.68 / 8.74 / 8.78 / 8.81 against
-//     6.94 / 7.03 / 7.37 / 7.47 / 9.00
-//   4 rows of 2^21 keys, 2048 buckets of 32768; 4 / 8 / 16 / 24: 13.38 / 13.91 / 13.93 / 14.00 against
-//     12.44 / 12.66 / 13.79 / 14.25
+//     13.1 / 12.8 / 13.3 / 13.5 / 13.5 against 11.2 / 11.3 / 12.6 / 13.3 / 18.9 and 7.4 / 7.3 / 8.1 / 9.6 / 18.9
+//   4 rows of 2^21 keys, 2048 buckets of 32768; 4 / 8 / 16 / 24 / 32: 14.0 / 14.0 / 14.4 / 14.4 / 14.5 against
+//     13.1 / 13.1 / 14.0 / 14.5 / 18.9 and 7.3 / 7.4 / 8.0 / 9.4 / 18.0
+//   8 rows of 2^20 keys, 4096 buckets of 4096; 4 / 8 / 16 / 24 / 32: 8.5 / 8.7 / 8.7 / 8.8 / 8.8 against
+//     7.1 / 7.2 / 7.4 / 7.6 / 9.0 and the same paced (launches too short for a schedule to pay)
 //   8 rows of 2^18 keys, 1024 buckets of 4096 (1024 items a row: four waves per compute unit), the queries of
-//     the 256 K-key benchmark workload (8 per bucket on average): 1.21 against 1.41; at random 4 / 8 / 16:
-//     1.54 / 1.51 / 1.52 against 1.26 / 1.44 / 1.60
+//     the 256 K-key benchmark workload (8 per bucket on average): 1.22 against 1.46 (paced the same)
+//   16 rows of 2^19 keys, 1024 buckets of 8192; 4 / 8 / 16: 5.84 / 5.83 / 5.89 against 5.12 / 5.56 / 6.20
 static bool wave_per_item_pays(int H, int Sq, int N, int C) {
-  return row_launches_pay(4, H, Sq, N, C) && (C < Sq ? C : Sq) >= 2048 && int64_t(Sq) <= int64_t(16) * C;
+  return row_launches_pay(4, H, Sq, N, C) && (C < Sq ? C : Sq) >= 2048 && int64_t(Sq) <= int64_t(24) * C;
 }
 
 int hash_attn_mfma_choice(int H, int Sq, int N, int C) {

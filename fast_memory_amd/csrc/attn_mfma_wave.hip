@@ -23,7 +23,7 @@ extern std::atomic<int> g_force_generic;  // attn_api.hip; 13: a launch per row 
 //   * searching: a kept schedule is followed by one 2 % faster; the first one missed ends the search -- the
 //     slot holds the fastest schedule kept + 4 % (if none was kept: 5 % slower and on with the search);
 //   * holding, for 16 launches the first time and twice as long after every search, up to 256: a launch that
-//     misses the held schedule makes it 3 % slower; every 33rd launch runs unpaced and renews the unpaced
+//     misses the held schedule makes it 3 % slower; every 129th launch runs unpaced and renews the unpaced
 //     duration; then the search goes on from the held schedule;
 //   * the held schedule's launches take more than 0.97 x the unpaced duration on average, or a schedule would
 //     have to be slower than that: the slot gives up for 1024 launches (they run unpaced and cost nothing),
@@ -105,6 +105,7 @@ __device__ inline void wave_pace_update(WavePaceSlot* s, unsigned long long key,
       s->good = 0.f;
       s->hold = s->hold_len;
       s->hold_len = s->hold_len < 128 ? 2 * s->hold_len : 256;
+      s->since_refresh = int((key >> 20) & 127);  // (the rows of a memory renew their unpaced durations in different calls)
     } else {
       s->tpk = 1.05f * tpk_used;
     }
@@ -115,7 +116,7 @@ __device__ inline void wave_pace_update(WavePaceSlot* s, unsigned long long key,
     } else {
       s->tpk = 1.03f * tpk_used;
     }
-    if (++s->since_refresh >= 32) s->refresh = 1;
+    if (++s->since_refresh >= 128) s->refresh = 1;
     if (s->held > 0.97f * s->base) give_up();
   }
   if (s->mode == 1 && s->tpk > 0.97f * s->base) give_up();
@@ -174,20 +175,24 @@ __global__ void wave_pace_step_kernel(WavePaceSlot* __restrict__ pace, unsigned 
   pace->t0 = 0;
 }
 
-// The table's address on the current device (in host code its name only stands for the symbol).
-static WavePaceSlot* wave_pace_table() {
+// The table's address on the current device (in host code its name only stands for the symbol); null while it
+// is not known and cannot be asked for (a stream that is being captured: the launches then go unpaced).
+static WavePaceSlot* wave_pace_table(hipStream_t st) {
   constexpr int kMaxDevices = 64;
   static std::mutex mu;
   static WavePaceSlot* table[kMaxDevices];
-  static bool asked[kMaxDevices];
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
     (void)hipGetLastError();
     return nullptr;
   }
   std::lock_guard<std::mutex> lock(mu);
-  if (!asked[dev]) {
-    asked[dev] = true;
+  if (!table[dev]) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
     void* p = nullptr;
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_wave_pace)) == hipSuccess)
       table[dev] = static_cast<WavePaceSlot*>(p);
@@ -229,7 +234,7 @@ int hash_attn_mfma_wave(const void* q, const void* k, const void* v, const int32
                         const int32_t* n_items, int64_t max_items, void* out, float* lse, int Sq, int N, int C,
                         float sm_scale, bool f16, int H, bool per_row, hipStream_t st) {
   // paced sweeps for the launches per row (a single launch over all rows has no common sweep to pace)
-  WavePaceSlot* const table = per_row && g_force_generic != 13 ? wave_pace_table() : nullptr;
+  WavePaceSlot* const table = per_row && g_force_generic != 13 ? wave_pace_table(st) : nullptr;
 #define FM_WAVE_LAUNCH(F16, ITEMS, ROW)                                                                           \
   do {                                                                                                            \
     FM_ALLOW_LDS((hash_attn_wave_kernel<F16>), kWaveLdsBytes, "fm_hash_attn_fwd: lds");                           \
@@ -268,7 +273,7 @@ int hash_attn_mfma_wave(const void* q, const void* k, const void* v, const int32
 // last launch's ticks per key and the schedule it ran on, of the slot of (N, C, Sq, lists, row); all zero where there is none yet.  A synchronous copy.
 int wave_pace_state(int N, int C, int Sq, const void* lists, int row, float* out) {
   for (int i = 0; i < 8; ++i) out[i] = 0.f;
-  WavePaceSlot* const table = wave_pace_table();
+  WavePaceSlot* const table = wave_pace_table(nullptr);
   if (!table) return FM_ERR_LAUNCH;
   const unsigned long long key = wave_pace_key(N, C, Sq, lists, row);
   WavePaceSlot h;

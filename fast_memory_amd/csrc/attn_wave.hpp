@@ -43,8 +43,9 @@ constexpr size_t kWaveLdsBytes = size_t(4) * kWWaveBytes;
 // and a wave asks for a tile only once its first key is due (less a margin).  Waves that are behind run free,
 // waves that are ahead wait, and if the schedule is one the launch can keep, all of them sweep the key range
 // together and the launch ends on schedule -- sooner than it ends unpaced (2^20 keys, 2048 buckets of 16384:
-// 1.32 ms per launch unpaced, 1.05 ms on a schedule of 1.0 ms; on a schedule it cannot keep, 1.43 ms).  Which
-// schedule a launch can keep is found by trying (WavePaceSlot).  A wait ends after kWaveGateTicks at the
+// 1.32 ms per launch unpaced, 0.94 ms on a schedule of 0.93 ms; on a schedule it cannot keep, a fifth to a half
+// longer than unpaced: the waves that get behind no longer find their rows in the L2 and get further behind).
+// Which schedule a launch can keep is found by trying (WavePaceSlot in attn_mfma_wave.hip).  A wait ends after kWaveGateTicks at the
 // latest and a wave stops pacing after kWaveLongWaits such waits or kWaveSpinLimit looks at the clock in all
 // (lists that do not ascend; a clock that stands still), so every wave ends whatever the clock says.  The
 // clock only delays loads: results do not depend on it.

@@ -41,7 +41,7 @@ int fm_debug_hooks_enabled(void);
  * the staged kernel beyond; one launch per row when K and V of all rows are 512 MB
  * or more, those of a row 32 MB or more, and a row has 1024 (staged kernel: 1536)
  * or more buckets and queries; where the launches go per row, a row has 2048 or
- * more buckets and queries and a bucket receives 16 queries or fewer on average,
+ * more buckets and queries and a bucket receives 24 queries or fewer on average,
  * the kernel with a wave per work item in place of the direct loads. */
 void fm_debug_force_generic(int on);
 

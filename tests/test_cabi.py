@@ -123,7 +123,8 @@ def test_grouped_forward_dispatch_rule():
     name = lambda *a: lib.fm_hash_attn_fwd_kernel(*a).decode()
     assert name(8, 32768, 1048576, 128, 2048, 1) == "hash_attn_wave_kernel"           # 1 M keys, 16 queries / bucket
     assert name(8, 32768, 1048576, 128, 2048, 2) == "hash_attn_wave_kernel<f16>"
-    assert name(8, 32769, 1048576, 128, 2048, 1) == "hash_attn_ring_kernel"           # ... more than 16
+    assert name(8, 24 * 2048, 1048576, 128, 2048, 1) == "hash_attn_wave_kernel"       # ... 24
+    assert name(8, 24 * 2048 + 1, 1048576, 128, 2048, 1) == "hash_attn_ring_kernel"   # ... more than 24
     assert name(1, 32768, 1048576, 128, 2048, 1) == "hash_attn_ring_kernel"           # ... a single row (one launch)
     assert name(8, 16384, 262144, 128, 1024, 1) == "hash_attn_ring_kernel"            # 256 K keys, 16 queries / bucket
     assert name(8, 8192, 262144, 128, 1024, 1) == "hash_attn_ring_kernel"             # ... 8 / bucket: too few buckets per row

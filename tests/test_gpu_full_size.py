@@ -161,6 +161,27 @@ def test_config5_one_million_keys_full_size(ops):
     out, lse = mem.attend(q, scale, q_hash=qh)
     assert bool(torch.isfinite(out.float()).all()) and bool((lse > -1e30).all())      # every bucket is full
     check_attention_sampled(mem, q, qh, out, lse, scale, per_head=8)
+    # The launches of this shape (one per row, a wave per work item) pace their sweeps against the device's
+    # clock, on a schedule the library looks for from call to call: whatever the schedule, the same bits -- and
+    # after 40 calls every row either runs on a schedule faster than its unpaced launch or has stopped pacing.
+    assert ops.hash_attn_fwd_kernel_name(H, G * S, N, d, C, torch.bfloat16) == "hash_attn_wave_kernel"
+    for _ in range(40):
+        o_again, l_again = mem.attend(q, scale, q_hash=qh)
+        assert torch.equal(o_again, out) and torch.equal(l_again, lse)
+    del o_again, l_again
+    lists = mem.attention_lists(G * S)
+    states = [ops.wave_pace_state(N, C, G * S, lists, r) for r in range(H)]
+    print("c5 paced sweeps:", [(st["mode"], round(st["ticks_per_key"], 4), round(st["unpaced"], 4)) for st in states])
+    for st in states:
+        assert st["mode"] in (1, 2) and st["unpaced"] > 0
+        assert st["mode"] == 2 or 0 < st["ticks_per_key"] <= 0.97 * st["unpaced"] + 1e-6
+    ops.grouped_forward_kernel("wave-per-row-unpaced")
+    try:
+        o_un, l_un = mem.attend(q, scale, q_hash=qh)
+    finally:
+        ops.grouped_forward_kernel(None)
+    assert torch.equal(o_un, out) and torch.equal(l_un, lse)
+    del o_un, l_un
     # equivariance: the queries in another order give the same rows
     perm = torch.randperm(q.shape[1], device="cuda")
     o2, l2 = mem.attend(q[:, perm].contiguous(), scale)

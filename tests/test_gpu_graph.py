@@ -115,3 +115,53 @@ def test_build_hash_and_attention_in_one_graph():
     # the deferred check of the Python wrapper: same lists, nothing read back until asked
     idx2, st2 = ops.build_index(A, k, Z, fused=True, defer_check=True)
     assert st2.unresolved() == 0 and torch.equal(idx2, gb["idx"])
+
+
+@pytest.mark.parametrize("eager_first", [True, False])
+def test_paced_per_row_launches_replayed_from_a_graph(eager_first):
+    """The kernel that gives every work item a wave of its own, in one launch per row (forced here on a small
+    memory; dispatch takes it on large ones): each launch is followed by a one-thread kernel that sets the next
+    launch's schedule from this one's duration, and both are recorded.  The schedules live in a table of the
+    library whose address is asked for once per device -- not while a stream is being captured: captured
+    first, the launches go unpaced.  Either way every replay gives the bits of the eager call."""
+    H, S, N, C, Z, d = 5, 700, 9000, 64, 512, 128
+    q, k, v, kh, cnt, qh = make_attn_case(77, H, S, N, C, Z, d, torch.bfloat16, window="all")   # full lists
+    q, k, v = dev(q, k, v)
+    kh, cnt, qh = dev(kh.int(), cnt.int(), qh.int())
+    kh = kh.reshape(H, C, Z).sort(-1).values.reshape(-1).contiguous()      # ascending lists: what the pacing expects
+    scale = d ** -0.5
+    lib = _lib.load()
+
+    def run(out_buf, lse_buf):
+        st = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.fm_attention_hash_varlen_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), kh.data_ptr(),
+                                                       cnt.data_ptr(), qh.data_ptr(), out_buf.data_ptr(),
+                                                       lse_buf.data_ptr(), H, S, N, d, C, scale, 1, st))
+
+    bufs = lambda: (torch.zeros_like(q), torch.zeros(H, S, dtype=torch.float32, device="cuda"))
+    out_e, lse_e = bufs()
+    out_g, lse_g = bufs()
+    ref_out, ref_lse = ops.attention_hash_varlen_i32(q, k, v, kh, cnt, qh, scale)   # (dispatch's kernel; also the
+    torch.cuda.synchronize()                                                       # first use of the static array)
+    ops.grouped_forward_kernel("wave-per-row")
+    try:
+        assert ops.hash_attn_fwd_kernel_name(H, S, N, d, C, torch.bfloat16) == "hash_attn_wave_kernel"
+        if eager_first:
+            run(out_e, lse_e)
+            torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run(out_g, lse_g)
+        for rep in range(5):
+            if rep:
+                q.copy_((torch.randn(H, S, d, generator=gen(90 + rep)) * 0.5).to(torch.bfloat16))
+            graph.replay()
+            torch.cuda.synchronize()
+            run(out_e, lse_e)
+            torch.cuda.synchronize()
+            assert torch.equal(out_g.view(torch.int16), out_e.view(torch.int16)), f"replay {rep}: out differs"
+            assert torch.equal(lse_g.view(torch.int32), lse_e.view(torch.int32)), f"replay {rep}: lse differs"
+            assert float(out_g.float().abs().sum()) > 0
+    finally:
+        ops.grouped_forward_kernel(None)
+    del ref_out, ref_lse

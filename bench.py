@@ -820,7 +820,10 @@ def main():
         roofline["note"] = ("achieved = algorithmic bytes / time is not an HBM rate here: a key row listed in several "
                             "buckets comes from HBM once and from the last-level cache or an L2 for the others "
                             "(reuse_factor = algorithmic / distinct bytes); no_reuse_control is the same kernel where "
-                            "nothing can be re-used")
+                            "nothing can be re-used.  Where the launches pace their sweeps (paced_sweeps) four of five "
+                            "row requests are answered by an L2 and frac, the share of the fabric's rate the remaining "
+                            "misses take, is well below 1: such a launch is bound by the latency of its loads with one "
+                            "tile per wave in flight, not by a rate")
     log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M {'keys/s' if args.config == 'c4' else 'query-heads/s'}"
         f"; attention kernel "
         f"{attn_ms:.2f} ms = {achieved:.0f} GB/s algorithmic ({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak); "

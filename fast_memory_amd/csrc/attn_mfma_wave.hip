@@ -51,8 +51,8 @@ struct WavePaceSlot {
 constexpr int kWavePaceSlots = 1024;
 static __device__ __align__(256) WavePaceSlot g_wave_pace[kWavePaceSlots];
 
-// What the last wave of a launch does with the slot (one lane).  elapsed: ticks since the launch's first wave
-// started; tpk_used: the schedule the launch ran on (0: unpaced).
+// What wave_pace_step_kernel does with the slot.  elapsed: ticks since the launch's first wave started;
+// tpk_used: the schedule the launch ran on (0: unpaced).
 __device__ inline void wave_pace_update(WavePaceSlot* s, unsigned long long key, float elapsed, float tpk_used, int N) {
   const float e = elapsed / float(N);  // ticks per key of this launch
   if (s->key != key) {  // (first use, or another memory's slot: start over)

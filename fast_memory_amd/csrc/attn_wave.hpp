@@ -179,7 +179,7 @@ __device__ __forceinline__ void attend_wave(const bf16_t* __restrict__ Qb, const
       read_rows(0);
       gate();
       issue_tile(0);
-      // two tiles per round, so that the buffers are compile-time constants
+      // two tiles per trip of the loop, so that the buffers are compile-time constants
       for (int t0 = 0; t0 < ntiles; t0 += 2) {
 #pragma unroll
         for (int par = 0; par < 2; ++par) {
@@ -189,7 +189,7 @@ __device__ __forceinline__ void attend_wave(const bf16_t* __restrict__ Qb, const
           if (t + 1 < ntiles) {
             read_rows(t + 1);
             gate();
-            // block b + 1 of the list entries takes the buffer of block b - 1, last read for tile 4 b - 1 (in round 4 b - 2)
+            // block b + 1 of the list entries takes the buffer of block b - 1, last read for tile 4 b - 1 (in iteration 4 b - 2)
             if (par == 0 && (t & 3) == 0 && t > 0 && (t >> 2) + 1 < nblk) issue_ids((t >> 2) + 1);
             issue_tile(1 - par);
           }

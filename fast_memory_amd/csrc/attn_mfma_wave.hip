@@ -21,7 +21,7 @@ extern std::atomic<int> g_force_generic;  // attn_api.hip; 13: a launch per row 
 //   * no schedule yet: the launch runs unpaced; the second such launch (the first on a memory is a cold one)
 //     gives the unpaced duration, and the next launch a schedule of 0.92 x that;
 //   * searching: a kept schedule is followed by one 2 % faster; the first one missed ends the search -- the
-//     slot holds the fastest schedule kept + 4 % (if none was kept: 5 % slower and on with the search);
+//     slot holds the fastest schedule kept + 2 % (if none was kept: 5 % slower and on with the search);
 //   * holding, for 16 launches the first time and twice as long after every search, up to 256: a launch that
 //     misses the held schedule makes it 3 % slower; every 129th launch runs unpaced and renews the unpaced
 //     duration; then the search goes on from the held schedule;
@@ -100,7 +100,7 @@ __device__ inline void wave_pace_update(WavePaceSlot* s, unsigned long long key,
       s->good = tpk_used;
       s->tpk = fmaxf(0.98f * tpk_used, 0.4f * s->base);
     } else if (s->good > 0.f) {
-      s->tpk = 1.04f * s->good;
+      s->tpk = 1.02f * s->good;
       s->held = 1.02f * s->tpk;  // (what a launch on it should take; the launches will tell)
       s->good = 0.f;
       s->hold = s->hold_len;

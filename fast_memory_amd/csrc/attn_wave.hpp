@@ -283,6 +283,12 @@ __device__ __forceinline__ void attend_wave(const bf16_t* __restrict__ Qb, const
       }
     }
   };
+  // A wave with more queries has more to do per tile and sets the pace of its launch: it goes first where it
+  // shares a SIMD with a lighter one.
+  if (n_qt >= 3)
+    __builtin_amdgcn_s_setprio(3);
+  else if (n_qt == 2)
+    __builtin_amdgcn_s_setprio(1);
   if (n_qt <= 1)
     run(std::integral_constant<int, 1>{});
   else if (NQW >= 2 && n_qt == 2)
@@ -291,6 +297,7 @@ __device__ __forceinline__ void attend_wave(const bf16_t* __restrict__ Qb, const
     run(std::integral_constant<int, (NQW >= 3 ? 3 : 1)>{});
   else
     run(std::integral_constant<int, NQW>{});
+  __builtin_amdgcn_s_setprio(0);
 }
 
 }  // namespace fm

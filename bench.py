@@ -224,7 +224,7 @@ def fabric_gather_probe(dev, region_mib=64, passes=64):
     call = lambda: _lib.check(lib.fm_debug_gather(src.data_ptr(), src.numel(), passes, sink.data_ptr(),
                                                   torch.cuda.current_stream().cuda_stream))
     best_ms = min(timed(call, reps=1, warm=1)[0] for _ in range(5))
-    return src.numel() * passes / best_ms / 1e6
+    return max(src.numel(), 32 << 20) * passes / best_ms / 1e6
 
 
 def distinct_rows_per_launch(lists, hit_mask, N):
@@ -808,6 +808,14 @@ def main():
     if traffic is not None:
         roofline["fabric_gbs"] = traffic / avg_launch_ms / 1e6
         roofline["fabric_probe_gbs"] = fabric_gather_probe(dev)
+        # the same gather out of 2 MiB, which every L2 holds: what the path L2 -> compute unit gives scattered rows
+        roofline["l2_gather_probe_gbs"] = fabric_gather_probe(dev, region_mib=2, passes=128)
+        roofline["achieved_over_l2_gather_probe"] = roofline["achieved"] / roofline["l2_gather_probe_gbs"]
+        # every algorithmic byte passes from an L2 into a compute unit, the misses also from the fabric into an L2:
+        # the time the two probes' rates give for a launch's bytes if the two transfers did not overlap at all
+        roofline["two_path_ms"] = (alg_bytes / launches / roofline["l2_gather_probe_gbs"]
+                                   + traffic / roofline["fabric_probe_gbs"]) / 1e6
+        roofline["two_path_over_launch"] = roofline["two_path_ms"] / avg_launch_ms
     if achieved > HBM_PEAK_GBS * 0.8 and traffic is not None:
         # Algorithmic bytes count a bucket's rows once per hit bucket; where every row is listed in many buckets
         # most of those requests are answered by an L2 or by the last-level cache, and algorithmic bytes / time
@@ -823,7 +831,9 @@ def main():
                             "nothing can be re-used.  Where the launches pace their sweeps (paced_sweeps) four of five "
                             "row requests are answered by an L2 and frac, the share of the fabric's rate the remaining "
                             "misses take, is well below 1: such a launch is bound by the latency of its loads with one "
-                            "tile per wave in flight, not by a rate")
+                            "tile per wave in flight, not by a rate (l2_gather_probe_gbs: what the L2s give the same "
+                            "row fetches when every one hits; two_path_ms: the launch's bytes at the two probes' "
+                            "rates, one after the other)")
     log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M {'keys/s' if args.config == 'c4' else 'query-heads/s'}"
         f"; attention kernel "
         f"{attn_ms:.2f} ms = {achieved:.0f} GB/s algorithmic ({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak); "

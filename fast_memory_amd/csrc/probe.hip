@@ -37,7 +37,8 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict
 // region (an odd multiplier modulo a power of two), so no row is read twice in a pass, and the groups move on by
 // 17 places from pass to pass, so the next reader of a row sits behind another L2.  Nothing is written.  From
 // the second pass on every byte comes out of the last-level cache through the fabric into an L2: the rate is
-// what that path sustains for scattered rows.
+// what that path sustains for scattered rows.  With a region that every L2 holds (1 or 2 MiB) the same loads
+// are answered by the L2s: the rate of the path L2 -> compute unit for scattered rows.
 __global__ __launch_bounds__(256) void gather_probe_kernel(const uint4* __restrict__ src, uint32_t region_rows,
                                                            int passes, uint32_t* __restrict__ sink) {
   constexpr int U = 8;
@@ -46,7 +47,9 @@ __global__ __launch_bounds__(256) void gather_probe_kernel(const uint4* __restri
   uint32_t acc = 0;
   for (int pass = 0; pass < passes; ++pass) {
     const uint32_t grp = (grp0 + uint32_t(pass) * 17u) % n_grp;
-    for (uint32_t r = grp; r + (U - 1) * n_grp < region_rows; r += U * n_grp) {
+    // (a region of fewer rows than a sweep of the grid, 2^17, is read 2^17 / region_rows times per pass)
+    const uint32_t sweep_rows = max(region_rows, U * n_grp);
+    for (uint32_t r = grp; r + (U - 1) * n_grp < sweep_rows; r += U * n_grp) {
       uint4 x[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -127,9 +130,9 @@ extern "C" int fm_debug_read(const void* src, int64_t nbytes, void* sink, void* 
 extern "C" int fm_debug_gather(const void* src, int64_t region_bytes, int passes, void* sink, void* stream) {
   using namespace fm;
   const int64_t rows = region_bytes / 256;
-  FM_REQUIRE(src && sink && passes >= 0 && rows >= (1 << 17) && rows <= (int64_t(1) << 31) && (rows & (rows - 1)) == 0 &&
+  FM_REQUIRE(src && sink && passes >= 0 && rows >= (1 << 10) && rows <= (int64_t(1) << 31) && (rows & (rows - 1)) == 0 &&
                  region_bytes % 256 == 0,
-             FM_ERR_ARG, "fm_debug_gather: region_bytes=%lld must be 256 x a power of two >= 2^17, passes=%d",
+             FM_ERR_ARG, "fm_debug_gather: region_bytes=%lld must be 256 x a power of two >= 2^10, passes=%d",
              (long long)region_bytes, passes);
   if (passes == 0) return FM_OK;
   // 1024 workgroups x 16 groups x 8 rows = 2^17 rows per sweep of the grid

@@ -106,9 +106,12 @@ int fm_debug_copy(void* dst, const void* src, int64_t nbytes, void* stream);
  * read bandwidth a kernel reaches on the device. */
 int fm_debug_read(const void* src, int64_t nbytes, void* sink, void* stream);
 
-/* Diagnostic: `passes` sweeps over region_bytes (256 x a power of two >= 2^17) of device memory in which every
+/* Diagnostic: `passes` sweeps over region_bytes (256 x a power of two >= 2^10) of device memory in which every
  * 256-byte row is read exactly once per sweep, in a scattered order, by sixteen lanes with a 16-byte load each
  * (the row fetch of the gathered attention); from one sweep to the next a row's reader moves behind another L2.
+ * (A sweep is 2^17 rows at least: a region of fewer rows is read 2^17 / rows times per sweep, and the bytes a call
+ * reads are passes * max(region_bytes, 32 MiB).  With a region that every L2 holds, 1 or 2 MiB, the rate is that
+ * of the path from an L2 into the compute units for scattered rows.)
  * With a region that the last-level cache holds and an L2 does not (say 64 MiB), the bytes of every sweep after the
  * first come out of the last-level cache: region_bytes * passes / time is the rate the path from that cache into
  * the L2s sustains for scattered rows.  Nothing is written (sink: 4 bytes, left untouched). */

@@ -221,6 +221,14 @@ def test_probe_kernels_run_and_write_nothing(ops):
     _lib.check(lib.fm_debug_read(src.data_ptr(), src.numel(), sink.data_ptr(), st))
     _lib.check(lib.fm_debug_mfma(operands.data_ptr(), operands.numel(), 3, sink.data_ptr(), st))
     _lib.check(lib.fm_debug_mfma(operands.data_ptr(), operands.numel(), 0, sink.data_ptr(), st))
+    # the gather of 256-byte rows: a region every L2 holds (read 2^17 / rows times per sweep), one a sweep
+    # covers exactly, and sizes it does not take
+    big = torch.ones(32 << 20, dtype=torch.uint8, device="cuda")
+    _lib.check(lib.fm_debug_gather(src.data_ptr(), src.numel(), 2, sink.data_ptr(), st))
+    _lib.check(lib.fm_debug_gather(big.data_ptr(), big.numel(), 2, sink.data_ptr(), st))
+    _lib.check(lib.fm_debug_gather(big.data_ptr(), big.numel(), 0, sink.data_ptr(), st))
+    for bad in (256 * 1000, 256 * 512, (1 << 20) + 128):
+        assert lib.fm_debug_gather(big.data_ptr(), bad, 1, sink.data_ptr(), st) != 0
     sync()
     assert sink.tolist() == [0.0, 0.0]
 

@@ -811,11 +811,6 @@ def main():
         # the same gather out of 2 MiB, which every L2 holds: what the path L2 -> compute unit gives scattered rows
         roofline["l2_gather_probe_gbs"] = fabric_gather_probe(dev, region_mib=2, passes=128)
         roofline["achieved_over_l2_gather_probe"] = roofline["achieved"] / roofline["l2_gather_probe_gbs"]
-        # every algorithmic byte passes from an L2 into a compute unit, the misses also from the fabric into an L2:
-        # the time the two probes' rates give for a launch's bytes if the two transfers did not overlap at all
-        roofline["two_path_ms"] = (alg_bytes / launches / roofline["l2_gather_probe_gbs"]
-                                   + traffic / roofline["fabric_probe_gbs"]) / 1e6
-        roofline["two_path_over_launch"] = roofline["two_path_ms"] / avg_launch_ms
     if achieved > HBM_PEAK_GBS * 0.8 and traffic is not None:
         # Algorithmic bytes count a bucket's rows once per hit bucket; where every row is listed in many buckets
         # most of those requests are answered by an L2 or by the last-level cache, and algorithmic bytes / time
@@ -832,8 +827,8 @@ def main():
                             "row requests are answered by an L2 and frac, the share of the fabric's rate the remaining "
                             "misses take, is well below 1: such a launch is bound by the latency of its loads with one "
                             "tile per wave in flight, not by a rate (l2_gather_probe_gbs: what the L2s give the same "
-                            "row fetches when every one hits; two_path_ms: the launch's bytes at the two probes' "
-                            "rates, one after the other)")
+                            "row fetches when every one hits).  traffic is the average over a step's launches, "
+                            "paced or not")
     log(f"[bench] step {ms_per_step:.2f} ms -> {value / 1e6:.2f} M {'keys/s' if args.config == 'c4' else 'query-heads/s'}"
         f"; attention kernel "
         f"{attn_ms:.2f} ms = {achieved:.0f} GB/s algorithmic ({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak); "

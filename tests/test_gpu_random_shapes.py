@@ -353,3 +353,40 @@ def test_forced_forward_kernels_against_generic_and_themselves_random_extents(wh
     assert torch.equal(l1 < -1e30, empty)
     assert torch.allclose(o1.float(), o2.float(), atol=2e-2, rtol=1e-2)
     assert (l1[~empty] - l2[~empty]).abs().max().item() < 1e-3 if (~empty).any() else True
+
+
+@pytest.mark.parametrize("C,S", [(1025, 5000), (1500, 9000), (2048, 40000), (2600, 12000), (4200, 30000)])
+def test_wave_per_row_takes_every_item_once_in_the_paired_order(C, S):
+    """Rows of more than 1024 work items: a launch of the wave-per-item kernel takes them in an order of its own
+    (heavy and light items paired), chunk by chunk of 2048 slots -- a last chunk of any length, items of one to
+    four tiles of queries and items swept twice.  Against the generic kernel, and bit for bit against the
+    single launch over all rows, which takes the items in the order they come."""
+    from fast_memory_amd import attention_hash_varlen, ops
+    B, N, Z = 2, 4096, 48
+    g = torch.Generator(device="cuda").manual_seed(C * 7 + S)
+    mk = lambda *s: (torch.randn(*s, generator=g, device="cuda") * 0.6).to(torch.bfloat16)
+    q, k, v = mk(B, S, 128), mk(B, N, 128), mk(B, N, 128)
+    lists = torch.randint(0, N, (B, C, Z), generator=g, device="cuda", dtype=torch.int32).sort(-1).values
+    cnt = torch.randint(1, Z + 1, (B, C), generator=g, device="cuda", dtype=torch.int32)
+    keep = torch.arange(Z, device="cuda")[None, None, :] < cnt[..., None]
+    flat = lists[keep].contiguous()
+    qh = torch.randint(0, C, (B, S), generator=g, device="cuda", dtype=torch.int32)
+    qh[0, : S // 8] = 3                                            # a bucket of many items
+    qh[1, : 60] = C - 1                                            # one of 60 queries: swept twice
+    run = lambda: attention_hash_varlen(q, k, v, flat, cnt, qh, 128 ** -0.5, lse_dtype=torch.float32)
+    outs = {}
+    for which in ("wave-per-row", "wave"):
+        ops.grouped_forward_kernel(which)
+        try:
+            outs[which] = run()
+        finally:
+            ops.grouped_forward_kernel(None)
+    assert torch.equal(outs["wave-per-row"][0], outs["wave"][0]) and torch.equal(outs["wave-per-row"][1], outs["wave"][1])
+    ops.force_generic_kernels(True)
+    try:
+        o2, l2 = run()
+    finally:
+        ops.force_generic_kernels(False)
+    o1, l1 = outs["wave-per-row"]
+    assert torch.allclose(o1.float(), o2.float(), atol=2e-2, rtol=1e-2)
+    assert (l1 - l2).abs().max().item() < 1e-3

@@ -163,14 +163,16 @@ int fm_group_queries(const int32_t* q_hash, int H, int C, int Sq, int32_t* q_per
  * that is part of no item (hash outside [0, C), see fm_group_queries).
  * On large memories (bf16 / fp16, d = 128, K and V of all rows 512 MB or more, rows
  * of 2048 or more buckets that receive 24 queries or fewer each) the call is one
- * launch per row whose waves sweep the row's key range on a common schedule against
- * the device's clock (lists in ascending key order are what this is for: see
- * fm_lists_key_order).  The library looks for the fastest schedule such a launch
- * keeps from call to call, per (N, C, Sq, k_idx, row), in a table of its own in
- * device memory (64 KB per GPU, no allocation; its address is asked for at the first
- * such call outside stream capture -- calls captured before that run unpaced); the
- * first calls on a memory are slower than the settled ones (about 15).  Results do
- * not depend on the schedule: the same bits paced and unpaced. */
+ * launch per row, which takes the row's work items in an order of its own (heavy
+ * and light ones paired) and whose waves may sweep the row's key range on a common
+ * schedule against the device's clock (lists in ascending key order are what this is
+ * for: see fm_lists_key_order).  The library looks for the fastest schedule such a
+ * launch keeps from call to call, per (N, C, Sq, k_idx, row), in a table of its own
+ * in device memory (64 KB per GPU, no allocation; its address is asked for at the
+ * first such call outside stream capture -- calls captured before that run unpaced),
+ * and holds it only while it is faster than the launch left to itself; the first
+ * calls on a memory can be slower than the settled ones (about 15).  Results do not
+ * depend on the schedule or the order: the same bits paced and unpaced. */
 int fm_hash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* k_idx,
                      const int64_t* bucket_off, const int32_t* bucket_cnt, const int32_t* q_perm,
                      const fm_item* items, const int32_t* n_items, int64_t max_items, void* out,
